@@ -1,0 +1,202 @@
+/*
+ * skainet_hip.h -- C ABI of libskainet_hip.so, the MI355X (gfx950) kernel library behind SKaiNET's
+ * kernel SPI (skainet-backend-api). Plain pointers and sizes only; a JVM binds it through Panama FFM
+ * or JNI exactly as it binds the reference's libskainet_kernels.
+ *
+ * Two families of entry points:
+ *
+ *  1. Host-pointer entries with the reference's own signatures (names `skainet_hip_<ref name>`): every
+ *     pointer is host memory, the call stages operands to the device, runs, copies the result back
+ *     and returns when `output` is complete. They return void like the functions they replace: each
+ *     clears the thread's error text on entry, and on a failure nothing is written and
+ *     skainet_hip_last_error() tells why. Non-positive dimensions
+ *     are no-ops, as in the reference.
+ *
+ *  2. Device entries (`*_dev`, weight handles): operands are device pointers owned by the caller (or by
+ *     this library's allocator), launches are asynchronous on the calling thread's stream
+ *     (skainet_hip_set_stream, default: the null stream) and return 0 / -1.
+ *
+ * Reference paths below are relative to
+ *   REF = /root/reference/skainet-backends
+ *   NAT = REF/skainet-backend-native-cpu/native/include/skainet_kernels.h
+ *   API = REF/skainet-backend-api/src/commonMain/kotlin/sk/ainet/backend/api/kernel
+ *
+ * Threading: every entry point may be called from any thread. Error text, the current stream and
+ * staging buffers are per thread; a weight handle may be shared by threads once uploaded.
+ */
+#ifndef SKAINET_HIP_H
+#define SKAINET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SKAINET_HIP_API __attribute__((visibility("default")))
+
+/* Weight encodings: the GGML tensor-type ids StreamingGGUFReader maps to TensorEncoding
+ * (REF/../skainet-io/skainet-io-gguf/src/commonMain/kotlin/sk/ainet/io/gguf/StreamingGGUFReader.kt:190-211). */
+#define SKAINET_HIP_ENC_Q8_0 8
+#define SKAINET_HIP_ENC_Q4_K 12
+#define SKAINET_HIP_ENC_Q6_K 14
+
+/* Block orders of a packed weight (REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/memory/Layout.kt:21-27). */
+#define SKAINET_HIP_ORDER_ROW_MAJOR 0         /* canonical GGUF order: block (o, b) at (o * blocksPerRow + b) */
+#define SKAINET_HIP_ORDER_INPUT_BLOCK_MAJOR 1 /* kernel feed order: block (b, o) at (b * rows + o) */
+
+/* ------------------------------------------------------------------------------------------------
+ * Runtime. Replaces what NativeLibraryLoader / KernelProvider.isAvailable() probe on the CPU side
+ * (REF/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/NativeKernelProvider.kt:98-150):
+ * "unavailable" is an answer, never a crash.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* 1 when a gfx950 device is present and usable, else 0. Cheap after the first call; never aborts. */
+SKAINET_HIP_API int32_t skainet_hip_available(void);
+/* Select the device (default 0) for this process. 0 on success. */
+SKAINET_HIP_API int32_t skainet_hip_init(int32_t device);
+/* Message of the calling thread's last failed call ("" when none). Valid until that thread's next failure. */
+SKAINET_HIP_API const char* skainet_hip_last_error(void);
+/* Device name ("" when unavailable) and compute-unit count. */
+SKAINET_HIP_API const char* skainet_hip_device_name(void);
+SKAINET_HIP_API int32_t skainet_hip_compute_units(void);
+/* Stream (a hipStream_t, NULL = the null stream) used by this thread's later device entries. */
+SKAINET_HIP_API int32_t skainet_hip_set_stream(void* stream);
+/* Wait for this thread's stream. */
+SKAINET_HIP_API int32_t skainet_hip_sync(void);
+
+/* Device buffers: the backing store of a Storage.Device
+ * (REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/memory/Storage.kt:230). */
+SKAINET_HIP_API void* skainet_hip_malloc(size_t bytes);
+SKAINET_HIP_API int32_t skainet_hip_free(void* device_ptr);
+SKAINET_HIP_API int32_t skainet_hip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
+SKAINET_HIP_API int32_t skainet_hip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
+SKAINET_HIP_API int32_t skainet_hip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes);
+
+/* Elapsed-time measurement on the calling thread's stream (HIP events): begin, launch, end -> milliseconds. */
+SKAINET_HIP_API int32_t skainet_hip_timer_begin(void);
+SKAINET_HIP_API float skainet_hip_timer_end_ms(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Packed weights resident on the device. The device-side analogue of the weight caches keyed by array
+ * identity (WASM sidecar handles, REF/skainet-backend-wasm-simd/src/wasmJsMain/kotlin/sk/ainet/exec/wasm/WasmKernels.kt:206-223):
+ * upload once, multiply many times.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct skainet_hip_weight skainet_hip_weight;
+
+/* Copy `nbytes` packed bytes of a [rows, cols] weight to the device. `order` says how the host bytes are
+ * laid out; the device copy is always canonical row-major (an input-block-major source is permuted on
+ * the device, the inverse of API/PackedWeights.kt:63-93 toKernelOrder). NULL on failure. */
+SKAINET_HIP_API skainet_hip_weight* skainet_hip_weight_upload(
+    const uint8_t* bytes, int64_t nbytes, int32_t encoding, int32_t order, int32_t rows, int32_t cols);
+/* Describe packed row-major bytes that already live on the device (not owned, not freed). */
+SKAINET_HIP_API skainet_hip_weight* skainet_hip_weight_wrap(
+    const void* device_bytes, int32_t encoding, int32_t rows, int32_t cols);
+SKAINET_HIP_API void skainet_hip_weight_free(skainet_hip_weight* w);
+SKAINET_HIP_API const void* skainet_hip_weight_data(const skainet_hip_weight* w);
+SKAINET_HIP_API int64_t skainet_hip_weight_nbytes(const skainet_hip_weight* w);
+
+/* out[m, rows] = x[m, cols] . W^T, fp32 in and out, device pointers. What a ViewKernel registered for
+ * matmul(F32 dense x packed BLOCKED_ROW_MAJOR) runs (API/MatmulKernels.kt:11-40; CPU twin
+ * REF/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/FfmRowMajorKernels.kt:52-106).
+ * m <= 8 streams the weight once per 4 rows (GEMV kernels, fp32 arithmetic); larger m uses the MFMA
+ * dequant-GEMM (bf16 operands, fp32 accumulation). */
+SKAINET_HIP_API int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out);
+/* Same product, forcing one of the two kernels (kind 0 = GEMV path, 1 = MFMA GEMM path). */
+SKAINET_HIP_API int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out, int32_t kind);
+/* Measurement aid: `iters` such products back to back on this thread's stream, weight number i % nweights at
+ * step i, timed with HIP events; returns the elapsed milliseconds (< 0 on failure). use_graph != 0 captures the
+ * launches into a HIP graph first and times one replay, so host launch cost stays off the GPU timeline.
+ * (The reference times its kernels the same way, in a loop around the call: NativeKernel microbench,
+ * REF/skainet-backend-native-cpu/src/jvmTest/kotlin/sk/ainet/exec/kernel/Q4KMatmulMicrobenchTest.kt:53-70.) */
+SKAINET_HIP_API float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, int32_t nweights,
+    const float* x, int32_t m, float* out, int32_t iters, int32_t kind, int32_t use_graph);
+/* Bit-exact decode of the whole weight to fp32 [rows, cols] (the TensorData.dequantizeBlock semantics,
+ * REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/data/Q4_KTensorData.kt:120,
+ * Q6_KTensorData.kt:112, Q8_0TensorData.kt:80). */
+SKAINET_HIP_API int32_t skainet_hip_dequantize_dev(const skainet_hip_weight* w, float* out);
+/* Decode `count` rows picked by `row_ids` (device int32) into out[count, cols]: the packed embedding
+ * lookup (RowDequantSource.dequantRow, .../tensor/data/Q8_0TensorData.kt:91-100). */
+SKAINET_HIP_API int32_t skainet_hip_dequantize_rows_dev(const skainet_hip_weight* w, const int32_t* row_ids, int32_t count, float* out);
+
+/* ------------------------------------------------------------------------------------------------
+ * Host-pointer entries with the reference's signatures.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* NAT:57 skainet_q4k_matmul / NAT:80 skainet_q4k_matmul_rm (Q4KMatmulKernel.matmul, API/Q4KMatmulKernel.kt:54-59).
+ * The plain name takes the SPI's input-block-major weight, `_rm` the canonical GGUF order. */
+SKAINET_HIP_API void skainet_hip_q4k_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q4k_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+/* NAT:135 / NAT:157 (Q6KMatmulKernel.matmul, API/Q6KMatmulKernel.kt:34). */
+SKAINET_HIP_API void skainet_hip_q6k_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q6k_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+/* NAT:327 / NAT:179 (Q8_0MatmulKernel.matmul, API/Q8_0MatmulKernel.kt:42). */
+SKAINET_HIP_API void skainet_hip_q8_0_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q8_0_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+
+/* NAT:271 skainet_fp32_matmul (Fp32MatmulKernel.matmul, API/Fp32MatmulKernel.kt:25-50): C(m,n) = A(m,k) B(k,n),
+ * strides in floats, full overwrite; k == 0 zeroes C. */
+SKAINET_HIP_API void skainet_hip_fp32_matmul(const float* a, int32_t a_offset, int32_t a_stride,
+    const float* b, int32_t b_offset, int32_t b_stride, float* c, int32_t c_offset, int32_t c_stride,
+    int32_t m, int32_t n, int32_t k);
+/* NAT:510 skainet_fp32_matmul_wt (Fp32MatmulWtKernel, API/Fp32MatmulWtKernel.kt:21-28): out[i,o] = sum_p in[i,p] w[o,p]. */
+SKAINET_HIP_API void skainet_hip_fp32_matmul_wt(const float* in, int32_t in_offset, const float* w, int32_t w_offset,
+    float* out, int32_t out_offset, int32_t m, int32_t n, int32_t k);
+
+/* NAT:573 skainet_f32_rms_norm (Fp32NormKernel.rmsNorm, API/Fp32FusedKernels.kt:37-53); gamma may be NULL. */
+SKAINET_HIP_API void skainet_hip_f32_rms_norm(const float* in, const float* gamma, float* out,
+    int32_t rows, int32_t cols, float eps);
+/* NAT:568 skainet_f32_layer_norm (Fp32NormKernel.layerNorm, API/Fp32FusedKernels.kt:37-53); gamma / beta may be NULL. */
+SKAINET_HIP_API void skainet_hip_f32_layer_norm(const float* in, const float* gamma, const float* beta, float* out,
+    int32_t rows, int32_t cols, float eps);
+/* NAT:566 skainet_f32_softmax_rows (Fp32SoftmaxKernel, API/Fp32FusedKernels.kt:15-35). */
+SKAINET_HIP_API void skainet_hip_f32_softmax_rows(const float* in, float* out, int32_t rows, int32_t cols, int32_t log_form);
+/* NAT:577-584 skainet_f32_sdpa (Fp32AttentionKernel.sdpa, API/Fp32FusedKernels.kt:54-85). */
+SKAINET_HIP_API void skainet_hip_f32_sdpa(const float* q, const float* k, const float* v, float* out,
+    int32_t batch, int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t head_dim,
+    float scale, int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths,
+    const float* mask, int32_t mask_b, int32_t mask_h, int32_t mask_q, int32_t mask_k);
+
+/* ------------------------------------------------------------------------------------------------
+ * Device entries of the same kernels (all pointers on the device, asynchronous, 0 / -1).
+ * ---------------------------------------------------------------------------------------------- */
+SKAINET_HIP_API int32_t skainet_hip_fp32_matmul_dev(const float* a, int32_t a_offset, int32_t a_stride,
+    const float* b, int32_t b_offset, int32_t b_stride, float* c, int32_t c_offset, int32_t c_stride,
+    int32_t m, int32_t n, int32_t k);
+SKAINET_HIP_API int32_t skainet_hip_fp32_matmul_wt_dev(const float* in, int32_t in_offset, const float* w, int32_t w_offset,
+    float* out, int32_t out_offset, int32_t m, int32_t n, int32_t k);
+SKAINET_HIP_API int32_t skainet_hip_f32_rms_norm_dev(const float* in, const float* gamma, float* out,
+    int32_t rows, int32_t cols, float eps);
+SKAINET_HIP_API int32_t skainet_hip_f32_layer_norm_dev(const float* in, const float* gamma, const float* beta, float* out,
+    int32_t rows, int32_t cols, float eps);
+SKAINET_HIP_API int32_t skainet_hip_f32_softmax_rows_dev(const float* in, float* out, int32_t rows, int32_t cols, int32_t log_form);
+SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_dev(const float* q, const float* k, const float* v, float* out,
+    int32_t batch, int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t head_dim,
+    float scale, int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths,
+    const float* mask, int32_t mask_b, int32_t mask_h, int32_t mask_q, int32_t mask_k);
+
+/* Decoder glue with the reference ops' semantics (device pointers):
+ *   silu_mul: out[i] = gate[i] * (1 / (1 + exp(-gate[i]))) * up[i]   (NAT:532-539 unary op 2 then binary mul,
+ *             REF/skainet-backend-native-cpu/native/src/f32_ops.c:222-244)
+ *   add:      out[i] = a[i] + b[i]                                  (NAT:532 binary op 0)
+ *   argmax:   index of the first maximum of each row, int32          (TensorOps.argMax ties -> lowest index,
+ *             REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/ops/TensorOps.kt:263-277) */
+SKAINET_HIP_API int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* out, int64_t n);
+SKAINET_HIP_API int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int64_t n);
+SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
+
+/* Tuning knob for experiments: resident GEMV waves per compute unit used to size the row shares (default 8). */
+SKAINET_HIP_API void skainet_hip_set_gemv_waves_per_cu(int32_t waves);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SKAINET_HIP_H */

@@ -1,0 +1,354 @@
+// Decode-time dequant-GEMV for GGUF Q4_K / Q6_K / Q8_0 weights in canonical row-major block order:
+//   y[b, o] = sum_j x[b, j] * dequant(W[o, j])     b < batch <= 4 per launch, fp32 activations and sums.
+//
+// Semantics follow the reference's exact-fp32 kernels (same products, different summation order):
+//   /root/reference/skainet-backends/skainet-backend-cpu/src/commonMain/kotlin/sk/ainet/exec/kernel/
+//   ScalarQ4_KMatmulKernel.kt:40-78, ScalarQ6_KMatmulKernel.kt:33-44, ScalarQ8_0MatmulKernel.kt:41-62
+// and the row-major weight addressing of the native entries
+//   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/q4k_matmul.c:294-309.
+//
+// Mapping (HBM-bound, one pass over the weight, nothing staged in LDS):
+//   * A weight row is cut into "slots" of SLOT_ELEMS consecutive-in-memory quants (Q4_K: one 16-byte
+//     nibble chunk = 16 + 16 elements of two sub-blocks; Q6_K: 4 x 4 elements sharing 12 code bytes;
+//     Q8_0: one 34-byte block). Lane l of wave s in a workgroup owns slot s * 64 + l of EVERY row the
+//     workgroup processes, so the activation slice that slot needs lives in registers for the whole
+//     kernel and each wave-wide load instruction covers one contiguous span of the row.
+//   * Rows are streamed R at a time with all loads issued before the arithmetic; the R * B per-lane
+//     partial sums are folded across the wave with a multi-value butterfly (log2(R*B) halving steps,
+//     then plain xor-shuffles), written to LDS per (wave, row) and summed over the waves in a fixed
+//     order, so results are deterministic.
+//   * Grid: contiguous row ranges, sized so the whole chip gets an even share (rows_per_wg from the host).
+#include "common.h"
+
+namespace skh {
+
+constexpr int GEMV_MAX_WAVES = 8;    // waves per workgroup = K segments processed concurrently (2 per SIMD: 256 VGPRs each)
+constexpr int GEMV_MAX_ROWS = 64;    // rows per workgroup (bounds the LDS partial-sum buffer)
+
+// ---------------------------------------------------------------------------------------------- Q4_K
+struct Q4KSlot {
+    static constexpr int BLOCK_BYTES = Q4K_BYTES, SLOTS_PER_BLOCK = 8, SLOT_ELEMS = 32, NX = 32;
+    struct Raw { uint4 hdr, qs; };
+    struct Lane {
+        int blk_off, qs_off;   // byte offsets inside a row
+        int g;                 // 32-byte nibble group of this slot (sub-blocks 2g and 2g + 1)
+    };
+    __device__ static void init(Lane& ln, int slot) {
+        const int blk = slot >> 3, c = slot & 7;
+        ln.blk_off = blk * BLOCK_BYTES;
+        ln.qs_off = ln.blk_off + 16 + c * 16;
+        ln.g = c >> 1;
+    }
+    // Element index (inside the row) of activation register i for this slot: 16 of sub-block 2g then 16 of 2g+1.
+    __device__ static int x_index(int slot, int i) {
+        const int blk = slot >> 3, c = slot & 7;
+        return blk * 256 + (c >> 1) * 64 + (c & 1) * 16 + (i >> 4) * 32 + (i & 15);
+    }
+    __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
+        r.hdr = *reinterpret_cast<const uint4*>(row + ln.blk_off);
+        r.qs = *reinterpret_cast<const uint4*>(row + ln.qs_off);
+    }
+    // xsum[0] = sum of the 16 low-nibble activations, xsum[1] = sum of the 16 high-nibble activations.
+    __device__ static void prep(const float* x, float* xsum) {
+        float a = 0.f, b = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { a += x[i]; b += x[16 + i]; }
+        xsum[0] = a; xsum[1] = b;
+    }
+    struct Scales { float dlo, dhi, mlo, mhi; };
+    // The 6-bit (scale, min) pairs of sub-blocks 2g and 2g+1 (ggml get_scale_min_k4), folded with d / dmin.
+    __device__ static Scales scales(const Raw& r, const Lane& ln) {
+        const float d = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
+        const int sh = (ln.g & 1) * 16;
+        const uint32_t u = (r.hdr.y >> sh) & 0xFFFFu;   // scale bytes s[2g'], s[2g'+1]
+        const uint32_t v = (r.hdr.z >> sh) & 0xFFFFu;   // scale bytes s[4+2g'], s[5+2g']
+        const uint32_t t = (r.hdr.w >> sh) & 0xFFFFu;   // scale bytes s[8+2g'], s[9+2g']
+        uint32_t sc, mn;
+        if (ln.g < 2) {
+            sc = u & 0x3F3Fu;
+            mn = v & 0x3F3Fu;
+        } else {
+            sc = (t & 0x0F0Fu) | ((u >> 2) & 0x3030u);
+            mn = ((t >> 4) & 0x0F0Fu) | ((v >> 2) & 0x3030u);
+        }
+        Scales s;
+        s.dlo = d * (float)(sc & 0xFFu);
+        s.dhi = d * (float)(sc >> 8) * 0.0625f;   // high nibbles are accumulated as 16 * code
+        s.mlo = dmin * (float)(mn & 0xFFu);
+        s.mhi = dmin * (float)(mn >> 8);
+        return s;
+    }
+    template <int B>
+    __device__ static void dot(const Raw& r, const Lane& ln, const float (*x)[NX], const float (*xsum)[2], float* acc) {
+        const Scales s = scales(r, ln);
+        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+        float lo[B], hi[B];
+#pragma unroll
+        for (int b = 0; b < B; ++b) lo[b] = hi[b] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t l4 = q[i] & 0x0F0F0F0Fu, h4 = q[i] & 0xF0F0F0F0u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float cl = (float)((l4 >> (8 * j)) & 0xFFu), ch = (float)((h4 >> (8 * j)) & 0xFFu);
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    lo[b] = fmaf(x[b][i * 4 + j], cl, lo[b]);
+                    hi[b] = fmaf(x[b][16 + i * 4 + j], ch, hi[b]);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b)
+            acc[b] = s.dlo * lo[b] + s.dhi * hi[b] - (s.mlo * xsum[b][0] + s.mhi * xsum[b][1]);
+    }
+};
+
+// ---------------------------------------------------------------------------------------------- Q6_K
+struct Q6KSlot {
+    static constexpr int BLOCK_BYTES = Q6K_BYTES, SLOTS_PER_BLOCK = 16, SLOT_ELEMS = 16, NX = 16;
+    struct Raw { uint32_t qla, qlb, qh, sc0, sc1, d; };
+    struct Lane { int blk_off, ql_off, qh_off, sc_off, sc_shift; };
+    __device__ static void init(Lane& ln, int slot) {
+        const int blk = slot >> 4, t = slot & 15, half = t >> 3, l0 = (t & 7) * 4;
+        ln.blk_off = blk * BLOCK_BYTES;
+        ln.ql_off = ln.blk_off + half * 64 + l0;
+        ln.qh_off = ln.blk_off + 128 + half * 32 + l0;
+        ln.sc_off = ln.blk_off + 192 + half * 8;
+        ln.sc_shift = (l0 >> 4) * 8;
+    }
+    // Register i = 4 * k + j pairs with element half*128 + 32*k + l0 + j.
+    __device__ static int x_index(int slot, int i) {
+        const int blk = slot >> 4, t = slot & 15, half = t >> 3, l0 = (t & 7) * 4;
+        return blk * 256 + half * 128 + (i >> 2) * 32 + l0 + (i & 3);
+    }
+    __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
+        r.qla = load_u32_a2(row + ln.ql_off);
+        r.qlb = load_u32_a2(row + ln.ql_off + 32);
+        r.qh = load_u32_a2(row + ln.qh_off);
+        r.sc0 = load_u32_a2(row + ln.sc_off);
+        r.sc1 = load_u32_a2(row + ln.sc_off + 4);
+        r.d = load_u16(row + ln.blk_off + 208);
+    }
+    __device__ static void prep(const float* x, float* xsum) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) xsum[k] = 32.f * (x[4 * k] + x[4 * k + 1] + x[4 * k + 2] + x[4 * k + 3]);
+    }
+    template <int B>
+    __device__ static void dot(const Raw& r, const Lane& ln, const float (*x)[NX], const float (*xsum)[4], float* acc) {
+        const float d = half_bits_to_float(r.d);
+        // signed scales of the four quarters: bytes is, is+2, is+4, is+6 of the half's 8 scale bytes
+        const uint32_t s0 = r.sc0 >> ln.sc_shift, s1 = r.sc1 >> ln.sc_shift;
+        const float sc[4] = {d * (float)(int8_t)(s0), d * (float)(int8_t)(s0 >> 16),
+                             d * (float)(int8_t)(s1), d * (float)(int8_t)(s1 >> 16)};
+        const uint32_t c[4] = {
+            (r.qla & 0x0F0F0F0Fu) | ((r.qh << 4) & 0x30303030u),
+            (r.qlb & 0x0F0F0F0Fu) | ((r.qh << 2) & 0x30303030u),
+            ((r.qla >> 4) & 0x0F0F0F0Fu) | (r.qh & 0x30303030u),
+            ((r.qlb >> 4) & 0x0F0F0F0Fu) | ((r.qh >> 2) & 0x30303030u)};
+#pragma unroll
+        for (int b = 0; b < B; ++b) acc[b] = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float s[B];
+#pragma unroll
+            for (int b = 0; b < B; ++b) s[b] = -xsum[b][k];   // the -32 bias of every code, taken out of the loop
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float cf = (float)((c[k] >> (8 * j)) & 0xFFu);
+#pragma unroll
+                for (int b = 0; b < B; ++b) s[b] = fmaf(x[b][4 * k + j], cf, s[b]);
+            }
+#pragma unroll
+            for (int b = 0; b < B; ++b) acc[b] = fmaf(sc[k], s[b], acc[b]);
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------- Q8_0
+struct Q80Slot {
+    static constexpr int BLOCK_BYTES = Q80_BYTES, SLOTS_PER_BLOCK = 1, SLOT_ELEMS = 32, NX = 32;
+    struct Raw { uint32_t d; uint32_t q[8]; };
+    struct Lane { int blk_off; };
+    __device__ static void init(Lane& ln, int slot) { ln.blk_off = slot * BLOCK_BYTES; }
+    __device__ static int x_index(int slot, int i) { return slot * 32 + i; }
+    __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
+        const uint8_t* p = row + ln.blk_off;
+        r.d = load_u16(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r.q[i] = load_u32_a2(p + 2 + 4 * i);
+    }
+    __device__ static void prep(const float*, float*) {}
+    template <int B>
+    __device__ static void dot(const Raw& r, const Lane&, const float (*x)[NX], const float (*)[1], float* acc) {
+        const float d = half_bits_to_float(r.d);
+        float s[B];
+#pragma unroll
+        for (int b = 0; b < B; ++b) s[b] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float cf = (float)(int8_t)(r.q[i] >> (8 * j));
+#pragma unroll
+                for (int b = 0; b < B; ++b) s[b] = fmaf(x[b][i * 4 + j], cf, s[b]);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b) acc[b] = s[b] * d;
+    }
+};
+
+template <class F> struct XSumCount { static constexpr int N = 1; };
+template <> struct XSumCount<Q4KSlot> { static constexpr int N = 2; };
+template <> struct XSumCount<Q6KSlot> { static constexpr int N = 4; };
+
+// Fold NV per-lane values across the 64 lanes. On return v[0] of lane l holds the wave total of value
+// index bitrev(l & (NV-1)) over log2(NV) bits (see gemv_value_of_lane).
+template <int NV>
+__device__ __forceinline__ void wave_fold(float* v, int lane) {
+    int mask = 1;
+#pragma unroll
+    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) {
+        const int half = nv >> 1;
+        const bool upper = (lane & mask) != 0;
+#pragma unroll
+        for (int i = 0; i < half; ++i) {
+            const float send = upper ? v[i] : v[i + half];
+            const float keep = upper ? v[i + half] : v[i];
+            v[i] = keep + __shfl_xor(send, mask, 64);
+        }
+    }
+#pragma unroll
+    for (int m = NV; m < 64; m <<= 1) v[0] += __shfl_xor(v[0], m, 64);
+}
+template <int NV>
+__device__ __forceinline__ int gemv_value_of_lane(int lane) {
+    int idx = 0, mask = 1;
+#pragma unroll
+    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) idx += (lane & mask) ? (nv >> 1) : 0;
+    return idx;
+}
+
+// F: slot policy, B: activation rows per launch (1, 2 or 4; unused ones are zero), R: weight rows in flight.
+template <class F, int B, int R>
+__global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
+    const uint8_t* __restrict__ w, const float* __restrict__ x, float* __restrict__ y,
+    int k, int n, int batch, int64_t row_bytes, int rows_per_wg) {
+    constexpr int NX = F::NX, NS = XSumCount<F>::N, NV = R * B;
+    __shared__ float partial[GEMV_MAX_WAVES][GEMV_MAX_ROWS][B];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int nslots = k / F::SLOT_ELEMS;
+    const int nseg = (nslots + 63) >> 6;
+    const int r0 = blockIdx.x * rows_per_wg;
+    const int r1 = min(n, r0 + rows_per_wg);
+    const int nrows = r1 - r0;
+    if (nrows <= 0) return;
+    const uint8_t* wbase = w + (int64_t)r0 * row_bytes;
+    const int my_value = gemv_value_of_lane<NV>(lane);
+
+    for (int seg = wave, pass = 0; seg < nseg; seg += nwaves, ++pass) {
+        const int slot = seg * 64 + lane;
+        const bool active = slot < nslots;
+        typename F::Lane ln;
+        F::init(ln, active ? slot : 0);
+
+        // First rows' weight loads are issued before the activation slice is fetched.
+        typename F::Raw raw[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) F::load(raw[i], wbase + (int64_t)min(i, nrows - 1) * row_bytes, ln);
+
+        float xs[B][NX], xsum[B][NS];
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const bool have = active && b < batch;
+#pragma unroll
+            for (int i = 0; i < NX; i += 4) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (have) v = *reinterpret_cast<const float4*>(x + (int64_t)b * k + F::x_index(slot, i));
+                xs[b][i] = v.x; xs[b][i + 1] = v.y; xs[b][i + 2] = v.z; xs[b][i + 3] = v.w;
+            }
+            F::prep(xs[b], xsum[b]);
+        }
+
+        for (int r = 0; r < nrows; r += R) {
+            float acc[NV];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                float a[B];
+                F::template dot<B>(raw[i], ln, xs, xsum, a);
+#pragma unroll
+                for (int b = 0; b < B; ++b) acc[i * B + b] = active ? a[b] : 0.f;
+                // refill this register set with the row R ahead (clamped: a repeated last row is discarded)
+                F::load(raw[i], wbase + (int64_t)min(r + R + i, nrows - 1) * row_bytes, ln);
+            }
+            wave_fold<NV>(acc, lane);
+            if (lane < NV) {
+                const int i = my_value / B, b = my_value % B;
+                if (r + i < nrows) {
+                    float* dst = &partial[wave][r + i][b];
+                    *dst = pass == 0 ? acc[0] : *dst + acc[0];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int used_waves = min(nwaves, nseg);
+    for (int t = threadIdx.x; t < nrows * B; t += blockDim.x) {
+        const int rr = t / B, b = t % B;
+        if (b >= batch) continue;
+        float s = 0.f;
+        for (int wv = 0; wv < used_waves; ++wv) s += partial[wv][rr][b];
+        y[(int64_t)b * n + r0 + rr] = s;
+    }
+}
+
+template <class F, int B, int R>
+static int launch_one(const uint8_t* w, const float* x, float* y, int k, int n, int batch, int waves_per_cu) {
+    const int nslots = k / F::SLOT_ELEMS;
+    const int nseg = (nslots + 63) / 64;
+    const int nwaves = nseg < GEMV_MAX_WAVES ? nseg : GEMV_MAX_WAVES;
+    const int64_t row_bytes = (int64_t)(k / (F::SLOT_ELEMS * F::SLOTS_PER_BLOCK)) * F::BLOCK_BYTES;
+    // Even contiguous row shares: about waves_per_cu resident waves on every CU.
+    int target_wgs = (num_cus() * waves_per_cu) / nwaves;
+    if (target_wgs < 1) target_wgs = 1;
+    int rows_per_wg = (n + target_wgs - 1) / target_wgs;
+    if (rows_per_wg < 1) rows_per_wg = 1;
+    if (rows_per_wg > GEMV_MAX_ROWS) rows_per_wg = GEMV_MAX_ROWS;
+    const int grid = (n + rows_per_wg - 1) / rows_per_wg;
+    gemv_kernel<F, B, R><<<dim3(grid), dim3(64 * nwaves), 0, current_stream()>>>(w, x, y, k, n, batch, row_bytes, rows_per_wg);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
+template <class F>
+static int launch_format(const uint8_t* w, const float* x, float* y, int k, int n, int batch, int waves_per_cu) {
+    if (batch == 1) return launch_one<F, 1, 8>(w, x, y, k, n, batch, waves_per_cu);
+    if (batch == 2) return launch_one<F, 2, 4>(w, x, y, k, n, batch, waves_per_cu);
+    return launch_one<F, 4, 2>(w, x, y, k, n, batch, waves_per_cu);
+}
+
+static int g_gemv_waves_per_cu = 8;
+void set_gemv_waves_per_cu(int v) { if (v > 0) g_gemv_waves_per_cu = v; }
+
+// y[m, n] = x[m, k] . W^T for m activation rows, at most 4 per pass over the weight.
+int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y) {
+    if (m <= 0 || n <= 0) return 0;
+    if (!is_packed(enc)) return set_error("gemv: unsupported encoding %d", enc);
+    if (k <= 0 || k % block_elems(enc) != 0)
+        return set_error("gemv: inputDim must be a positive multiple of %d; got %d", block_elems(enc), k);
+    for (int b0 = 0; b0 < m; b0 += 4) {
+        const int nb = m - b0 < 4 ? m - b0 : 4;
+        const float* xb = x + (int64_t)b0 * k;
+        float* yb = y + (int64_t)b0 * n;
+        int rc;
+        if (enc == ENC_Q4_K) rc = launch_format<Q4KSlot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
+        else if (enc == ENC_Q6_K) rc = launch_format<Q6KSlot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
+        else rc = launch_format<Q80Slot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+}  // namespace skh

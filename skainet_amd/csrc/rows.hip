@@ -1,0 +1,192 @@
+// Row kernels a decoder needs around the matmuls: RMSNorm, softmax, SiLU*up, residual add, arg-max,
+// the packed-weight block permutation and the packed embedding lookup. All fp32, all HBM-bound:
+// one pass in, one pass out, reductions inside a workgroup.
+//
+// Semantics (paths under /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/):
+//   rms_norm      out = x / sqrt(mean(x^2) + eps) * gamma      f32_fused.c:255-286
+//   layer_norm    (x - mean) / sqrt(var + eps) * gamma + beta  f32_fused.c:255-279
+//   softmax_rows  exp(x - max) / sum, or x - (log sum + max)   f32_fused.c:199-222
+//   silu_mul      x * (1 / (1 + exp(-x))) * up                 f32_ops.c:222-244 (silu), binary mul
+//   argmax        first index of the row maximum               TensorOps.kt:263-277 (ties -> lowest index)
+#include "common.h"
+
+namespace skh {
+
+constexpr int ROW_THREADS = 256;
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += red[i];
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) t = fmaxf(t, red[i]);
+    return t;
+}
+
+// One workgroup per row.
+__global__ __launch_bounds__(ROW_THREADS) void rms_norm_kernel(const float* __restrict__ in, const float* __restrict__ gamma,
+                                                               float* __restrict__ out, int cols, float eps) {
+    __shared__ float red[ROW_THREADS / 64];
+    const float* x = in + (int64_t)blockIdx.x * cols;
+    float* o = out + (int64_t)blockIdx.x * cols;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = x[i]; s = fmaf(v, v, s); }
+    s = block_sum(s, red);
+    const float scale = 1.0f / sqrtf(s * (1.0f / (float)cols) + eps);
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        float y = x[i] * scale;
+        if (gamma) y *= gamma[i];
+        o[i] = y;
+    }
+}
+
+// out = (x - mean) / sqrt(var + eps) * gamma + beta with the biased variance; gamma / beta may be null.
+// Reference: f32_fused.c:255-279 (two passes: mean, then centred sum of squares).
+__global__ __launch_bounds__(ROW_THREADS) void layer_norm_kernel(const float* __restrict__ in, const float* __restrict__ gamma,
+                                                                 const float* __restrict__ beta, float* __restrict__ out,
+                                                                 int cols, float eps) {
+    __shared__ float red[ROW_THREADS / 64];
+    const float* x = in + (int64_t)blockIdx.x * cols;
+    float* o = out + (int64_t)blockIdx.x * cols;
+    const float inv_n = 1.0f / (float)cols;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) s += x[i];
+    const float mean = block_sum(s, red) * inv_n;
+    float v = 0.f;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float d = x[i] - mean; v = fmaf(d, d, v); }
+    const float scale = 1.0f / sqrtf(block_sum(v, red) * inv_n + eps);
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        float y = (x[i] - mean) * scale;
+        if (gamma) y *= gamma[i];
+        if (beta) y += beta[i];
+        o[i] = y;
+    }
+}
+
+__global__ __launch_bounds__(ROW_THREADS) void softmax_rows_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                                   int cols, int log_form) {
+    __shared__ float red[ROW_THREADS / 64];
+    const float* x = in + (int64_t)blockIdx.x * cols;
+    float* o = out + (int64_t)blockIdx.x * cols;
+    float m = -INFINITY;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) m = fmaxf(m, x[i]);
+    m = block_max(m, red);
+    float s = 0.f;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) s += expf(x[i] - m);
+    s = block_sum(s, red);
+    if (log_form) {
+        const float lse = logf(s) + m;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) o[i] = x[i] - lse;
+    } else {
+        const float inv = s > 0.f ? 1.0f / s : 1.0f;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) o[i] = expf(x[i] - m) * inv;
+    }
+}
+
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       float* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) { const float g = gate[i]; out[i] = g * (1.0f / (1.0f + expf(-g))) * up[i]; }
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                  float* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] + b[i];
+}
+
+// One workgroup per row; (value, index) pairs reduced with "larger value, then lower index" so ties keep the first.
+__global__ __launch_bounds__(ROW_THREADS) void argmax_rows_kernel(const float* __restrict__ in, int cols, int32_t* __restrict__ out) {
+    __shared__ float rv[ROW_THREADS / 64];
+    __shared__ int ri[ROW_THREADS / 64];
+    const float* x = in + (int64_t)blockIdx.x * cols;
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        const float v = x[i];
+        if (v > bv || (v == bv && i < bi) || bi == 0x7FFFFFFF) { bv = v; bi = i; }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const float ov = __shfl_xor(bv, m, 64);
+        const int oi = __shfl_xor(bi, m, 64);
+        if (oi != 0x7FFFFFFF && (bi == 0x7FFFFFFF || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { rv[wave] = bv; ri[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w) {
+            if (ri[w] != 0x7FFFFFFF && (bi == 0x7FFFFFFF || rv[w] > bv || (rv[w] == bv && ri[w] < bi))) { bv = rv[w]; bi = ri[w]; }
+        }
+        out[blockIdx.x] = bi == 0x7FFFFFFF ? 0 : bi;
+    }
+}
+
+// dst (row-major) block (o, b) <- src (input-block-major) block (b, o); 2 bytes per thread-step because
+// Q8_0 / Q6_K blocks are only 2-byte aligned.
+__global__ __launch_bounds__(256) void relayout_to_row_major_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                                    int rows, int bpr, int block_bytes) {
+    const int64_t blk = blockIdx.x;   // destination block index o * bpr + b
+    const int o = (int)(blk / bpr), b = (int)(blk % bpr);
+    const uint16_t* s = reinterpret_cast<const uint16_t*>(src + ((int64_t)b * rows + o) * block_bytes);
+    uint16_t* d = reinterpret_cast<uint16_t*>(dst + blk * block_bytes);
+    for (int i = threadIdx.x; i < block_bytes / 2; i += blockDim.x) d[i] = s[i];
+}
+
+int launch_rms_norm(const float* in, const float* gamma, float* out, int rows, int cols, float eps) {
+    if (rows <= 0 || cols <= 0) return 0;
+    rms_norm_kernel<<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, gamma, out, cols, eps);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int rows, int cols, float eps) {
+    if (rows <= 0 || cols <= 0) return 0;
+    layer_norm_kernel<<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, gamma, beta, out, cols, eps);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_softmax_rows(const float* in, float* out, int rows, int cols, int log_form) {
+    if (rows <= 0 || cols <= 0) return 0;
+    softmax_rows_kernel<<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, out, cols, log_form);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_silu_mul(const float* gate, const float* up, float* out, int64_t n) {
+    if (n <= 0) return 0;
+    silu_mul_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(gate, up, out, n);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_add(const float* a, const float* b, float* out, int64_t n) {
+    if (n <= 0) return 0;
+    add_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(a, b, out, n);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out) {
+    if (rows <= 0 || cols <= 0) return 0;
+    argmax_rows_kernel<<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, cols, out);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes) {
+    if (rows <= 0 || bpr <= 0) return 0;
+    relayout_to_row_major_kernel<<<dim3((unsigned)((int64_t)rows * bpr)), dim3(64), 0, current_stream()>>>(src, dst, rows, bpr, block_bytes);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
+}  // namespace skh

@@ -1,0 +1,509 @@
+// C ABI of libskainet_hip.so (declared in include/skainet_hip.h): device selection, allocation, one-time
+// packed-weight upload, stream and launch. No arithmetic lives here.
+//
+// Contract mirrored from the reference's native provider: a missing device or library is an answer
+// ("unavailable"), never a crash
+//   /root/reference/skainet-backends/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/NativeLibraryLoader.kt:24-29
+// and the C functions return void, ignore non-positive dimensions and leave the output untouched on a
+// resource failure
+//   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/q4k_matmul.c:326-333.
+#include "common.h"
+#include "../../include/skainet_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+namespace skh {
+
+// kernels (one translation unit each)
+int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr);
+int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
+int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
+void set_gemv_waves_per_cu(int v);
+int launch_rms_norm(const float* in, const float* gamma, float* out, int rows, int cols, float eps);
+int launch_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int rows, int cols, float eps);
+int launch_softmax_rows(const float* in, float* out, int rows, int cols, int log_form);
+int launch_silu_mul(const float* gate, const float* up, float* out, int64_t n);
+int launch_add(const float* a, const float* b, float* out, int64_t n);
+int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out);
+int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes);
+int launch_fp32_matmul(const float* a, int64_t a_stride, const float* b, int64_t b_stride, float* c, int64_t c_stride,
+                       int m, int n, int k, bool b_transposed);
+int launch_sdpa(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
+                int seq_q, int seq_kv, int head_dim, float scale, int causal, int window, int right_context,
+                const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k);
+
+// ------------------------------------------------------------------------------------------ state
+static thread_local char t_error[512] = "";
+static thread_local hipStream_t t_stream = nullptr;
+static thread_local hipEvent_t t_ev0 = nullptr, t_ev1 = nullptr;
+
+struct Scratch { void* ptr = nullptr; size_t cap = 0; };
+static thread_local Scratch t_workspace;          // kernel scratch (attention split-K partials, GEMM staging)
+static thread_local Scratch t_stage[6];           // device staging of the host-pointer entries
+
+static std::mutex g_mutex;
+static int g_state = 0;        // 0 = not probed, 1 = usable, -1 = unusable
+static int g_device = 0;
+static int g_cus = 0;
+static char g_name[256] = "";
+
+int set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_error, sizeof(t_error), fmt, ap);
+    va_end(ap);
+    return -1;
+}
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return 0;
+    (void)hipGetLastError();   // clear the sticky error so later calls report their own
+    return set_error("%s failed: %s", what, hipGetErrorString(e));
+}
+hipStream_t current_stream() { return t_stream; }
+int num_cus() { return g_cus > 0 ? g_cus : 256; }
+
+static int probe_locked(int device) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        g_state = -1;
+        return set_error("no HIP device visible");
+    }
+    if (device < 0 || device >= count) { g_state = -1; return set_error("device %d out of range (%d visible)", device, count); }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) { (void)hipGetLastError(); g_state = -1; return set_error("cannot query device %d", device); }
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        g_state = -1;
+        return set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    }
+    if (hipSetDevice(device) != hipSuccess) { (void)hipGetLastError(); g_state = -1; return set_error("cannot select device %d", device); }
+    g_device = device;
+    g_cus = prop.multiProcessorCount;
+    snprintf(g_name, sizeof(g_name), "%s (%s)", prop.name, prop.gcnArchName);
+    g_state = 1;
+    return 0;
+}
+
+int ensure_device() {
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        if (g_state == 0) probe_locked(0);
+        if (g_state != 1) return t_error[0] ? -1 : set_error("HIP backend unavailable");
+    }
+    // hipSetDevice is per thread
+    static thread_local bool bound = false;
+    if (!bound) { if (check_hip(hipSetDevice(g_device), "hipSetDevice") != 0) return -1; bound = true; }
+    return 0;
+}
+
+static void* scratch_get(Scratch& s, size_t bytes) {
+    if (bytes <= s.cap) return s.ptr;
+    // the old buffer may still be read by queued kernels of this thread's stream
+    if (s.ptr) { (void)hipStreamSynchronize(t_stream); (void)hipFree(s.ptr); s.ptr = nullptr; s.cap = 0; }
+    const size_t cap = (bytes + (1u << 20) - 1) & ~((size_t)(1u << 20) - 1);
+    void* p = nullptr;
+    if (check_hip(hipMalloc(&p, cap), "hipMalloc(scratch)") != 0) return nullptr;
+    s.ptr = p; s.cap = cap;
+    return p;
+}
+float* sdpa_workspace(size_t bytes) { return static_cast<float*>(scratch_get(t_workspace, bytes)); }
+void* kernel_workspace(size_t bytes) { return scratch_get(t_workspace, bytes); }
+
+}  // namespace skh
+
+using namespace skh;
+
+struct skainet_hip_weight {
+    uint8_t* data;
+    int64_t nbytes;
+    int32_t encoding, rows, cols;
+    bool owned;
+};
+
+extern "C" {
+
+// ------------------------------------------------------------------------------------------ runtime
+int32_t skainet_hip_available(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_state == 0) probe_locked(0);
+    return g_state == 1 ? 1 : 0;
+}
+int32_t skainet_hip_init(int32_t device) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_state == 1 && device == g_device) return 0;
+    return probe_locked(device);
+}
+const char* skainet_hip_last_error(void) { return t_error; }
+const char* skainet_hip_device_name(void) { return g_name; }
+int32_t skainet_hip_compute_units(void) { return g_cus; }
+int32_t skainet_hip_set_stream(void* stream) { t_stream = static_cast<hipStream_t>(stream); return 0; }
+int32_t skainet_hip_sync(void) {
+    if (ensure_device() != 0) return -1;
+    return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+void* skainet_hip_malloc(size_t bytes) {
+    if (ensure_device() != 0) return nullptr;
+    void* p = nullptr;
+    if (check_hip(hipMalloc(&p, bytes ? bytes : 1), "hipMalloc") != 0) return nullptr;
+    return p;
+}
+int32_t skainet_hip_free(void* p) {
+    if (!p) return 0;
+    if (ensure_device() != 0) return -1;
+    return check_hip(hipFree(p), "hipFree");
+}
+int32_t skainet_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    if (ensure_device() != 0) return -1;
+    if (bytes == 0) return 0;
+    if (check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, t_stream), "hipMemcpy h2d") != 0) return -1;
+    return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+int32_t skainet_hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    if (ensure_device() != 0) return -1;
+    if (bytes == 0) return 0;
+    if (check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, t_stream), "hipMemcpy d2h") != 0) return -1;
+    return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+int32_t skainet_hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    if (ensure_device() != 0) return -1;
+    if (bytes == 0) return 0;
+    return check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, t_stream), "hipMemcpy d2d");
+}
+int32_t skainet_hip_timer_begin(void) {
+    if (ensure_device() != 0) return -1;
+    if (!t_ev0) {
+        if (check_hip(hipEventCreate(&t_ev0), "hipEventCreate") != 0) return -1;
+        if (check_hip(hipEventCreate(&t_ev1), "hipEventCreate") != 0) return -1;
+    }
+    return check_hip(hipEventRecord(t_ev0, t_stream), "hipEventRecord");
+}
+float skainet_hip_timer_end_ms(void) {
+    if (!t_ev0) { set_error("timer_end without timer_begin"); return -1.f; }
+    if (check_hip(hipEventRecord(t_ev1, t_stream), "hipEventRecord") != 0) return -1.f;
+    if (check_hip(hipEventSynchronize(t_ev1), "hipEventSynchronize") != 0) return -1.f;
+    float ms = -1.f;
+    if (check_hip(hipEventElapsedTime(&ms, t_ev0, t_ev1), "hipEventElapsedTime") != 0) return -1.f;
+    return ms;
+}
+void skainet_hip_set_gemv_waves_per_cu(int32_t waves) { set_gemv_waves_per_cu(waves); }
+
+// ------------------------------------------------------------------------------------------ weights
+static int check_weight_shape(const char* who, int32_t encoding, int32_t rows, int32_t cols, int64_t* nbytes) {
+    if (!is_packed(encoding)) return set_error("%s: unsupported encoding %d", who, encoding);
+    if (rows <= 0 || cols <= 0) return set_error("%s: rows and cols must be positive; got %d x %d", who, rows, cols);
+    if (cols % block_elems(encoding) != 0)
+        return set_error("%s: inputDim must be a multiple of %d; got %d", who, block_elems(encoding), cols);
+    *nbytes = (int64_t)rows * (cols / block_elems(encoding)) * block_bytes(encoding);
+    return 0;
+}
+
+skainet_hip_weight* skainet_hip_weight_upload(const uint8_t* bytes, int64_t nbytes, int32_t encoding, int32_t order,
+                                              int32_t rows, int32_t cols) {
+    if (ensure_device() != 0) return nullptr;
+    int64_t need = 0;
+    if (check_weight_shape("weight_upload", encoding, rows, cols, &need) != 0) return nullptr;
+    if (!bytes || nbytes < need) { set_error("weight_upload: %lld bytes given, %lld needed", (long long)nbytes, (long long)need); return nullptr; }
+    if (order != SKAINET_HIP_ORDER_ROW_MAJOR && order != SKAINET_HIP_ORDER_INPUT_BLOCK_MAJOR) { set_error("weight_upload: unknown block order %d", order); return nullptr; }
+    void* dev = nullptr;
+    if (check_hip(hipMalloc(&dev, (size_t)need), "hipMalloc(weight)") != 0) return nullptr;
+    bool ok;
+    if (order == SKAINET_HIP_ORDER_ROW_MAJOR) {
+        ok = check_hip(hipMemcpy(dev, bytes, (size_t)need, hipMemcpyHostToDevice), "hipMemcpy(weight)") == 0;
+    } else {
+        void* tmp = nullptr;
+        ok = check_hip(hipMalloc(&tmp, (size_t)need), "hipMalloc(weight staging)") == 0;
+        ok = ok && check_hip(hipMemcpy(tmp, bytes, (size_t)need, hipMemcpyHostToDevice), "hipMemcpy(weight)") == 0;
+        ok = ok && launch_relayout_to_row_major(static_cast<uint8_t*>(tmp), static_cast<uint8_t*>(dev), rows,
+                                                cols / block_elems(encoding), block_bytes(encoding)) == 0;
+        ok = ok && check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize") == 0;
+        if (tmp) (void)hipFree(tmp);
+    }
+    if (!ok) { (void)hipFree(dev); return nullptr; }
+    return new skainet_hip_weight{static_cast<uint8_t*>(dev), need, encoding, rows, cols, true};
+}
+
+skainet_hip_weight* skainet_hip_weight_wrap(const void* device_bytes, int32_t encoding, int32_t rows, int32_t cols) {
+    int64_t need = 0;
+    if (check_weight_shape("weight_wrap", encoding, rows, cols, &need) != 0) return nullptr;
+    if (!device_bytes) { set_error("weight_wrap: null device pointer"); return nullptr; }
+    if (reinterpret_cast<uintptr_t>(device_bytes) & 15) { set_error("weight_wrap: device bytes must be 16-byte aligned"); return nullptr; }
+    return new skainet_hip_weight{static_cast<uint8_t*>(const_cast<void*>(device_bytes)), need, encoding, rows, cols, false};
+}
+void skainet_hip_weight_free(skainet_hip_weight* w) {
+    if (!w) return;
+    if (w->owned && w->data) (void)hipFree(w->data);
+    delete w;
+}
+const void* skainet_hip_weight_data(const skainet_hip_weight* w) { return w ? w->data : nullptr; }
+int64_t skainet_hip_weight_nbytes(const skainet_hip_weight* w) { return w ? w->nbytes : 0; }
+
+int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out, int32_t kind) {
+    if (ensure_device() != 0) return -1;
+    if (!w) return set_error("matmul: null weight handle");
+    if (m <= 0) return 0;
+    if (!x || !out) return set_error("matmul: null activation or output pointer");
+    if (kind == 0) return launch_gemv(w->encoding, w->data, x, m, w->cols, w->rows, out);
+    if (kind == 1) return launch_gemm(w->encoding, w->data, x, m, w->cols, w->rows, out);
+    return set_error("matmul: unknown kernel kind %d", kind);
+}
+int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out) {
+    return skainet_hip_matmul_kind_dev(w, x, m, out, m <= 8 ? 0 : 1);
+}
+// `iters` products back to back on this thread's stream, weight i % nweights each time (several copies of one
+// weight defeat the memory-side cache), bracketed by HIP events. With use_graph the launches are captured once
+// into a HIP graph (kernel nodes only) and replayed, which removes the host's per-launch cost from the GPU timeline.
+float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, int32_t nweights, const float* x, int32_t m,
+                                    float* out, int32_t iters, int32_t kind, int32_t use_graph) {
+    if (ensure_device() != 0) return -1.f;
+    if (!weights || nweights <= 0 || iters <= 0 || m <= 0) { set_error("matmul_repeat: bad arguments"); return -1.f; }
+    hipStream_t prev = t_stream, cap = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    float ms = -1.f;
+    bool ok = true;
+    if (use_graph) {
+        // capture needs a real (non-null) stream; the graph is then launched on it as well
+        ok = check_hip(hipStreamCreateWithFlags(&cap, hipStreamNonBlocking), "hipStreamCreate") == 0;
+        if (ok) {
+            t_stream = cap;
+            ok = check_hip(hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture") == 0;
+            for (int i = 0; ok && i < iters; ++i) ok = skainet_hip_matmul_kind_dev(weights[i % nweights], x, m, out, kind) == 0;
+            hipError_t e = hipStreamEndCapture(cap, &graph);
+            ok = ok && check_hip(e, "hipStreamEndCapture") == 0;
+            ok = ok && check_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate") == 0;
+            // one untimed replay (uploads the graph), then the timed one
+            ok = ok && check_hip(hipGraphLaunch(exec, cap), "hipGraphLaunch") == 0;
+            ok = ok && check_hip(hipStreamSynchronize(cap), "hipStreamSynchronize") == 0;
+            ok = ok && skainet_hip_timer_begin() == 0;
+            ok = ok && check_hip(hipGraphLaunch(exec, cap), "hipGraphLaunch") == 0;
+            if (ok) ms = skainet_hip_timer_end_ms();
+        }
+    } else {
+        ok = skainet_hip_timer_begin() == 0;
+        for (int i = 0; ok && i < iters; ++i) ok = skainet_hip_matmul_kind_dev(weights[i % nweights], x, m, out, kind) == 0;
+        if (ok) ms = skainet_hip_timer_end_ms();
+    }
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    t_stream = prev;
+    if (cap) { (void)hipStreamSynchronize(cap); (void)hipStreamDestroy(cap); }
+    return ok ? ms : -1.f;
+}
+
+int32_t skainet_hip_dequantize_dev(const skainet_hip_weight* w, float* out) {
+    if (ensure_device() != 0) return -1;
+    if (!w || !out) return set_error("dequantize: null argument");
+    return launch_dequant(w->encoding, w->data, (int64_t)w->rows * (w->cols / block_elems(w->encoding)), out, nullptr, 1);
+}
+int32_t skainet_hip_dequantize_rows_dev(const skainet_hip_weight* w, const int32_t* row_ids, int32_t count, float* out) {
+    if (ensure_device() != 0) return -1;
+    if (!w || !out || !row_ids) return set_error("dequantize_rows: null argument");
+    if (count <= 0) return 0;
+    const int bpr = w->cols / block_elems(w->encoding);
+    return launch_dequant(w->encoding, w->data, (int64_t)count * bpr, out, row_ids, bpr);
+}
+
+// ------------------------------------------------------------------------------------------ device entries
+int32_t skainet_hip_fp32_matmul_dev(const float* a, int32_t a_offset, int32_t a_stride, const float* b, int32_t b_offset,
+                                    int32_t b_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k) {
+    if (ensure_device() != 0) return -1;
+    if (m <= 0 || n <= 0) return 0;
+    return launch_fp32_matmul(a + a_offset, a_stride, b + b_offset, b_stride, c + c_offset, c_stride, m, n, k, false);
+}
+int32_t skainet_hip_fp32_matmul_wt_dev(const float* in, int32_t in_offset, const float* w, int32_t w_offset, float* out,
+                                       int32_t out_offset, int32_t m, int32_t n, int32_t k) {
+    if (ensure_device() != 0) return -1;
+    if (m <= 0 || n <= 0 || k < 0) return 0;
+    return launch_fp32_matmul(in + in_offset, k, w + w_offset, k, out + out_offset, n, m, n, k, true);
+}
+int32_t skainet_hip_f32_rms_norm_dev(const float* in, const float* gamma, float* out, int32_t rows, int32_t cols, float eps) {
+    if (ensure_device() != 0) return -1;
+    return launch_rms_norm(in, gamma, out, rows, cols, eps);
+}
+int32_t skainet_hip_f32_layer_norm_dev(const float* in, const float* gamma, const float* beta, float* out, int32_t rows,
+                                      int32_t cols, float eps) {
+    if (ensure_device() != 0) return -1;
+    return launch_layer_norm(in, gamma, beta, out, rows, cols, eps);
+}
+int32_t skainet_hip_f32_softmax_rows_dev(const float* in, float* out, int32_t rows, int32_t cols, int32_t log_form) {
+    if (ensure_device() != 0) return -1;
+    return launch_softmax_rows(in, out, rows, cols, log_form);
+}
+int32_t skainet_hip_f32_sdpa_dev(const float* q, const float* k, const float* v, float* out, int32_t batch, int32_t heads,
+                                 int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t head_dim, float scale,
+                                 int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths,
+                                 const float* mask, int32_t mask_b, int32_t mask_h, int32_t mask_q, int32_t mask_k) {
+    if (ensure_device() != 0) return -1;
+    return launch_sdpa(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, scale, causal, window, right_context,
+                       lengths, mask, mask_b, mask_h, mask_q, mask_k);
+}
+int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* out, int64_t n) {
+    if (ensure_device() != 0) return -1;
+    return launch_silu_mul(gate, up, out, n);
+}
+int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int64_t n) {
+    if (ensure_device() != 0) return -1;
+    return launch_add(a, b, out, n);
+}
+int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out) {
+    if (ensure_device() != 0) return -1;
+    return launch_argmax_rows(in, rows, cols, out);
+}
+
+// ------------------------------------------------------------------------------------------ host-pointer entries
+// Each stages its operands into per-thread device buffers, runs on this thread's stream and copies the
+// result back before returning. Each clears the thread's error text first; a failure leaves `output`
+// untouched and the reason in last_error().
+
+static void* stage_in(int slot, const void* host, size_t bytes) {
+    void* d = scratch_get(t_stage[slot], bytes ? bytes : 1);
+    if (!d) return nullptr;
+    if (bytes && check_hip(hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, t_stream), "hipMemcpy h2d") != 0) return nullptr;
+    return d;
+}
+static int stage_out(void* host, const void* dev, size_t bytes) {
+    if (check_hip(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, t_stream), "hipMemcpy d2h") != 0) return -1;
+    return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+
+static void packed_matmul_host(int enc, int order, const float* input, int32_t input_offset, const uint8_t* weight,
+                               int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output,
+                               int32_t output_offset) {
+    t_error[0] = 0;
+    if (output_dim <= 0) return;
+    if (ensure_device() != 0) return;
+    if (input_dim % block_elems(enc) != 0) { set_error("matmul: inputDim must be a multiple of %d; got %d", block_elems(enc), input_dim); return; }
+    if (input_dim <= 0) {   // an empty contraction is a row of zeros (Q8_0 scalar kernel) / a no-op (K-quants): write zeros
+        for (int32_t o = 0; o < output_dim; ++o) output[output_offset + o] = 0.f;
+        return;
+    }
+    const int bpr = input_dim / block_elems(enc);
+    const size_t wbytes = (size_t)output_dim * bpr * block_bytes(enc);
+    uint8_t* wd = static_cast<uint8_t*>(stage_in(0, weight + weight_byte_offset, wbytes));
+    float* xd = static_cast<float*>(stage_in(1, input + input_offset, sizeof(float) * (size_t)input_dim));
+    float* yd = static_cast<float*>(scratch_get(t_stage[2], sizeof(float) * (size_t)output_dim));
+    if (!wd || !xd || !yd) return;
+    if (order == SKAINET_HIP_ORDER_INPUT_BLOCK_MAJOR) {
+        uint8_t* rm = static_cast<uint8_t*>(scratch_get(t_stage[3], wbytes));
+        if (!rm || launch_relayout_to_row_major(wd, rm, output_dim, bpr, block_bytes(enc)) != 0) return;
+        wd = rm;
+    }
+    if (launch_gemv(enc, wd, xd, 1, input_dim, output_dim, yd) != 0) return;
+    stage_out(output + output_offset, yd, sizeof(float) * (size_t)output_dim);
+}
+
+#define SKH_PACKED_ENTRY(name, enc)                                                                                        \
+    void skainet_hip_##name##_matmul(const float* input, int32_t input_offset, const uint8_t* weight,                        \
+                                     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output,       \
+                                     int32_t output_offset) {                                                               \
+        packed_matmul_host(enc, SKAINET_HIP_ORDER_INPUT_BLOCK_MAJOR, input, input_offset, weight, weight_byte_offset,      \
+                           input_dim, output_dim, output, output_offset);                                                  \
+    }                                                                                                                      \
+    void skainet_hip_##name##_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,                     \
+                                        int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output,    \
+                                        int32_t output_offset) {                                                            \
+        packed_matmul_host(enc, SKAINET_HIP_ORDER_ROW_MAJOR, input, input_offset, weight, weight_byte_offset, input_dim,   \
+                           output_dim, output, output_offset);                                                             \
+    }
+SKH_PACKED_ENTRY(q4k, ENC_Q4_K)
+SKH_PACKED_ENTRY(q6k, ENC_Q6_K)
+SKH_PACKED_ENTRY(q8_0, ENC_Q8_0)
+
+void skainet_hip_fp32_matmul(const float* a, int32_t a_offset, int32_t a_stride, const float* b, int32_t b_offset,
+                             int32_t b_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k) {
+    t_error[0] = 0;
+    if (m <= 0 || n <= 0) return;
+    if (ensure_device() != 0) return;
+    if (k < 0) k = 0;
+    // Strided operands are staged as their bounding spans: (rows - 1) * stride + cols floats.
+    const size_t a_span = k > 0 ? (size_t)(m - 1) * a_stride + k : 0, b_span = k > 0 ? (size_t)(k - 1) * b_stride + n : 0;
+    float* ad = static_cast<float*>(stage_in(0, a + a_offset, sizeof(float) * a_span));
+    float* bd = static_cast<float*>(stage_in(1, b + b_offset, sizeof(float) * b_span));
+    float* cd = static_cast<float*>(scratch_get(t_stage[2], sizeof(float) * (size_t)m * n));
+    if (!ad || !bd || !cd) return;
+    if (launch_fp32_matmul(ad, a_stride, bd, b_stride, cd, n, m, n, k, false) != 0) return;
+    if (c_stride == n) { stage_out(c + c_offset, cd, sizeof(float) * (size_t)m * n); return; }
+    if (check_hip(hipMemcpy2DAsync(c + c_offset, sizeof(float) * (size_t)c_stride, cd, sizeof(float) * (size_t)n,
+                                   sizeof(float) * (size_t)n, (size_t)m, hipMemcpyDeviceToHost, t_stream), "hipMemcpy2D d2h") != 0) return;
+    check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+
+void skainet_hip_fp32_matmul_wt(const float* in, int32_t in_offset, const float* w, int32_t w_offset, float* out,
+                                int32_t out_offset, int32_t m, int32_t n, int32_t k) {
+    t_error[0] = 0;
+    if (m <= 0 || n <= 0 || k < 0) return;
+    if (ensure_device() != 0) return;
+    float* xd = static_cast<float*>(stage_in(0, in + in_offset, sizeof(float) * (size_t)m * k));
+    float* wd = static_cast<float*>(stage_in(1, w + w_offset, sizeof(float) * (size_t)n * k));
+    float* od = static_cast<float*>(scratch_get(t_stage[2], sizeof(float) * (size_t)m * n));
+    if (!xd || !wd || !od) return;
+    if (launch_fp32_matmul(xd, k, wd, k, od, n, m, n, k, true) != 0) return;
+    stage_out(out + out_offset, od, sizeof(float) * (size_t)m * n);
+}
+
+void skainet_hip_f32_rms_norm(const float* in, const float* gamma, float* out, int32_t rows, int32_t cols, float eps) {
+    t_error[0] = 0;
+    if (rows <= 0 || cols <= 0) return;
+    if (ensure_device() != 0) return;
+    const size_t bytes = sizeof(float) * (size_t)rows * cols;
+    float* xd = static_cast<float*>(stage_in(0, in, bytes));
+    float* gd = gamma ? static_cast<float*>(stage_in(1, gamma, sizeof(float) * (size_t)cols)) : nullptr;
+    float* od = static_cast<float*>(scratch_get(t_stage[2], bytes));
+    if (!xd || (gamma && !gd) || !od) return;
+    if (launch_rms_norm(xd, gd, od, rows, cols, eps) != 0) return;
+    stage_out(out, od, bytes);
+}
+
+void skainet_hip_f32_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int32_t rows, int32_t cols,
+                                float eps) {
+    t_error[0] = 0;
+    if (rows <= 0 || cols <= 0) return;
+    if (ensure_device() != 0) return;
+    const size_t bytes = sizeof(float) * (size_t)rows * cols;
+    float* xd = static_cast<float*>(stage_in(0, in, bytes));
+    float* gd = gamma ? static_cast<float*>(stage_in(1, gamma, sizeof(float) * (size_t)cols)) : nullptr;
+    float* bd = beta ? static_cast<float*>(stage_in(3, beta, sizeof(float) * (size_t)cols)) : nullptr;
+    float* od = static_cast<float*>(scratch_get(t_stage[2], bytes));
+    if (!xd || (gamma && !gd) || (beta && !bd) || !od) return;
+    if (launch_layer_norm(xd, gd, bd, od, rows, cols, eps) != 0) return;
+    stage_out(out, od, bytes);
+}
+
+void skainet_hip_f32_softmax_rows(const float* in, float* out, int32_t rows, int32_t cols, int32_t log_form) {
+    t_error[0] = 0;
+    if (rows <= 0 || cols <= 0) return;
+    if (ensure_device() != 0) return;
+    const size_t bytes = sizeof(float) * (size_t)rows * cols;
+    float* xd = static_cast<float*>(stage_in(0, in, bytes));
+    float* od = static_cast<float*>(scratch_get(t_stage[2], bytes));
+    if (!xd || !od) return;
+    if (launch_softmax_rows(xd, od, rows, cols, log_form) != 0) return;
+    stage_out(out, od, bytes);
+}
+
+void skainet_hip_f32_sdpa(const float* q, const float* k, const float* v, float* out, int32_t batch, int32_t heads,
+                          int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t head_dim, float scale, int32_t causal,
+                          int32_t window, int32_t right_context, const int32_t* lengths, const float* mask, int32_t mask_b,
+                          int32_t mask_h, int32_t mask_q, int32_t mask_k) {
+    t_error[0] = 0;
+    if (batch <= 0 || heads <= 0 || kv_heads <= 0 || seq_q <= 0 || head_dim <= 0) return;
+    const size_t qn = (size_t)batch * heads * seq_q * head_dim;
+    if (seq_kv <= 0) { for (size_t i = 0; i < qn; ++i) out[i] = 0.f; return; }
+    if (ensure_device() != 0) return;
+    const size_t kn = (size_t)batch * kv_heads * seq_kv * head_dim;
+    float* qd = static_cast<float*>(stage_in(0, q, sizeof(float) * qn));
+    float* kd = static_cast<float*>(stage_in(1, k, sizeof(float) * kn));
+    float* vd = static_cast<float*>(stage_in(3, v, sizeof(float) * kn));
+    float* od = static_cast<float*>(scratch_get(t_stage[2], sizeof(float) * qn));
+    int32_t* ld = lengths ? static_cast<int32_t*>(stage_in(4, lengths, sizeof(int32_t) * (size_t)batch)) : nullptr;
+    float* md = mask ? static_cast<float*>(stage_in(5, mask, sizeof(float) * (size_t)mask_b * mask_h * mask_q * mask_k)) : nullptr;
+    if (!qd || !kd || !vd || !od || (lengths && !ld) || (mask && !md)) return;
+    if (launch_sdpa(qd, kd, vd, od, batch, heads, kv_heads, seq_q, seq_kv, head_dim, scale, causal, window, right_context, ld,
+                    md, mask_b, mask_h, mask_q, mask_k) != 0) return;
+    stage_out(out, od, sizeof(float) * qn);
+}
+
+}  // extern "C"
