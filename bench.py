@@ -91,7 +91,7 @@ def main():
     ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
-    ap.add_argument("--gemv-waves-per-cu", type=int, default=0)
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE", help="launch-shape knob (skainet_hip_set_tuning)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this backend is a single-GPU kernel library (no collectives); run with --gpus 1", file=sys.stderr)
@@ -102,8 +102,9 @@ def main():
     if not kernels.is_available():
         print("bench.py: HIP backend unavailable: " + _lib.last_error(), file=sys.stderr)
         sys.exit(1)
-    if a.gemv_waves_per_cu > 0:
-        _lib.hip().skainet_hip_set_gemv_waves_per_cu(a.gemv_waves_per_cu)
+    for kv in a.tune:
+        key, _, val = kv.partition("=")
+        _lib.check(_lib.hip().skainet_hip_set_tuning(key.encode(), int(val)), "set_tuning")
 
     enc, n, k, m = WORKLOADS[a.workload]
     rng = np.random.default_rng(20251125)
@@ -134,6 +135,10 @@ def main():
     ms = run(weights, a.steps)              # exactly K timed steps, HIP events on the launch stream
     wall = time.perf_counter() - t0
     ms_warm = run(weights[:1], a.steps)     # same K steps on one copy: served by the memory-side cache
+    # ceiling for a read-once pass over the same rotating copies: a kernel that only loads (no arithmetic)
+    probe_iters = min(a.steps, 500)
+    ms_probe = min(kernels.read_probe(store, packed.size, probe_iters, g) for g in (512, 2048))
+    gbs_probe = packed.size / (ms_probe / probe_iters * 1e-3) / 1e9
     ms_per_step = ms / a.steps
     gbs = alg / (ms_per_step * 1e-3) / 1e9
     gbs_warm = alg / (ms_warm / a.steps * 1e-3) / 1e9
@@ -157,6 +162,8 @@ def main():
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)},
         "extra": {"algorithmic_bytes_per_step": alg, "cache_warm_GBps": round(gbs_warm, 2),
                   "cache_warm_ms_per_step": round(ms_warm / a.steps, 6), "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+                  "read_only_probe_GBps_same_buffers": round(gbs_probe, 2),
+                  "frac_of_read_only_probe": round(gbs / gbs_probe, 4),
                   "wall_s_timed_region": round(wall, 4), "max_normalized_err_vs_fp64_decode_matmul": err,
                   "device": _lib.hip().skainet_hip_device_name().decode()},
     }

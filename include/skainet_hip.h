@@ -112,6 +112,11 @@ SKAINET_HIP_API int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w,
  * REF/skainet-backend-native-cpu/src/jvmTest/kotlin/sk/ainet/exec/kernel/Q4KMatmulMicrobenchTest.kt:53-70.) */
 SKAINET_HIP_API float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, int32_t nweights,
     const float* x, int32_t m, float* out, int32_t iters, int32_t kind, int32_t use_graph);
+/* Calibration aid with no reference counterpart: `iters` launches of a pure streaming-read kernel (16-byte loads,
+ * no arithmetic) over buffers[i % nbuffers], each `bytes` long, timed with HIP events; returns milliseconds.
+ * The rate it reaches on rotating copies of a weight is the device's ceiling for a read-once pass of that size. */
+SKAINET_HIP_API float skainet_hip_read_probe_dev(const void* const* buffers, int32_t nbuffers, int64_t bytes,
+    int32_t iters, int32_t grid);
 /* Bit-exact decode of the whole weight to fp32 [rows, cols] (the TensorData.dequantizeBlock semantics,
  * REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/data/Q4_KTensorData.kt:120,
  * Q6_KTensorData.kt:112, Q8_0TensorData.kt:80). */
@@ -192,8 +197,10 @@ SKAINET_HIP_API int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const fl
 SKAINET_HIP_API int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int64_t n);
 SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
 
-/* Tuning knob for experiments: resident GEMV waves per compute unit used to size the row shares (default 8). */
-SKAINET_HIP_API void skainet_hip_set_gemv_waves_per_cu(int32_t waves);
+/* Launch-shape knobs for experiments (defaults are the measured best). Keys: "gemv_waves_per_cu",
+ * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares), "q4k_rows_enable".
+ * 0 when the key is known. No reference counterpart. */
+SKAINET_HIP_API int32_t skainet_hip_set_tuning(const char* key, int32_t value);
 
 #ifdef __cplusplus
 }

@@ -6,7 +6,9 @@ The product path has no CPU fallback: `hip()` raises when the library is missing
 from __future__ import annotations
 
 import ctypes as C
+import importlib.util
 import os
+import sys
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 _vp, _i32, _i64, _f32, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_size_t
@@ -40,6 +42,7 @@ SIGNATURES = {
     "skainet_hip_matmul_dev": (_i32, [_vp, _vp, _i32, _vp]),
     "skainet_hip_matmul_kind_dev": (_i32, [_vp, _vp, _i32, _vp, _i32]),
     "skainet_hip_matmul_repeat_dev": (_f32, [_vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32]),
+    "skainet_hip_read_probe_dev": (_f32, [_vp, _i32, _i64, _i32, _i32]),
     "skainet_hip_dequantize_dev": (_i32, [_vp, _vp]),
     "skainet_hip_dequantize_rows_dev": (_i32, [_vp, _vp, _i32, _vp]),
     "skainet_hip_q4k_matmul": (None, _GEMV),
@@ -63,7 +66,7 @@ SIGNATURES = {
     "skainet_hip_f32_silu_mul_dev": (_i32, [_vp, _vp, _vp, _i64]),
     "skainet_hip_f32_add_dev": (_i32, [_vp, _vp, _vp, _i64]),
     "skainet_hip_f32_argmax_rows_dev": (_i32, [_vp, _i32, _i32, _vp]),
-    "skainet_hip_set_gemv_waves_per_cu": (None, [_i32]),
+    "skainet_hip_set_tuning": (_i32, [C.c_char_p, _i32]),
 }
 
 HIP_LIB_PATH = os.path.join(_PKG, "libskainet_hip.so")
@@ -76,12 +79,34 @@ class HipError(RuntimeError):
     """A device call failed, or the HIP library / a gfx950 device is missing."""
 
 
+def _share_hip_runtime_with_torch() -> None:
+    """One HIP runtime per process: PyTorch wheels carry their own libamdhip64.so.7, and the dynamic loader hands
+    whichever copy was loaded first to every later client of that soname. When torch is installed, load ITS copy
+    before this library so that device pointers, streams and the device count agree whichever is imported first
+    (with the system copy loaded first, torch reports no GPU). Without torch the system runtime is used."""
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    for loc in (spec.submodule_search_locations if spec and spec.submodule_search_locations else []):
+        path = os.path.join(loc, "lib", "libamdhip64.so")
+        if os.path.exists(path):
+            try:
+                C.CDLL(path, mode=C.RTLD_GLOBAL)
+            except OSError:
+                pass
+            return
+
+
 def hip() -> C.CDLL:
     """The loaded kernel library. Raises HipError when it was not built (python -m skainet_amd.build)."""
     global _hip
     if _hip is None:
         if not os.path.exists(HIP_LIB_PATH):
             raise HipError(f"{HIP_LIB_PATH} is missing: build it with `python -m skainet_amd.build`")
+        _share_hip_runtime_with_torch()
         lib = C.CDLL(HIP_LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)

@@ -58,6 +58,27 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
     return __uint_as_float(bits);
 }
 
+// Hardware fp16 -> fp32 (v_cvt_f32_f16): one instruction; used where the result feeds tolerance-checked sums.
+__device__ __forceinline__ float half_bits_to_float_fast(uint32_t h) {
+    const uint16_t b = (uint16_t)h;
+    _Float16 v;
+    __builtin_memcpy(&v, &b, 2);
+    return (float)v;
+}
+
+// Byte N of a dword as float (v_cvt_f32_ubyteN). Written as asm so the compiler keeps one pre-masked dword
+// and four conversions instead of re-deriving a shift/mask per byte.
+__device__ __forceinline__ float ubyte0_to_float(uint32_t v) { float f; asm("v_cvt_f32_ubyte0_e32 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ubyte1_to_float(uint32_t v) { float f; asm("v_cvt_f32_ubyte1_e32 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ubyte2_to_float(uint32_t v) { float f; asm("v_cvt_f32_ubyte2_e32 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ubyte3_to_float(uint32_t v) { float f; asm("v_cvt_f32_ubyte3_e32 %0, %1" : "=v"(f) : "v"(v)); return f; }
+template <int J> __device__ __forceinline__ float ubyte_to_float(uint32_t v) {
+    if constexpr (J == 0) return ubyte0_to_float(v);
+    else if constexpr (J == 1) return ubyte1_to_float(v);
+    else if constexpr (J == 2) return ubyte2_to_float(v);
+    else return ubyte3_to_float(v);
+}
+
 // Loads that tolerate the 2-byte alignment of Q8_0 / Q6_K blocks (34 and 210 bytes per block).
 struct __attribute__((packed, aligned(2))) u32_a2 { uint32_t v; };
 __device__ __forceinline__ uint32_t load_u32_a2(const uint8_t* p) { return reinterpret_cast<const u32_a2*>(p)->v; }
@@ -68,6 +89,38 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
     return v;
 }
+// Fold NV (a power of two, <= 64) per-lane values across the 64 lanes of a wave with a multi-value butterfly:
+// each of the first log2(NV) steps halves the number of live values (a lane keeps the half selected by one bit of
+// its lane id and hands the other half to its partner), the remaining steps are plain xor-shuffle adds. On return
+// v[0] of lane l holds the wave-wide total of value wave_fold_index<NV>(l). The selects are written as bit-field
+// inserts on the raw bits so they stay one instruction each (a ?: on array elements is turned into an indexed
+// register read, which this target expands into a compare/select chain per element).
+template <int NV>
+__device__ __forceinline__ void wave_fold(float* v, int lane) {
+    int mask = 1;
+#pragma unroll
+    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) {
+        const int half = nv >> 1;
+        const uint32_t up = (lane & mask) ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+        for (int i = 0; i < half; ++i) {
+            const uint32_t a = __float_as_uint(v[i]), b = __float_as_uint(v[i + half]);
+            const float send = __uint_as_float((a & up) | (b & ~up));
+            const float keep = __uint_as_float((b & up) | (a & ~up));
+            v[i] = keep + __shfl_xor(send, mask, 64);
+        }
+    }
+#pragma unroll
+    for (int m = NV; m < 64; m <<= 1) v[0] += __shfl_xor(v[0], m, 64);
+}
+template <int NV>
+__device__ __forceinline__ int wave_fold_index(int lane) {
+    int idx = 0, mask = 1;
+#pragma unroll
+    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) idx += (lane & mask) ? (nv >> 1) : 0;
+    return idx;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));

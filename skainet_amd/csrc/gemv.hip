@@ -20,6 +20,8 @@
 //   * Grid: contiguous row ranges, sized so the whole chip gets an even share (rows_per_wg from the host).
 #include "common.h"
 
+#include <cstring>
+
 namespace skh {
 
 constexpr int GEMV_MAX_WAVES = 8;    // waves per workgroup = K segments processed concurrently (2 per SIMD: 256 VGPRs each)
@@ -31,13 +33,15 @@ struct Q4KSlot {
     struct Raw { uint4 hdr, qs; };
     struct Lane {
         int blk_off, qs_off;   // byte offsets inside a row
-        int g;                 // 32-byte nibble group of this slot (sub-blocks 2g and 2g + 1)
+        int sh;                // bit offset of this slot's scale-byte pair inside the header dwords (0 or 16)
+        uint32_t hi_mask;      // all ones when the slot's sub-blocks are 4..7 (split 6-bit packing), else 0
     };
     __device__ static void init(Lane& ln, int slot) {
         const int blk = slot >> 3, c = slot & 7;
         ln.blk_off = blk * BLOCK_BYTES;
         ln.qs_off = ln.blk_off + 16 + c * 16;
-        ln.g = c >> 1;
+        ln.sh = ((c >> 1) & 1) * 16;
+        ln.hi_mask = (c >> 1) >= 2 ? 0xFFFFFFFFu : 0u;
     }
     // Element index (inside the row) of activation register i for this slot: 16 of sub-block 2g then 16 of 2g+1.
     __device__ static int x_index(int slot, int i) {
@@ -58,24 +62,19 @@ struct Q4KSlot {
     struct Scales { float dlo, dhi, mlo, mhi; };
     // The 6-bit (scale, min) pairs of sub-blocks 2g and 2g+1 (ggml get_scale_min_k4), folded with d / dmin.
     __device__ static Scales scales(const Raw& r, const Lane& ln) {
-        const float d = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
-        const int sh = (ln.g & 1) * 16;
-        const uint32_t u = (r.hdr.y >> sh) & 0xFFFFu;   // scale bytes s[2g'], s[2g'+1]
-        const uint32_t v = (r.hdr.z >> sh) & 0xFFFFu;   // scale bytes s[4+2g'], s[5+2g']
-        const uint32_t t = (r.hdr.w >> sh) & 0xFFFFu;   // scale bytes s[8+2g'], s[9+2g']
-        uint32_t sc, mn;
-        if (ln.g < 2) {
-            sc = u & 0x3F3Fu;
-            mn = v & 0x3F3Fu;
-        } else {
-            sc = (t & 0x0F0Fu) | ((u >> 2) & 0x3030u);
-            mn = ((t >> 4) & 0x0F0Fu) | ((v >> 2) & 0x3030u);
-        }
+        const float d = half_bits_to_float_fast(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(r.hdr.x >> 16);
+        const uint32_t u = r.hdr.y >> ln.sh;   // low 16 bits: scale bytes s[2g'], s[2g'+1]
+        const uint32_t v = r.hdr.z >> ln.sh;   // scale bytes s[4+2g'], s[5+2g']
+        const uint32_t t = r.hdr.w >> ln.sh;   // scale bytes s[8+2g'], s[9+2g']
+        // g < 2: (u & 0x3F3F, v & 0x3F3F); g >= 2: low nibbles of t / high nibbles of t, top two bits from u / v.
+        // Both forms are evaluated and picked by the lane-constant mask, so no branch diverges.
+        const uint32_t sc = ((u & 0x3F3Fu) & ~ln.hi_mask) | (((t & 0x0F0Fu) | ((u >> 2) & 0x3030u)) & ln.hi_mask);
+        const uint32_t mn = ((v & 0x3F3Fu) & ~ln.hi_mask) | ((((t >> 4) & 0x0F0Fu) | ((v >> 2) & 0x3030u)) & ln.hi_mask);
         Scales s;
-        s.dlo = d * (float)(sc & 0xFFu);
-        s.dhi = d * (float)(sc >> 8) * 0.0625f;   // high nibbles are accumulated as 16 * code
-        s.mlo = dmin * (float)(mn & 0xFFu);
-        s.mhi = dmin * (float)(mn >> 8);
+        s.dlo = d * ubyte0_to_float(sc);
+        s.dhi = d * ubyte1_to_float(sc) * 0.0625f;   // high nibbles are accumulated as 16 * code
+        s.mlo = dmin * ubyte0_to_float(mn);
+        s.mhi = dmin * ubyte1_to_float(mn);
         return s;
     }
     template <int B>
@@ -88,13 +87,14 @@ struct Q4KSlot {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t l4 = q[i] & 0x0F0F0F0Fu, h4 = q[i] & 0xF0F0F0F0u;
+            const float cl[4] = {ubyte0_to_float(l4), ubyte1_to_float(l4), ubyte2_to_float(l4), ubyte3_to_float(l4)};
+            const float ch[4] = {ubyte0_to_float(h4), ubyte1_to_float(h4), ubyte2_to_float(h4), ubyte3_to_float(h4)};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float cl = (float)((l4 >> (8 * j)) & 0xFFu), ch = (float)((h4 >> (8 * j)) & 0xFFu);
 #pragma unroll
                 for (int b = 0; b < B; ++b) {
-                    lo[b] = fmaf(x[b][i * 4 + j], cl, lo[b]);
-                    hi[b] = fmaf(x[b][16 + i * 4 + j], ch, hi[b]);
+                    lo[b] = fmaf(x[b][i * 4 + j], cl[j], lo[b]);
+                    hi[b] = fmaf(x[b][16 + i * 4 + j], ch[j], hi[b]);
                 }
             }
         }
@@ -136,7 +136,7 @@ struct Q6KSlot {
     }
     template <int B>
     __device__ static void dot(const Raw& r, const Lane& ln, const float (*x)[NX], const float (*xsum)[4], float* acc) {
-        const float d = half_bits_to_float(r.d);
+        const float d = half_bits_to_float_fast(r.d);
         // signed scales of the four quarters: bytes is, is+2, is+4, is+6 of the half's 8 scale bytes
         const uint32_t s0 = r.sc0 >> ln.sc_shift, s1 = r.sc1 >> ln.sc_shift;
         const float sc[4] = {d * (float)(int8_t)(s0), d * (float)(int8_t)(s0 >> 16),
@@ -153,11 +153,11 @@ struct Q6KSlot {
             float s[B];
 #pragma unroll
             for (int b = 0; b < B; ++b) s[b] = -xsum[b][k];   // the -32 bias of every code, taken out of the loop
+            const float cf[4] = {ubyte0_to_float(c[k]), ubyte1_to_float(c[k]), ubyte2_to_float(c[k]), ubyte3_to_float(c[k])};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float cf = (float)((c[k] >> (8 * j)) & 0xFFu);
 #pragma unroll
-                for (int b = 0; b < B; ++b) s[b] = fmaf(x[b][4 * k + j], cf, s[b]);
+                for (int b = 0; b < B; ++b) s[b] = fmaf(x[b][4 * k + j], cf[j], s[b]);
             }
 #pragma unroll
             for (int b = 0; b < B; ++b) acc[b] = fmaf(sc[k], s[b], acc[b]);
@@ -181,7 +181,7 @@ struct Q80Slot {
     __device__ static void prep(const float*, float*) {}
     template <int B>
     __device__ static void dot(const Raw& r, const Lane&, const float (*x)[NX], const float (*)[1], float* acc) {
-        const float d = half_bits_to_float(r.d);
+        const float d = half_bits_to_float_fast(r.d);
         float s[B];
 #pragma unroll
         for (int b = 0; b < B; ++b) s[b] = 0.f;
@@ -203,33 +203,6 @@ template <class F> struct XSumCount { static constexpr int N = 1; };
 template <> struct XSumCount<Q4KSlot> { static constexpr int N = 2; };
 template <> struct XSumCount<Q6KSlot> { static constexpr int N = 4; };
 
-// Fold NV per-lane values across the 64 lanes. On return v[0] of lane l holds the wave total of value
-// index bitrev(l & (NV-1)) over log2(NV) bits (see gemv_value_of_lane).
-template <int NV>
-__device__ __forceinline__ void wave_fold(float* v, int lane) {
-    int mask = 1;
-#pragma unroll
-    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) {
-        const int half = nv >> 1;
-        const bool upper = (lane & mask) != 0;
-#pragma unroll
-        for (int i = 0; i < half; ++i) {
-            const float send = upper ? v[i] : v[i + half];
-            const float keep = upper ? v[i + half] : v[i];
-            v[i] = keep + __shfl_xor(send, mask, 64);
-        }
-    }
-#pragma unroll
-    for (int m = NV; m < 64; m <<= 1) v[0] += __shfl_xor(v[0], m, 64);
-}
-template <int NV>
-__device__ __forceinline__ int gemv_value_of_lane(int lane) {
-    int idx = 0, mask = 1;
-#pragma unroll
-    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) idx += (lane & mask) ? (nv >> 1) : 0;
-    return idx;
-}
-
 // F: slot policy, B: activation rows per launch (1, 2 or 4; unused ones are zero), R: weight rows in flight.
 template <class F, int B, int R>
 __global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
@@ -246,7 +219,7 @@ __global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
     const int nrows = r1 - r0;
     if (nrows <= 0) return;
     const uint8_t* wbase = w + (int64_t)r0 * row_bytes;
-    const int my_value = gemv_value_of_lane<NV>(lane);
+    const int my_value = wave_fold_index<NV>(lane);
 
     for (int seg = wave, pass = 0; seg < nseg; seg += nwaves, ++pass) {
         const int slot = seg * 64 + lane;
@@ -277,7 +250,9 @@ __global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
 #pragma unroll
             for (int i = 0; i < R; ++i) {
                 float a[B];
-                F::template dot<B>(raw[i], ln, xs, xsum, a);
+#pragma unroll
+                for (int b = 0; b < B; ++b) a[b] = 0.f;
+                if (r + i < nrows) F::template dot<B>(raw[i], ln, xs, xsum, a);   // wave-uniform: no arithmetic on padding rows
 #pragma unroll
                 for (int b = 0; b < B; ++b) acc[i * B + b] = active ? a[b] : 0.f;
                 // refill this register set with the row R ahead (clamped: a repeated last row is discarded)
@@ -330,7 +305,17 @@ static int launch_format(const uint8_t* w, const float* x, float* y, int k, int 
 }
 
 static int g_gemv_waves_per_cu = 8;
-void set_gemv_waves_per_cu(int v) { if (v > 0) g_gemv_waves_per_cu = v; }
+static int g_q4k_rows_enable = 1;
+void set_q4k_rows_waves_per_cu(int v);
+int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch);   // gemv_q4k.hip
+
+// Experiment knobs (defaults are the measured best): returns 0 when the key is known.
+int set_tuning(const char* key, int value) {
+    if (!strcmp(key, "gemv_waves_per_cu")) { if (value > 0) g_gemv_waves_per_cu = value; return 0; }
+    if (!strcmp(key, "q4k_rows_waves_per_cu")) { set_q4k_rows_waves_per_cu(value); return 0; }
+    if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }
+    return -1;
+}
 
 // y[m, n] = x[m, k] . W^T for m activation rows, at most 4 per pass over the weight.
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y) {
@@ -343,6 +328,11 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
         const float* xb = x + (int64_t)b0 * k;
         float* yb = y + (int64_t)b0 * n;
         int rc;
+        if (enc == ENC_Q4_K && g_q4k_rows_enable) {
+            rc = launch_q4k_gemv_rows(w, xb, yb, k, n, nb);
+            if (rc < 0) return rc;
+            if (rc == 1) continue;
+        }
         if (enc == ENC_Q4_K) rc = launch_format<Q4KSlot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
         else if (enc == ENC_Q6_K) rc = launch_format<Q6KSlot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
         else rc = launch_format<Q80Slot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);

@@ -1,0 +1,182 @@
+// Q4_K dequant-GEMV, decode shape (1 or 2 activation rows), canonical row-major GGUF weight.
+//
+//   y[b, o] = sum_j x[b, j] * dequant(W[o, j]),   W[o, j] = code * (d * sc) - dmin * m  per 32-element sub-block
+//
+// Same products as the reference's exact-fp32 kernel, other summation order
+//   /root/reference/skainet-backends/skainet-backend-cpu/src/commonMain/kotlin/sk/ainet/exec/kernel/ScalarQ4_KMatmulKernel.kt:40-78
+// (per sub-block: codeSum * (d * sc) - inputSum * (dmin * m)); weight addressing (o * blocksPerRow + b) * 144 as in
+//   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/q4k_matmul.c:294-309.
+//
+// HBM-bound design (algorithmic bytes = 144 B per 256 weights + 4 B per activation / output element):
+//   * One wave owns a contiguous range of output rows and walks K in passes of 16 super-blocks (4096 elements).
+//     Lane l owns 32-byte nibble group g = l % 4 of super-block l / 4 of the pass: 64 weights (sub-blocks 2g and
+//     2g + 1) whose 64 activations it keeps in registers for all of its rows. A row costs the lane two 16-byte
+//     loads of quants and one of the block header; across the wave these are one contiguous 2304-byte span.
+//   * The four waves of a workgroup work on the same K pass, so the pass's 4096 activations are fetched once per
+//     workgroup with coalesced 16-byte loads, parked in LDS (one padded 64-float slice per lane) and read back by
+//     each lane into registers. Weights never touch LDS. Per-row partial sums stay in registers across passes and
+//     are folded across the 64 lanes once, at the end, with a multi-value butterfly.
+//   * R rows are in flight per wave (loads issued before the arithmetic of the previous rows), rows are spread
+//     evenly over all waves of the chip by the host.
+#include "common.h"
+
+namespace skh {
+
+constexpr int Q4K_RMAX = 12;   // rows a wave can own (bounds the per-row accumulators)
+
+struct Q4KRow { uint4 hdr, q0, q1; };
+
+template <int B>
+__device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi_mask, const float (*x)[64],
+                                            const float (*xsum)[2], float* out) {
+    const float d = half_bits_to_float_fast(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(r.hdr.x >> 16);
+    // 6-bit (scale, min) pairs of sub-blocks 2g, 2g+1 (ggml get_scale_min_k4); both packings evaluated, lane-constant pick
+    const uint32_t u = r.hdr.y >> sh, v = r.hdr.z >> sh, t = r.hdr.w >> sh;
+    const uint32_t sc = ((u & 0x3F3Fu) & ~hi_mask) | (((t & 0x0F0Fu) | ((u >> 2) & 0x3030u)) & hi_mask);
+    const uint32_t mn = ((v & 0x3F3Fu) & ~hi_mask) | ((((t >> 4) & 0x0F0Fu) | ((v >> 2) & 0x3030u)) & hi_mask);
+    const float dlo = d * ubyte0_to_float(sc), dhi = d * ubyte1_to_float(sc) * 0.0625f;   // high nibbles summed as 16 * code
+    const float mlo = dmin * ubyte0_to_float(mn), mhi = dmin * ubyte1_to_float(mn);
+    const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+    float lo[B], hi[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) lo[b] = hi[b] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t l4 = q[i] & 0x0F0F0F0Fu, h4 = q[i] & 0xF0F0F0F0u;
+        const float cl[4] = {ubyte0_to_float(l4), ubyte1_to_float(l4), ubyte2_to_float(l4), ubyte3_to_float(l4)};
+        const float ch[4] = {ubyte0_to_float(h4), ubyte1_to_float(h4), ubyte2_to_float(h4), ubyte3_to_float(h4)};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int b = 0; b < B; ++b) {
+                lo[b] = fmaf(x[b][i * 4 + j], cl[j], lo[b]);
+                hi[b] = fmaf(x[b][32 + i * 4 + j], ch[j], hi[b]);
+            }
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) out[b] += dlo * lo[b] + dhi * hi[b] - (mlo * xsum[b][0] + mhi * xsum[b][1]);
+}
+
+template <int B, int R>
+__global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                            float* __restrict__ y, int k, int n, int rows_per_wave) {
+    constexpr int NV = 16 * B;   // Q4K_RMAX rows padded to 16, times B
+    constexpr int SLICE = 68;    // 64 activations + 4 floats of padding: 16-byte aligned and bank-conflict free
+    __shared__ __attribute__((aligned(16))) float xlds[B][64 * SLICE];
+    const int lane = threadIdx.x & 63;
+    // readfirstlane: the wave index is uniform across a wave, and saying so keeps every row guard a scalar branch
+    const int gw = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
+    const int r0 = gw * rows_per_wave;
+    const int nrows = max(0, min(n, r0 + rows_per_wave) - r0);   // a wave without rows still helps stage activations
+    const int bpr = k >> 8;
+    const int64_t row_bytes = (int64_t)bpr * Q4K_BYTES;
+    const uint8_t* wbase = w + (int64_t)r0 * row_bytes;
+    const int g = lane & 3;
+    const int sh = (g & 1) * 16;
+    const uint32_t hi_mask = g >= 2 ? 0xFFFFFFFFu : 0u;
+
+    float acc[16][B];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int b = 0; b < B; ++b) acc[i][b] = 0.f;
+
+    for (int blk0 = 0; blk0 < bpr; blk0 += 16) {
+        const int blk = blk0 + (lane >> 2);
+        const int blk_c = min(blk, bpr - 1);                // lanes past K re-read a valid block and multiply it by zero activations
+        const uint8_t* lane_base = wbase + blk_c * Q4K_BYTES;
+        const int q_off = 16 + g * 32;
+
+        // the first rows' weight loads go out before anything else
+        Q4KRow raw[R];
+        if (nrows > 0) {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const uint8_t* p = lane_base + (int64_t)min(i, nrows - 1) * row_bytes;
+                raw[i].hdr = *reinterpret_cast<const uint4*>(p);
+                raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+            }
+        }
+
+        // stage this pass's activations: float4 number f of the pass goes to slice f / 16, position f % 16
+        if (blk0 > 0) __syncthreads();   // the previous pass's slices have been read
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int f = threadIdx.x + 256 * j;
+                const int e = blk0 * 256 + f * 4;
+                float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (e < k) v4 = *reinterpret_cast<const float4*>(x + (int64_t)b * k + e);
+                *reinterpret_cast<float4*>(&xlds[b][(f >> 4) * SLICE + (f & 15) * 4]) = v4;
+            }
+        }
+        __syncthreads();
+
+        float xs[B][64], xsum[B][2];
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float4 v4 = *reinterpret_cast<const float4*>(&xlds[b][lane * SLICE + i * 4]);   // zeros past K
+                xs[b][4 * i] = v4.x; xs[b][4 * i + 1] = v4.y; xs[b][4 * i + 2] = v4.z; xs[b][4 * i + 3] = v4.w;
+            }
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) { s0 += xs[b][i]; s1 += xs[b][32 + i]; }
+            xsum[b][0] = s0; xsum[b][1] = s1;
+        }
+
+#pragma unroll
+        for (int c = 0; c < Q4K_RMAX; c += R) {
+            if (c < nrows) {                                  // wave-uniform
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    if (c + i < nrows) q4k_row_dot<B>(raw[i], sh, hi_mask, xs, xsum, acc[c + i]);
+                    if (c + R + i < nrows) {                  // refill with the row R ahead
+                        const uint8_t* p = lane_base + (int64_t)(c + R + i) * row_bytes;
+                        raw[i].hdr = *reinterpret_cast<const uint4*>(p);
+                        raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                        raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+                    }
+                }
+            }
+        }
+    }
+
+    float v[NV];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int b = 0; b < B; ++b) v[i * B + b] = acc[i][b];
+    wave_fold<NV>(v, lane);
+    if (lane < NV) {
+        const int idx = wave_fold_index<NV>(lane);
+        const int row = idx / B, b = idx % B;
+        if (row < nrows) y[(int64_t)b * n + r0 + row] = v[0];
+    }
+}
+
+static int g_q4k_rows_waves_per_cu = 8;
+void set_q4k_rows_waves_per_cu(int v) { if (v > 0) g_q4k_rows_waves_per_cu = v; }
+
+// Returns 1 when this kernel took the product, 0 when the shape is outside its range (caller falls back to the
+// slot kernel), -1 on a launch error.
+int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch) {
+    if (batch < 1 || batch > 2) return 0;
+    if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 3)) return 0;
+    int total_waves = num_cus() * g_q4k_rows_waves_per_cu;
+    int rows_per_wave = (n + total_waves - 1) / total_waves;
+    if (rows_per_wave > Q4K_RMAX) rows_per_wave = Q4K_RMAX;
+    const int waves = (n + rows_per_wave - 1) / rows_per_wave;
+    const int grid = (waves + 3) / 4;
+    hipStream_t s = current_stream();
+    if (batch == 1) q4k_gemv_rows_kernel<1, 6><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave);
+    else q4k_gemv_rows_kernel<2, 3><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave);
+    SKH_CHECK(hipGetLastError());
+    return 1;
+}
+
+}  // namespace skh

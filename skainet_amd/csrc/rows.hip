@@ -146,6 +146,27 @@ __global__ __launch_bounds__(256) void relayout_to_row_major_kernel(const uint8_
     for (int i = threadIdx.x; i < block_bytes / 2; i += blockDim.x) d[i] = s[i];
 }
 
+// Calibration kernel: every thread streams 16-byte loads over a buffer with four independent loads in flight and
+// almost no arithmetic. Its rate is what this device sustains for a read-once pass of that size.
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ p, int64_t n16, uint32_t* __restrict__ sink) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    uint32_t acc = 0;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const uint4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], d = p[i + 3 * stride];
+        acc += a.x ^ b.y ^ c.z ^ d.w;
+    }
+    for (; i < n16; i += stride) acc += p[i].x;
+    if (acc == 0x9E3779B9u) sink[0] = acc;   // keeps the loads alive; practically never true
+}
+
+int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink) {
+    if (bytes < 16) return 0;
+    stream_read_kernel<<<dim3(grid > 0 ? grid : 2 * num_cus()), dim3(256), 0, current_stream()>>>(static_cast<const uint4*>(p), bytes / 16, sink);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
 int launch_rms_norm(const float* in, const float* gamma, float* out, int rows, int cols, float eps) {
     if (rows <= 0 || cols <= 0) return 0;
     rms_norm_kernel<<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, gamma, out, cols, eps);

@@ -21,13 +21,14 @@ namespace skh {
 int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr);
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
 int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
-void set_gemv_waves_per_cu(int v);
+int set_tuning(const char* key, int value);
 int launch_rms_norm(const float* in, const float* gamma, float* out, int rows, int cols, float eps);
 int launch_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int rows, int cols, float eps);
 int launch_softmax_rows(const float* in, float* out, int rows, int cols, int log_form);
 int launch_silu_mul(const float* gate, const float* up, float* out, int64_t n);
 int launch_add(const float* a, const float* b, float* out, int64_t n);
 int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out);
+int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink);
 int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes);
 int launch_fp32_matmul(const float* a, int64_t a_stride, const float* b, int64_t b_stride, float* c, int64_t c_stride,
                        int m, int n, int k, bool b_transposed);
@@ -188,7 +189,11 @@ float skainet_hip_timer_end_ms(void) {
     if (check_hip(hipEventElapsedTime(&ms, t_ev0, t_ev1), "hipEventElapsedTime") != 0) return -1.f;
     return ms;
 }
-void skainet_hip_set_gemv_waves_per_cu(int32_t waves) { set_gemv_waves_per_cu(waves); }
+int32_t skainet_hip_set_tuning(const char* key, int32_t value) {
+    if (!key) return set_error("set_tuning: null key");
+    if (set_tuning(key, value) != 0) return set_error("set_tuning: unknown key '%s'", key);
+    return 0;
+}
 
 // ------------------------------------------------------------------------------------------ weights
 static int check_weight_shape(const char* who, int32_t encoding, int32_t rows, int32_t cols, int64_t* nbytes) {
@@ -291,6 +296,19 @@ float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, in
     t_stream = prev;
     if (cap) { (void)hipStreamSynchronize(cap); (void)hipStreamDestroy(cap); }
     return ok ? ms : -1.f;
+}
+
+// Read-rate calibration: `iters` launches of a pure streaming-read kernel over buffers[i % nbuffers] (each `bytes`
+// long), timed with HIP events on this thread's stream. Returns milliseconds, < 0 on failure.
+float skainet_hip_read_probe_dev(const void* const* buffers, int32_t nbuffers, int64_t bytes, int32_t iters, int32_t grid) {
+    if (ensure_device() != 0) return -1.f;
+    if (!buffers || nbuffers <= 0 || iters <= 0 || bytes < 16) { set_error("read_probe: bad arguments"); return -1.f; }
+    uint32_t* sink = static_cast<uint32_t*>(scratch_get(t_workspace, 256));
+    if (!sink) return -1.f;
+    for (int i = 0; i < 3; ++i) if (launch_stream_read(buffers[i % nbuffers], bytes, grid, sink) != 0) return -1.f;
+    if (skainet_hip_timer_begin() != 0) return -1.f;
+    for (int i = 0; i < iters; ++i) if (launch_stream_read(buffers[i % nbuffers], bytes, grid, sink) != 0) return -1.f;
+    return skainet_hip_timer_end_ms();
 }
 
 int32_t skainet_hip_dequantize_dev(const skainet_hip_weight* w, float* out) {

@@ -177,6 +177,20 @@ def matmul_repeat(weights, x, m: int, out, iters: int, kind: int = 0, use_graph:
 
 # ---------------------------------------------------------------------------------------------- device ops
 
+def read_probe(buffers, nbytes: int, iters: int, grid: int = 0) -> float:
+    """Milliseconds for `iters` launches of the pure streaming-read kernel rotating over `buffers` (device addresses/tensors)."""
+    arr = (C.c_void_p * len(buffers))(*[_ptr(b) for b in buffers])
+    ms = _lib.hip().skainet_hip_read_probe_dev(arr, len(buffers), nbytes, iters, grid)
+    if ms < 0:
+        raise HipError("read_probe: " + _lib.last_error())
+    return ms
+
+
+def set_tuning(key: str, value: int) -> None:
+    """Launch-shape / kernel-variant knob of the library (skainet_hip_set_tuning); unknown keys raise."""
+    check(_lib.hip().skainet_hip_set_tuning(key.encode(), int(value)), "set_tuning")
+
+
 def sync() -> None:
     check(_lib.hip().skainet_hip_sync(), "sync")
 

@@ -114,6 +114,25 @@ def test_gemv_at_config_sizes(hip_backend, torch_cuda, enc, n, k, batches):
         assert err <= GEMV_TOL
 
 
+@pytest.mark.parametrize("mode", ["slot-fp32", "rows-fp32"])
+@pytest.mark.parametrize("n,k,m", [(11008, 4096, 1), (11008, 4096, 2), (4096, 14336, 1), (1000, 11008, 1), (77, 2304, 2), (5, 256, 1)])
+def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cuda, mode, n, k, m):
+    """Both Q4_K decode kernels (the generic slot kernel and the row-streaming kernel) are held to the same bound
+    against the exact-fp32 oracle, on quantised Gaussian weights and on random valid blocks with large scales."""
+    hip_backend.set_tuning("q4k_rows_enable", 1 if mode == "rows-fp32" else 0)
+    try:
+        for packed in (gaussian_weight(hip_backend, "Q4_K", n, k, 71), random_valid_blocks("Q4_K", n * k // 256, 72)):
+            x = np.random.default_rng(73 + m).standard_normal((m, k)).astype(np.float32)
+            x[0, :64] = 0.0          # a constant slice (zero range) and an outlier
+            x[0, 100] = 37.5
+            got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+            err = normalized_err(got, L.gemv("Q4_K", x, packed, n))
+            print(f"{mode} {n}x{k} m={m}: {err:.2e}")
+            assert err <= GEMV_TOL
+    finally:
+        hip_backend.set_tuning("q4k_rows_enable", 1)
+
+
 def test_gemv_is_linear_and_deterministic_at_full_size(hip_backend, torch_cuda):
     """Size-independent properties at the benchmark shape: y(a*x1 + x2) == a*y(x1) + y(x2) within rounding; two runs agree bit for bit."""
     n, k = 11008, 4096
@@ -127,7 +146,7 @@ def test_gemv_is_linear_and_deterministic_at_full_size(hip_backend, torch_cuda):
     assert np.array_equal(y1, gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x1))
     # a batch row equals the same row run alone
     yb = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, np.concatenate([x1, x2, x1, x2]))
-    assert np.array_equal(yb[1], y2[0]) or normalized_err(yb[1], y2[0]) <= 1e-5
+    assert normalized_err(yb[1], y2[0]) <= 1e-4   # another kernel (4 rows per pass) sums in another order
 
 
 @pytest.mark.parametrize("enc", ENCS)
