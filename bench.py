@@ -38,8 +38,9 @@ WORKLOADS = {
     "q8_0_gemv_4096x4096_b1": ("Q8_0", 4096, 4096, 1),
     "q6k_gemv_32000x4096_b1": ("Q6_K", 32000, 4096, 1),
 }
-# HBM bytes per launch of the b1 workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.9973, calibrated on a plain copy) + WRITE_SIZE (x1.0);
+# the runs and their raw readings are in profiles/q4k_gemv_11008x4096_b1.md. Workloads not measured report null.
+MEASURED_TRAFFIC_BYTES = {"q4k_gemv_11008x4096_b1": 25666560}
 
 
 def algorithmic_bytes(enc, n, k, m):
@@ -91,6 +92,8 @@ def main():
     ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
+    ap.add_argument("--hbm-only", action="store_true", help="skip the cache-warm pass and the read probe, so every launch of the "
+                    "kernel in a profile is one of the rotating-copy (HBM) kind")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE", help="launch-shape knob (skainet_hip_set_tuning)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -134,10 +137,15 @@ def main():
     t0 = time.perf_counter()
     ms = run(weights, a.steps)              # exactly K timed steps, HIP events on the launch stream
     wall = time.perf_counter() - t0
-    ms_warm = run(weights[:1], a.steps)     # same K steps on one copy: served by the memory-side cache
+    ms_probe = float("nan")
+    if a.hbm_only:
+        ms_warm = float("nan")
+    else:
+        ms_warm = run(weights[:1], a.steps)     # same K steps on one copy: served by the memory-side cache
     # ceiling for a read-once pass over the same rotating copies: a kernel that only loads (no arithmetic)
     probe_iters = min(a.steps, 500)
-    ms_probe = min(kernels.read_probe(store, packed.size, probe_iters, g) for g in (512, 2048))
+    if not a.hbm_only:
+        ms_probe = min(kernels.read_probe(store, packed.size, probe_iters, g) for g in (512, 2048))
     gbs_probe = packed.size / (ms_probe / probe_iters * 1e-3) / 1e9
     ms_per_step = ms / a.steps
     gbs = alg / (ms_per_step * 1e-3) / 1e9
@@ -171,7 +179,7 @@ def main():
         out["extra"]["PARITY_FAILED"] = True
     if not a.skip_cpu:
         out["cpu_baseline"] = cpu_baseline(enc, n, k, m, packed, x)
-    print(json.dumps(out))
+    print(json.dumps(out).replace("NaN", "null"))
     sys.exit(0 if err <= 1e-3 else 1)
 
 
