@@ -37,7 +37,12 @@ WORKLOADS = {
     "q4k_gemv_11008x4096_b8": ("Q4_K", 11008, 4096, 8),
     "q8_0_gemv_4096x4096_b1": ("Q8_0", 4096, 4096, 1),
     "q6k_gemv_32000x4096_b1": ("Q6_K", 32000, 4096, 1),
+    # prefill: batch > 8 goes to the MFMA dequant-GEMM and is reported in TFLOP/s against the bf16 MFMA peak
+    "q4k_gemm_512x4096x4096": ("Q4_K", 4096, 4096, 512),
+    "q6k_gemm_512x32000x4096": ("Q6_K", 32000, 4096, 512),
+    "q4k_gemm_512x14336x4096": ("Q4_K", 14336, 4096, 512),
 }
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.9973, calibrated on a plain copy) + WRITE_SIZE (x1.0);
 # the runs and their raw readings are in profiles/q4k_gemv_11008x4096_b1.md. Workloads not measured report null.
 MEASURED_TRAFFIC_BYTES = {"q4k_gemv_11008x4096_b1": 25666560}
@@ -51,7 +56,10 @@ def algorithmic_bytes(enc, n, k, m):
 
 def cpu_baseline(enc, n, k, m, packed, x, budget_s=12.0):
     """The reference's native row-major kernel (int8-activation path for K-quants, 4-participant row pool) on this
-    host; protocol of the reference microbench: >= 20 warm-ups, median of >= 21 samples. m rows = m calls."""
+    host; protocol of the reference microbench: >= 20 warm-ups, median of >= 21 samples. m rows = m calls (the
+    reference has no packed GEMM); for a prefill batch a bounded sample of rows is timed and scaled to the batch."""
+    m_full = m
+    m = min(m, 16)
     from oracle import lib as L
     short = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k"}[enc]
     ref = L.ref()
@@ -78,6 +86,12 @@ def cpu_baseline(enc, n, k, m, packed, x, budget_s=12.0):
         call()
         samples.append(time.perf_counter() - t0)
     med = float(np.median(samples))
+    if m_full > 8:
+        tflops = 2.0 * m * n * k / med / 1e12
+        return {"value": round(tflops, 5), "unit": "TFLOP/s", "cores": cores, "kind": kind,
+                "sample": f"{m} of the {m_full} activation rows, one skainet_{short}_matmul_rm call per row, {warm} warm-ups + "
+                          f"median of {samples_n} samples ({med / m * 1e3:.3f} ms/row -> {med / m * m_full * 1e3:.1f} ms/step, "
+                          f"host has {os.cpu_count()} logical cores)"}
     gbs = algorithmic_bytes(enc, n, k, m) / med / 1e9
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": cores, "kind": kind,
             "sample": f"same workload, {warm} warm-ups + median of {samples_n} calls of skainet_{short}_matmul_rm "
@@ -87,7 +101,7 @@ def cpu_baseline(enc, n, k, m, packed, x, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--steps", type=int, default=2000, help="timed steps (default 2000; 200 for the GEMM workloads)")
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
@@ -123,8 +137,13 @@ def main():
     weights = [kernels.DeviceWeight.wrap(enc, t, n, k) for t in store]
     xd = torch.from_numpy(x).cuda()
     yd = torch.empty((m, n), dtype=torch.float32, device="cuda")
-    kind = 0
+    kind = 0 if m <= 8 else 1
     graph = not a.no_graph
+    is_gemm = kind == 1
+    if is_gemm and a.steps == 2000:
+        a.steps, a.warmup = 200, 20
+    weights[0].matmul(xd, m, yd, kind)      # sizes the library's scratch before any stream capture
+    torch.cuda.synchronize()
 
     def run(ws, iters):
         torch.cuda.synchronize()
@@ -156,18 +175,26 @@ def main():
     weights[0].dequantize(dense)
     want = (dense.double() @ xd[0].double()).cpu().numpy()
     got = yd[0].cpu().numpy()
-    err = float((np.abs(got - want) / np.maximum(np.abs(want), 1e-2 * np.abs(want).max())).max())
+    floor = 1.0 if is_gemm else 1e-2        # bf16 operands: error taken against the largest output
+    err = float((np.abs(got - want) / np.maximum(np.abs(want), floor * np.abs(want).max())).max())
+    tol = 2e-2 if is_gemm else 1e-3
     del dense
 
+    flops = 2.0 * m * n * k
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
     out = {
-        "metric": "Q4_K GEMV GB/s" if enc == "Q4_K" else f"{enc} GEMV GB/s",
-        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "metric": f"{enc} GEMM TFLOP/s" if is_gemm else f"{enc} GEMV GB/s",
+        "value": round(tflops if is_gemm else gbs, 2), "unit": "TFLOP/s" if is_gemm else "GB/s", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "bf16 x bf16 -> f32" if is_gemm else "f32", "data": "synthetic",
         "config": {"workload": a.workload, "encoding": enc, "rows": n, "cols": k, "batch": m,
                    "weight_copies_rotated": copies, "launch": "hip-graph replay" if graph else "host loop"},
-        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)},
+        "roofline": ({"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                      "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}
+                     if is_gemm else
+                     {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}),
         "extra": {"algorithmic_bytes_per_step": alg, "cache_warm_GBps": round(gbs_warm, 2),
                   "cache_warm_ms_per_step": round(ms_warm / a.steps, 6), "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
                   "read_only_probe_GBps_same_buffers": round(gbs_probe, 2),
@@ -175,12 +202,15 @@ def main():
                   "wall_s_timed_region": round(wall, 4), "max_normalized_err_vs_fp64_decode_matmul": err,
                   "device": _lib.hip().skainet_hip_device_name().decode()},
     }
-    if err > 1e-3:
+    if is_gemm:
+        out["extra"]["flops_per_step"] = flops
+        out["extra"]["step_includes"] = "fp32->bf16 activation pass + (split-K only) zero fill + dequant-GEMM kernel"
+    if err > tol:
         out["extra"]["PARITY_FAILED"] = True
     if not a.skip_cpu:
         out["cpu_baseline"] = cpu_baseline(enc, n, k, m, packed, x)
     print(json.dumps(out).replace("NaN", "null"))
-    sys.exit(0 if err <= 1e-3 else 1)
+    sys.exit(0 if err <= tol else 1)
 
 
 if __name__ == "__main__":

@@ -198,7 +198,8 @@ SKAINET_HIP_API int32_t skainet_hip_f32_add_dev(const float* a, const float* b, 
 SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
 
 /* Launch-shape knobs for experiments (defaults are the measured best). Keys: "gemv_waves_per_cu",
- * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares), "q4k_rows_enable".
+ * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares), "q4k_rows_enable",
+ * "gemm_ksplit" (K splits of the MFMA GEMM, 0 = automatic).
  * 0 when the key is known. No reference counterpart. */
 SKAINET_HIP_API int32_t skainet_hip_set_tuning(const char* key, int32_t value);
 

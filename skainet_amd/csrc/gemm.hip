@@ -1,9 +1,290 @@
-// Prefill dequant-GEMM entry (placeholder body until the MFMA kernel lands in this file).
+// Prefill dequant-GEMM on the matrix cores:  C[m, n] = sum_k A[m, k] * dequant(W[n, k])
+//   A fp32 [M, K] (rounded once to bf16), W packed Q4_K / Q6_K / Q8_0 in canonical row-major GGUF order,
+//   products bf16 x bf16 on v_mfma_f32_32x32x16_bf16, fp32 accumulation, C fp32 [M, N].
+//
+// What it replaces: the reference has no packed GEMM -- a [rows, k] activation is `rows` GEMV calls
+//   /root/reference/skainet-backends/skainet-backend-api/src/commonMain/kotlin/sk/ainet/backend/api/kernel/PackedViewMatmulKernel.kt:69-108
+//   /root/reference/skainet-backends/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/FfmRowMajorKernels.kt:94-104
+// so the weight is re-streamed once per row. Here a weight tile is decoded once into LDS and reused by 256 rows.
+// The decode is the reference's block arithmetic (code * (d * sc) - dmin * m, (d * sc) * q, code * d) in fp32,
+// rounded to bf16 (nearest even) when it is parked in LDS.
+//
+// Tiling (MFMA-bound): workgroup tile 256 (M) x 128 (N), K step 64, 256 threads = 4 waves in a 2 x 2 grid, each wave
+// owning a 128 x 64 patch = 4 x 2 MFMA tiles of 32 x 32 (128 accumulator registers per lane). Per K step a thread
+// decodes 32 consecutive weights of one row (one Q4_K sub-block / one Q6_K quarter / one Q8_0 block) and copies
+// 8 x 16 bytes of the bf16 activation tile; LDS rows are padded to 144 bytes so the 16-byte fragment reads of 32
+// consecutive rows fall on distinct banks. Two LDS stages: the next step's global loads and decode overlap the
+// current step's MFMAs, one barrier per step. When the tile grid is smaller than the chip, K is split across
+// gridDim.z and the partial tiles are combined with fp32 atomic adds into a zeroed C.
 #include "common.h"
 
 namespace skh {
-int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
-int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y) {
-    return launch_gemv(enc, w, x, m, k, n, y);
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int GM = 256, GN = 128, GK = 64;
+constexpr int GSTRIDE = GK + 8;                               // bf16 elements per LDS row (144 bytes)
+constexpr int G_A_ELEMS = GM * GSTRIDE, G_W_ELEMS = GN * GSTRIDE;
+constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16);
+
+void* kernel_workspace(size_t bytes);   // shim.hip
+int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);   // gemv.hip
+
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, __bf16* __restrict__ out, int64_t n4) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const float4 v = reinterpret_cast<const float4*>(in)[i];
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    bf16x4 o = {(__bf16)v.x, (__bf16)v.y, (__bf16)v.z, (__bf16)v.w};
+    reinterpret_cast<bf16x4*>(out)[i] = o;
 }
+
+__global__ __launch_bounds__(256) void zero_f32_kernel(float* out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = 0.f;
+}
+
+// ---- raw bytes a thread needs to decode 32 consecutive weights of one row, per encoding ----
+struct RawQ4K { uint4 hdr, q0, q1; };
+struct RawQ6K { uint32_t ql[8], qh[8]; uint32_t sc, d; };
+struct RawQ80 { uint32_t d; uint32_t q[8]; };
+
+// `e` = element offset inside the row, a multiple of 32.
+__device__ __forceinline__ void load_raw(RawQ4K& r, const uint8_t* row, int e) {
+    const uint8_t* blk = row + (e >> 8) * Q4K_BYTES;
+    const int g = (e & 255) >> 6;                     // 32-byte nibble group holding sub-blocks 2g, 2g+1
+    r.hdr = *reinterpret_cast<const uint4*>(blk);
+    r.q0 = *reinterpret_cast<const uint4*>(blk + 16 + g * 32);
+    r.q1 = *reinterpret_cast<const uint4*>(blk + 32 + g * 32);
+}
+__device__ __forceinline__ void decode32(const RawQ4K& r, int e, float* w) {
+    const int sb = (e & 255) >> 5;
+    const float d = half_bits_to_float_fast(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(r.hdr.x >> 16);
+    // ggml get_scale_min_k4 on the 12 scale bytes s[0..11] (hdr.y = s[0..3], hdr.z = s[4..7], hdr.w = s[8..11])
+    const int sh = (sb & 3) * 8;
+    const uint32_t sa = (r.hdr.y >> sh) & 0xFFu, sbm = (r.hdr.z >> sh) & 0xFFu, st = (r.hdr.w >> sh) & 0xFFu;
+    const uint32_t sc = sb < 4 ? (sa & 63u) : ((st & 0xFu) | ((sa >> 6) << 4));
+    const uint32_t mn = sb < 4 ? (sbm & 63u) : ((st >> 4) | ((sbm >> 6) << 4));
+    const float scale = d * (float)sc, offset = dmin * (float)mn;
+    const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+    const int shift = (sb & 1) * 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t v = (q[i] >> shift) & 0x0F0F0F0Fu;
+        w[4 * i + 0] = fmaf(ubyte0_to_float(v), scale, -offset);
+        w[4 * i + 1] = fmaf(ubyte1_to_float(v), scale, -offset);
+        w[4 * i + 2] = fmaf(ubyte2_to_float(v), scale, -offset);
+        w[4 * i + 3] = fmaf(ubyte3_to_float(v), scale, -offset);
+    }
+}
+
+__device__ __forceinline__ void load_raw(RawQ6K& r, const uint8_t* row, int e) {
+    const uint8_t* blk = row + (e >> 8) * Q6K_BYTES;
+    const int half = (e & 255) >> 7, kq = (e & 127) >> 5;   // quarter kq of the half: output offset 32 * kq
+    const uint8_t* ql = blk + half * 64 + (kq & 1) * 32;
+    const uint8_t* qh = blk + 128 + half * 32;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { r.ql[i] = load_u32_a2(ql + 4 * i); r.qh[i] = load_u32_a2(qh + 4 * i); }
+    // the two int8 scales of this quarter: sc[half * 8 + 2 * kq] (elements 0..15) and [.. + 1] (elements 16..31)
+    r.sc = load_u16(blk + 192 + half * 8 + 2 * kq);
+    r.d = load_u16(blk + 208);
+}
+__device__ __forceinline__ void decode32(const RawQ6K& r, int e, float* w) {
+    const int kq = (e & 127) >> 5;
+    const float d = half_bits_to_float_fast(r.d);
+    const float s0 = d * (float)(int8_t)(r.sc & 0xFF), s1 = d * (float)(int8_t)(r.sc >> 8);
+    const int nib = (kq >> 1) * 4, hs = 2 * kq;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t lo = (r.ql[i] >> nib) & 0x0F0F0F0Fu;
+        const uint32_t hi = ((r.qh[i] >> hs) & 0x03030303u) << 4;
+        const uint32_t c = lo | hi;                          // four 6-bit codes, one per byte
+        const float sc = i < 4 ? s0 : s1;
+        w[4 * i + 0] = sc * (ubyte0_to_float(c) - 32.f);
+        w[4 * i + 1] = sc * (ubyte1_to_float(c) - 32.f);
+        w[4 * i + 2] = sc * (ubyte2_to_float(c) - 32.f);
+        w[4 * i + 3] = sc * (ubyte3_to_float(c) - 32.f);
+    }
+}
+
+__device__ __forceinline__ void load_raw(RawQ80& r, const uint8_t* row, int e) {
+    const uint8_t* blk = row + (e >> 5) * Q80_BYTES;
+    r.d = load_u16(blk);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.q[i] = load_u32_a2(blk + 2 + 4 * i);
+}
+__device__ __forceinline__ void decode32(const RawQ80& r, int, float* w) {
+    const float d = half_bits_to_float_fast(r.d);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[4 * i + j] = (float)(int8_t)(r.q[i] >> (8 * j)) * d;
+    }
+}
+
+template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES>
+__global__ __launch_bounds__(256) void dequant_gemm_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
+                                                           float* __restrict__ c, int m, int n, int k, int k_chunk,
+                                                           int use_atomics) {
+    extern __shared__ __attribute__((aligned(16))) __bf16 smem[];
+    // stage `buf` (0 / 1): activation tile, then weight tile
+    auto a_tile = [&](int buf) { return smem + buf * (G_A_ELEMS + G_W_ELEMS); };
+    auto w_tile = [&](int buf) { return smem + buf * (G_A_ELEMS + G_W_ELEMS) + G_A_ELEMS; };
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * GM, n0 = blockIdx.x * GN;
+    const int k_begin = blockIdx.z * k_chunk;
+    const int k_end = min(k, k_begin + k_chunk);
+    const int nsteps = (k_end - k_begin) / GK;
+    const int64_t row_bytes = (int64_t)(k / BLOCK_ELEMS) * BLOCK_BYTES;
+
+    // this thread's share of the weight tile: 32 consecutive elements of one row per K step
+    const int wrow = tid >> 1, wsub = tid & 1;
+    const uint8_t* wrow_ptr = w + (int64_t)min(n0 + wrow, n - 1) * row_bytes;   // rows past N decode a valid row, never stored
+
+    uint4 areg[8];
+    Raw wraw;
+    auto load_global = [&](int step) {
+        const int k0 = k_begin + step * GK;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int p = tid + 256 * j, row = p >> 3, kp = p & 7;
+            areg[j] = make_uint4(0u, 0u, 0u, 0u);
+            if (m0 + row < m) areg[j] = *reinterpret_cast<const uint4*>(a + (int64_t)(m0 + row) * k + k0 + 8 * kp);
+        }
+        load_raw(wraw, wrow_ptr, k0 + 32 * wsub);
+    };
+    auto store_lds = [&](int buf, int step) {
+        const int k0 = k_begin + step * GK;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int p = tid + 256 * j, row = p >> 3, kp = p & 7;
+            *reinterpret_cast<uint4*>(a_tile(buf) + row * GSTRIDE + 8 * kp) = areg[j];
+        }
+        float wv[32];
+        decode32(wraw, k0 + 32 * wsub, wv);
+        __bf16* dst = w_tile(buf) + wrow * GSTRIDE + 32 * wsub;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bf16x8 o;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = (__bf16)wv[8 * i + j];
+            *reinterpret_cast<bf16x8*>(dst + 8 * i) = o;
+        }
+    };
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    if (nsteps > 0) {
+        load_global(0);
+        store_lds(0, 0);
+    }
+    __syncthreads();
+
+    const int fr = lane & 31, fk = (lane >> 5) * 8;   // fragment row inside a 32-row tile, first k of this lane's 8
+    for (int step = 0; step < nsteps; ++step) {
+        const int buf = step & 1;
+        if (step + 1 < nsteps) load_global(step + 1);
+        const __bf16* at = a_tile(buf) + (128 * wm + fr) * GSTRIDE + fk;
+        const __bf16* wt = w_tile(buf) + (64 * wn + fr) * GSTRIDE + fk;
+#pragma unroll
+        for (int kk = 0; kk < GK; kk += 16) {
+            bf16x8 af[4], bf[2];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(at + 32 * i * GSTRIDE + kk);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(wt + 32 * j * GSTRIDE + kk);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        if (step + 1 < nsteps) store_lds(buf ^ 1, step + 1);
+        __syncthreads();
+    }
+
+    // accumulator element e of lane l sits at row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32 of its 32 x 32 tile
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + 64 * wn + 32 * j + (lane & 31);
+            if (col >= n) continue;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = m0 + 128 * wm + 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (row < m) {
+                    float* dst = c + (int64_t)row * n + col;
+                    if (use_atomics) atomicAdd(dst, acc[i][j][e]);
+                    else *dst = acc[i][j][e];
+                }
+            }
+        }
+}
+
+template <class Raw, int BE, int BB>
+static int launch_gemm_enc(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk, int atomics,
+                           hipStream_t s) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&dequant_gemm_kernel<Raw, BE, BB>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)G_SMEM));
+        attr_set = true;
+    }
+    dequant_gemm_kernel<Raw, BE, BB><<<grid, dim3(256), G_SMEM, s>>>(a, w, c, m, n, k, k_chunk, atomics);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
+static int g_gemm_ksplit = 0;   // 0 = choose from the tile count
+void set_gemm_ksplit(int v) { g_gemm_ksplit = v; }
+
+int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y) {
+    if (m <= 0 || n <= 0) return 0;
+    if (!is_packed(enc)) return set_error("gemm: unsupported encoding %d", enc);
+    if (k <= 0 || k % block_elems(enc) != 0)
+        return set_error("gemm: inputDim must be a positive multiple of %d; got %d", block_elems(enc), k);
+    // shapes the tile loader cannot take (a Q8_0 row that is not a whole number of 64-element steps, unaligned
+    // operands) go through the row kernels: same result to fp32 rounding, the weight streamed once per 4 rows
+    if (k % GK != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15))
+        return launch_gemv(enc, w, x, m, k, n, y);
+    hipStream_t s = current_stream();
+    __bf16* a = static_cast<__bf16*>(kernel_workspace((size_t)m * k * sizeof(__bf16)));
+    if (!a) return -1;
+    const int64_t n4 = (int64_t)m * k / 4;
+    f32_to_bf16_kernel<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s>>>(x, a, n4);
+    SKH_CHECK(hipGetLastError());
+
+    const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;
+    const int tiles = tiles_m * tiles_n;
+    // K chunks are whole 256-element groups so every encoding's blocks stay intact
+    const int kgroups = (k + 255) / 256;
+    int ksplit = g_gemm_ksplit;
+    if (ksplit <= 0) {
+        ksplit = 1;
+        if (tiles < num_cus()) ksplit = (num_cus() + tiles - 1) / tiles;
+        if (ksplit > 8) ksplit = 8;
+    }
+    if (ksplit > kgroups) ksplit = kgroups;
+    const int k_chunk = ((kgroups + ksplit - 1) / ksplit) * 256;
+    ksplit = (k + k_chunk - 1) / k_chunk;
+    if (ksplit > 1) {
+        const int64_t cn = (int64_t)m * n;
+        zero_f32_kernel<<<dim3((unsigned)((cn + 255) / 256)), dim3(256), 0, s>>>(y, cn);
+        SKH_CHECK(hipGetLastError());
+    }
+    const dim3 grid(tiles_n, tiles_m, ksplit);
+    if (enc == ENC_Q4_K) return launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(a, w, y, m, n, k, grid, k_chunk, ksplit > 1, s);
+    if (enc == ENC_Q6_K) return launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(a, w, y, m, n, k, grid, k_chunk, ksplit > 1, s);
+    return launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(a, w, y, m, n, k, grid, k_chunk, ksplit > 1, s);
+}
+
 }  // namespace skh
