@@ -98,12 +98,126 @@ def cpu_baseline(enc, n, k, m, packed, x, budget_s=12.0):
                       f"({med * 1e3:.3f} ms/step, host has {os.cpu_count()} logical cores)"}
 
 
+DECODER_WORKLOADS = {
+    # name -> (config overrides, prompt tokens, layers with values of their own)
+    "llama3_8b_decode": ({}, 512, 1),
+    # a quarter-depth stack for quick runs; same per-layer shapes
+    "llama3_8b_8layers_decode": ({"layers": 8}, 512, 1),
+}
+
+
+def cpu_baseline_decode(cfg, host, ctx):
+    """Reference native kernels over one decoder layer's four Q4_K products and the Q6_K head, scaled to the stack:
+    the CPU cost of the packed products of one decode step (attention, norms and RoPE left out, which favours the CPU)."""
+    from oracle import lib as L
+    ref = L.ref()
+    if ref is not None:
+        q4, q6, kind, cores = ref.skainet_q4k_matmul_rm, ref.skainet_q6k_matmul_rm, "reference", 4
+    else:
+        lib = L.oracle(fast=True)
+        q4, q6, kind, cores = lib.orc_native_q4k_matmul_rm, lib.orc_native_q6k_matmul_rm, "port", 1
+    rng = np.random.default_rng(1)
+    shapes = [("l0.wqkv", cfg.q_dim + 2 * cfg.kv_dim, cfg.hidden), ("l0.wo", cfg.hidden, cfg.q_dim),
+              ("l0.w_gate_up", 2 * cfg.ffn, cfg.hidden), ("l0.w_down", cfg.hidden, cfg.ffn)]
+    xs = {k: rng.standard_normal(k).astype(np.float32) for k in {s[2] for s in shapes} | {cfg.hidden}}
+    ys = {n: np.empty(n, np.float32) for n in {s[1] for s in shapes} | {cfg.vocab}}
+
+    def layer():
+        for name, n, k in shapes:
+            q4(L.fp(xs[k]), 0, L.u8(host[name]), 0, k, n, L.fp(ys[n]), 0)
+
+    def head():
+        q6(L.fp(xs[cfg.hidden]), 0, L.u8(host["head"]), 0, cfg.hidden, cfg.vocab, L.fp(ys[cfg.vocab]), 0)
+
+    def med(fn, reps):
+        fn()
+        t = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            t.append(time.perf_counter() - t0)
+        return float(np.median(t))
+
+    t_layer, t_head = med(layer, 41), med(head, 21)
+    per_token = cfg.layers * t_layer + t_head
+    return {"value": round(1.0 / per_token, 3), "unit": "tok/s", "cores": cores, "kind": kind,
+            "sample": f"one layer's four Q4_K products (median of 41: {t_layer * 1e3:.2f} ms) x {cfg.layers} layers + the Q6_K head "
+                      f"(median of 21: {t_head * 1e3:.2f} ms); attention, norms, RoPE not included; host has {os.cpu_count()} logical cores"}
+
+
+def bench_decoder(a):
+    """Synthetic Llama-3-8B-shape stack: prefill of 512 random token ids, then greedy decode; a step = one decoded token."""
+    from dataclasses import replace
+    from skainet_amd import _lib, kernels
+    from skainet_amd.decoder import LLAMA3_8B, LlamaDecoder, LlamaWeights
+    overrides, prompt_len, distinct = DECODER_WORKLOADS[a.workload]
+    cfg = replace(LLAMA3_8B, **overrides)
+    steps = 128 if a.steps == 2000 else a.steps
+    warmup = 8 if a.warmup == 200 else a.warmup
+    t0 = time.perf_counter()
+    w = LlamaWeights(cfg, seed=20251125, keep_host=not a.skip_cpu, distinct_layers=distinct)
+    t_weights = time.perf_counter() - t0
+    dec = LlamaDecoder(w, max_prefill=prompt_len)
+    prompt = np.random.default_rng(7).integers(0, cfg.vocab, prompt_len)
+    dec.prefill(prompt)                      # warm-up pass: sizes the library's scratch
+    kernels.sync()
+    with kernels.Timer() as t:
+        first = dec.prefill(prompt)
+    prefill_ms = t.ms
+    toks = [first] + [int(x) for x in dec.decode(max(1, warmup), use_graph=not a.no_graph)]
+    kernels.sync()
+    pos0 = dec.position()
+    t0 = time.perf_counter()
+    with kernels.Timer() as t:               # HIP events on the launch stream around exactly K decode steps
+        if a.no_graph:
+            for _ in range(steps):
+                dec._decode_step()
+        else:
+            for _ in range(steps):
+                dec._graph.launch()
+    wall = time.perf_counter() - t0
+    ms = t.ms
+    assert dec.position() == pos0 + steps
+    generated = dec.generated_tokens()
+    ms_per_tok = ms / steps
+    ctx_mid = pos0 + steps // 2
+    alg = w.decode_bytes_per_token(ctx_mid)
+    gbs = alg / (ms_per_tok * 1e-3) / 1e9
+    # sanity of the timed path: the last emitted token is the first arg-max of the logits left on the device
+    logits = dec.last_logits()
+    ok = bool(np.isfinite(logits).all()) and int(np.argmax(logits)) == int(generated[-1])
+    out = {
+        "metric": "decode tok/s", "value": round(1e3 / ms_per_tok, 2), "unit": "tok/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(ms_per_tok, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 (packed Q4_K / Q6_K weights)", "data": "synthetic",
+        "config": {"workload": a.workload, "layers": cfg.layers, "hidden": cfg.hidden, "heads": cfg.heads,
+                   "kv_heads": cfg.kv_heads, "head_dim": cfg.head_dim, "ffn": cfg.ffn, "vocab": cfg.vocab, "batch": 1,
+                   "prompt_tokens": prompt_len, "decoded_tokens": steps, "context_at_end": pos0 + steps,
+                   "weights": f"random init N(0, 0.02^2), Q4_K linears + Q6_K head; {distinct} layer(s) of distinct values, "
+                              f"every layer in its own HBM allocation",
+                   "launch": "host loop" if a.no_graph else "hip-graph replay of one decode step"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "extra": {"algorithmic_bytes_per_token": alg, "packed_weight_bytes": w.packed_bytes(),
+                  "prefill_ms": round(prefill_ms, 3), "prefill_tok_per_s": round(prompt_len / (prefill_ms * 1e-3), 1),
+                  "hbm_bound_ms_per_token": round(alg / (HBM_PEAK_GBS * 1e9) * 1e3, 5),
+                  "wall_s_timed_region": round(wall, 4), "weight_build_s": round(t_weights, 1),
+                  "first_tokens": toks[:8], "device": _lib.hip().skainet_hip_device_name().decode()},
+    }
+    if not ok:
+        out["extra"]["PARITY_FAILED"] = True
+    if not a.skip_cpu:
+        out["cpu_baseline"] = cpu_baseline_decode(cfg, w.host, ctx_mid)
+    print(json.dumps(out).replace("NaN", "null"))
+    sys.exit(0 if ok else 1)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000, help="timed steps (default 2000; 200 for the GEMM workloads)")
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
     ap.add_argument("--hbm-only", action="store_true", help="skip the cache-warm pass and the read probe, so every launch of the "
@@ -123,6 +237,8 @@ def main():
         key, _, val = kv.partition("=")
         _lib.check(_lib.hip().skainet_hip_set_tuning(key.encode(), int(val)), "set_tuning")
 
+    if a.workload in DECODER_WORKLOADS:
+        bench_decoder(a)
     enc, n, k, m = WORKLOADS[a.workload]
     rng = np.random.default_rng(20251125)
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)

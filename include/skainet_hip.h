@@ -186,6 +186,13 @@ SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_dev(const float* q, const float* k,
     int32_t batch, int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t head_dim,
     float scale, int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths,
     const float* mask, int32_t mask_b, int32_t mask_h, int32_t mask_q, int32_t mask_k);
+/* The same attention reading K / V in place from a cache laid out [batch, kv_heads, kv_capacity, head_dim] (the
+ * per-layer layout KvCacheStore.readKeys / readValues return,
+ * skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/storage/KvCacheStore.kt:125-149): only the
+ * first seq_kv rows of every head are keys, kv_capacity >= seq_kv is the row count of the storage. No additive mask. */
+SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_cache_dev(const float* q, const float* k_cache, const float* v_cache, float* out,
+    int32_t batch, int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t kv_capacity, int32_t head_dim,
+    float scale, int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths);
 
 /* Decoder glue with the reference ops' semantics (device pointers):
  *   silu_mul: out[i] = gate[i] * (1 / (1 + exp(-gate[i]))) * up[i]   (NAT:532-539 unary op 2 then binary mul,
@@ -196,6 +203,39 @@ SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_dev(const float* q, const float* k,
 SKAINET_HIP_API int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* out, int64_t n);
 SKAINET_HIP_API int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int64_t n);
 SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
+
+/* Decoder glue the reference keeps in its external transformer repository (no counterpart in /root/reference; the
+ * semantics are the standard Llama ones and are checked against closed forms):
+ *   rope_scatter: token t, head h read at in + t*in_row_pitch + h*head_dim (a column slice of a token-major projection
+ *                 output) -> out element (h, row0 + t, d) at h*out_head_stride + (row0+t)*head_dim + d,
+ *                 row0 = *pos_dev when pos_dev != NULL else pos_start if out_row_is_pos, else 0; rotate != 0 rotates the
+ *                 adjacent pairs (x[2i], x[2i+1]) by (pos + t) * theta^(-2i/head_dim), rotate == 0 copies (cache values).
+ *                 Writes straight into the [kv_heads, positions, head_dim] layout KvCacheStore.readKeys/readValues expose
+ *                 (REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/storage/KvCacheStore.kt:125-149).
+ *   heads_to_rows: [heads, tokens, head_dim] -> [tokens, heads*head_dim].
+ *   swiglu_rows:   rows of [gate | up] (2*ffn floats) -> out[r, i] = silu(gate[r, i]) * up[r, i], silu as in silu_mul.
+ *   i32_increment: *value += delta on the device (the position counter of a recorded decode step). */
+SKAINET_HIP_API int32_t skainet_hip_f32_rope_scatter_dev(const float* in, int64_t in_row_pitch, float* out, int32_t tokens,
+    int32_t heads, int32_t head_dim, int32_t pos_start, const int32_t* pos_dev, float theta, int32_t rotate,
+    int64_t out_head_stride, int32_t out_row_is_pos);
+SKAINET_HIP_API int32_t skainet_hip_f32_swiglu_rows_dev(const float* gate_up, float* out, int32_t rows, int32_t ffn);
+SKAINET_HIP_API int32_t skainet_hip_f32_heads_to_rows_dev(const float* in, float* out, int32_t heads, int32_t tokens, int32_t head_dim);
+SKAINET_HIP_API int32_t skainet_hip_i32_increment_dev(int32_t* value, int32_t delta);
+/* dst[index_dev[0] + offset] = src[0], all on the device: appends a sampled token to a log at the device-side position. */
+SKAINET_HIP_API int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t* index_dev, int32_t offset, const int32_t* src);
+
+/* HIP graphs (no reference counterpart; for launch-bound loops such as a decode step): graph_begin redirects this
+ * thread's device entries into a stream capture, graph_end closes it and returns an executable graph (NULL on
+ * failure), graph_launch replays it on the calling thread's stream (in order with that thread's eager device
+ * entries), graph_sync waits for that stream. Nothing that
+ * allocates (a first call that grows the library's scratch) may run between begin and end: run the sequence once
+ * eagerly first. Only kernel launches are recorded. */
+typedef struct skainet_hip_graph skainet_hip_graph;
+SKAINET_HIP_API int32_t skainet_hip_graph_begin(void);
+SKAINET_HIP_API skainet_hip_graph* skainet_hip_graph_end(void);
+SKAINET_HIP_API int32_t skainet_hip_graph_launch(skainet_hip_graph* graph);
+SKAINET_HIP_API int32_t skainet_hip_graph_sync(skainet_hip_graph* graph);
+SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
 
 /* Launch-shape knobs for experiments (defaults are the measured best). Keys: "gemv_waves_per_cu",
  * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares), "q4k_rows_enable",

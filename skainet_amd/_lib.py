@@ -63,9 +63,21 @@ SIGNATURES = {
     "skainet_hip_f32_layer_norm_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _f32]),
     "skainet_hip_f32_softmax_rows_dev": (_i32, [_vp, _vp, _i32, _i32, _i32]),
     "skainet_hip_f32_sdpa_dev": (_i32, _SDPA),
+    "skainet_hip_f32_sdpa_cache_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _i32,
+                                              _vp]),
     "skainet_hip_f32_silu_mul_dev": (_i32, [_vp, _vp, _vp, _i64]),
     "skainet_hip_f32_add_dev": (_i32, [_vp, _vp, _vp, _i64]),
     "skainet_hip_f32_argmax_rows_dev": (_i32, [_vp, _i32, _i32, _vp]),
+    "skainet_hip_f32_rope_scatter_dev": (_i32, [_vp, _i64, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _i32, _i64, _i32]),
+    "skainet_hip_i32_store_at_dev": (_i32, [_vp, _vp, _i32, _vp]),
+    "skainet_hip_f32_swiglu_rows_dev": (_i32, [_vp, _vp, _i32, _i32]),
+    "skainet_hip_f32_heads_to_rows_dev": (_i32, [_vp, _vp, _i32, _i32, _i32]),
+    "skainet_hip_i32_increment_dev": (_i32, [_vp, _i32]),
+    "skainet_hip_graph_begin": (_i32, []),
+    "skainet_hip_graph_end": (_vp, []),
+    "skainet_hip_graph_launch": (_i32, [_vp]),
+    "skainet_hip_graph_sync": (_i32, [_vp]),
+    "skainet_hip_graph_free": (None, [_vp]),
     "skainet_hip_set_tuning": (_i32, [C.c_char_p, _i32]),
 }
 

@@ -101,6 +101,15 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
     if (i < n) { const float g = gate[i]; out[i] = g * (1.0f / (1.0f + expf(-g))) * up[i]; }
 }
 
+// SwiGLU over rows holding [gate | up]: out[r, i] = silu(gu[r, i]) * gu[r, ffn + i].
+__global__ __launch_bounds__(256) void swiglu_rows_kernel(const float* __restrict__ gu, float* __restrict__ out, int64_t n, int ffn) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t r = i / ffn, c = i % ffn;
+    const float g = gu[r * 2 * ffn + c];
+    out[i] = g * (1.0f / (1.0f + expf(-g))) * gu[r * 2 * ffn + ffn + c];
+}
+
 __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                   float* __restrict__ out, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -146,6 +155,90 @@ __global__ __launch_bounds__(256) void relayout_to_row_major_kernel(const uint8_
     for (int i = threadIdx.x; i < block_bytes / 2; i += blockDim.x) d[i] = s[i];
 }
 
+// Rotary position embedding fused with the head-major scatter a KV cache / attention operand needs.
+//   in  token t, head h at in + t * in_row_pitch + h * head_dim (a column slice of a projection's token-major output;
+//       in_row_pitch == heads * head_dim when the slice is the whole row)
+//   out [heads, *, head_dim]: element (h, row0 + t, d) at h * out_head_stride + (row0 + t) * head_dim + d,
+//       row0 = *pos_dev (when given) or pos_start: the absolute position of token 0, which is also its cache row
+//       when out_row_is_pos != 0 (else rows start at 0).
+//   rotate != 0: pairs (x[2i], x[2i+1]) of every head are rotated by (row0 + t) * theta^(-2i / head_dim)
+//       (the adjacent-pair convention GGUF Llama weights use); rotate == 0 copies (values of the cache).
+// The reference has no RoPE (it lives in the external transformer repo), so this op has no reference parity; the
+// tests check it against the closed form in float64.
+__global__ __launch_bounds__(256) void rope_scatter_kernel(const float* __restrict__ in, int64_t in_row_pitch,
+                                                           float* __restrict__ out, int tokens,
+                                                           int heads, int head_dim, int pos_start,
+                                                           const int32_t* __restrict__ pos_dev, float theta, int rotate,
+                                                           int64_t out_head_stride, int out_row_is_pos) {
+    const int half = head_dim >> 1;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (token, head, pair)
+    if (idx >= (int64_t)tokens * heads * half) return;
+    const int i = (int)(idx % half);
+    const int h = (int)((idx / half) % heads);
+    const int t = (int)(idx / ((int64_t)half * heads));
+    const int p0 = pos_dev ? pos_dev[0] : pos_start;
+    const float2 x = *reinterpret_cast<const float2*>(in + (int64_t)t * in_row_pitch + h * head_dim + 2 * i);
+    float2 y = x;
+    if (rotate) {
+        const float freq = powf(theta, -2.0f * (float)i / (float)head_dim);
+        float sn, cs;
+        sincosf((float)(p0 + t) * freq, &sn, &cs);
+        y.x = x.x * cs - x.y * sn;
+        y.y = x.x * sn + x.y * cs;
+    }
+    const int row = (out_row_is_pos ? p0 : 0) + t;
+    *reinterpret_cast<float2*>(out + h * out_head_stride + (int64_t)row * head_dim + 2 * i) = y;
+}
+
+// [heads, tokens, head_dim] -> [tokens, heads * head_dim]: attention output back to the token-major rows a projection takes.
+__global__ __launch_bounds__(256) void heads_to_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int heads,
+                                                            int tokens, int head_dim) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per float4 of the output
+    const int d4 = head_dim >> 2;
+    if (idx >= (int64_t)heads * tokens * d4) return;
+    const int d = (int)(idx % d4);
+    const int h = (int)((idx / d4) % heads);
+    const int t = (int)(idx / ((int64_t)d4 * heads));
+    reinterpret_cast<float4*>(out)[idx] = reinterpret_cast<const float4*>(in)[((int64_t)h * tokens + t) * d4 + d];
+}
+
+__global__ void i32_increment_kernel(int32_t* v, int32_t delta) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) v[0] += delta;
+}
+
+__global__ void i32_store_at_kernel(int32_t* dst, const int32_t* __restrict__ index, int32_t offset, const int32_t* __restrict__ src) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) dst[index[0] + offset] = src[0];
+}
+
+int launch_rope_scatter(const float* in, int64_t in_row_pitch, float* out, int tokens, int heads, int head_dim, int pos_start,
+                        const int32_t* pos_dev, float theta, int rotate, int64_t out_head_stride, int out_row_is_pos) {
+    if (tokens <= 0 || heads <= 0 || head_dim <= 0) return 0;
+    if ((head_dim & 1) || (in_row_pitch & 1)) return set_error("rope: head_dim and the row pitch must be even; got %d, %lld", head_dim, (long long)in_row_pitch);
+    const int64_t n = (int64_t)tokens * heads * (head_dim / 2);
+    rope_scatter_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(
+        in, in_row_pitch, out, tokens, heads, head_dim, pos_start, pos_dev, theta, rotate, out_head_stride, out_row_is_pos);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim) {
+    if (tokens <= 0 || heads <= 0 || head_dim <= 0) return 0;
+    if (head_dim & 3) return set_error("heads_to_rows: head_dim must be a multiple of 4; got %d", head_dim);
+    const int64_t n = (int64_t)heads * tokens * (head_dim / 4);
+    heads_to_rows_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(in, out, heads, tokens, head_dim);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_i32_store_at(int32_t* dst, const int32_t* index, int32_t offset, const int32_t* src) {
+    i32_store_at_kernel<<<dim3(1), dim3(64), 0, current_stream()>>>(dst, index, offset, src);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_i32_increment(int32_t* v, int32_t delta) {
+    i32_increment_kernel<<<dim3(1), dim3(64), 0, current_stream()>>>(v, delta);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
 // Calibration kernel: every thread streams 16-byte loads over a buffer with four independent loads in flight and
 // almost no arithmetic. Its rate is what this device sustains for a read-once pass of that size.
 __global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ p, int64_t n16, uint32_t* __restrict__ sink) {
@@ -188,6 +281,13 @@ int launch_softmax_rows(const float* in, float* out, int rows, int cols, int log
 int launch_silu_mul(const float* gate, const float* up, float* out, int64_t n) {
     if (n <= 0) return 0;
     silu_mul_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(gate, up, out, n);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_swiglu_rows(const float* gate_up, float* out, int rows, int ffn) {
+    if (rows <= 0 || ffn <= 0) return 0;
+    const int64_t n = (int64_t)rows * ffn;
+    swiglu_rows_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(gate_up, out, n, ffn);
     SKH_CHECK(hipGetLastError());
     return 0;
 }

@@ -27,6 +27,7 @@ struct SdpaParams {
     const float *q, *k, *v;
     float* out;
     int batch, heads, kv_heads, seq_q, seq_kv, head_dim;
+    int kv_capacity;  // key rows of storage per kv head (>= seq_kv): a KV cache holds more rows than are attended
     float scale;
     int causal, window, right_context;
     const int32_t* lengths;
@@ -55,8 +56,8 @@ __global__ __launch_bounds__(64 * SDPA_MAX_GROUP) void sdpa_rows_kernel(SdpaPara
     const int h = kvh * per_kv + gsel * p.group + wave;
 
     const float* qrow = p.q + (((int64_t)b * p.heads + h) * p.seq_q + qi) * d;
-    const float* kb = p.k + ((int64_t)b * p.kv_heads + kvh) * p.seq_kv * d;
-    const float* vb = p.v + ((int64_t)b * p.kv_heads + kvh) * p.seq_kv * d;
+    const float* kb = p.k + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * d;
+    const float* vb = p.v + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * d;
     float* orow = p.out + (((int64_t)b * p.heads + h) * p.seq_q + qi) * d;
 
     // Attended key range [first, end) of this query position.
@@ -176,12 +177,13 @@ __global__ __launch_bounds__(256) void zero_kernel(float* out, int64_t n) {
 float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
 
 int launch_sdpa(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
-                int seq_q, int seq_kv, int head_dim, float scale, int causal, int window, int right_context,
+                int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window, int right_context,
                 const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k) {
     if (batch <= 0 || heads <= 0 || kv_heads <= 0 || seq_q <= 0 || head_dim <= 0) return 0;
     if (heads % kv_heads != 0) return set_error("sdpa: heads (%d) must be a multiple of kv_heads (%d)", heads, kv_heads);
     if (window < 0 || right_context < 0) return set_error("sdpa: window and rightContext must be >= 0");
     if (right_context != 0 && window == 0) return set_error("sdpa: rightContext (%d) is only meaningful with window > 0", right_context);
+    if (kv_capacity < seq_kv) return set_error("sdpa: kv capacity %d is below seq_kv %d", kv_capacity, seq_kv);
     if (head_dim > SDPA_MAX_D) return set_error("sdpa: head_dim %d exceeds %d", head_dim, SDPA_MAX_D);
     const int64_t rows = (int64_t)batch * heads * seq_q;
     hipStream_t s = current_stream();
@@ -197,7 +199,7 @@ int launch_sdpa(const float* q, const float* k, const float* v, float* out, int 
         if (!ok) return set_error("sdpa: mask dims [%d,%d,%d,%d] do not broadcast over [%d,%d|%d,%d,%d]", mask_b, mask_h,
                                   mask_q, mask_k, batch, heads, kv_heads, seq_q, seq_kv);
     }
-    SdpaParams p{q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, scale, causal, window, right_context,
+    SdpaParams p{q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, kv_capacity, scale, causal, window, right_context,
                  lengths, mask, mask_b, mask_h, mask_q, mask_k, 1, 1, nullptr};
     const int per_kv = heads / kv_heads;
     int group = per_kv;

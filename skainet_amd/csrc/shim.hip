@@ -28,12 +28,18 @@ int launch_softmax_rows(const float* in, float* out, int rows, int cols, int log
 int launch_silu_mul(const float* gate, const float* up, float* out, int64_t n);
 int launch_add(const float* a, const float* b, float* out, int64_t n);
 int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out);
+int launch_rope_scatter(const float* in, int64_t in_row_pitch, float* out, int tokens, int heads, int head_dim, int pos_start,
+                        const int32_t* pos_dev, float theta, int rotate, int64_t out_head_stride, int out_row_is_pos);
+int launch_swiglu_rows(const float* gate_up, float* out, int rows, int ffn);
+int launch_i32_store_at(int32_t* dst, const int32_t* index, int32_t offset, const int32_t* src);
+int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim);
+int launch_i32_increment(int32_t* v, int32_t delta);
 int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink);
 int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes);
 int launch_fp32_matmul(const float* a, int64_t a_stride, const float* b, int64_t b_stride, float* c, int64_t c_stride,
                        int m, int n, int k, bool b_transposed);
 int launch_sdpa(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
-                int seq_q, int seq_kv, int head_dim, float scale, int causal, int window, int right_context,
+                int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window, int right_context,
                 const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k);
 
 // ------------------------------------------------------------------------------------------ state
@@ -355,8 +361,16 @@ int32_t skainet_hip_f32_sdpa_dev(const float* q, const float* k, const float* v,
                                  int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths,
                                  const float* mask, int32_t mask_b, int32_t mask_h, int32_t mask_q, int32_t mask_k) {
     if (ensure_device() != 0) return -1;
-    return launch_sdpa(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, scale, causal, window, right_context,
+    return launch_sdpa(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, seq_kv, head_dim, scale, causal, window, right_context,
                        lengths, mask, mask_b, mask_h, mask_q, mask_k);
+}
+int32_t skainet_hip_f32_sdpa_cache_dev(const float* q, const float* k_cache, const float* v_cache, float* out, int32_t batch,
+                                       int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t kv_capacity,
+                                       int32_t head_dim, float scale, int32_t causal, int32_t window, int32_t right_context,
+                                       const int32_t* lengths) {
+    if (ensure_device() != 0) return -1;
+    return launch_sdpa(q, k_cache, v_cache, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale, causal,
+                       window, right_context, lengths, nullptr, 0, 0, 0, 0);
 }
 int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* out, int64_t n) {
     if (ensure_device() != 0) return -1;
@@ -369,6 +383,81 @@ int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int6
 int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out) {
     if (ensure_device() != 0) return -1;
     return launch_argmax_rows(in, rows, cols, out);
+}
+
+int32_t skainet_hip_f32_rope_scatter_dev(const float* in, int64_t in_row_pitch, float* out, int32_t tokens, int32_t heads,
+                                         int32_t head_dim, int32_t pos_start, const int32_t* pos_dev, float theta,
+                                         int32_t rotate, int64_t out_head_stride, int32_t out_row_is_pos) {
+    if (ensure_device() != 0) return -1;
+    return launch_rope_scatter(in, in_row_pitch, out, tokens, heads, head_dim, pos_start, pos_dev, theta, rotate, out_head_stride,
+                               out_row_is_pos);
+}
+int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t* index_dev, int32_t offset, const int32_t* src) {
+    if (ensure_device() != 0) return -1;
+    return launch_i32_store_at(dst, index_dev, offset, src);
+}
+int32_t skainet_hip_f32_swiglu_rows_dev(const float* gate_up, float* out, int32_t rows, int32_t ffn) {
+    if (ensure_device() != 0) return -1;
+    return launch_swiglu_rows(gate_up, out, rows, ffn);
+}
+int32_t skainet_hip_f32_heads_to_rows_dev(const float* in, float* out, int32_t heads, int32_t tokens, int32_t head_dim) {
+    if (ensure_device() != 0) return -1;
+    return launch_heads_to_rows(in, out, heads, tokens, head_dim);
+}
+int32_t skainet_hip_i32_increment_dev(int32_t* value, int32_t delta) {
+    if (ensure_device() != 0) return -1;
+    return launch_i32_increment(value, delta);
+}
+
+// ---- HIP graphs: record this thread's device entries once, replay them with one launch ----
+struct skainet_hip_graph { hipGraph_t graph; hipGraphExec_t exec; };
+static thread_local hipStream_t t_capture_prev = nullptr;
+static thread_local hipStream_t t_capture_stream = nullptr;
+
+int32_t skainet_hip_graph_begin(void) {
+    if (ensure_device() != 0) return -1;
+    if (t_capture_stream) return set_error("graph_begin: a capture is already open on this thread");
+    hipStream_t cap = nullptr;
+    if (check_hip(hipStreamCreateWithFlags(&cap, hipStreamNonBlocking), "hipStreamCreate") != 0) return -1;
+    if (check_hip(hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture") != 0) {
+        (void)hipStreamDestroy(cap);
+        return -1;
+    }
+    t_capture_prev = t_stream;
+    t_capture_stream = cap;
+    t_stream = cap;
+    return 0;
+}
+skainet_hip_graph* skainet_hip_graph_end(void) {
+    if (!t_capture_stream) { set_error("graph_end without graph_begin"); return nullptr; }
+    hipStream_t cap = t_capture_stream;
+    t_stream = t_capture_prev;
+    t_capture_stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (check_hip(hipStreamEndCapture(cap, &graph), "hipStreamEndCapture") != 0 ||
+        check_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate") != 0) {
+        if (graph) (void)hipGraphDestroy(graph);
+        (void)hipStreamDestroy(cap);
+        return nullptr;
+    }
+    (void)hipStreamDestroy(cap);   // replays run on the calling thread's stream, in order with its eager work
+    return new skainet_hip_graph{graph, exec};
+}
+int32_t skainet_hip_graph_launch(skainet_hip_graph* g) {
+    if (!g) return set_error("graph_launch: null graph");
+    return check_hip(hipGraphLaunch(g->exec, t_stream), "hipGraphLaunch");
+}
+int32_t skainet_hip_graph_sync(skainet_hip_graph* g) {
+    if (!g) return set_error("graph_sync: null graph");
+    return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+void skainet_hip_graph_free(skainet_hip_graph* g) {
+    if (!g) return;
+    (void)hipStreamSynchronize(t_stream);
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->graph);
+    delete g;
 }
 
 // ------------------------------------------------------------------------------------------ host-pointer entries
@@ -519,7 +608,7 @@ void skainet_hip_f32_sdpa(const float* q, const float* k, const float* v, float*
     int32_t* ld = lengths ? static_cast<int32_t*>(stage_in(4, lengths, sizeof(int32_t) * (size_t)batch)) : nullptr;
     float* md = mask ? static_cast<float*>(stage_in(5, mask, sizeof(float) * (size_t)mask_b * mask_h * mask_q * mask_k)) : nullptr;
     if (!qd || !kd || !vd || !od || (lengths && !ld) || (mask && !md)) return;
-    if (launch_sdpa(qd, kd, vd, od, batch, heads, kv_heads, seq_q, seq_kv, head_dim, scale, causal, window, right_context, ld,
+    if (launch_sdpa(qd, kd, vd, od, batch, heads, kv_heads, seq_q, seq_kv, seq_kv, head_dim, scale, causal, window, right_context, ld,
                     md, mask_b, mask_h, mask_q, mask_k) != 0) return;
     stage_out(out, od, sizeof(float) * qn);
 }

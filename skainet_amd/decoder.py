@@ -1,0 +1,344 @@
+"""A Llama-shaped decoder stack driven entirely through the backend's SPI-level device entries.
+
+The reference repository has no transformer (RoPE, the decoder block and the sampler live in the external
+SKaiNET-transformers repo; the nearest in-repo thing is the synthetic DecodeHarness,
+/root/reference/skainet-backends/skainet-backend-cpu/src/commonTest/kotlin/sk/ainet/exec/harness/DecodeHarness.kt:49).
+This driver is what such a model does with the kernel SPI: every linear layer is a packed-weight matmul
+(`DeviceWeight.matmul`: GEMV kernels for decode, the MFMA GEMM for prefill), attention is the fused SDPA kernel over a
+device KV cache laid out `[kv_heads, positions, head_dim]` per layer (the layout KvCacheStore.readKeys/readValues
+return, .../lang/tensor/storage/KvCacheStore.kt:125-149), RMSNorm / SiLU*up / residual add / arg-max are the
+reference ops' device twins. Activations never leave the device; a decode step can be recorded once into a HIP
+graph and replayed (the position lives in device memory).
+
+Block (standard Llama-3):  h += Wo . attn(rope(Wq n1), rope(Wk n1), Wv n1),  n1 = rmsnorm(h) * g1
+                           h += Wdown . (silu(Wgate n2) * (Wup n2)),        n2 = rmsnorm(h) * g2
+                           logits = Whead . (rmsnorm(h) * g_out);  greedy = first arg-max.
+q/k/v and gate/up weights are stored concatenated along the output rows ([q; k; v] and [gate; up]) so each pair is
+one pass over the activations.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Optional
+
+import numpy as np
+
+from . import _lib, kernels
+from ._lib import HipError, check
+
+
+@dataclass
+class LlamaConfig:
+    layers: int = 32
+    hidden: int = 4096
+    heads: int = 32
+    kv_heads: int = 8
+    head_dim: int = 128
+    ffn: int = 14336
+    vocab: int = 128256
+    rms_eps: float = 1e-5
+    rope_theta: float = 500000.0
+    ctx_max: int = 2048
+    linear_encoding: str = "Q4_K"
+    head_encoding: str = "Q6_K"
+
+    @property
+    def q_dim(self) -> int:
+        return self.heads * self.head_dim
+
+    @property
+    def kv_dim(self) -> int:
+        return self.kv_heads * self.head_dim
+
+
+LLAMA3_8B = LlamaConfig()
+
+
+class DeviceBuffer:
+    """Device memory from the library's allocator (skainet_hip_malloc), with numpy upload / download."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        self.ptr = _lib.hip().skainet_hip_malloc(self.nbytes)
+        if not self.ptr:
+            raise HipError("malloc: " + _lib.last_error())
+
+    def data_ptr(self) -> int:
+        return self.ptr
+
+    def at(self, byte_offset: int) -> int:
+        return self.ptr + int(byte_offset)
+
+    def upload(self, a: np.ndarray, byte_offset: int = 0) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        check(_lib.hip().skainet_hip_memcpy_h2d(self.ptr + byte_offset, a.ctypes.data, a.nbytes), "h2d")
+        return self
+
+    def download(self, dtype, count: int, byte_offset: int = 0) -> np.ndarray:
+        out = np.empty(count, dtype=dtype)
+        check(_lib.hip().skainet_hip_memcpy_d2h(out.ctypes.data, self.ptr + byte_offset, out.nbytes), "d2h")
+        return out
+
+    def close(self) -> None:
+        if self.ptr:
+            _lib.hip().skainet_hip_free(self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+@dataclass
+class LayerWeights:
+    attn_norm: DeviceBuffer      # fp32 [hidden]
+    wqkv: kernels.DeviceWeight   # [(heads + 2 kv_heads) * head_dim, hidden]
+    wo: kernels.DeviceWeight     # [hidden, heads * head_dim]
+    ffn_norm: DeviceBuffer       # fp32 [hidden]
+    w_gate_up: kernels.DeviceWeight   # [2 * ffn, hidden]
+    w_down: kernels.DeviceWeight      # [hidden, ffn]
+
+
+class LlamaWeights:
+    """Random-init weights of the architecture, quantised on the host and resident on the device.
+
+    `host` keeps the packed bytes and norm gains when `keep_host` is set, so a CPU checker can consume the very
+    same bytes."""
+
+    def __init__(self, cfg: LlamaConfig, seed: int = 0, sigma: float = 0.02, keep_host: bool = False, progress=None,
+                 distinct_layers: int = 0):
+        """distinct_layers > 0: only that many layers get values of their own; layer i re-uses the packed bytes of
+        layer i % distinct_layers in a device allocation of its own (same HBM traffic, far less host-side
+        generation and quantisation time for a benchmark)."""
+        kernels._require_available()
+        self.cfg = cfg
+        self.host = {} if keep_host else None
+        rng = np.random.default_rng(seed)
+        bytes_of = {}
+
+        def packed(name, enc, rows, cols, same_as=None):
+            if same_as is not None:
+                return kernels.DeviceWeight.upload(enc, bytes_of[same_as], rows, cols)
+            # generated and quantised in row chunks so the fp32 source never exceeds ~256 MB
+            _, bs, nb = kernels.ENCODINGS[enc]
+            out = np.empty(rows * (cols // bs) * nb, dtype=np.uint8)
+            step = max(1, (64 << 20) // cols)
+            row_bytes = (cols // bs) * nb
+            for r0 in range(0, rows, step):
+                r1 = min(rows, r0 + step)
+                w = rng.standard_normal((r1 - r0, cols), dtype=np.float32) * np.float32(sigma)
+                out[r0 * row_bytes:r1 * row_bytes] = kernels.quantize(enc, w)
+            if self.host is not None:
+                self.host[name] = out
+            if distinct_layers > 0:
+                bytes_of[name] = out
+            if progress:
+                progress(name)
+            return kernels.DeviceWeight.upload(enc, out, rows, cols)
+
+        def gain(name, same_as=None):
+            if same_as is not None:
+                return DeviceBuffer(bytes_of[same_as].nbytes).upload(bytes_of[same_as])
+            g = (1.0 + 0.1 * rng.standard_normal(cfg.hidden)).astype(np.float32)
+            if distinct_layers > 0:
+                bytes_of[name] = g
+            if self.host is not None:
+                self.host[name] = g
+            return DeviceBuffer(g.nbytes).upload(g)
+
+        le = cfg.linear_encoding
+        self.tok_embd = packed("tok_embd", le, cfg.vocab, cfg.hidden)
+        self.layers: List[LayerWeights] = []
+        for i in range(cfg.layers):
+            src = None if distinct_layers <= 0 or i < distinct_layers else f"l{i % distinct_layers}"
+
+            def same(part):
+                return None if src is None else f"{src}.{part}"
+
+            self.layers.append(LayerWeights(
+                attn_norm=gain(f"l{i}.attn_norm", same("attn_norm")),
+                wqkv=packed(f"l{i}.wqkv", le, cfg.q_dim + 2 * cfg.kv_dim, cfg.hidden, same("wqkv")),
+                wo=packed(f"l{i}.wo", le, cfg.hidden, cfg.q_dim, same("wo")),
+                ffn_norm=gain(f"l{i}.ffn_norm", same("ffn_norm")),
+                w_gate_up=packed(f"l{i}.w_gate_up", le, 2 * cfg.ffn, cfg.hidden, same("w_gate_up")),
+                w_down=packed(f"l{i}.w_down", le, cfg.hidden, cfg.ffn, same("w_down")),
+            ))
+        self.out_norm = gain("out_norm")
+        self.head = packed("head", cfg.head_encoding, cfg.vocab, cfg.hidden)
+
+    def packed_bytes(self) -> int:
+        n = self.tok_embd.nbytes + self.head.nbytes
+        for l in self.layers:
+            n += l.wqkv.nbytes + l.wo.nbytes + l.w_gate_up.nbytes + l.w_down.nbytes
+        return n
+
+    def decode_bytes_per_token(self, context: int) -> int:
+        """Algorithmic HBM bytes of one decode step: every linear weight and the head once, the KV cache up to `context`."""
+        c = self.cfg
+        return (self.packed_bytes() - self.tok_embd.nbytes) + 2 * c.layers * c.kv_heads * context * c.head_dim * 4
+
+
+class LlamaDecoder:
+    """Prefill + greedy decode for batch 1, state (KV cache, position, current token) on the device."""
+
+    def __init__(self, weights: LlamaWeights, max_prefill: int = 512):
+        c = self.cfg = weights.cfg
+        self.w = weights
+        self.max_rows = max(1, max_prefill)
+        f = 4
+        rows = self.max_rows
+        self.h = DeviceBuffer(rows * c.hidden * f)
+        self.norm = DeviceBuffer(rows * c.hidden * f)
+        self.qkv = DeviceBuffer(rows * (c.q_dim + 2 * c.kv_dim) * f)
+        self.q = DeviceBuffer(rows * c.q_dim * f)            # [heads, rows, head_dim]
+        self.attn = DeviceBuffer(rows * c.q_dim * f)         # [heads, rows, head_dim]
+        self.attn_rows = DeviceBuffer(rows * c.q_dim * f)    # [rows, heads * head_dim]
+        self.proj = DeviceBuffer(rows * c.hidden * f)
+        self.gate_up = DeviceBuffer(rows * 2 * c.ffn * f)
+        self.act = DeviceBuffer(rows * c.ffn * f)
+        self.logits = DeviceBuffer(c.vocab * f)
+        self.kv_layer_floats = c.kv_heads * c.ctx_max * c.head_dim
+        self.k_cache = DeviceBuffer(c.layers * self.kv_layer_floats * f)
+        self.v_cache = DeviceBuffer(c.layers * self.kv_layer_floats * f)
+        self.pos = DeviceBuffer(4).upload(np.zeros(1, np.int32))        # tokens already in the cache
+        self.kv_len = DeviceBuffer(4).upload(np.zeros(1, np.int32))     # = pos + 1 during a decode step
+        self.token = DeviceBuffer(4).upload(np.zeros(1, np.int32))
+        self.generated = DeviceBuffer(4 * (c.ctx_max + 1))   # generated[p] = the token predicted for position p
+        self.prompt_len = 0
+        self._graph: Optional[kernels.Graph] = None
+
+    # ------------------------------------------------------------------ building blocks
+    def _block(self, li: int, rows: int, pos_start: int, pos_dev, seq_kv: int, kv_len_dev) -> None:
+        """One decoder block over `rows` token rows already in self.h. Prefill: positions pos_start.., K/V rows
+        written at those positions, causal attention over seq_kv = pos_start + rows keys. Decode: one row at the
+        device-side position, attention over the whole cache bounded by the device-side key length."""
+        c, w, L = self.cfg, self.w, self.w.layers[li]
+        f = 4
+        kx = kernels
+        kx.rms_norm_dev(self.h, L.attn_norm, self.norm, rows, c.hidden, c.rms_eps)
+        L.wqkv.matmul(self.norm, rows, self.qkv)
+        qkv_dim = c.q_dim + 2 * c.kv_dim
+        kc = self.k_cache.at(li * self.kv_layer_floats * f)
+        vc = self.v_cache.at(li * self.kv_layer_floats * f)
+        # the three column slices of each token's [q | k | v] row go to the query buffer and into the cache
+        self._rope(self.qkv.ptr, self.q.ptr, rows, c.heads, qkv_dim, 0, pos_start, pos_dev, True, rows * c.head_dim, False)
+        self._rope(self.qkv.ptr, kc, rows, c.kv_heads, qkv_dim, c.q_dim, pos_start, pos_dev, True, c.ctx_max * c.head_dim, True)
+        self._rope(self.qkv.ptr, vc, rows, c.kv_heads, qkv_dim, c.q_dim + c.kv_dim, pos_start, pos_dev, False, c.ctx_max * c.head_dim, True)
+        scale = float(1.0 / np.sqrt(c.head_dim))
+        kx.sdpa_cache_dev(self.q, kc, vc, self.attn, 1, c.heads, c.kv_heads, rows, seq_kv, c.ctx_max, c.head_dim, scale,
+                          True, 0, 0, kv_len_dev)
+        if rows > 1:
+            kx.heads_to_rows_dev(self.attn, self.attn_rows, c.heads, rows, c.head_dim)
+            attn_rows = self.attn_rows
+        else:
+            attn_rows = self.attn                  # one token: [heads, 1, head_dim] is already the row
+        L.wo.matmul(attn_rows, rows, self.proj)
+        kx.add_dev(self.h, self.proj, self.h, rows * c.hidden)
+        kx.rms_norm_dev(self.h, L.ffn_norm, self.norm, rows, c.hidden, c.rms_eps)
+        L.w_gate_up.matmul(self.norm, rows, self.gate_up)
+        kx.swiglu_rows_dev(self.gate_up, self.act, rows, c.ffn)
+        L.w_down.matmul(self.act, rows, self.proj)
+        kx.add_dev(self.h, self.proj, self.h, rows * c.hidden)
+
+    def _rope(self, src, dst, rows, heads, row_pitch, col0, pos_start, pos_dev, rotate, head_stride, row_is_pos):
+        """rope_scatter over the column slice [col0, col0 + heads * head_dim) of token rows `row_pitch` floats apart."""
+        c = self.cfg
+        kernels.rope_scatter_dev(src + 4 * col0, dst, rows, heads, c.head_dim, pos_start, pos_dev, c.rope_theta, rotate,
+                                 head_stride, row_is_pos, in_row_pitch=row_pitch)
+
+    def _head(self, row: int) -> None:
+        c = self.cfg
+        kernels.rms_norm_dev(self.h.at(4 * row * c.hidden), self.w.out_norm, self.norm, 1, c.hidden, c.rms_eps)
+        self.w.head.matmul(self.norm, 1, self.logits)
+        kernels.argmax_rows_dev(self.logits, 1, c.vocab, self.token)
+
+    # ------------------------------------------------------------------ public API
+    def prefill(self, token_ids) -> int:
+        """Run the prompt through the stack, fill the KV cache, return the greedy next token."""
+        c = self.cfg
+        ids = np.ascontiguousarray(token_ids, dtype=np.int32)
+        rows = int(ids.size)
+        if rows < 1 or rows > self.max_rows or rows > c.ctx_max:
+            raise ValueError(f"prompt of {rows} tokens does not fit (max_prefill {self.max_rows}, ctx {c.ctx_max})")
+        ids_dev = DeviceBuffer(ids.nbytes).upload(ids)
+        self.w.tok_embd.dequantize_rows(ids_dev, rows, self.h)
+        for li in range(c.layers):
+            self._block(li, rows, 0, None, rows, None)
+        self._head(rows - 1)
+        kernels.sync()
+        self.pos.upload(np.array([rows], np.int32))
+        self.kv_len.upload(np.array([rows + 1], np.int32))
+        self.prompt_len = rows
+        kernels.i32_store_at_dev(self.generated, self.pos, 0, self.token)
+        kernels.sync()
+        ids_dev.close()
+        return int(self.token.download(np.int32, 1)[0])
+
+    def _decode_step(self) -> None:
+        """Consumes self.token at device position self.pos, leaves the next token in self.token, advances the position."""
+        c = self.cfg
+        self.w.tok_embd.dequantize_rows(self.token, 1, self.h)
+        for li in range(c.layers):
+            self._block(li, 1, 0, self.pos, c.ctx_max, self.kv_len)
+        self._head(0)
+        kernels.i32_increment_dev(self.pos, 1)
+        kernels.i32_increment_dev(self.kv_len, 1)
+        kernels.i32_store_at_dev(self.generated, self.pos, 0, self.token)
+
+    def decode(self, steps: int, use_graph: bool = True) -> np.ndarray:
+        """Greedy-decode `steps` tokens after prefill(); returns them. With use_graph the step is recorded once and replayed."""
+        c = self.cfg
+        if self.position() + steps > c.ctx_max:
+            raise ValueError(f"{steps} more tokens would pass the context limit {c.ctx_max}")
+        out = np.empty(steps, np.int32)
+        if use_graph and self._graph is None:
+            self._decode_step()                       # eager once: sizes every scratch buffer
+            kernels.sync()
+            out0 = int(self.token.download(np.int32, 1)[0])
+            with kernels.Graph() as g:
+                self._decode_step()
+            self._graph = g
+            first = 1
+            out[0] = out0
+        else:
+            first = 0
+        for i in range(first, steps):
+            if use_graph:
+                self._graph.launch()
+                self._graph.sync()
+            else:
+                self._decode_step()
+                kernels.sync()
+            out[i] = int(self.token.download(np.int32, 1)[0])
+        return out
+
+    def decode_timed(self, steps: int) -> float:
+        """Replay the recorded step `steps` times without reading tokens back; returns seconds (host clock around
+        launch + sync). Tokens stay on the device (greedy feedback happens there)."""
+        import time
+        if self._graph is None:
+            self.decode(1, use_graph=True)
+        kernels.sync()
+        self._graph.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self._graph.launch()
+        self._graph.sync()
+        return time.perf_counter() - t0
+
+    def generated_tokens(self) -> np.ndarray:
+        """Every token emitted since the last prefill (the prefill's own next-token first), read from the device log."""
+        n = self.position() - self.prompt_len + 1
+        return self.generated.download(np.int32, n, 4 * self.prompt_len)
+
+    def position(self) -> int:
+        return int(self.pos.download(np.int32, 1)[0])
+
+    def last_logits(self) -> np.ndarray:
+        return self.logits.download(np.float32, self.cfg.vocab)
+
+    def hidden_rows(self, rows: int) -> np.ndarray:
+        return self.h.download(np.float32, rows * self.cfg.hidden).reshape(rows, self.cfg.hidden)

@@ -214,6 +214,14 @@ def sdpa_dev(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, scal
                                               _ptr(mask), *mask_dims), "sdpa")
 
 
+def sdpa_cache_dev(q, k_cache, v_cache, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale,
+                   causal=False, window=0, right_context=0, key_lengths=None) -> None:
+    """SDPA over K / V stored [batch, kv_heads, kv_capacity, head_dim] of which the first seq_kv rows are keys."""
+    check(_lib.hip().skainet_hip_f32_sdpa_cache_dev(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), batch, heads, kv_heads,
+                                                    seq_q, seq_kv, kv_capacity, head_dim, scale, int(causal), window,
+                                                    right_context, _ptr(key_lengths)), "sdpa_cache")
+
+
 def silu_mul_dev(gate, up, out, n: int) -> None:
     check(_lib.hip().skainet_hip_f32_silu_mul_dev(_ptr(gate), _ptr(up), _ptr(out), n), "silu_mul")
 
@@ -224,6 +232,62 @@ def add_dev(a, b, out, n: int) -> None:
 
 def argmax_rows_dev(x, rows: int, cols: int, out) -> None:
     check(_lib.hip().skainet_hip_f32_argmax_rows_dev(_ptr(x), rows, cols, _ptr(out)), "argmax_rows")
+
+
+def rope_scatter_dev(x, out, tokens, heads, head_dim, pos_start=0, pos_dev=None, theta=10000.0, rotate=True,
+                     out_head_stride=None, out_row_is_pos=False, in_row_pitch=None) -> None:
+    if out_head_stride is None:
+        out_head_stride = tokens * head_dim
+    if in_row_pitch is None:
+        in_row_pitch = heads * head_dim
+    check(_lib.hip().skainet_hip_f32_rope_scatter_dev(_ptr(x), in_row_pitch, _ptr(out), tokens, heads, head_dim, pos_start,
+                                                      _ptr(pos_dev), theta, int(rotate), out_head_stride, int(out_row_is_pos)),
+          "rope_scatter")
+
+
+def swiglu_rows_dev(gate_up, out, rows: int, ffn: int) -> None:
+    check(_lib.hip().skainet_hip_f32_swiglu_rows_dev(_ptr(gate_up), _ptr(out), rows, ffn), "swiglu_rows")
+
+
+def heads_to_rows_dev(x, out, heads, tokens, head_dim) -> None:
+    check(_lib.hip().skainet_hip_f32_heads_to_rows_dev(_ptr(x), _ptr(out), heads, tokens, head_dim), "heads_to_rows")
+
+
+def i32_increment_dev(value, delta: int) -> None:
+    check(_lib.hip().skainet_hip_i32_increment_dev(_ptr(value), delta), "i32_increment")
+
+
+def i32_store_at_dev(dst, index_dev, offset: int, src) -> None:
+    check(_lib.hip().skainet_hip_i32_store_at_dev(_ptr(dst), _ptr(index_dev), offset, _ptr(src)), "i32_store_at")
+
+
+class Graph:
+    """Records the device entries issued inside the `with` block into a HIP graph; `launch()` replays them."""
+
+    def __init__(self):
+        self._g = 0
+
+    def __enter__(self):
+        check(_lib.hip().skainet_hip_graph_begin(), "graph_begin")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        g = _lib.hip().skainet_hip_graph_end()
+        if not g and exc_type is None:
+            raise HipError("graph_end: " + _lib.last_error())
+        self._g = g or 0
+        return False
+
+    def launch(self) -> None:
+        check(_lib.hip().skainet_hip_graph_launch(self._g), "graph_launch")
+
+    def sync(self) -> None:
+        check(_lib.hip().skainet_hip_graph_sync(self._g), "graph_sync")
+
+    def close(self) -> None:
+        if self._g:
+            _lib.hip().skainet_hip_graph_free(self._g)
+            self._g = 0
 
 
 def fp32_matmul_dev(a, a_offset, a_stride, b, b_offset, b_stride, out, out_offset, out_stride, m, n, k) -> None:

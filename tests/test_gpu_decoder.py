@@ -1,0 +1,239 @@
+"""The decoder glue ops and the Llama-shaped decoder stack on the device against CPU checkers.
+
+RoPE has no counterpart in the reference repository, so it is checked against the closed form in float64; the
+decoder as a whole is checked against tests/decoder_check.py (float64 numpy over oracle-dequantised weights).
+Tolerances: fp32 paths (decode rows, prompts of at most 8 tokens) 1e-3 of the largest reference magnitude; the
+bf16-operand MFMA prefill path 2e-2."""
+import numpy as np
+import pytest
+
+from decoder_check import CheckDecoder
+from gpu_util import dev
+
+pytestmark = pytest.mark.gpu
+
+
+def max_norm_err(got, ref):
+    ref = np.asarray(ref, np.float64)
+    return float(np.abs(np.asarray(got, np.float64) - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def small_config():
+    from skainet_amd.decoder import LlamaConfig
+    return LlamaConfig(layers=2, hidden=512, heads=8, kv_heads=2, head_dim=64, ffn=1024, vocab=1024, ctx_max=64,
+                       rope_theta=10000.0)
+
+
+@pytest.fixture(scope="module")
+def small_model(hip_backend):
+    from skainet_amd.decoder import LlamaWeights
+    cfg = small_config()
+    w = LlamaWeights(cfg, seed=11, sigma=0.05, keep_host=True)
+    return cfg, w
+
+
+@pytest.mark.parametrize("tokens,heads,head_dim,pos0,pitch_extra", [(1, 8, 64, 0, 0), (5, 4, 128, 17, 0), (7, 2, 64, 3, 192)])
+def test_rope_scatter_closed_form(hip_backend, torch_cuda, tokens, heads, head_dim, pos0, pitch_extra):
+    torch = torch_cuda
+    kx = hip_backend
+    rng = np.random.default_rng(5)
+    pitch = heads * head_dim + pitch_extra
+    src = rng.standard_normal((tokens, pitch)).astype(np.float32)
+    col0 = pitch_extra // 2
+    theta = 500000.0
+    x = src[:, col0:col0 + heads * head_dim].reshape(tokens, heads, head_dim).astype(np.float64)
+    ang = (np.arange(tokens)[:, None, None] + pos0) * theta ** (-2.0 * np.arange(head_dim // 2)[None, None, :] / head_dim)
+    want = np.empty_like(x)
+    want[..., 0::2] = x[..., 0::2] * np.cos(ang) - x[..., 1::2] * np.sin(ang)
+    want[..., 1::2] = x[..., 0::2] * np.sin(ang) + x[..., 1::2] * np.cos(ang)
+    d_src = dev(torch, src)
+    cap = 32
+    # query layout: [heads, tokens, head_dim], rows from 0
+    out_q = torch.zeros(heads * tokens * head_dim, dtype=torch.float32, device="cuda")
+    kx.rope_scatter_dev(d_src.data_ptr() + 4 * col0, out_q, tokens, heads, head_dim, pos0, None, theta, True,
+                        tokens * head_dim, False, in_row_pitch=pitch)
+    # cache layout: [heads, cap, head_dim], rows at the absolute position, position read from the device
+    out_c = torch.full((heads, cap, head_dim), 7.0, dtype=torch.float32, device="cuda")
+    pos_dev = dev(torch, np.array([pos0], np.int32))
+    kx.rope_scatter_dev(d_src.data_ptr() + 4 * col0, out_c, tokens, heads, head_dim, 0, pos_dev, theta, True,
+                        cap * head_dim, True, in_row_pitch=pitch)
+    # values: copied, not rotated
+    out_v = torch.full((heads, cap, head_dim), 7.0, dtype=torch.float32, device="cuda")
+    kx.rope_scatter_dev(d_src.data_ptr() + 4 * col0, out_v, tokens, heads, head_dim, pos0, None, theta, False,
+                        cap * head_dim, True, in_row_pitch=pitch)
+    kx.sync()
+    got_q = out_q.cpu().numpy().reshape(heads, tokens, head_dim).transpose(1, 0, 2)
+    assert np.abs(got_q - want).max() < 2e-5
+    got_c = out_c.cpu().numpy()
+    assert np.abs(got_c[:, pos0:pos0 + tokens].transpose(1, 0, 2) - want).max() < 2e-5
+    untouched = np.ones(cap, bool)
+    untouched[pos0:pos0 + tokens] = False
+    assert (got_c[:, untouched] == 7.0).all()
+    got_v = out_v.cpu().numpy()
+    assert np.array_equal(got_v[:, pos0:pos0 + tokens].transpose(1, 0, 2), x.astype(np.float32))
+    assert (got_v[:, untouched] == 7.0).all()
+
+
+def test_rope_rejects_odd_head_dim(hip_backend, torch_cuda):
+    from skainet_amd._lib import HipError
+    t = torch_cuda.zeros(64, device="cuda")
+    with pytest.raises(HipError):
+        hip_backend.rope_scatter_dev(t, t, 1, 1, 7)
+
+
+def test_heads_to_rows_and_swiglu_and_increment(hip_backend, torch_cuda):
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(9)
+    heads, tokens, hd = 6, 5, 32
+    a = rng.standard_normal((heads, tokens, hd)).astype(np.float32)
+    out = torch.empty(tokens * heads * hd, dtype=torch.float32, device="cuda")
+    kx.heads_to_rows_dev(dev(torch, a), out, heads, tokens, hd)
+    rows, ffn = 3, 130
+    gu = (rng.standard_normal((rows, 2 * ffn)) * 3).astype(np.float32)
+    act = torch.empty(rows * ffn, dtype=torch.float32, device="cuda")
+    kx.swiglu_rows_dev(dev(torch, gu), act, rows, ffn)
+    ctr = dev(torch, np.array([41], np.int32))
+    kx.i32_increment_dev(ctr, 1)
+    kx.i32_increment_dev(ctr, 3)
+    kx.sync()
+    assert np.array_equal(out.cpu().numpy().reshape(tokens, heads, hd), a.transpose(1, 0, 2))
+    g, u = gu[:, :ffn].astype(np.float64), gu[:, ffn:].astype(np.float64)
+    assert max_norm_err(act.cpu().numpy().reshape(rows, ffn), g / (1 + np.exp(-g)) * u) < 1e-6
+    assert int(ctr.cpu()[0]) == 45
+
+
+def test_sdpa_cache_layout_matches_contiguous(hip_backend, torch_cuda):
+    """K / V read in place from a cache with spare rows == the contiguous-operand kernel on the gathered rows."""
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(21)
+    b, h, hkv, sq, skv, cap, d = 2, 8, 2, 3, 37, 50, 64
+    q = rng.standard_normal((b, h, sq, d)).astype(np.float32)
+    kc = rng.standard_normal((b, hkv, cap, d)).astype(np.float32)
+    vc = rng.standard_normal((b, hkv, cap, d)).astype(np.float32)
+    lens = np.array([37, 20], np.int32)
+    out_c = torch.empty(b * h * sq * d, dtype=torch.float32, device="cuda")
+    out_p = torch.empty_like(out_c)
+    kx.sdpa_cache_dev(dev(torch, q), dev(torch, kc), dev(torch, vc), out_c, b, h, hkv, sq, skv, cap, d, 0.125, True, 0, 0,
+                      dev(torch, lens))
+    kx.sdpa_dev(dev(torch, q), dev(torch, kc[:, :, :skv]), dev(torch, vc[:, :, :skv]), out_p, b, h, hkv, sq, skv, d, 0.125,
+                True, 0, 0, dev(torch, lens))
+    kx.sync()
+    assert np.array_equal(out_c.cpu().numpy(), out_p.cpu().numpy())
+    from skainet_amd._lib import HipError
+    with pytest.raises(HipError):
+        kx.sdpa_cache_dev(out_c, out_c, out_c, out_p, 1, 8, 2, 1, 40, 39, 64, 1.0)
+
+
+def test_graph_replays_match_eager(hip_backend, torch_cuda):
+    """A recorded sequence (norm -> packed GEMV -> add -> counter) replayed several times, with eager work and
+    synchronisation between the replays, gives the eager result every time."""
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(2)
+    n, k = 768, 512
+    w = kx.DeviceWeight.upload("Q4_K", kx.quantize("Q4_K", (rng.standard_normal((n, k)) * 0.05).astype(np.float32)), n, k)
+    gain = dev(torch, np.ones(k, np.float32))
+    x = dev(torch, rng.standard_normal(k).astype(np.float32))
+    xn = torch.empty(k, dtype=torch.float32, device="cuda")
+    y = torch.empty(n, dtype=torch.float32, device="cuda")
+    acc = torch.zeros(n, dtype=torch.float32, device="cuda")
+    ctr = dev(torch, np.zeros(1, np.int32))
+
+    def step():
+        kx.rms_norm_dev(x, gain, xn, 1, k, 1e-5)
+        w.matmul(xn, 1, y)
+        kx.add_dev(acc, y, acc, n)
+        kx.i32_increment_dev(ctr, 1)
+
+    step()
+    kx.sync()
+    y1 = y.cpu().numpy().copy()
+    with kx.Graph() as g:
+        step()
+    kx.sync()
+    assert int(ctr.cpu()[0]) == 1, "recording must not execute the step"
+    for i in range(4):
+        g.launch()
+        g.sync()
+        kx.rms_norm_dev(x, gain, xn, 1, k, 1e-5)      # eager work between replays
+        kx.sync()
+        assert int(ctr.cpu()[0]) == 2 + i
+        assert np.array_equal(y.cpu().numpy(), y1)
+        assert max_norm_err(acc.cpu().numpy(), y1.astype(np.float64) * (2 + i)) < 1e-6
+    g.close()
+
+
+@pytest.mark.parametrize("prompt_len,tol", [(6, 1e-3), (24, 2e-2)])
+def test_prefill_matches_cpu_checker(small_model, prompt_len, tol):
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    prompt = np.random.default_rng(prompt_len).integers(0, cfg.vocab, prompt_len)
+    dec = LlamaDecoder(w, max_prefill=32)
+    tok = dec.prefill(prompt)
+    chk = CheckDecoder(cfg, w.host)
+    h_ref, logits_ref = chk.forward(prompt)
+    assert max_norm_err(dec.hidden_rows(prompt_len), h_ref) < tol
+    logits = dec.last_logits()
+    assert max_norm_err(logits, logits_ref) < tol
+    assert tok == int(np.argmax(logits)), "greedy token is the first arg-max of the device logits"
+    assert dec.position() == prompt_len
+    # the cache holds the rotated keys / raw values at rows [0, prompt_len) of every kv head
+    for li in (0, cfg.layers - 1):
+        kc = dec.k_cache.download(np.float32, dec.kv_layer_floats, 4 * li * dec.kv_layer_floats)
+        vc = dec.v_cache.download(np.float32, dec.kv_layer_floats, 4 * li * dec.kv_layer_floats)
+        kc = kc.reshape(cfg.kv_heads, cfg.ctx_max, cfg.head_dim)[:, :prompt_len]
+        vc = vc.reshape(cfg.kv_heads, cfg.ctx_max, cfg.head_dim)[:, :prompt_len]
+        assert max_norm_err(kc, chk.k[li]) < tol
+        assert max_norm_err(vc, chk.v[li]) < tol
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_greedy_decode_matches_cpu_checker(small_model, use_graph):
+    """Teacher-forced on the device's own tokens: after every step the device logits match the checker's for the
+    same token history, the emitted token is the first arg-max of the device logits, and it equals the checker's
+    arg-max whenever the checker's top-2 gap is clear of the tolerance."""
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    prompt = np.random.default_rng(77).integers(0, cfg.vocab, 5)
+    dec = LlamaDecoder(w, max_prefill=8)
+    chk = CheckDecoder(cfg, w.host)
+    tok = dec.prefill(prompt)
+    _, logits_ref = chk.forward(prompt)
+    steps = 12
+    for i in range(steps):
+        assert max_norm_err(dec.last_logits(), logits_ref) < 1e-3, f"step {i}"
+        top2 = np.sort(logits_ref)[-2:]
+        if top2[1] - top2[0] > 2e-3 * np.abs(logits_ref).max():
+            assert tok == int(np.argmax(logits_ref)), f"step {i}"
+        _, logits_ref = chk.forward([tok])
+        nxt = int(dec.decode(1, use_graph=use_graph)[0])
+        assert nxt == int(np.argmax(dec.last_logits()))
+        assert dec.position() == len(prompt) + i + 1
+        tok = nxt
+    assert max_norm_err(dec.last_logits(), logits_ref) < 1e-3
+
+
+def test_graph_and_eager_decode_agree(small_model):
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    prompt = np.random.default_rng(3).integers(0, cfg.vocab, 7)
+    outs = []
+    for use_graph in (False, True):
+        dec = LlamaDecoder(w, max_prefill=8)
+        first = dec.prefill(prompt)
+        toks = dec.decode(10, use_graph=use_graph)
+        assert np.array_equal(dec.generated_tokens(), np.concatenate([[first], toks]))   # the device-side token log
+        outs.append((first, toks, dec.last_logits()))
+    assert outs[0][0] == outs[1][0]
+    assert np.array_equal(outs[0][1], outs[1][1])
+    assert np.array_equal(outs[0][2], outs[1][2])
+
+
+def test_prefill_rejects_oversized_prompt(small_model):
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    dec = LlamaDecoder(w, max_prefill=4)
+    with pytest.raises(ValueError):
+        dec.prefill(np.zeros(5, np.int32))
+    dec.prefill(np.zeros(4, np.int32))
+    with pytest.raises(ValueError):
+        dec.decode(cfg.ctx_max, use_graph=False)
