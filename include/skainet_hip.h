@@ -105,6 +105,14 @@ SKAINET_HIP_API int64_t skainet_hip_weight_nbytes(const skainet_hip_weight* w);
 SKAINET_HIP_API int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out);
 /* Same product, forcing one of the two kernels (kind 0 = GEMV path, 1 = MFMA GEMM path). */
 SKAINET_HIP_API int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out, int32_t kind);
+/* out = epilogue(W . prologue(x)): a product with the row ops a decoder block puts around it folded in (no reference
+ * counterpart as one call; the parts are f32_fused.c:255-286 RMSNorm, f32_ops.c:222-244 SiLU, binary add / mul).
+ *   gain != NULL: every activation row is RMS-normalised first, x / sqrt(mean(x^2) + eps) * gain;
+ *   epilogue 0: out [m, rows] = product; 1: out = residual + product (residual [m, rows], may alias out);
+ *   2: out [m, rows/2], out[j] = silu(p[2j]) * p[2j+1] -- for a weight whose rows alternate gate row, up row.
+ * Q4_K weights with m <= 2 run as one kernel; other shapes run the same arithmetic as separate launches. */
+SKAINET_HIP_API int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out,
+    const float* gain, float eps, const float* residual, int32_t epilogue);
 /* Measurement aid: `iters` such products back to back on this thread's stream, weight number i % nweights at
  * step i, timed with HIP events; returns the elapsed milliseconds (< 0 on failure). use_graph != 0 captures the
  * launches into a HIP graph first and times one replay, so host launch cost stays off the GPU timeline.
@@ -213,12 +221,18 @@ SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t
  *                 Writes straight into the [kv_heads, positions, head_dim] layout KvCacheStore.readKeys/readValues expose
  *                 (REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/storage/KvCacheStore.kt:125-149).
  *   heads_to_rows: [heads, tokens, head_dim] -> [tokens, heads*head_dim].
- *   swiglu_rows:   rows of [gate | up] (2*ffn floats) -> out[r, i] = silu(gate[r, i]) * up[r, i], silu as in silu_mul.
+ *   swiglu_pairs:  interleaved (gate, up) pairs -> out[i] = silu(gu[2i]) * gu[2i+1] for i < n, silu as in silu_mul
+ *                  (the output of one product against a weight whose rows alternate gate row, up row).
+ *   rope_qkv:      the three rope_scatter calls of a decoder block in one launch: token rows [q | k | v] -> rotated
+ *                  q [heads, tokens, head_dim], rotated k and raw v into rows pos + t of [kv_heads, kv_capacity, head_dim].
  *   i32_increment: *value += delta on the device (the position counter of a recorded decode step). */
 SKAINET_HIP_API int32_t skainet_hip_f32_rope_scatter_dev(const float* in, int64_t in_row_pitch, float* out, int32_t tokens,
     int32_t heads, int32_t head_dim, int32_t pos_start, const int32_t* pos_dev, float theta, int32_t rotate,
     int64_t out_head_stride, int32_t out_row_is_pos);
-SKAINET_HIP_API int32_t skainet_hip_f32_swiglu_rows_dev(const float* gate_up, float* out, int32_t rows, int32_t ffn);
+SKAINET_HIP_API int32_t skainet_hip_f32_swiglu_pairs_dev(const float* gate_up, float* out, int64_t n);
+SKAINET_HIP_API int32_t skainet_hip_f32_rope_qkv_dev(const float* qkv, float* q_out, float* k_cache, float* v_cache,
+    int32_t tokens, int32_t heads, int32_t kv_heads, int32_t head_dim, int32_t kv_capacity, int32_t pos_start,
+    const int32_t* pos_dev, float theta);
 SKAINET_HIP_API int32_t skainet_hip_f32_heads_to_rows_dev(const float* in, float* out, int32_t heads, int32_t tokens, int32_t head_dim);
 SKAINET_HIP_API int32_t skainet_hip_i32_increment_dev(int32_t* value, int32_t delta);
 /* dst[index_dev[0] + offset] = src[0], all on the device: appends a sampled token to a log at the device-side position. */

@@ -18,6 +18,11 @@
 //     are folded across the 64 lanes once, at the end, with a multi-value butterfly.
 //   * R rows are in flight per wave (loads issued before the arithmetic of the previous rows), rows are spread
 //     evenly over all waves of the chip by the host.
+//   * Optional fusions, so a decoder block needs no separate row kernels around its products:
+//       prologue RMSNorm  y = W . (x * gain / sqrt(mean(x^2) + eps)): every workgroup stages all of x anyway, so it
+//                         sums the squares while staging x * gain and scales its outputs at the end;
+//       epilogue residual y = residual + W . x  (residual may alias y);
+//       epilogue SwiGLU   out[j] = silu(y[2j]) * y[2j + 1] for a weight whose rows alternate gate row, up row.
 #include "common.h"
 
 namespace skh {
@@ -58,9 +63,12 @@ __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi
     for (int b = 0; b < B; ++b) out[b] += dlo * lo[b] + dhi * hi[b] - (mlo * xsum[b][0] + mhi * xsum[b][1]);
 }
 
-template <int B, int R>
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+
+template <int B, int R, int PRO, int EPI>
 __global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                                            float* __restrict__ y, int k, int n, int rows_per_wave) {
+                                                            float* y, int k, int n, int rows_per_wave,
+                                                            const float* __restrict__ gain, float eps, const float* residual) {
     constexpr int NV = 16 * B;   // Q4K_RMAX rows padded to 16, times B
     constexpr int SLICE = 68;    // 64 activations + 4 floats of padding: 16-byte aligned and bank-conflict free
     __shared__ __attribute__((aligned(16))) float xlds[B][64 * SLICE];
@@ -82,6 +90,10 @@ __global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __res
 #pragma unroll
         for (int b = 0; b < B; ++b) acc[i][b] = 0.f;
 
+    float ssq[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) ssq[b] = 0.f;
+
     for (int blk0 = 0; blk0 < bpr; blk0 += 16) {
         const int blk = blk0 + (lane >> 2);
         const int blk_c = min(blk, bpr - 1);                // lanes past K re-read a valid block and multiply it by zero activations
@@ -90,10 +102,10 @@ __global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __res
 
         // the first rows' weight loads go out before anything else
         Q4KRow raw[R];
-        if (nrows > 0) {
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                const uint8_t* p = lane_base + (int64_t)min(i, nrows - 1) * row_bytes;
+        for (int i = 0; i < R; ++i) {
+            if (i < nrows) {                                    // wave-uniform
+                const uint8_t* p = lane_base + (int64_t)i * row_bytes;
                 raw[i].hdr = *reinterpret_cast<const uint4*>(p);
                 raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
                 raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
@@ -110,6 +122,13 @@ __global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __res
                 const int e = blk0 * 256 + f * 4;
                 float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (e < k) v4 = *reinterpret_cast<const float4*>(x + (int64_t)b * k + e);
+                if (PRO) {
+                    ssq[b] = fmaf(v4.x, v4.x, fmaf(v4.y, v4.y, fmaf(v4.z, v4.z, fmaf(v4.w, v4.w, ssq[b]))));
+                    if (e < k) {
+                        const float4 g4 = *reinterpret_cast<const float4*>(gain + e);
+                        v4.x *= g4.x; v4.y *= g4.y; v4.z *= g4.z; v4.w *= g4.w;
+                    }
+                }
                 *reinterpret_cast<float4*>(&xlds[b][(f >> 4) * SLICE + (f & 15) * 4]) = v4;
             }
         }
@@ -146,16 +165,41 @@ __global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __res
         }
     }
 
+    float xscale[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) xscale[b] = 1.0f;
+    if (PRO) {
+        // every workgroup has seen all of x: total the squares over its four waves
+        __syncthreads();                                        // the last pass's slices have been read
+        float* red = &xlds[0][0];
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const float t = wave_sum(ssq[b]);
+            if (lane == 0) red[(threadIdx.x >> 6) * B + b] = t;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < B; ++b)
+            xscale[b] = 1.0f / sqrtf((red[b] + red[B + b] + red[2 * B + b] + red[3 * B + b]) * (1.0f / (float)k) + eps);
+    }
+
     float v[NV];
 #pragma unroll
     for (int i = 0; i < 16; ++i)
 #pragma unroll
         for (int b = 0; b < B; ++b) v[i * B + b] = acc[i][b];
     wave_fold<NV>(v, lane);
-    if (lane < NV) {
-        const int idx = wave_fold_index<NV>(lane);
-        const int row = idx / B, b = idx % B;
-        if (row < nrows) y[(int64_t)b * n + r0 + row] = v[0];
+    const int idx = wave_fold_index<NV>(lane);
+    const int row = idx / B, b = idx % B;
+    float val = v[0] * (B == 1 ? xscale[0] : (b == 0 ? xscale[0] : xscale[B - 1]));
+    if (EPI == EPI_SWIGLU) {
+        // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
+        const float up = __shfl_xor(val, NV / (2 * B), 64);
+        if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
+    } else if (lane < NV && row < nrows) {
+        const int64_t o = (int64_t)b * n + r0 + row;
+        if (EPI == EPI_RESIDUAL) val += residual[o];
+        y[o] = val;
     }
 }
 
@@ -164,19 +208,43 @@ void set_q4k_rows_waves_per_cu(int v) { if (v > 0) g_q4k_rows_waves_per_cu = v; 
 
 // Returns 1 when this kernel took the product, 0 when the shape is outside its range (caller falls back to the
 // slot kernel), -1 on a launch error.
-int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch) {
+template <int PRO, int EPI>
+static void launch_variant(int batch, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n,
+                           int rows_per_wave, const float* gain, float eps, const float* residual) {
+    if (batch == 1) q4k_gemv_rows_kernel<1, 6, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, gain, eps, residual);
+    else q4k_gemv_rows_kernel<2, 3, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, gain, eps, residual);
+}
+
+// y = epilogue(W . prologue(x)); gain != null selects the RMSNorm prologue, epilogue is one of EPI_*.
+int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k, int n, int batch, const float* gain, float eps,
+                               const float* residual, int epilogue) {
     if (batch < 1 || batch > 2) return 0;
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 3)) return 0;
+    if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return 0;
+    if (epilogue == EPI_SWIGLU && (n & 1)) return 0;
     int total_waves = num_cus() * g_q4k_rows_waves_per_cu;
     int rows_per_wave = (n + total_waves - 1) / total_waves;
+    if (epilogue == EPI_SWIGLU) rows_per_wave = (rows_per_wave + 1) & ~1;   // a (gate, up) pair never straddles two waves
     if (rows_per_wave > Q4K_RMAX) rows_per_wave = Q4K_RMAX;
     const int waves = (n + rows_per_wave - 1) / rows_per_wave;
     const int grid = (waves + 3) / 4;
     hipStream_t s = current_stream();
-    if (batch == 1) q4k_gemv_rows_kernel<1, 6><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave);
-    else q4k_gemv_rows_kernel<2, 3><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave);
+    const int variant = (gain ? 3 : 0) + epilogue;
+    switch (variant) {
+        case 0: launch_variant<0, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
+        case 1: launch_variant<0, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
+        case 2: launch_variant<0, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
+        case 3: launch_variant<1, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
+        case 4: launch_variant<1, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
+        case 5: launch_variant<1, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
+        default: return set_error("q4k gemv: unknown epilogue %d", epilogue);
+    }
     SKH_CHECK(hipGetLastError());
     return 1;
+}
+
+int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch) {
+    return launch_q4k_gemv_rows_fused(w, x, y, k, n, batch, nullptr, 0.f, nullptr, EPI_NONE);
 }
 
 }  // namespace skh

@@ -12,6 +12,8 @@
 
 namespace skh {
 
+void* sync_scratch(size_t bytes);   // shim.hip: persistent zero-initialised device memory for cross-workgroup counters
+
 constexpr int ROW_THREADS = 256;
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
@@ -49,6 +51,36 @@ __global__ __launch_bounds__(ROW_THREADS) void rms_norm_kernel(const float* __re
         float y = x[i] * scale;
         if (gamma) y *= gamma[i];
         o[i] = y;
+    }
+}
+
+// Rows of at most 4 * ROW_THREADS * V floats (cols a multiple of 4, 16-byte aligned): every load of the row is in
+// flight at once and the row stays in registers between the two passes, so a single row costs one memory
+// round trip instead of one per 256 elements.
+template <int V>
+__global__ __launch_bounds__(ROW_THREADS) void rms_norm_cached_kernel(const float* __restrict__ in, const float* __restrict__ gamma,
+                                                                      float* __restrict__ out, int cols, float eps) {
+    __shared__ float red[ROW_THREADS / 64];
+    const float4* x = reinterpret_cast<const float4*>(in + (int64_t)blockIdx.x * cols);
+    float4* o = reinterpret_cast<float4*>(out + (int64_t)blockIdx.x * cols);
+    const float4* g4 = reinterpret_cast<const float4*>(gamma);
+    const int c4 = cols >> 2;
+    float4 xr[V], gr[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + ROW_THREADS * j;
+        xr[j] = i < c4 ? x[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        gr[j] = (gamma && i < c4) ? g4[i] : make_float4(1.f, 1.f, 1.f, 1.f);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j) { s = fmaf(xr[j].x, xr[j].x, s); s = fmaf(xr[j].y, xr[j].y, s); s = fmaf(xr[j].z, xr[j].z, s); s = fmaf(xr[j].w, xr[j].w, s); }
+    s = block_sum(s, red);
+    const float scale = 1.0f / sqrtf(s * (1.0f / (float)cols) + eps);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + ROW_THREADS * j;
+        if (i < c4) o[i] = make_float4(xr[j].x * scale * gr[j].x, xr[j].y * scale * gr[j].y, xr[j].z * scale * gr[j].z, xr[j].w * scale * gr[j].w);
     }
 }
 
@@ -101,13 +133,12 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
     if (i < n) { const float g = gate[i]; out[i] = g * (1.0f / (1.0f + expf(-g))) * up[i]; }
 }
 
-// SwiGLU over rows holding [gate | up]: out[r, i] = silu(gu[r, i]) * gu[r, ffn + i].
-__global__ __launch_bounds__(256) void swiglu_rows_kernel(const float* __restrict__ gu, float* __restrict__ out, int64_t n, int ffn) {
+// SwiGLU over rows of interleaved (gate, up) pairs: out[i] = silu(gu[2i]) * gu[2i + 1].
+__global__ __launch_bounds__(256) void swiglu_pairs_kernel(const float2* __restrict__ gu, float* __restrict__ out, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const int64_t r = i / ffn, c = i % ffn;
-    const float g = gu[r * 2 * ffn + c];
-    out[i] = g * (1.0f / (1.0f + expf(-g))) * gu[r * 2 * ffn + ffn + c];
+    const float2 p = gu[i];
+    out[i] = p.x * (1.0f / (1.0f + expf(-p.x))) * p.y;
 }
 
 __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
@@ -143,6 +174,58 @@ __global__ __launch_bounds__(ROW_THREADS) void argmax_rows_kernel(const float* _
         out[blockIdx.x] = bi == 0x7FFFFFFF ? 0 : bi;
     }
 }
+
+// Few long rows (the logits of a decode step): ARGMAX_SPLIT workgroups per row each reduce a slice to one
+// (value, index) pair; the workgroup that finishes last for a row (an agent-scope counter tells it) merges the
+// pairs and resets the counter for the next launch. Same ordering rule as above, so ties still keep the first.
+constexpr int ARGMAX_SPLIT = 64;
+constexpr int ARGMAX_MAX_ROWS = 64;
+struct ArgmaxScratch { float val[ARGMAX_MAX_ROWS][ARGMAX_SPLIT]; int idx[ARGMAX_MAX_ROWS][ARGMAX_SPLIT]; unsigned done[ARGMAX_MAX_ROWS]; };
+
+__device__ __forceinline__ void argmax_merge(float& bv, int& bi, float ov, int oi) {
+    if (oi != 0x7FFFFFFF && (bi == 0x7FFFFFFF || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+}
+
+__global__ __launch_bounds__(ROW_THREADS) void argmax_split_kernel(const float* __restrict__ in, int cols, int32_t* __restrict__ out,
+                                                                   ArgmaxScratch* __restrict__ sc) {
+    __shared__ float rv[ROW_THREADS / 64];
+    __shared__ int ri[ROW_THREADS / 64];
+    __shared__ unsigned ticket;
+    const int row = blockIdx.y, part = blockIdx.x;
+    const float* x = in + (int64_t)row * cols;
+    const int per = ((cols + ARGMAX_SPLIT - 1) / ARGMAX_SPLIT + 3) & ~3;
+    const int lo = part * per, hi = min(cols, lo + per);
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+        const float v = x[i];
+        if (v > bv || bi == 0x7FFFFFFF) { bv = v; bi = i; }     // a thread walks upwards: an equal value later is never lower
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) argmax_merge(bv, bi, __shfl_xor(bv, m, 64), __shfl_xor(bi, m, 64));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { rv[wave] = bv; ri[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < ROW_THREADS / 64; ++w) argmax_merge(bv, bi, rv[w], ri[w]);
+        __hip_atomic_store(&sc->val[row][part], bv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&sc->idx[row][part], bi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ticket = __hip_atomic_fetch_add(&sc->done[row], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (ticket != ARGMAX_SPLIT - 1) return;      // uniform over the workgroup
+    if (threadIdx.x < 64) {
+        bv = __hip_atomic_load(&sc->val[row][threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bi = __hip_atomic_load(&sc->idx[row][threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) argmax_merge(bv, bi, __shfl_xor(bv, m, 64), __shfl_xor(bi, m, 64));
+        if (threadIdx.x == 0) {
+            out[row] = bi == 0x7FFFFFFF ? 0 : bi;
+            __hip_atomic_store(&sc->done[row], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+static_assert(ARGMAX_SPLIT == 64, "the merge step reads one pair per lane of a wave");
 
 // dst (row-major) block (o, b) <- src (input-block-major) block (b, o); 2 bytes per thread-step because
 // Q8_0 / Q6_K blocks are only 2-byte aligned.
@@ -190,6 +273,37 @@ __global__ __launch_bounds__(256) void rope_scatter_kernel(const float* __restri
     *reinterpret_cast<float2*>(out + h * out_head_stride + (int64_t)row * head_dim + 2 * i) = y;
 }
 
+// The three scatters of a decoder block in one launch: token rows of [q | k | v] (heads, kv_heads, kv_heads heads of
+// head_dim) -> rotated queries [heads, tokens, head_dim], rotated keys and raw values into cache rows p0 + t of
+// [kv_heads, kv_capacity, head_dim] caches. p0 = *pos_dev when given, else pos_start.
+__global__ __launch_bounds__(256) void rope_qkv_kernel(const float* __restrict__ qkv, float* __restrict__ q_out,
+                                                       float* __restrict__ k_cache, float* __restrict__ v_cache, int tokens,
+                                                       int heads, int kv_heads, int head_dim, int kv_capacity, int pos_start,
+                                                       const int32_t* __restrict__ pos_dev, float theta) {
+    const int half = head_dim >> 1;
+    const int slots = heads + 2 * kv_heads;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (token, head slot, pair)
+    if (idx >= (int64_t)tokens * slots * half) return;
+    const int i = (int)(idx % half);
+    const int hs = (int)((idx / half) % slots);
+    const int t = (int)(idx / ((int64_t)half * slots));
+    const int p0 = pos_dev ? pos_dev[0] : pos_start;
+    const float2 x = *reinterpret_cast<const float2*>(qkv + ((int64_t)t * slots + hs) * head_dim + 2 * i);
+    float2 y = x;
+    if (hs < heads + kv_heads) {
+        const float freq = powf(theta, -2.0f * (float)i / (float)head_dim);
+        float sn, cs;
+        sincosf((float)(p0 + t) * freq, &sn, &cs);
+        y.x = x.x * cs - x.y * sn;
+        y.y = x.x * sn + x.y * cs;
+    }
+    float* dst;
+    if (hs < heads) dst = q_out + ((int64_t)hs * tokens + t) * head_dim;
+    else if (hs < heads + kv_heads) dst = k_cache + ((int64_t)(hs - heads) * kv_capacity + p0 + t) * head_dim;
+    else dst = v_cache + ((int64_t)(hs - heads - kv_heads) * kv_capacity + p0 + t) * head_dim;
+    *reinterpret_cast<float2*>(dst + 2 * i) = y;
+}
+
 // [heads, tokens, head_dim] -> [tokens, heads * head_dim]: attention output back to the token-major rows a projection takes.
 __global__ __launch_bounds__(256) void heads_to_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int heads,
                                                             int tokens, int head_dim) {
@@ -217,6 +331,18 @@ int launch_rope_scatter(const float* in, int64_t in_row_pitch, float* out, int t
     const int64_t n = (int64_t)tokens * heads * (head_dim / 2);
     rope_scatter_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(
         in, in_row_pitch, out, tokens, heads, head_dim, pos_start, pos_dev, theta, rotate, out_head_stride, out_row_is_pos);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+int launch_rope_qkv(const float* qkv, float* q_out, float* k_cache, float* v_cache, int tokens, int heads, int kv_heads,
+                    int head_dim, int kv_capacity, int pos_start, const int32_t* pos_dev, float theta) {
+    if (tokens <= 0 || heads <= 0 || kv_heads <= 0 || head_dim <= 0) return 0;
+    if (head_dim & 1) return set_error("rope: head_dim must be even; got %d", head_dim);
+    if (!pos_dev && (pos_start < 0 || pos_start + tokens > kv_capacity))
+        return set_error("rope_qkv: positions [%d, %d) do not fit a cache of %d rows", pos_start, pos_start + tokens, kv_capacity);
+    const int64_t n = (int64_t)tokens * (heads + 2 * kv_heads) * (head_dim / 2);
+    rope_qkv_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(
+        qkv, q_out, k_cache, v_cache, tokens, heads, kv_heads, head_dim, kv_capacity, pos_start, pos_dev, theta);
     SKH_CHECK(hipGetLastError());
     return 0;
 }
@@ -262,6 +388,13 @@ int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink) {
 
 int launch_rms_norm(const float* in, const float* gamma, float* out, int rows, int cols, float eps) {
     if (rows <= 0 || cols <= 0) return 0;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(gamma)) & 15) == 0;
+    if (aligned && (cols & 3) == 0 && cols <= 4 * ROW_THREADS * 8) {
+        if (cols <= 4 * ROW_THREADS * 4) rms_norm_cached_kernel<4><<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, gamma, out, cols, eps);
+        else rms_norm_cached_kernel<8><<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, gamma, out, cols, eps);
+        SKH_CHECK(hipGetLastError());
+        return 0;
+    }
     rms_norm_kernel<<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, gamma, out, cols, eps);
     SKH_CHECK(hipGetLastError());
     return 0;
@@ -284,10 +417,9 @@ int launch_silu_mul(const float* gate, const float* up, float* out, int64_t n) {
     SKH_CHECK(hipGetLastError());
     return 0;
 }
-int launch_swiglu_rows(const float* gate_up, float* out, int rows, int ffn) {
-    if (rows <= 0 || ffn <= 0) return 0;
-    const int64_t n = (int64_t)rows * ffn;
-    swiglu_rows_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(gate_up, out, n, ffn);
+int launch_swiglu_pairs(const float* gate_up, float* out, int64_t n) {
+    if (n <= 0) return 0;
+    swiglu_pairs_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(reinterpret_cast<const float2*>(gate_up), out, n);
     SKH_CHECK(hipGetLastError());
     return 0;
 }
@@ -299,6 +431,13 @@ int launch_add(const float* a, const float* b, float* out, int64_t n) {
 }
 int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out) {
     if (rows <= 0 || cols <= 0) return 0;
+    if (rows <= ARGMAX_MAX_ROWS && cols >= 16384) {
+        ArgmaxScratch* sc = static_cast<ArgmaxScratch*>(sync_scratch(sizeof(ArgmaxScratch)));
+        if (!sc) return -1;
+        argmax_split_kernel<<<dim3(ARGMAX_SPLIT, rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, cols, out, sc);
+        SKH_CHECK(hipGetLastError());
+        return 0;
+    }
     argmax_rows_kernel<<<dim3(rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, cols, out);
     SKH_CHECK(hipGetLastError());
     return 0;

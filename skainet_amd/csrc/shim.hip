@@ -30,7 +30,11 @@ int launch_add(const float* a, const float* b, float* out, int64_t n);
 int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out);
 int launch_rope_scatter(const float* in, int64_t in_row_pitch, float* out, int tokens, int heads, int head_dim, int pos_start,
                         const int32_t* pos_dev, float theta, int rotate, int64_t out_head_stride, int out_row_is_pos);
-int launch_swiglu_rows(const float* gate_up, float* out, int rows, int ffn);
+int launch_swiglu_pairs(const float* gate_up, float* out, int64_t n);
+int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k, int n, int batch, const float* gain, float eps,
+                               const float* residual, int epilogue);
+int launch_rope_qkv(const float* qkv, float* q_out, float* k_cache, float* v_cache, int tokens, int heads, int kv_heads,
+                    int head_dim, int kv_capacity, int pos_start, const int32_t* pos_dev, float theta);
 int launch_i32_store_at(int32_t* dst, const int32_t* index, int32_t offset, const int32_t* src);
 int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim);
 int launch_i32_increment(int32_t* v, int32_t delta);
@@ -50,6 +54,7 @@ static thread_local hipEvent_t t_ev0 = nullptr, t_ev1 = nullptr;
 struct Scratch { void* ptr = nullptr; size_t cap = 0; };
 static thread_local Scratch t_workspace;          // kernel scratch (attention split-K partials, GEMM staging)
 static thread_local Scratch t_stage[6];           // device staging of the host-pointer entries
+static thread_local Scratch t_fuse[2];            // normalised input / raw product of the unfused route of matmul_fused
 
 static std::mutex g_mutex;
 static int g_state = 0;        // 0 = not probed, 1 = usable, -1 = unusable
@@ -115,6 +120,20 @@ static void* scratch_get(Scratch& s, size_t bytes) {
     if (check_hip(hipMalloc(&p, cap), "hipMalloc(scratch)") != 0) return nullptr;
     s.ptr = p; s.cap = cap;
     return p;
+}
+// Persistent, zero-initialised device memory for cross-workgroup counters (a kernel that uses one leaves it at zero).
+// One allocation per host thread, made on first use and never moved, so recorded graphs keep a valid address.
+constexpr size_t SYNC_SCRATCH_BYTES = 1u << 20;
+static thread_local void* t_sync = nullptr;
+void* sync_scratch(size_t bytes) {
+    if (bytes > SYNC_SCRATCH_BYTES) { set_error("sync scratch request of %zu bytes exceeds %zu", bytes, SYNC_SCRATCH_BYTES); return nullptr; }
+    if (!t_sync) {
+        void* p = nullptr;
+        if (check_hip(hipMalloc(&p, SYNC_SCRATCH_BYTES), "hipMalloc(sync scratch)") != 0) return nullptr;
+        if (check_hip(hipMemset(p, 0, SYNC_SCRATCH_BYTES), "hipMemset(sync scratch)") != 0) { (void)hipFree(p); return nullptr; }
+        t_sync = p;
+    }
+    return t_sync;
 }
 float* sdpa_workspace(size_t bytes) { return static_cast<float*>(scratch_get(t_workspace, bytes)); }
 void* kernel_workspace(size_t bytes) { return scratch_get(t_workspace, bytes); }
@@ -263,6 +282,40 @@ int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w, const float* x,
 int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out) {
     return skainet_hip_matmul_kind_dev(w, x, m, out, m <= 8 ? 0 : 1);
 }
+// out = epilogue(W . prologue(x)), the products of a decoder block with their neighbouring row ops folded in:
+//   gain != NULL: x is RMS-normalised first (x / sqrt(mean(x^2) + eps) * gain, per activation row);
+//   epilogue 0: out [m, rows] = product; 1: out = residual + product (residual [m, rows], may be `out`);
+//   2: out [m, rows / 2], out[j] = silu(p[2j]) * p[2j + 1] (the weight's rows alternate gate row, up row).
+// Decode shapes of Q4_K weights run as ONE kernel; everything else runs the same arithmetic as separate launches.
+int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out, const float* gain,
+                                     float eps, const float* residual, int32_t epilogue) {
+    if (ensure_device() != 0) return -1;
+    if (!w) return set_error("matmul_fused: null weight handle");
+    if (m <= 0) return 0;
+    if (!x || !out) return set_error("matmul_fused: null activation or output pointer");
+    if (epilogue < 0 || epilogue > 2) return set_error("matmul_fused: unknown epilogue %d", epilogue);
+    if (epilogue == 1 && !residual) return set_error("matmul_fused: the residual epilogue needs a residual pointer");
+    if (epilogue == 2 && (w->rows & 1)) return set_error("matmul_fused: the SwiGLU epilogue needs an even row count; got %d", w->rows);
+    if (w->encoding == ENC_Q4_K && m <= 2) {
+        const int r = launch_q4k_gemv_rows_fused(w->data, x, out, w->cols, w->rows, m, gain, eps, residual, epilogue);
+        if (r != 0) return r < 0 ? -1 : 0;
+    }
+    const float* xin = x;
+    if (gain) {
+        float* xn = static_cast<float*>(scratch_get(t_fuse[0], sizeof(float) * (size_t)m * w->cols));
+        if (!xn || launch_rms_norm(x, gain, xn, m, w->cols, eps) != 0) return -1;
+        xin = xn;
+    }
+    float* y = out;
+    if (epilogue != 0) {
+        y = static_cast<float*>(scratch_get(t_fuse[1], sizeof(float) * (size_t)m * w->rows));
+        if (!y) return -1;
+    }
+    if (skainet_hip_matmul_dev(w, xin, m, y) != 0) return -1;
+    if (epilogue == 1) return launch_add(residual, y, out, (int64_t)m * w->rows);
+    if (epilogue == 2) return launch_swiglu_pairs(y, out, (int64_t)m * (w->rows / 2));
+    return 0;
+}
 // `iters` products back to back on this thread's stream, weight i % nweights each time (several copies of one
 // weight defeat the memory-side cache), bracketed by HIP events. With use_graph the launches are captured once
 // into a HIP graph (kernel nodes only) and replayed, which removes the host's per-launch cost from the GPU timeline.
@@ -396,9 +449,15 @@ int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t* index_dev, int
     if (ensure_device() != 0) return -1;
     return launch_i32_store_at(dst, index_dev, offset, src);
 }
-int32_t skainet_hip_f32_swiglu_rows_dev(const float* gate_up, float* out, int32_t rows, int32_t ffn) {
+int32_t skainet_hip_f32_swiglu_pairs_dev(const float* gate_up, float* out, int64_t n) {
     if (ensure_device() != 0) return -1;
-    return launch_swiglu_rows(gate_up, out, rows, ffn);
+    return launch_swiglu_pairs(gate_up, out, n);
+}
+int32_t skainet_hip_f32_rope_qkv_dev(const float* qkv, float* q_out, float* k_cache, float* v_cache, int32_t tokens, int32_t heads,
+                                     int32_t kv_heads, int32_t head_dim, int32_t kv_capacity, int32_t pos_start,
+                                     const int32_t* pos_dev, float theta) {
+    if (ensure_device() != 0) return -1;
+    return launch_rope_qkv(qkv, q_out, k_cache, v_cache, tokens, heads, kv_heads, head_dim, kv_capacity, pos_start, pos_dev, theta);
 }
 int32_t skainet_hip_f32_heads_to_rows_dev(const float* in, float* out, int32_t heads, int32_t tokens, int32_t head_dim) {
     if (ensure_device() != 0) return -1;

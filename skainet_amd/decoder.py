@@ -13,8 +13,10 @@ graph and replayed (the position lives in device memory).
 Block (standard Llama-3):  h += Wo . attn(rope(Wq n1), rope(Wk n1), Wv n1),  n1 = rmsnorm(h) * g1
                            h += Wdown . (silu(Wgate n2) * (Wup n2)),        n2 = rmsnorm(h) * g2
                            logits = Whead . (rmsnorm(h) * g_out);  greedy = first arg-max.
-q/k/v and gate/up weights are stored concatenated along the output rows ([q; k; v] and [gate; up]) so each pair is
-one pass over the activations.
+q/k/v weights are stored concatenated along the output rows ([q; k; v]) and gate/up interleaved row by row
+(gate row j, up row j, gate row j + 1, ...), so each group is one pass over the activations and the SwiGLU pairs
+come out of the product side by side. The norms, the residual adds and SwiGLU ride inside the products
+(`DeviceWeight.matmul_fused`): a decode step is six launches per block.
 """
 from __future__ import annotations
 
@@ -98,7 +100,7 @@ class LayerWeights:
     wqkv: kernels.DeviceWeight   # [(heads + 2 kv_heads) * head_dim, hidden]
     wo: kernels.DeviceWeight     # [hidden, heads * head_dim]
     ffn_norm: DeviceBuffer       # fp32 [hidden]
-    w_gate_up: kernels.DeviceWeight   # [2 * ffn, hidden]
+    w_gate_up: kernels.DeviceWeight   # [2 * ffn, hidden], row 2j = gate row j, row 2j + 1 = up row j
     w_down: kernels.DeviceWeight      # [hidden, ffn]
 
 
@@ -196,8 +198,6 @@ class LlamaDecoder:
         self.q = DeviceBuffer(rows * c.q_dim * f)            # [heads, rows, head_dim]
         self.attn = DeviceBuffer(rows * c.q_dim * f)         # [heads, rows, head_dim]
         self.attn_rows = DeviceBuffer(rows * c.q_dim * f)    # [rows, heads * head_dim]
-        self.proj = DeviceBuffer(rows * c.hidden * f)
-        self.gate_up = DeviceBuffer(rows * 2 * c.ffn * f)
         self.act = DeviceBuffer(rows * c.ffn * f)
         self.logits = DeviceBuffer(c.vocab * f)
         self.kv_layer_floats = c.kv_heads * c.ctx_max * c.head_dim
@@ -218,15 +218,12 @@ class LlamaDecoder:
         c, w, L = self.cfg, self.w, self.w.layers[li]
         f = 4
         kx = kernels
-        kx.rms_norm_dev(self.h, L.attn_norm, self.norm, rows, c.hidden, c.rms_eps)
-        L.wqkv.matmul(self.norm, rows, self.qkv)
-        qkv_dim = c.q_dim + 2 * c.kv_dim
+        L.wqkv.matmul_fused(self.h, rows, self.qkv, gain=L.attn_norm, eps=c.rms_eps)
         kc = self.k_cache.at(li * self.kv_layer_floats * f)
         vc = self.v_cache.at(li * self.kv_layer_floats * f)
-        # the three column slices of each token's [q | k | v] row go to the query buffer and into the cache
-        self._rope(self.qkv.ptr, self.q.ptr, rows, c.heads, qkv_dim, 0, pos_start, pos_dev, True, rows * c.head_dim, False)
-        self._rope(self.qkv.ptr, kc, rows, c.kv_heads, qkv_dim, c.q_dim, pos_start, pos_dev, True, c.ctx_max * c.head_dim, True)
-        self._rope(self.qkv.ptr, vc, rows, c.kv_heads, qkv_dim, c.q_dim + c.kv_dim, pos_start, pos_dev, False, c.ctx_max * c.head_dim, True)
+        # rotated queries to [heads, rows, head_dim]; rotated keys and raw values into the cache rows of these positions
+        kx.rope_qkv_dev(self.qkv, self.q, kc, vc, rows, c.heads, c.kv_heads, c.head_dim, c.ctx_max, pos_start, pos_dev,
+                        c.rope_theta)
         scale = float(1.0 / np.sqrt(c.head_dim))
         kx.sdpa_cache_dev(self.q, kc, vc, self.attn, 1, c.heads, c.kv_heads, rows, seq_kv, c.ctx_max, c.head_dim, scale,
                           True, 0, 0, kv_len_dev)
@@ -235,19 +232,9 @@ class LlamaDecoder:
             attn_rows = self.attn_rows
         else:
             attn_rows = self.attn                  # one token: [heads, 1, head_dim] is already the row
-        L.wo.matmul(attn_rows, rows, self.proj)
-        kx.add_dev(self.h, self.proj, self.h, rows * c.hidden)
-        kx.rms_norm_dev(self.h, L.ffn_norm, self.norm, rows, c.hidden, c.rms_eps)
-        L.w_gate_up.matmul(self.norm, rows, self.gate_up)
-        kx.swiglu_rows_dev(self.gate_up, self.act, rows, c.ffn)
-        L.w_down.matmul(self.act, rows, self.proj)
-        kx.add_dev(self.h, self.proj, self.h, rows * c.hidden)
-
-    def _rope(self, src, dst, rows, heads, row_pitch, col0, pos_start, pos_dev, rotate, head_stride, row_is_pos):
-        """rope_scatter over the column slice [col0, col0 + heads * head_dim) of token rows `row_pitch` floats apart."""
-        c = self.cfg
-        kernels.rope_scatter_dev(src + 4 * col0, dst, rows, heads, c.head_dim, pos_start, pos_dev, c.rope_theta, rotate,
-                                 head_stride, row_is_pos, in_row_pitch=row_pitch)
+        L.wo.matmul_fused(attn_rows, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
+        L.w_gate_up.matmul_fused(self.h, rows, self.act, gain=L.ffn_norm, eps=c.rms_eps, epilogue=kx.EPI_SWIGLU)
+        L.w_down.matmul_fused(self.act, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
 
     def _head(self, row: int) -> None:
         c = self.cfg

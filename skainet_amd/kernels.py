@@ -105,6 +105,9 @@ def to_kernel_order(encoding: str, row_major: np.ndarray, rows: int, blocks_per_
 
 # ---------------------------------------------------------------------------------------------- device weights
 
+EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
+
+
 class DeviceWeight:
     """A packed [rows, cols] weight resident on the device (canonical row-major blocks)."""
 
@@ -147,6 +150,11 @@ class DeviceWeight:
             check(_lib.hip().skainet_hip_matmul_dev(self._h, _ptr(x), m, _ptr(out)), "matmul")
         else:
             check(_lib.hip().skainet_hip_matmul_kind_dev(self._h, _ptr(x), m, _ptr(out), kind), "matmul")
+
+    def matmul_fused(self, x, m: int, out, gain=None, eps: float = 0.0, residual=None, epilogue: int = 0) -> None:
+        """out = epilogue(W . rmsnorm(x) if gain is given else W . x); epilogue EPI_NONE / EPI_RESIDUAL / EPI_SWIGLU."""
+        check(_lib.hip().skainet_hip_matmul_fused_dev(self._h, _ptr(x), m, _ptr(out), _ptr(gain), eps, _ptr(residual), epilogue),
+              "matmul_fused")
 
     def dequantize(self, out) -> None:
         check(_lib.hip().skainet_hip_dequantize_dev(self._h, _ptr(out)), "dequantize")
@@ -245,8 +253,15 @@ def rope_scatter_dev(x, out, tokens, heads, head_dim, pos_start=0, pos_dev=None,
           "rope_scatter")
 
 
-def swiglu_rows_dev(gate_up, out, rows: int, ffn: int) -> None:
-    check(_lib.hip().skainet_hip_f32_swiglu_rows_dev(_ptr(gate_up), _ptr(out), rows, ffn), "swiglu_rows")
+def swiglu_pairs_dev(gate_up, out, n: int) -> None:
+    """out[i] = silu(gate_up[2i]) * gate_up[2i + 1] for i < n."""
+    check(_lib.hip().skainet_hip_f32_swiglu_pairs_dev(_ptr(gate_up), _ptr(out), n), "swiglu_pairs")
+
+
+def rope_qkv_dev(qkv, q_out, k_cache, v_cache, tokens, heads, kv_heads, head_dim, kv_capacity, pos_start=0, pos_dev=None,
+                 theta=10000.0) -> None:
+    check(_lib.hip().skainet_hip_f32_rope_qkv_dev(_ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), tokens, heads, kv_heads,
+                                                  head_dim, kv_capacity, pos_start, _ptr(pos_dev), theta), "rope_qkv")
 
 
 def heads_to_rows_dev(x, out, heads, tokens, head_dim) -> None:

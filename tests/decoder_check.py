@@ -72,7 +72,7 @@ class CheckDecoder:
             h = h + att.reshape(n, c.q_dim) @ L["wo"].T
             x = self._rms(h, L["ffn_norm"])
             gu = x @ L["w_gate_up"].T
-            g, u = gu[:, :c.ffn], gu[:, c.ffn:]
+            g, u = gu[:, 0::2], gu[:, 1::2]          # rows of w_gate_up alternate gate row, up row
             h = h + (g / (1.0 + np.exp(-g)) * u) @ L["w_down"].T
         logits = self._rms(h[-1], self.out_norm) @ self.head.T
         return h, logits

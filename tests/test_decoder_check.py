@@ -72,6 +72,6 @@ def test_single_token_reduces_to_matrix_algebra():
     h1 = x0 + L["wo"] @ att
     n2 = h1 / np.sqrt((h1 ** 2).mean() + cfg.rms_eps) * L["ffn_norm"]
     gu = L["w_gate_up"] @ n2
-    g, u = gu[:cfg.ffn], gu[cfg.ffn:]
+    g, u = gu[0::2], gu[1::2]
     want = h1 + L["w_down"] @ (g / (1 + np.exp(-g)) * u)
     assert np.abs(h[0] - want).max() < 1e-10

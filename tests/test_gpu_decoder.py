@@ -91,15 +91,79 @@ def test_heads_to_rows_and_swiglu_and_increment(hip_backend, torch_cuda):
     rows, ffn = 3, 130
     gu = (rng.standard_normal((rows, 2 * ffn)) * 3).astype(np.float32)
     act = torch.empty(rows * ffn, dtype=torch.float32, device="cuda")
-    kx.swiglu_rows_dev(dev(torch, gu), act, rows, ffn)
+    kx.swiglu_pairs_dev(dev(torch, gu), act, rows * ffn)
     ctr = dev(torch, np.array([41], np.int32))
     kx.i32_increment_dev(ctr, 1)
     kx.i32_increment_dev(ctr, 3)
     kx.sync()
     assert np.array_equal(out.cpu().numpy().reshape(tokens, heads, hd), a.transpose(1, 0, 2))
-    g, u = gu[:, :ffn].astype(np.float64), gu[:, ffn:].astype(np.float64)
+    g, u = gu[:, 0::2].astype(np.float64), gu[:, 1::2].astype(np.float64)
     assert max_norm_err(act.cpu().numpy().reshape(rows, ffn), g / (1 + np.exp(-g)) * u) < 1e-6
     assert int(ctr.cpu()[0]) == 45
+
+
+def test_rope_qkv_equals_three_scatters(hip_backend, torch_cuda):
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(31)
+    tokens, heads, kvh, hd, cap, pos0, theta = 5, 8, 2, 64, 40, 9, 500000.0
+    width = (heads + 2 * kvh) * hd
+    qkv = dev(torch, rng.standard_normal((tokens, width)).astype(np.float32))
+    pos_dev = dev(torch, np.array([pos0], np.int32))
+    for use_dev_pos in (False, True):
+        q1 = torch.zeros(heads * tokens * hd, device="cuda")
+        k1 = torch.full((kvh * cap * hd,), 3.0, device="cuda")
+        v1 = torch.full((kvh * cap * hd,), 3.0, device="cuda")
+        q2, k2, v2 = torch.zeros_like(q1), torch.full_like(k1, 3.0), torch.full_like(v1, 3.0)
+        pd = pos_dev if use_dev_pos else None
+        ps = 0 if use_dev_pos else pos0
+        kx.rope_qkv_dev(qkv, q1, k1, v1, tokens, heads, kvh, hd, cap, ps, pd, theta)
+        base = qkv.data_ptr()
+        kx.rope_scatter_dev(base, q2, tokens, heads, hd, ps, pd, theta, True, tokens * hd, False, in_row_pitch=width)
+        kx.rope_scatter_dev(base + 4 * heads * hd, k2, tokens, kvh, hd, ps, pd, theta, True, cap * hd, True, in_row_pitch=width)
+        kx.rope_scatter_dev(base + 4 * (heads + kvh) * hd, v2, tokens, kvh, hd, ps, pd, theta, False, cap * hd, True,
+                            in_row_pitch=width)
+        kx.sync()
+        for a, b in ((q1, q2), (k1, k2), (v1, v2)):
+            assert np.array_equal(a.cpu().numpy(), b.cpu().numpy())
+    from skainet_amd._lib import HipError
+    with pytest.raises(HipError):
+        kx.rope_qkv_dev(qkv, q1, k1, v1, tokens, heads, kvh, hd, cap, cap - 2, None, theta)   # rows past the cache
+
+
+@pytest.mark.parametrize("enc,n,k,m", [("Q4_K", 1536, 1024, 1), ("Q4_K", 1030, 512, 2), ("Q4_K", 24, 4096 + 256, 1),
+                                        ("Q4_K", 640, 512, 5), ("Q6_K", 512, 512, 1), ("Q4_K", 768, 1024, 24)])
+def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
+    """Every prologue / epilogue combination against float64 arithmetic on the oracle-decoded weight; the decode
+    shapes of Q4_K run the one-kernel route, the other cases the composed route of the same entry."""
+    from oracle import lib as O
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(n + k + m)
+    packed = kx.quantize(enc, (rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+    wd = O.dequant(enc, packed).reshape(n, k).astype(np.float64)
+    w = kx.DeviceWeight.upload(enc, packed, n, k)
+    x = (rng.standard_normal((m, k)) * 2).astype(np.float32)
+    gain = (1 + 0.2 * rng.standard_normal(k)).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    eps = 1e-5
+    tol = 2e-2 if m > 8 else 1e-3
+    xd = x.astype(np.float64)
+    xn = xd / np.sqrt((xd * xd).mean(1, keepdims=True) + eps) * gain
+    d_x, d_gain = dev(torch, x), dev(torch, gain)
+    for use_gain in (False, True):
+        p = (xn if use_gain else xd) @ wd.T
+        for epi in (kx.EPI_NONE, kx.EPI_RESIDUAL, kx.EPI_SWIGLU):
+            want = p if epi == kx.EPI_NONE else p + res if epi == kx.EPI_RESIDUAL else \
+                p[:, 0::2] / (1 + np.exp(-p[:, 0::2])) * p[:, 1::2]
+            out = dev(torch, res.copy()) if epi == kx.EPI_RESIDUAL else torch.full((m, want.shape[1]), 9.0, device="cuda")
+            w.matmul_fused(d_x, m, out, gain=d_gain if use_gain else None, eps=eps,
+                           residual=out if epi == kx.EPI_RESIDUAL else None, epilogue=epi)   # residual aliases the output
+            kx.sync()
+            assert max_norm_err(out.cpu().numpy(), want) < tol, (use_gain, epi)
+    from skainet_amd._lib import HipError
+    with pytest.raises(HipError):
+        w.matmul_fused(d_x, m, out, epilogue=kx.EPI_RESIDUAL)          # residual epilogue without a residual
+    with pytest.raises(HipError):
+        w.matmul_fused(d_x, m, out, epilogue=7)
 
 
 def test_sdpa_cache_layout_matches_contiguous(hip_backend, torch_cuda):

@@ -182,6 +182,38 @@ def test_norms_softmax_and_glue(hip_backend, torch_cuda):
     close(ho[:rows].sum(1), np.ones(rows), rel=1e-5)
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 8192), (3, 4099), (2, 100), (7, 6144), (1, 12288)])
+def test_rms_norm_row_shapes(hip_backend, torch_cuda, rows, cols):
+    """Register-cached rows (cols % 4 == 0 up to 8192) and the looping kernel (everything else) against the oracle."""
+    torch, kx = torch_cuda, hip_backend
+    x = (np.random.default_rng(cols).standard_normal((rows, cols)) * 2).astype(np.float32)
+    g = np.random.default_rng(cols + 1).standard_normal(cols).astype(np.float32)
+    out = torch.empty(rows, cols, device="cuda")
+    kx.rms_norm_dev(dev(torch, x), dev(torch, g), out, rows, cols, 1e-6)
+    ref = np.empty_like(x)
+    L.oracle().orc_f32_rms_norm(L.fp(x), L.fp(g), L.fp(ref), rows, cols, 1e-6)
+    close(out.cpu().numpy(), ref, rel=2e-5, abs_=1e-6)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 16384), (64, 20000), (65, 20000), (2, 16383), (3, 128256)])
+def test_argmax_split_and_single_kernels(hip_backend, torch_cuda, rows, cols):
+    """Few long rows take the many-workgroups-per-row kernel (twice in a row: its counters must come back to zero),
+    other shapes the one-workgroup-per-row kernel; ties keep the lowest index, also across slice borders."""
+    torch, kx = torch_cuda, hip_backend
+    lg = np.random.default_rng(rows * cols).standard_normal((rows, cols)).astype(np.float32)
+    lg[0, cols - 1] = lg[0, cols // 2] = 40.0          # tie in two different slices
+    if rows > 1:
+        lg[1, :] = 1.5                                  # all equal: index 0
+    idx = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+    want = [int(r.argmax()) for r in lg]
+    assert want[0] == cols // 2
+    d = dev(torch, lg)
+    for _ in range(2):
+        idx.fill_(-1)
+        kx.argmax_rows_dev(d, rows, cols, idx)
+        assert idx.cpu().tolist() == want
+
+
 def test_dense_matmuls(hip_backend, torch_cuda):
     prov = hip_backend.HipKernelProvider()
     rng = np.random.default_rng(9)
