@@ -175,6 +175,9 @@ __global__ __launch_bounds__(256) void zero_kernel(float* out, int64_t n) {
 }
 
 float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
+int launch_sdpa_decode(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
+                       int seq_kv, int kv_capacity, int head_dim, float scale, int window, int right_context,
+                       const int32_t* lengths);   // sdpa_decode.hip
 
 int launch_sdpa(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                 int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window, int right_context,
@@ -198,6 +201,11 @@ int launch_sdpa(const float* q, const float* k, const float* v, float* out, int 
                         (mask_q == 1 || mask_q == seq_q) && (mask_k == 1 || mask_k == seq_kv);
         if (!ok) return set_error("sdpa: mask dims [%d,%d,%d,%d] do not broadcast over [%d,%d|%d,%d,%d]", mask_b, mask_h,
                                   mask_q, mask_k, batch, heads, kv_heads, seq_q, seq_kv);
+    }
+    if (seq_q == 1 && !mask) {   // decode shape: the split-K cache-streaming kernel, when the head shape is one it carries
+        const int r = launch_sdpa_decode(q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, head_dim, scale, window,
+                                         right_context, lengths);
+        if (r != 0) return r < 0 ? -1 : 0;
     }
     SdpaParams p{q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, kv_capacity, scale, causal, window, right_context,
                  lengths, mask, mask_b, mask_h, mask_q, mask_k, 1, 1, nullptr};

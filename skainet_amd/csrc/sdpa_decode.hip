@@ -1,0 +1,257 @@
+// Decode-shape attention (one query position per sequence) over a KV cache: bandwidth-bound split-K.
+//
+// Same contract as the general kernel in sdpa.hip (reference: skainet_f32_sdpa,
+//   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/f32_fused.c:290-396, rules of
+//   /root/reference/skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/ops/AttentionMask.kt:24-104)
+// for seq_q == 1 and no additive mask: the attended keys are one range [first, end) per sequence (window, causal
+// and key-length rules all cut a range), an empty range means uniform weights over every key.
+//
+// The K/V rows of a cache are read exactly once, straight from HBM into registers, no LDS staging:
+//   * grid (key splits, kv heads x head sub-groups, batch); a workgroup owns one split of the key range of one
+//     KV head and GS of the query heads that share it, so a K/V row is loaded once for GS heads;
+//   * 16 lanes hold one key row (D / 16 consecutive floats each), a wave covers 4 adjacent keys per load
+//     instruction (one contiguous span of 4 rows), the 4 waves interleave groups of 4 keys;
+//   * every 16-lane group keeps its own online-softmax state (running max, sum, output slice) for its keys, so
+//     the key loop has no cross-lane traffic beyond the 4-step dot-product reduction; states are merged across
+//     lane groups by shuffles, across waves through LDS;
+//   * splits > 1: each workgroup writes an unnormalised partial (output, max, sum); the workgroup that arrives
+//     last for its (sequence, head group) -- an agent-scope counter tells it -- merges the partials and writes
+//     the result, so there is no second launch.
+#include "common.h"
+
+namespace skh {
+
+constexpr float SDPA_DECODE_MASKED = -1.0e30f;
+constexpr int SDPA_DECODE_MAX_SPLITS = 64;
+
+struct SdpaDecodeParams {
+    const float *q, *k, *v;
+    float* out;
+    int batch, heads, kv_heads, seq_kv, kv_capacity;
+    float scale;
+    int window, right_context;
+    const int32_t* lengths;
+    int splits;
+    float* part;          // [batch * heads][splits][D + 2]
+    unsigned* counters;   // one per (batch, kv head, head sub-group), zero between launches
+};
+
+__device__ __forceinline__ float exp_diff(float m_old, float m_new) { return m_old == -INFINITY ? 0.f : expf(m_old - m_new); }
+
+template <int GS, int DPL>
+__global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
+    constexpr int D = 16 * DPL;
+    constexpr int U = 2;                       // groups of 4 keys a wave has in flight
+    __shared__ float wacc[4][GS][D];
+    __shared__ float wm[4][GS], wl[4][GS];
+    __shared__ unsigned ticket;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane & 15, kg = lane >> 4;
+    const int split = blockIdx.x, b = blockIdx.z;
+    const int per_kv = p.heads / p.kv_heads;
+    const int subs = per_kv / GS;
+    const int kvh = blockIdx.y / subs;
+    const int h0 = kvh * per_kv + (blockIdx.y % subs) * GS;
+
+    // attended key range of this sequence's single query (absolute position seq_kv - 1, so causal cuts nothing)
+    int first = 0, end = p.seq_kv;
+    if (p.window > 0) {
+        first = max(first, p.seq_kv - p.window);
+        end = min(end, p.seq_kv + p.right_context);
+    }
+    if (p.lengths) end = min(end, p.lengths[b]);
+    end = max(end, 0);
+    const bool uniform = first >= end;         // nothing attended: every key scores the same finite value
+    if (uniform) { first = 0; end = p.seq_kv; }
+    const int chunk = ((end - first + p.splits - 1) / p.splits + 15) & ~15;
+    const int lo = first + split * chunk;
+    const int hi = min(end, lo + chunk);
+
+    float qr[GS][DPL];
+#pragma unroll
+    for (int g = 0; g < GS; ++g) {
+        const float* qp = p.q + ((int64_t)b * p.heads + h0 + g) * D + sub * DPL;
+#pragma unroll
+        for (int d = 0; d < DPL; d += 4) {
+            const float4 t = *reinterpret_cast<const float4*>(qp + d);
+            qr[g][d] = t.x * p.scale; qr[g][d + 1] = t.y * p.scale; qr[g][d + 2] = t.z * p.scale; qr[g][d + 3] = t.w * p.scale;
+        }
+    }
+    float m[GS], l[GS], acc[GS][DPL];
+#pragma unroll
+    for (int g = 0; g < GS; ++g) {
+        m[g] = -INFINITY; l[g] = 0.f;
+#pragma unroll
+        for (int d = 0; d < DPL; ++d) acc[g][d] = 0.f;
+    }
+
+    const float* kb = p.k + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * DPL;
+    const float* vb = p.v + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * DPL;
+    for (int k0 = lo + wave * 4; k0 < hi; k0 += 16 * U) {       // wave-uniform trip count
+        float kr[U][DPL], vr[U][DPL];
+        bool valid[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int key = k0 + 16 * u + kg;
+            valid[u] = key < hi;
+            const int64_t off = (int64_t)min(key, hi - 1) * D;   // a lane past the range re-reads the last row
+#pragma unroll
+            for (int d = 0; d < DPL; d += 4) {
+                const float4 a = *reinterpret_cast<const float4*>(kb + off + d);
+                const float4 c = *reinterpret_cast<const float4*>(vb + off + d);
+                kr[u][d] = a.x; kr[u][d + 1] = a.y; kr[u][d + 2] = a.z; kr[u][d + 3] = a.w;
+                vr[u][d] = c.x; vr[u][d + 1] = c.y; vr[u][d + 2] = c.z; vr[u][d + 3] = c.w;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int g = 0; g < GS; ++g) {
+                float s = 0.f;
+#pragma unroll
+                for (int d = 0; d < DPL; ++d) s = fmaf(qr[g][d], kr[u][d], s);
+                s += __shfl_xor(s, 1, 64);
+                s += __shfl_xor(s, 2, 64);
+                s += __shfl_xor(s, 4, 64);
+                s += __shfl_xor(s, 8, 64);
+                if (uniform) s = SDPA_DECODE_MASKED;
+                if (valid[u]) {
+                    const float m_new = fmaxf(m[g], s);
+                    const float alpha = exp_diff(m[g], m_new);
+                    const float pr = expf(s - m_new);
+                    l[g] = l[g] * alpha + pr;
+#pragma unroll
+                    for (int d = 0; d < DPL; ++d) acc[g][d] = fmaf(pr, vr[u][d], acc[g][d] * alpha);
+                    m[g] = m_new;
+                }
+            }
+        }
+    }
+
+    // merge the four lane groups of the wave (lanes 16 and 32 apart hold the same dims of other keys)
+#pragma unroll
+    for (int step = 16; step <= 32; step <<= 1) {
+#pragma unroll
+        for (int g = 0; g < GS; ++g) {
+            const float mo = __shfl_xor(m[g], step, 64), lo_ = __shfl_xor(l[g], step, 64);
+            const float mm = fmaxf(m[g], mo);
+            const float a = exp_diff(m[g], mm), c = exp_diff(mo, mm);
+            l[g] = l[g] * a + lo_ * c;
+#pragma unroll
+            for (int d = 0; d < DPL; ++d) acc[g][d] = acc[g][d] * a + __shfl_xor(acc[g][d], step, 64) * c;
+            m[g] = mm;
+        }
+    }
+    if (kg == 0) {
+#pragma unroll
+        for (int g = 0; g < GS; ++g) {
+#pragma unroll
+            for (int d = 0; d < DPL; ++d) wacc[wave][g][sub * DPL + d] = acc[g][d];
+            if (sub == 0) { wm[wave][g] = m[g]; wl[wave][g] = l[g]; }
+        }
+    }
+    __syncthreads();
+
+    // merge the four waves; element (g, d) by thread
+    for (int t = threadIdx.x; t < GS * D; t += 256) {
+        const int g = t / D, d = t % D;
+        const float mm = fmaxf(fmaxf(wm[0][g], wm[1][g]), fmaxf(wm[2][g], wm[3][g]));
+        float o = 0.f, ls = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float c = exp_diff(wm[w][g], mm);
+            o = fmaf(wacc[w][g][d], c, o);
+            ls = fmaf(wl[w][g], c, ls);
+        }
+        const int64_t row = (int64_t)b * p.heads + h0 + g;
+        if (p.splits == 1) {
+            p.out[row * D + d] = ls > 0.f ? o / ls : 0.f;
+        } else {
+            float* dst = p.part + (row * p.splits + split) * (D + 2);
+            dst[d] = o;
+            if (d == 0) { dst[D] = mm; dst[D + 1] = ls; }
+        }
+    }
+    if (p.splits == 1) return;
+
+    // publish the partial, take a ticket; the last workgroup of this (sequence, head group) merges all splits
+    __threadfence();
+    __syncthreads();
+    unsigned* counter = p.counters + (int64_t)b * gridDim.y + blockIdx.y;
+    if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket != (unsigned)p.splits - 1) return;      // uniform over the workgroup
+    __threadfence();
+    for (int t = threadIdx.x; t < GS * D; t += 256) {
+        const int g = t / D, d = t % D;
+        const int64_t row = (int64_t)b * p.heads + h0 + g;
+        const float* src = p.part + row * p.splits * (D + 2);
+        float mm = -INFINITY;
+        for (int s = 0; s < p.splits; ++s) mm = fmaxf(mm, src[s * (D + 2) + D]);
+        float o = 0.f, ls = 0.f;
+        for (int s = 0; s < p.splits; ++s) {
+            const float c = exp_diff(src[s * (D + 2) + D], mm);
+            o = fmaf(src[s * (D + 2) + d], c, o);
+            ls = fmaf(src[s * (D + 2) + D + 1], c, ls);
+        }
+        p.out[row * D + d] = ls > 0.f ? o / ls : 0.f;
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
+void* sync_scratch(size_t bytes);      // shim.hip: persistent zero-initialised device memory
+
+constexpr size_t SDPA_COUNTER_OFFSET = 64u << 10;   // the arg-max kernel owns the first 64 KiB of the sync scratch
+constexpr int SDPA_MAX_COUNTERS = 16384;
+
+template <int GS, int DPL>
+static int launch_decode_variant(const SdpaDecodeParams& p, int subs) {
+    sdpa_decode_kernel<GS, DPL><<<dim3(p.splits, p.kv_heads * subs, p.batch), dim3(256), 0, current_stream()>>>(p);
+    SKH_CHECK(hipGetLastError());
+    return 1;
+}
+
+// Returns 1 when this kernel took the call, 0 when the shape is outside its range (the caller uses the general
+// kernel), -1 on error.
+int launch_sdpa_decode(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
+                       int seq_kv, int kv_capacity, int head_dim, float scale, int window, int right_context,
+                       const int32_t* lengths) {
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return 0;
+    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) & 15) return 0;
+    const int per_kv = heads / kv_heads;
+    const int gs_max = head_dim == 256 ? 2 : 4;
+    int gs = gs_max;
+    while (per_kv % gs != 0) gs >>= 1;
+    const int subs = per_kv / gs;
+    if ((int64_t)batch * kv_heads * subs > SDPA_MAX_COUNTERS || batch > 65535) return 0;
+    SdpaDecodeParams p{q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, scale, window, right_context, lengths, 1,
+                       nullptr, nullptr};
+    // enough workgroups to put every CU on the cache, at least 64 keys per split
+    const int64_t groups = (int64_t)batch * kv_heads * subs;
+    int splits = (int)((2 * (int64_t)num_cus() + groups - 1) / groups);
+    splits = min(splits, min(SDPA_DECODE_MAX_SPLITS, (seq_kv + 63) / 64));
+    if (splits < 1) splits = 1;
+    p.splits = splits;
+    if (splits > 1) {
+        p.part = sdpa_workspace(sizeof(float) * (size_t)batch * heads * splits * (head_dim + 2));
+        char* base = static_cast<char*>(sync_scratch(SDPA_COUNTER_OFFSET + sizeof(unsigned) * SDPA_MAX_COUNTERS));
+        if (!p.part || !base) return -1;
+        p.counters = reinterpret_cast<unsigned*>(base + SDPA_COUNTER_OFFSET);
+    }
+    if (head_dim == 64) {
+        if (gs == 4) return launch_decode_variant<4, 4>(p, subs);
+        if (gs == 2) return launch_decode_variant<2, 4>(p, subs);
+        return launch_decode_variant<1, 4>(p, subs);
+    }
+    if (head_dim == 128) {
+        if (gs == 4) return launch_decode_variant<4, 8>(p, subs);
+        if (gs == 2) return launch_decode_variant<2, 8>(p, subs);
+        return launch_decode_variant<1, 8>(p, subs);
+    }
+    if (gs == 2) return launch_decode_variant<2, 16>(p, subs);
+    return launch_decode_variant<1, 16>(p, subs);
+}
+
+}  // namespace skh

@@ -100,6 +100,25 @@ def test_attention_decode_config(hip_backend, torch_cuda, batch):
     close(gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, True, 1024, 0, lengths), L.sdpa(q, k, v, scale, True, 1024, 0, lengths))
 
 
+@pytest.mark.parametrize("heads,kv_heads,d,skv,batch", [(8, 2, 64, 700, 2), (4, 4, 128, 33, 3), (16, 2, 128, 1500, 1),
+                                                         (6, 3, 256, 260, 2), (2, 1, 64, 16, 1), (32, 8, 128, 2048, 1),
+                                                         (12, 4, 64, 5000, 1), (5, 5, 96, 300, 2)])
+def test_attention_decode_kernel_shapes_and_rules(hip_backend, torch_cuda, heads, kv_heads, d, skv, batch):
+    """The one-query kernel over its head shapes (group sizes 1 / 2 / 4 / 8-as-2x4, head_dim 64 / 128 / 256; 96 stays
+    on the general kernel), split and unsplit key ranges, key lengths (one of them 0: uniform weights), windows,
+    and twice in a row so the split counters are known to come back to zero."""
+    rng = np.random.default_rng(heads * d + skv)
+    q = rng.standard_normal((batch, heads, 1, d)).astype(np.float32)
+    k = rng.standard_normal((batch, kv_heads, skv, d)).astype(np.float32)
+    v = rng.standard_normal((batch, kv_heads, skv, d)).astype(np.float32)
+    scale = float(1 / np.sqrt(d))
+    lengths = np.array([skv, 0, skv // 3][:batch], np.int32)
+    for causal, win, rc, lens in ((True, 0, 0, None), (False, 0, 0, lengths), (True, max(1, skv // 5), 0, None),
+                                  (True, max(2, skv // 2), 1, lengths), (True, 0, 0, None)):
+        got = gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, win, rc, lens)
+        close(got, L.sdpa(q, k, v, scale, causal, win, rc, lens), rel=2e-5, abs_=2e-6)
+
+
 def test_attention_prefill_config_against_torch_fp32(hip_backend, torch_cuda):
     """Prefill: seq 2048 causal, 32 / 8 heads, head_dim 128. The oracle checks a 256-long prefix problem exactly;
     the full size is compared with torch's fp32 attention on the same device (textbook softmax(QK^T)V)."""
