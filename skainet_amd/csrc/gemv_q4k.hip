@@ -65,9 +65,11 @@ __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi
 
 enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 
+// Two workgroups per CU is the occupancy the register budget is cut for (the row loads in flight, the pass's
+// activations and the per-row sums all live in registers); asking for more makes the compiler spill.
 template <int B, int R, int PRO, int EPI>
-__global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                                            float* y, int k, int n, int rows_per_wave,
+__global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                            float* y, int k, int n, int rows_per_wave, int chunk_rows,
                                                             const float* __restrict__ gain, float eps, const float* residual) {
     constexpr int NV = 16 * B;   // Q4K_RMAX rows padded to 16, times B
     constexpr int SLICE = 68;    // 64 activations + 4 floats of padding: 16-byte aligned and bank-conflict free
@@ -75,131 +77,141 @@ __global__ __launch_bounds__(256) void q4k_gemv_rows_kernel(const uint8_t* __res
     const int lane = threadIdx.x & 63;
     // readfirstlane: the wave index is uniform across a wave, and saying so keeps every row guard a scalar branch
     const int gw = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
-    const int r0 = gw * rows_per_wave;
-    const int nrows = max(0, min(n, r0 + rows_per_wave) - r0);   // a wave without rows still helps stage activations
+    const int wave_r0 = gw * rows_per_wave;
+    const int wave_end = min(n, wave_r0 + rows_per_wave);
     const int bpr = k >> 8;
     const int64_t row_bytes = (int64_t)bpr * Q4K_BYTES;
-    const uint8_t* wbase = w + (int64_t)r0 * row_bytes;
     const int g = lane & 3;
     const int sh = (g & 1) * 16;
     const uint32_t hi_mask = g >= 2 ? 0xFFFFFFFFu : 0u;
+    const int q_off = 16 + g * 32;
 
-    float acc[16][B];
+    float ssq[B], xscale[B];
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-#pragma unroll
-        for (int b = 0; b < B; ++b) acc[i][b] = 0.f;
+    for (int b = 0; b < B; ++b) { ssq[b] = 0.f; xscale[b] = 1.0f; }
 
-    float ssq[B];
-#pragma unroll
-    for (int b = 0; b < B; ++b) ssq[b] = 0.f;
+    // A wave's rows are taken in chunks of at most Q4K_RMAX (the per-row accumulators live in registers); every
+    // wave of the grid runs the same number of chunks and passes, so the barriers below are uniform.
+    for (int c0 = 0; c0 < rows_per_wave; c0 += chunk_rows) {
+        const int r0 = wave_r0 + c0;
+        const int nrows = max(0, min(wave_end, r0 + chunk_rows) - r0);   // a wave without rows still helps stage activations
+        const uint8_t* wbase = w + (int64_t)r0 * row_bytes;
 
-    for (int blk0 = 0; blk0 < bpr; blk0 += 16) {
-        const int blk = blk0 + (lane >> 2);
-        const int blk_c = min(blk, bpr - 1);                // lanes past K re-read a valid block and multiply it by zero activations
-        const uint8_t* lane_base = wbase + blk_c * Q4K_BYTES;
-        const int q_off = 16 + g * 32;
-
-        // the first rows' weight loads go out before anything else
-        Q4KRow raw[R];
+        float acc[16][B];
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            if (i < nrows) {                                    // wave-uniform
-                const uint8_t* p = lane_base + (int64_t)i * row_bytes;
-                raw[i].hdr = *reinterpret_cast<const uint4*>(p);
-                raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
-                raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+        for (int i = 0; i < 16; ++i)
+#pragma unroll
+            for (int b = 0; b < B; ++b) acc[i][b] = 0.f;
+
+        for (int blk0 = 0; blk0 < bpr; blk0 += 16) {
+            const int blk = blk0 + (lane >> 2);
+            const int blk_c = min(blk, bpr - 1);            // lanes past K re-read a valid block and multiply it by zero activations
+            const uint8_t* lane_base = wbase + blk_c * Q4K_BYTES;
+
+            // the first rows' weight loads go out before anything else
+            Q4KRow raw[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                if (i < nrows) {                                // wave-uniform
+                    const uint8_t* p = lane_base + (int64_t)i * row_bytes;
+                    raw[i].hdr = *reinterpret_cast<const uint4*>(p);
+                    raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                    raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+                }
             }
-        }
 
-        // stage this pass's activations: float4 number f of the pass goes to slice f / 16, position f % 16
-        if (blk0 > 0) __syncthreads();   // the previous pass's slices have been read
+            // stage this pass's activations: float4 number f of the pass goes to slice f / 16, position f % 16.
+            // All loads are issued unconditionally (clamped address, zeroed afterwards) so they overlap.
+            float4 xv[B][4], gv[4];
 #pragma unroll
-        for (int b = 0; b < B; ++b) {
+            for (int j = 0; j < 4; ++j) {
+                const int e = min(blk0 * 256 + (threadIdx.x + 256 * j) * 4, k - 4);
+#pragma unroll
+                for (int b = 0; b < B; ++b) xv[b][j] = *reinterpret_cast<const float4*>(x + (int64_t)b * k + e);
+                if (PRO) gv[j] = *reinterpret_cast<const float4*>(gain + e);
+            }
+            if (blk0 > 0 || c0 > 0) __syncthreads();   // the previous pass's slices have been read
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int f = threadIdx.x + 256 * j;
-                const int e = blk0 * 256 + f * 4;
-                float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (e < k) v4 = *reinterpret_cast<const float4*>(x + (int64_t)b * k + e);
-                if (PRO) {
-                    ssq[b] = fmaf(v4.x, v4.x, fmaf(v4.y, v4.y, fmaf(v4.z, v4.z, fmaf(v4.w, v4.w, ssq[b]))));
-                    if (e < k) {
-                        const float4 g4 = *reinterpret_cast<const float4*>(gain + e);
-                        v4.x *= g4.x; v4.y *= g4.y; v4.z *= g4.z; v4.w *= g4.w;
+                const bool inside = blk0 * 256 + f * 4 < k;
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    float4 v4 = xv[b][j];
+                    if (!inside) v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (PRO) {
+                        if (c0 == 0) ssq[b] = fmaf(v4.x, v4.x, fmaf(v4.y, v4.y, fmaf(v4.z, v4.z, fmaf(v4.w, v4.w, ssq[b]))));
+                        v4.x *= gv[j].x; v4.y *= gv[j].y; v4.z *= gv[j].z; v4.w *= gv[j].w;
                     }
-                }
-                *reinterpret_cast<float4*>(&xlds[b][(f >> 4) * SLICE + (f & 15) * 4]) = v4;
-            }
-        }
-        __syncthreads();
-
-        float xs[B][64], xsum[B][2];
-#pragma unroll
-        for (int b = 0; b < B; ++b) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float4 v4 = *reinterpret_cast<const float4*>(&xlds[b][lane * SLICE + i * 4]);   // zeros past K
-                xs[b][4 * i] = v4.x; xs[b][4 * i + 1] = v4.y; xs[b][4 * i + 2] = v4.z; xs[b][4 * i + 3] = v4.w;
-            }
-            float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-            for (int i = 0; i < 32; ++i) { s0 += xs[b][i]; s1 += xs[b][32 + i]; }
-            xsum[b][0] = s0; xsum[b][1] = s1;
-        }
-
-#pragma unroll
-        for (int c = 0; c < Q4K_RMAX; c += R) {
-            if (c < nrows) {                                  // wave-uniform
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    if (c + i < nrows) q4k_row_dot<B>(raw[i], sh, hi_mask, xs, xsum, acc[c + i]);
-                    if (c + R + i < nrows) {                  // refill with the row R ahead
-                        const uint8_t* p = lane_base + (int64_t)(c + R + i) * row_bytes;
-                        raw[i].hdr = *reinterpret_cast<const uint4*>(p);
-                        raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
-                        raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
-                    }
+                    *reinterpret_cast<float4*>(&xlds[b][(f >> 4) * SLICE + (f & 15) * 4]) = v4;
                 }
             }
-        }
-    }
+            __syncthreads();
 
-    float xscale[B];
+            float xs[B][64], xsum[B][2];
 #pragma unroll
-    for (int b = 0; b < B; ++b) xscale[b] = 1.0f;
-    if (PRO) {
-        // every workgroup has seen all of x: total the squares over its four waves
-        __syncthreads();                                        // the last pass's slices have been read
-        float* red = &xlds[0][0];
+            for (int b = 0; b < B; ++b) {
 #pragma unroll
-        for (int b = 0; b < B; ++b) {
-            const float t = wave_sum(ssq[b]);
-            if (lane == 0) red[(threadIdx.x >> 6) * B + b] = t;
-        }
-        __syncthreads();
+                for (int i = 0; i < 16; ++i) {
+                    const float4 v4 = *reinterpret_cast<const float4*>(&xlds[b][lane * SLICE + i * 4]);   // zeros past K
+                    xs[b][4 * i] = v4.x; xs[b][4 * i + 1] = v4.y; xs[b][4 * i + 2] = v4.z; xs[b][4 * i + 3] = v4.w;
+                }
+                float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-        for (int b = 0; b < B; ++b)
-            xscale[b] = 1.0f / sqrtf((red[b] + red[B + b] + red[2 * B + b] + red[3 * B + b]) * (1.0f / (float)k) + eps);
-    }
+                for (int i = 0; i < 32; ++i) { s0 += xs[b][i]; s1 += xs[b][32 + i]; }
+                xsum[b][0] = s0; xsum[b][1] = s1;
+            }
 
-    float v[NV];
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
+            for (int c = 0; c < Q4K_RMAX; c += R) {
+                if (c < nrows) {                                  // wave-uniform
 #pragma unroll
-        for (int b = 0; b < B; ++b) v[i * B + b] = acc[i][b];
-    wave_fold<NV>(v, lane);
-    const int idx = wave_fold_index<NV>(lane);
-    const int row = idx / B, b = idx % B;
-    float val = v[0] * (B == 1 ? xscale[0] : (b == 0 ? xscale[0] : xscale[B - 1]));
-    if (EPI == EPI_SWIGLU) {
-        // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
-        const float up = __shfl_xor(val, NV / (2 * B), 64);
-        if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
-    } else if (lane < NV && row < nrows) {
-        const int64_t o = (int64_t)b * n + r0 + row;
-        if (EPI == EPI_RESIDUAL) val += residual[o];
-        y[o] = val;
+                    for (int i = 0; i < R; ++i) {
+                        if (c + i < nrows) q4k_row_dot<B>(raw[i], sh, hi_mask, xs, xsum, acc[c + i]);
+                        if (c + R + i < nrows) {                  // refill with the row R ahead
+                            const uint8_t* p = lane_base + (int64_t)(c + R + i) * row_bytes;
+                            raw[i].hdr = *reinterpret_cast<const uint4*>(p);
+                            raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                            raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+                        }
+                    }
+                }
+            }
+        }
+
+        if (PRO && c0 == 0) {
+            // every workgroup has seen all of x: total the squares over its four waves
+            __syncthreads();                                    // the last pass's slices have been read
+            float* red = &xlds[0][0];
+#pragma unroll
+            for (int b = 0; b < B; ++b) {
+                const float t = wave_sum(ssq[b]);
+                if (lane == 0) red[(threadIdx.x >> 6) * B + b] = t;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int b = 0; b < B; ++b)
+                xscale[b] = 1.0f / sqrtf((red[b] + red[B + b] + red[2 * B + b] + red[3 * B + b]) * (1.0f / (float)k) + eps);
+        }
+
+        float v[NV];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+#pragma unroll
+            for (int b = 0; b < B; ++b) v[i * B + b] = acc[i][b];
+        wave_fold<NV>(v, lane);
+        const int idx = wave_fold_index<NV>(lane);
+        const int row = idx / B, b = idx % B;
+        float val = v[0] * (B == 1 ? xscale[0] : (b == 0 ? xscale[0] : xscale[B - 1]));
+        if (EPI == EPI_SWIGLU) {
+            // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
+            const float up = __shfl_xor(val, NV / (2 * B), 64);
+            if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
+        } else if (lane < NV && row < nrows) {
+            const int64_t o = (int64_t)b * n + r0 + row;
+            if (EPI == EPI_RESIDUAL) val += residual[o];
+            y[o] = val;
+        }
     }
 }
 
@@ -210,9 +222,11 @@ void set_q4k_rows_waves_per_cu(int v) { if (v > 0) g_q4k_rows_waves_per_cu = v; 
 // slot kernel), -1 on a launch error.
 template <int PRO, int EPI>
 static void launch_variant(int batch, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n,
-                           int rows_per_wave, const float* gain, float eps, const float* residual) {
-    if (batch == 1) q4k_gemv_rows_kernel<1, 6, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, gain, eps, residual);
-    else q4k_gemv_rows_kernel<2, 3, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, gain, eps, residual);
+                           int rows_per_wave, int chunk_rows, const float* gain, float eps, const float* residual) {
+    if (batch == 1)
+        q4k_gemv_rows_kernel<1, 4, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual);
+    else
+        q4k_gemv_rows_kernel<2, 2, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual);
 }
 
 // y = epilogue(W . prologue(x)); gain != null selects the RMSNorm prologue, epilogue is one of EPI_*.
@@ -225,18 +239,21 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     int total_waves = num_cus() * g_q4k_rows_waves_per_cu;
     int rows_per_wave = (n + total_waves - 1) / total_waves;
     if (epilogue == EPI_SWIGLU) rows_per_wave = (rows_per_wave + 1) & ~1;   // a (gate, up) pair never straddles two waves
-    if (rows_per_wave > Q4K_RMAX) rows_per_wave = Q4K_RMAX;
+    // one round of workgroups over the chip: a wave with more than Q4K_RMAX rows takes them in equal chunks
+    const int nchunks = (rows_per_wave + Q4K_RMAX - 1) / Q4K_RMAX;
+    int chunk_rows = (rows_per_wave + nchunks - 1) / nchunks;
+    if (epilogue == EPI_SWIGLU) chunk_rows = (chunk_rows + 1) & ~1;
     const int waves = (n + rows_per_wave - 1) / rows_per_wave;
     const int grid = (waves + 3) / 4;
     hipStream_t s = current_stream();
     const int variant = (gain ? 3 : 0) + epilogue;
     switch (variant) {
-        case 0: launch_variant<0, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
-        case 1: launch_variant<0, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
-        case 2: launch_variant<0, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
-        case 3: launch_variant<1, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
-        case 4: launch_variant<1, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
-        case 5: launch_variant<1, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, gain, eps, residual); break;
+        case 0: launch_variant<0, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
+        case 1: launch_variant<0, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
+        case 2: launch_variant<0, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
+        case 3: launch_variant<1, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
+        case 4: launch_variant<1, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
+        case 5: launch_variant<1, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
         default: return set_error("q4k gemv: unknown epilogue %d", epilogue);
     }
     SKH_CHECK(hipGetLastError());

@@ -14,9 +14,9 @@
 //   * every 16-lane group keeps its own online-softmax state (running max, sum, output slice) for its keys, so
 //     the key loop has no cross-lane traffic beyond the 4-step dot-product reduction; states are merged across
 //     lane groups by shuffles, across waves through LDS;
-//   * splits > 1: each workgroup writes an unnormalised partial (output, max, sum); the workgroup that arrives
-//     last for its (sequence, head group) -- an agent-scope counter tells it -- merges the partials and writes
-//     the result, so there is no second launch.
+//   * splits > 1: each workgroup writes an unnormalised partial (output, max, sum) and a second, small kernel
+//     merges them. (Merging in the last-arriving workgroup instead needs an agent-scope release / acquire per
+//     workgroup, which on this multi-die part writes back and invalidates whole L2s: measured slower.)
 #include "common.h"
 
 namespace skh {
@@ -33,7 +33,6 @@ struct SdpaDecodeParams {
     const int32_t* lengths;
     int splits;
     float* part;          // [batch * heads][splits][D + 2]
-    unsigned* counters;   // one per (batch, kv head, head sub-group), zero between launches
 };
 
 __device__ __forceinline__ float exp_diff(float m_old, float m_new) { return m_old == -INFINITY ? 0.f : expf(m_old - m_new); }
@@ -44,7 +43,6 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
     constexpr int U = 2;                       // groups of 4 keys a wave has in flight
     __shared__ float wacc[4][GS][D];
     __shared__ float wm[4][GS], wl[4][GS];
-    __shared__ unsigned ticket;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 15, kg = lane >> 4;
@@ -173,43 +171,53 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
             if (d == 0) { dst[D] = mm; dst[D + 1] = ls; }
         }
     }
-    if (p.splits == 1) return;
+}
 
-    // publish the partial, take a ticket; the last workgroup of this (sequence, head group) merges all splits
-    __threadfence();
-    __syncthreads();
-    unsigned* counter = p.counters + (int64_t)b * gridDim.y + blockIdx.y;
-    if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (ticket != (unsigned)p.splits - 1) return;      // uniform over the workgroup
-    __threadfence();
-    for (int t = threadIdx.x; t < GS * D; t += 256) {
-        const int g = t / D, d = t % D;
-        const int64_t row = (int64_t)b * p.heads + h0 + g;
-        const float* src = p.part + row * p.splits * (D + 2);
-        float mm = -INFINITY;
-        for (int s = 0; s < p.splits; ++s) mm = fmaxf(mm, src[s * (D + 2) + D]);
-        float o = 0.f, ls = 0.f;
-        for (int s = 0; s < p.splits; ++s) {
-            const float c = exp_diff(src[s * (D + 2) + D], mm);
-            o = fmaf(src[s * (D + 2) + d], c, o);
-            ls = fmaf(src[s * (D + 2) + D + 1], c, ls);
-        }
-        p.out[row * D + d] = ls > 0.f ? o / ls : 0.f;
+// Merge the per-split (unnormalised output, max, sum) triples of one query row. 4 * D threads: thread (j, d) folds
+// splits j, j + 4, ... of output element d (independent loads, all in flight together), LDS folds the four.
+template <int D>
+__global__ __launch_bounds__(4 * D) void sdpa_decode_combine_kernel(const float* __restrict__ part, float* __restrict__ out, int splits) {
+    __shared__ float sm[SDPA_DECODE_MAX_SPLITS], sl[SDPA_DECODE_MAX_SPLITS];
+    __shared__ float so[4][D];
+    const float* src = part + (int64_t)blockIdx.x * splits * (D + 2);
+    const int d = threadIdx.x % D, j = threadIdx.x / D;
+    if ((int)threadIdx.x < splits) { sm[threadIdx.x] = src[threadIdx.x * (D + 2) + D]; sl[threadIdx.x] = src[threadIdx.x * (D + 2) + D + 1]; }
+    float pv[SDPA_DECODE_MAX_SPLITS / 4];
+#pragma unroll
+    for (int i = 0; i < SDPA_DECODE_MAX_SPLITS / 4; ++i) {
+        const int sp = j + 4 * i;
+        pv[i] = sp < splits ? src[sp * (D + 2) + d] : 0.f;
     }
-    if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    float mm = -INFINITY;
+    for (int sp = 0; sp < splits; ++sp) mm = fmaxf(mm, sm[sp]);
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < SDPA_DECODE_MAX_SPLITS / 4; ++i) {
+        const int sp = j + 4 * i;
+        if (sp < splits) o = fmaf(pv[i], exp_diff(sm[sp], mm), o);
+    }
+    so[j][d] = o;
+    __syncthreads();
+    if (j == 0) {
+        float ls = 0.f;
+        for (int sp = 0; sp < splits; ++sp) ls = fmaf(sl[sp], exp_diff(sm[sp], mm), ls);
+        const float t = so[0][d] + so[1][d] + so[2][d] + so[3][d];
+        out[(int64_t)blockIdx.x * D + d] = ls > 0.f ? t / ls : 0.f;
+    }
 }
 
 float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
-void* sync_scratch(size_t bytes);      // shim.hip: persistent zero-initialised device memory
-
-constexpr size_t SDPA_COUNTER_OFFSET = 64u << 10;   // the arg-max kernel owns the first 64 KiB of the sync scratch
-constexpr int SDPA_MAX_COUNTERS = 16384;
 
 template <int GS, int DPL>
 static int launch_decode_variant(const SdpaDecodeParams& p, int subs) {
+    constexpr int D = 16 * DPL;
     sdpa_decode_kernel<GS, DPL><<<dim3(p.splits, p.kv_heads * subs, p.batch), dim3(256), 0, current_stream()>>>(p);
     SKH_CHECK(hipGetLastError());
+    if (p.splits > 1) {
+        sdpa_decode_combine_kernel<D><<<dim3(p.batch * p.heads), dim3(4 * D), 0, current_stream()>>>(p.part, p.out, p.splits);
+        SKH_CHECK(hipGetLastError());
+    }
     return 1;
 }
 
@@ -225,9 +233,9 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
     int gs = gs_max;
     while (per_kv % gs != 0) gs >>= 1;
     const int subs = per_kv / gs;
-    if ((int64_t)batch * kv_heads * subs > SDPA_MAX_COUNTERS || batch > 65535) return 0;
+    if (batch > 65535) return 0;
     SdpaDecodeParams p{q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, scale, window, right_context, lengths, 1,
-                       nullptr, nullptr};
+                       nullptr};
     // enough workgroups to put every CU on the cache, at least 64 keys per split
     const int64_t groups = (int64_t)batch * kv_heads * subs;
     int splits = (int)((2 * (int64_t)num_cus() + groups - 1) / groups);
@@ -236,9 +244,7 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
     p.splits = splits;
     if (splits > 1) {
         p.part = sdpa_workspace(sizeof(float) * (size_t)batch * heads * splits * (head_dim + 2));
-        char* base = static_cast<char*>(sync_scratch(SDPA_COUNTER_OFFSET + sizeof(unsigned) * SDPA_MAX_COUNTERS));
-        if (!p.part || !base) return -1;
-        p.counters = reinterpret_cast<unsigned*>(base + SDPA_COUNTER_OFFSET);
+        if (!p.part) return -1;
     }
     if (head_dim == 64) {
         if (gs == 4) return launch_decode_variant<4, 4>(p, subs);
