@@ -43,6 +43,7 @@ WORKLOADS = {
     "q4k_gemm_512x14336x4096": ("Q4_K", 14336, 4096, 512),
 }
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+ATTENTION_PREFILL_USES_MFMA = True    # the prompt-shape attention kernel runs bf16 operands on the matrix cores
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.9973, calibrated on a plain copy) + WRITE_SIZE (x1.0);
 # the runs and their raw readings are in profiles/q4k_gemv_11008x4096_b1.md. Workloads not measured report null.
 MEASURED_TRAFFIC_BYTES = {"q4k_gemv_11008x4096_b1": 25666560}
@@ -145,6 +146,140 @@ def cpu_baseline_decode(cfg, host, ctx):
                       f"(median of 21: {t_head * 1e3:.2f} ms); attention, norms, RoPE not included; host has {os.cpu_count()} logical cores"}
 
 
+ATTENTION_WORKLOADS = {
+    # name -> (batch, seq_q, seq_kv); 32 query heads, 8 KV heads, head_dim 128, fp32, scale 1/sqrt(128), causal
+    "sdpa_prefill_2048": (1, 2048, 2048),
+    "sdpa_decode_4096_b1": (1, 1, 4096),
+    "sdpa_decode_4096_b8": (8, 1, 4096),
+}
+FP32_VECTOR_PEAK_TFLOPS = 157.3
+
+
+def cpu_baseline_attention(batch, seq_q, seq_kv, heads, kv_heads, d, scale, budget_s=15.0):
+    """The reference's skainet_f32_sdpa on this host. Prefill is sampled on one KV head's group (heads / kv_heads
+    query heads) and scaled to all groups; decode runs the whole call."""
+    from oracle import lib as L
+    ref = L.ref()
+    fn, kind = (ref.skainet_f32_sdpa, "reference") if ref is not None else (L.oracle(fast=True).orc_f32_sdpa, "port")
+    h, hkv = (heads // kv_heads, 1) if seq_q > 1 else (heads, kv_heads)
+    rng = np.random.default_rng(3)
+    q = rng.standard_normal((batch, h, seq_q, d)).astype(np.float32)
+    k = rng.standard_normal((batch, hkv, seq_kv, d)).astype(np.float32)
+    v = rng.standard_normal((batch, hkv, seq_kv, d)).astype(np.float32)
+    o = np.empty_like(q)
+
+    def call():
+        fn(L.fp(q), L.fp(k), L.fp(v), L.fp(o), batch, h, hkv, seq_q, seq_kv, d, scale, 1, 0, 0, None, None, 0, 0, 0, 0)
+
+    t0 = time.perf_counter()
+    call()
+    one = time.perf_counter() - t0
+    reps = max(1, min(21, int(budget_s / max(one, 1e-6)) - 1))
+    t = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        call()
+        t.append(time.perf_counter() - t0)
+    med = float(np.median(t)) * (heads // h)
+    return med, kind, f"{'one KV head group (' + str(h) + ' query heads) scaled x' + str(heads // h) if seq_q > 1 else 'the whole call'}, " \
+                      f"median of {reps} after 1 warm-up ({med * 1e3:.2f} ms per call, host has {os.cpu_count()} logical cores)"
+
+
+def bench_attention(a):
+    """Fused causal GQA attention, fp32 operands: prefill at 2048 (MFMA-class, flops counted dense as the reference's
+    scenarios do) and one-token decode against a 4096-long KV cache (HBM-bound: K and V are read once)."""
+    import torch
+    from skainet_amd import _lib, kernels
+    batch, sq, skv = ATTENTION_WORKLOADS[a.workload]
+    heads, kvh, d = 32, 8, 128
+    scale = float(1.0 / np.sqrt(d))
+    decode = sq == 1
+    steps = (2000 if decode else 20) if a.steps == 2000 else a.steps
+    warmup = (200 if decode else 3) if a.warmup == 200 else a.warmup
+    gen = torch.Generator(device="cuda").manual_seed(20251125)
+    q = torch.randn((batch, heads, sq, d), device="cuda", generator=gen)
+    kv_bytes = 2 * batch * kvh * skv * d * 4
+    copies = max(2, -(-2 * LLC_BYTES // kv_bytes) + 1) if decode else 1
+    ks = [torch.randn((batch, kvh, skv, d), device="cuda", generator=gen) for _ in range(copies)]
+    vs = [torch.randn((batch, kvh, skv, d), device="cuda", generator=gen) for _ in range(copies)]
+    out = torch.empty_like(q)
+
+    def call(i):
+        kernels.sdpa_dev(q, ks[i % copies], vs[i % copies], out, batch, heads, kvh, sq, skv, d, scale, True)
+
+    call(0)                                   # sizes the library's scratch before any capture
+    kernels.sync()
+
+    def timed(n):
+        if a.no_graph:
+            with kernels.Timer() as t:
+                for i in range(n):
+                    call(i)
+            return t.ms
+        with kernels.Graph() as g:
+            for i in range(n):
+                call(i)
+        g.launch(); g.sync()
+        with kernels.Timer() as t:
+            g.launch()
+        g.close()
+        return t.ms
+
+    if warmup > 0:
+        timed(warmup)
+    t0 = time.perf_counter()
+    ms = timed(steps)
+    wall = time.perf_counter() - t0
+    ms_per_step = ms / steps
+    # sanity: torch's fp32 attention on the same operands (textbook softmax(QK^T)V with the causal rule)
+    call(0)
+    kernels.sync()
+    kk, vv = ks[0].repeat_interleave(heads // kvh, 1), vs[0].repeat_interleave(heads // kvh, 1)
+    sc = torch.matmul(q.double(), kk.double().transpose(-1, -2)) * scale
+    if not decode:
+        sc = sc.masked_fill(~torch.ones(sq, skv, dtype=torch.bool, device="cuda").tril(skv - sq), -1e30)
+    want = torch.matmul(torch.softmax(sc, -1), vv.double())
+    err = float(((out.double() - want).abs().max() / want.abs().max()).cpu())
+    tol = 2e-2
+    del sc, kk, vv, want
+    flops_dense = 4.0 * batch * heads * sq * skv * d
+    alg_bytes = kv_bytes + 2 * q.numel() * 4
+    if decode:
+        gbs = alg_bytes / (ms_per_step * 1e-3) / 1e9
+        value, unit, metric = gbs, "GB/s", "decode attention GB/s"
+        roof = {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}
+    else:
+        tf = flops_dense / (ms_per_step * 1e-3) / 1e12
+        value, unit, metric = tf, "TFLOP/s", "prefill attention TFLOP/s (dense-counted)"
+        peak = MFMA_BF16_PEAK_TFLOPS if ATTENTION_PREFILL_USES_MFMA else FP32_VECTOR_PEAK_TFLOPS
+        roof = {"bound": "mfma", "achieved": round(tf, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(tf / peak, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}
+    out_json = {
+        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if decode or not ATTENTION_PREFILL_USES_MFMA else "bf16 x bf16 -> f32", "data": "synthetic",
+        "config": {"workload": a.workload, "batch": batch, "heads": heads, "kv_heads": kvh, "head_dim": d, "seq_q": sq,
+                   "seq_kv": skv, "causal": True, "kv_copies_rotated": copies,
+                   "launch": "host loop" if a.no_graph else "hip-graph replay"},
+        "roofline": roof,
+        "extra": {"algorithmic_bytes_per_step": alg_bytes, "flops_dense_per_step": flops_dense,
+                  "flops_causal_useful_per_step": flops_dense if decode else flops_dense * (skv + 1) / (2 * skv),
+                  "wall_s_timed_region": round(wall, 4), "max_err_over_max_vs_torch_fp64": err,
+                  "device": _lib.hip().skainet_hip_device_name().decode()},
+    }
+    if err > tol:
+        out_json["extra"]["PARITY_FAILED"] = True
+    if not a.skip_cpu:
+        med, kind, sample = cpu_baseline_attention(batch, sq, skv, heads, kvh, d, scale)
+        cpu_val = alg_bytes / med / 1e9 if decode else flops_dense / med / 1e12
+        # the reference threads its attention rows over at most 4 pool participants once there are >= 512 rows
+        cores = 4 if (kind == "reference" and not decode) else 1
+        out_json["cpu_baseline"] = {"value": round(cpu_val, 4), "unit": unit, "cores": cores, "kind": kind, "sample": sample}
+    print(json.dumps(out_json).replace("NaN", "null"))
+    sys.exit(0 if err <= tol else 1)
+
+
 def bench_decoder(a):
     """Synthetic Llama-3-8B-shape stack: prefill of 512 random token ids, then greedy decode; a step = one decoded token."""
     from dataclasses import replace
@@ -217,7 +352,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000, help="timed steps (default 2000; 200 for the GEMM workloads)")
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS))
+    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
     ap.add_argument("--hbm-only", action="store_true", help="skip the cache-warm pass and the read probe, so every launch of the "
@@ -239,6 +374,8 @@ def main():
 
     if a.workload in DECODER_WORKLOADS:
         bench_decoder(a)
+    if a.workload in ATTENTION_WORKLOADS:
+        bench_attention(a)
     enc, n, k, m = WORKLOADS[a.workload]
     rng = np.random.default_rng(20251125)
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)

@@ -308,6 +308,7 @@ static int g_gemv_waves_per_cu = 8;
 static int g_q4k_rows_enable = 1;
 void set_q4k_rows_waves_per_cu(int v);
 void set_gemm_ksplit(int v);
+void set_sdpa_prefill_mfma(int v);
 int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch);   // gemv_q4k.hip
 
 // Experiment knobs (defaults are the measured best): returns 0 when the key is known.
@@ -316,6 +317,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q4k_rows_waves_per_cu")) { set_q4k_rows_waves_per_cu(value); return 0; }
     if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }
     if (!strcmp(key, "gemm_ksplit")) { set_gemm_ksplit(value); return 0; }
+    if (!strcmp(key, "sdpa_prefill_mfma")) { set_sdpa_prefill_mfma(value); return 0; }
     return -1;
 }
 

@@ -178,6 +178,8 @@ float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on
 int launch_sdpa_decode(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                        int seq_kv, int kv_capacity, int head_dim, float scale, int window, int right_context,
                        const int32_t* lengths);   // sdpa_decode.hip
+int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
+                        int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal);   // sdpa_prefill.hip
 
 int launch_sdpa(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                 int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window, int right_context,
@@ -205,6 +207,10 @@ int launch_sdpa(const float* q, const float* k, const float* v, float* out, int 
     if (seq_q == 1 && !mask) {   // decode shape: the split-K cache-streaming kernel, when the head shape is one it carries
         const int r = launch_sdpa_decode(q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, head_dim, scale, window,
                                          right_context, lengths);
+        if (r != 0) return r < 0 ? -1 : 0;
+    }
+    if (seq_q > 1 && !mask && !lengths && window == 0) {   // prompt shape: the matrix-core kernel, when it carries the shape
+        const int r = launch_sdpa_prefill(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale, causal);
         if (r != 0) return r < 0 ? -1 : 0;
     }
     SdpaParams p{q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, kv_capacity, scale, causal, window, right_context,

@@ -1,0 +1,315 @@
+// Prefill-shape attention on the matrix cores: out = softmax(q k^T * scale + causal rule) v, fp32 in and out,
+// bf16 operands on v_mfma_f32_32x32x16_bf16, fp32 accumulation and fp32 online softmax.
+//
+// Contract: the reference's skainet_f32_sdpa
+//   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/f32_fused.c:290-396
+// restricted to what a prompt pass uses: no additive mask, no key lengths, no window, seq_q <= seq_kv, causal or
+// full; head_dim 64 or 128. Every other call stays on the general fp32 kernel (sdpa.hip). Within these shapes
+// every query attends at least one key, so the reference's "-1e30 on excluded keys" and "excluded keys do not
+// take part" are the same function.
+//
+// Two launches:
+//   1. kv_to_bf16_kernel: K -> bf16 [kv head][key][D], V -> bf16 transposed [kv head][D][key], keys padded with
+//      zeros to a multiple of 64. (The PV product contracts over keys, and an MFMA operand wants 8 consecutive
+//      contraction values per lane: V has to be read along keys, hence the transpose, done once per call.)
+//   2. sdpa_prefill_kernel: one workgroup = 4 waves = up to 4 query heads that share a KV head x 32 query
+//      positions (fewer heads per KV head: more query blocks per workgroup). Keys in blocks of 64: the K and V^T
+//      tiles of a block go global -> registers -> LDS (double-buffered, one barrier per block) and are shared by
+//      the 4 waves. Per wave and block:
+//        S^T[key][query] = K_tile . Q^T           16 MFMAs (Q lives in registers, pre-multiplied by scale * log2 e)
+//        online softmax per query: a query is one accumulator COLUMN, so its 32 scores per 32-key tile sit in
+//          one lane pair (l, l ^ 32): the row statistics need a single cross-lane step
+//        O^T[d][query] += V^T_tile . P            16 MFMAs; P is the S^T accumulator converted in place: the MFMA
+//          contraction index is a free permutation, so the keys a lane holds (4h + {0..3}, 8 + 4h + {0..3} of each
+//          16) are simply declared to be its 8 k-slots and V^T is read in the same order.
+//      Blocks wholly above the diagonal are skipped, only blocks that cross it (or the end of the keys) mask.
+#include "common.h"
+
+namespace skh {
+
+typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 pf_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));   // a native 16-byte vector: staging registers stay registers
+
+constexpr int PF_KB = 64;          // keys per block
+constexpr int PF_QW = 32;          // query positions per wave
+
+// K [b][kvh][kv_capacity][D] fp32 -> kb [b*kvh][spad][D] bf16;  V -> vt [b*kvh][D][spad] bf16. One workgroup per
+// (64-key block, kv head, batch); keys >= seq_kv are written as zeros.
+template <int D>
+__global__ __launch_bounds__(256) void kv_to_bf16_kernel(const float* __restrict__ k, const float* __restrict__ v,
+                                                         __bf16* __restrict__ kb, __bf16* __restrict__ vt, int kv_heads,
+                                                         int seq_kv, int kv_capacity, int spad) {
+    __shared__ float tile[PF_KB][D + 1];
+    const int k0 = blockIdx.x * PF_KB;
+    const int64_t head = (int64_t)blockIdx.z * kv_heads + blockIdx.y;
+    const float* ksrc = k + head * kv_capacity * D;
+    const float* vsrc = v + head * kv_capacity * D;
+    // K: straight conversion, 4 floats per thread-step
+    for (int t = threadIdx.x; t < PF_KB * D / 4; t += 256) {
+        const int key = t / (D / 4), d4 = t % (D / 4);
+        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k0 + key < seq_kv) x = *reinterpret_cast<const float4*>(ksrc + (int64_t)(k0 + key) * D + 4 * d4);
+        pf_bf16x4 o;
+        o[0] = (__bf16)x.x; o[1] = (__bf16)x.y; o[2] = (__bf16)x.z; o[3] = (__bf16)x.w;
+        *reinterpret_cast<pf_bf16x4*>(kb + (head * spad + k0 + key) * D + 4 * d4) = o;
+        float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k0 + key < seq_kv) y = *reinterpret_cast<const float4*>(vsrc + (int64_t)(k0 + key) * D + 4 * d4);
+        tile[key][4 * d4] = y.x; tile[key][4 * d4 + 1] = y.y; tile[key][4 * d4 + 2] = y.z; tile[key][4 * d4 + 3] = y.w;
+    }
+    __syncthreads();
+    // V^T: thread-step = (d, 8 consecutive keys)
+    for (int t = threadIdx.x; t < D * PF_KB / 8; t += 256) {
+        const int d = t / (PF_KB / 8), kc = t % (PF_KB / 8);
+        pf_bf16x8 o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = (__bf16)tile[8 * kc + j][d];
+        *reinterpret_cast<pf_bf16x8*>(vt + (head * D + d) * spad + k0 + 8 * kc) = o;
+    }
+}
+
+struct PrefillParams {
+    const float* q;
+    const __bf16 *kb, *vt;
+    float* out;
+    int heads, kv_heads, seq_q, seq_kv, spad;
+    float scale_log2e;
+    int causal;
+    int heads_per_wg;      // 1, 2 or 4 query heads of one KV head per workgroup
+};
+
+// One 64-key block of the bf16 K and V^T copies: global -> registers, and registers -> the LDS tiles.
+template <int D>
+__device__ __forceinline__ void pf_load_block(pf_u32x4 (&kreg)[PF_KB * (D / 8) / 256], pf_u32x4 (&vreg)[D * (PF_KB / 8) / 256],
+                                              const __bf16* kbase, const __bf16* vbase, int spad, int k0, int tid) {
+    constexpr int KCH = D / 8;
+#pragma unroll
+    for (int j = 0; j < PF_KB * KCH / 256; ++j) {
+        const int c = tid + 256 * j, key = c / KCH, ch = c % KCH;
+        kreg[j] = *reinterpret_cast<const pf_u32x4*>(kbase + (int64_t)(k0 + key) * D + 8 * ch);
+    }
+#pragma unroll
+    for (int j = 0; j < D * (PF_KB / 8) / 256; ++j) {
+        const int c = tid + 256 * j, d = c / (PF_KB / 8), ch = c % (PF_KB / 8);
+        vreg[j] = *reinterpret_cast<const pf_u32x4*>(vbase + (int64_t)d * spad + k0 + 8 * ch);
+    }
+}
+template <int D>
+__device__ __forceinline__ void pf_store_block(const pf_u32x4 (&kreg)[PF_KB * (D / 8) / 256], const pf_u32x4 (&vreg)[D * (PF_KB / 8) / 256],
+                                               __bf16* kt, __bf16* vt, int tid) {
+    constexpr int KCH = D / 8, KP = D + 8, VP = PF_KB + 8;
+#pragma unroll
+    for (int j = 0; j < PF_KB * KCH / 256; ++j) {
+        const int c = tid + 256 * j, key = c / KCH, ch = c % KCH;
+        *reinterpret_cast<pf_u32x4*>(kt + key * KP + 8 * ch) = kreg[j];
+    }
+#pragma unroll
+    for (int j = 0; j < D * (PF_KB / 8) / 256; ++j) {
+        const int c = tid + 256 * j, d = c / (PF_KB / 8), ch = c % (PF_KB / 8);
+        *reinterpret_cast<pf_u32x4*>(vt + d * VP + 8 * ch) = vreg[j];
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
+    constexpr int KP = D + 8;          // K tile row pitch (bf16): 16-byte aligned rows, 16 lanes of a b128 read on distinct banks
+    constexpr int VP = PF_KB + 8;      // V^T tile row pitch (bf16)
+    constexpr int NT = D / 16;         // MFMA steps along head_dim for S
+    constexpr int ND = D / 32;         // 32-row tiles of O^T
+    constexpr int KCH = D / 8;         // 16-byte chunks per K row
+    constexpr int K_LOADS = PF_KB * KCH / 256;       // 16-byte loads per thread for the K tile
+    constexpr int V_LOADS = D * (PF_KB / 8) / 256;   // and for the V^T tile
+    extern __shared__ __attribute__((aligned(16))) uint8_t pf_smem[];       // 2 K tiles, then 2 V^T tiles
+    __bf16* const ktile0 = reinterpret_cast<__bf16*>(pf_smem);
+    __bf16* const vtile0 = ktile0 + 2 * PF_KB * KP;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int per_kv = p.heads / p.kv_heads;
+    const int hpw = p.heads_per_wg;
+    const int qblocks_per_wg = 4 / hpw;
+    const int head_groups = per_kv / hpw;
+    const int kvh = blockIdx.y / head_groups;
+    const int head = kvh * per_kv + (blockIdx.y % head_groups) * hpw + wave % hpw;
+    const int b = blockIdx.z;
+    // causal: the workgroups with the most keys start first
+    const int qb_wg = p.causal ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
+    const int q0 = (qb_wg * qblocks_per_wg + wave / hpw) * PF_QW;          // first query position of this wave
+    const int q_wg_last = min(p.seq_q, (qb_wg + 1) * qblocks_per_wg * PF_QW) - 1;
+    const int shift = p.seq_kv - p.seq_q;                                   // absolute position of query 0
+    // keys any wave of this workgroup needs: [0, kend)
+    const int kend = p.causal ? min(p.seq_kv, q_wg_last + shift + 1) : p.seq_kv;
+    const int nblocks = (kend + PF_KB - 1) / PF_KB;
+    const int my_q = q0 + col;
+    const int my_last_key = p.causal ? my_q + shift : p.seq_kv - 1;         // last key this lane's query attends
+    const int wave_last_key = p.causal ? min(p.seq_kv - 1, q0 + PF_QW - 1 + shift) : p.seq_kv - 1;
+
+    // Q fragment: lane (query col, half h) holds q[16 t + 8 h .. + 7] for every t, times scale * log2(e)
+    pf_bf16x8 qf[NT];
+    {
+        const int qrow = min(my_q, p.seq_q - 1);
+        const float* qp = p.q + (((int64_t)b * p.heads + head) * p.seq_q + qrow) * D + 8 * h;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const float4 a = *reinterpret_cast<const float4*>(qp + 16 * t);
+            const float4 c = *reinterpret_cast<const float4*>(qp + 16 * t + 4);
+            const float f = p.scale_log2e;
+            qf[t] = pf_bf16x8{(__bf16)(a.x * f), (__bf16)(a.y * f), (__bf16)(a.z * f), (__bf16)(a.w * f),
+                              (__bf16)(c.x * f), (__bf16)(c.y * f), (__bf16)(c.z * f), (__bf16)(c.w * f)};
+        }
+    }
+
+    const int64_t kvhead = (int64_t)b * p.kv_heads + kvh;
+    const __bf16* kbase = p.kb + kvhead * p.spad * D;
+    const __bf16* vbase = p.vt + kvhead * D * p.spad;
+    pf_u32x4 kreg[K_LOADS], vreg[V_LOADS];
+    pf_f32x16 oacc[ND];
+#pragma unroll
+    for (int i = 0; i < ND; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;     // per query (column); l_run is this lane's half of the keys
+
+    if (nblocks > 0) {
+        pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, 0, tid);
+        pf_store_block<D>(kreg, vreg, ktile0, vtile0, tid);
+    }
+    __syncthreads();
+
+    for (int blk = 0; blk < nblocks; ++blk) {
+        const int buf = blk & 1;
+        const int k0 = blk * PF_KB;
+        if (blk + 1 < nblocks) pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, k0 + PF_KB, tid);
+        if (k0 <= wave_last_key) {                                   // wave-uniform: this wave has keys in the block
+            // S^T tiles: s[j] covers keys k0 + 32 j .. + 31 (rows) x this wave's 32 queries (columns)
+            pf_f32x16 s[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[j][e] = 0.f;
+                const __bf16* kt = ktile0 + buf * (PF_KB * KP) + (32 * j + col) * KP + 8 * h;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const pf_bf16x8 kf = *reinterpret_cast<const pf_bf16x8*>(kt + 16 * t);
+                    s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s[j], 0, 0, 0);
+                }
+            }
+            // keys past this query's last key score -inf (they take no part)
+            const int first_last = p.causal ? q0 + shift : p.seq_kv - 1;     // the smallest last-key among this wave's queries
+            if (k0 + PF_KB - 1 > first_last || k0 + PF_KB > p.seq_kv) {      // wave-uniform: the block crosses a boundary
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = k0 + 32 * j + 8 * (e >> 2) + 4 * h + (e & 3);
+                        if (key > my_last_key) s[j][e] = -INFINITY;
+                    }
+            }
+            float mx = s[0][0];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[j][e]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);
+            // a query of a padded row past seq_q, or a block wholly past a query's keys, can leave m_new at -inf
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);                // m_run = -inf -> 0
+            float psum = 0.f;
+            pf_bf16x8 pf[4];                                         // pf[2 j + g]: keys 16 g .. of tile j, this lane's 8 slots
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                float pr[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) { pr[e] = __builtin_amdgcn_exp2f(s[j][e] - m_use); psum += pr[e]; }
+                pf[2 * j] = pf_bf16x8{(__bf16)pr[0], (__bf16)pr[1], (__bf16)pr[2], (__bf16)pr[3],
+                                      (__bf16)pr[4], (__bf16)pr[5], (__bf16)pr[6], (__bf16)pr[7]};
+                pf[2 * j + 1] = pf_bf16x8{(__bf16)pr[8], (__bf16)pr[9], (__bf16)pr[10], (__bf16)pr[11],
+                                          (__bf16)pr[12], (__bf16)pr[13], (__bf16)pr[14], (__bf16)pr[15]};
+            }
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+#pragma unroll
+            for (int i = 0; i < ND; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+            // O^T += V^T . P : A = V^T rows d, this lane's k-slots are keys 16 g + 4 h + {0..3} and 16 g + 8 + 4 h + {0..3}
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                for (int i = 0; i < ND; ++i) {
+                    const __bf16* vp = vtile0 + buf * (D * VP) + (32 * i + col) * VP + 16 * g + 4 * h;
+                    const pf_bf16x4 lo = *reinterpret_cast<const pf_bf16x4*>(vp);
+                    const pf_bf16x4 hi = *reinterpret_cast<const pf_bf16x4*>(vp + 8);
+                    const pf_bf16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[g], oacc[i], 0, 0, 0);
+                }
+            }
+        }
+        if (blk + 1 < nblocks) pf_store_block<D>(kreg, vreg, ktile0 + (buf ^ 1) * (PF_KB * KP), vtile0 + (buf ^ 1) * (D * VP), tid);
+        __syncthreads();
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    if (my_q < p.seq_q) {
+        float* op = p.out + (((int64_t)b * p.heads + head) * p.seq_q + my_q) * D;
+#pragma unroll
+        for (int i = 0; i < ND; ++i)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int d = 32 * i + 8 * e4 + 4 * h;
+                *reinterpret_cast<float4*>(op + d) = make_float4(oacc[i][4 * e4] * inv, oacc[i][4 * e4 + 1] * inv,
+                                                                 oacc[i][4 * e4 + 2] * inv, oacc[i][4 * e4 + 3] * inv);
+            }
+    }
+}
+
+void* kernel_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
+
+static int g_prefill_mfma = 1;
+void set_sdpa_prefill_mfma(int v) { g_prefill_mfma = v; }
+
+template <int D>
+static int launch_prefill_d(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
+                            int seq_q, int seq_kv, int kv_capacity, float scale, int causal) {
+    const int spad = (seq_kv + PF_KB - 1) / PF_KB * PF_KB;
+    const size_t elems = (size_t)batch * kv_heads * spad * D;
+    __bf16* ws = static_cast<__bf16*>(kernel_workspace(2 * elems * sizeof(__bf16)));
+    if (!ws) return -1;
+    __bf16 *kb = ws, *vt = ws + elems;
+    hipStream_t s = current_stream();
+    kv_to_bf16_kernel<D><<<dim3(spad / PF_KB, kv_heads, batch), dim3(256), 0, s>>>(k, v, kb, vt, kv_heads, seq_kv, kv_capacity, spad);
+    SKH_CHECK(hipGetLastError());
+    const int per_kv = heads / kv_heads;
+    const int hpw = per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1);
+    const int q_per_wg = (4 / hpw) * PF_QW;
+    PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, hpw};
+    const dim3 grid((seq_q + q_per_wg - 1) / q_per_wg, kv_heads * (per_kv / hpw), batch);
+    constexpr size_t smem = sizeof(__bf16) * (2 * PF_KB * (D + 8) + 2 * D * (PF_KB + 8));
+    static bool attr_set = false;
+    if (!attr_set) {
+        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_prefill_kernel<D>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    sdpa_prefill_kernel<D><<<grid, dim3(256), smem, s>>>(p);
+    SKH_CHECK(hipGetLastError());
+    return 1;
+}
+
+// Returns 1 when the MFMA path took the call, 0 when the shape is outside its range, -1 on error.
+int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
+                        int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal) {
+    if (!g_prefill_mfma) return 0;
+    if (head_dim != 64 && head_dim != 128) return 0;
+    if (seq_q < 16 || seq_q > seq_kv) return 0;          // a handful of rows is the row kernel's business
+    if (batch > 65535 || (int64_t)kv_heads * heads > 65535) return 0;
+    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+         reinterpret_cast<uintptr_t>(out)) & 15) return 0;
+    if (head_dim == 64) return launch_prefill_d<64>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal);
+    return launch_prefill_d<128>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal);
+}
+
+}  // namespace skh
