@@ -13,9 +13,9 @@
 // owning a 128 x 64 patch = 4 x 2 MFMA tiles of 32 x 32 (128 accumulator registers per lane). Per K step a thread
 // decodes 32 consecutive weights of one row (one Q4_K sub-block / one Q6_K quarter / one Q8_0 block) and copies
 // 8 x 16 bytes of the bf16 activation tile; LDS rows are padded to 144 bytes so the 16-byte fragment reads of 32
-// consecutive rows fall on distinct banks. Two LDS stages: the next step's global loads and decode overlap the
-// current step's MFMAs, one barrier per step. When the tile grid is smaller than the chip, K is split across
-// gridDim.z and the partial tiles are combined with fp32 atomic adds into a zeroed C.
+// consecutive rows fall on distinct banks. Two LDS stages (108 KB: one workgroup per CU); global loads run two
+// steps ahead in a two-slot register ring, one barrier per step. When the tile grid is smaller than the chip, K is split across gridDim.z and
+// the partial tiles are combined with fp32 atomic adds into a zeroed C.
 #include "common.h"
 
 namespace skh {
@@ -24,9 +24,11 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int GM = 256, GN = 128, GK = 64;
+constexpr int G_THREADS = (GM / 128) * (GN / 64) * 64;        // one wave per 128 x 64 patch
+constexpr int G_A_LOADS = GM * (GK / 8) / G_THREADS;          // 16-byte chunks of the activation tile per thread
 constexpr int GSTRIDE = GK + 8;                               // bf16 elements per LDS row (144 bytes)
 constexpr int G_A_ELEMS = GM * GSTRIDE, G_W_ELEMS = GN * GSTRIDE;
-constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16);
+constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16);   // two stages
 
 void* kernel_workspace(size_t bytes);   // shim.hip
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);   // gemv.hip
@@ -124,7 +126,7 @@ __device__ __forceinline__ void decode32(const RawQ80& r, int, float* w) {
 }
 
 template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES>
-__global__ __launch_bounds__(256) void dequant_gemm_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
+__global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
                                                            float* __restrict__ c, int m, int n, int k, int k_chunk,
                                                            int use_atomics) {
     extern __shared__ __attribute__((aligned(16))) __bf16 smem[];
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(256) void dequant_gemm_kernel(const __bf16* __restr
     auto w_tile = [&](int buf) { return smem + buf * (G_A_ELEMS + G_W_ELEMS) + G_A_ELEMS; };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / (GN / 64), wn = wave % (GN / 64);
     const int m0 = blockIdx.y * GM, n0 = blockIdx.x * GN;
     const int k_begin = blockIdx.z * k_chunk;
     const int k_end = min(k, k_begin + k_chunk);
@@ -144,27 +146,32 @@ __global__ __launch_bounds__(256) void dequant_gemm_kernel(const __bf16* __restr
     const int wrow = tid >> 1, wsub = tid & 1;
     const uint8_t* wrow_ptr = w + (int64_t)min(n0 + wrow, n - 1) * row_bytes;   // rows past N decode a valid row, never stored
 
-    uint4 areg[8];
-    Raw wraw;
-    auto load_global = [&](int step) {
+    // Staging registers: rings three steps deep of the activation tile (8 x 16 bytes per thread and step) and of the
+    // raw weight bytes, so a load has two full steps of MFMA work to arrive before it is written to LDS. One
+    // workgroup owns a CU (the double-buffered tiles fill its LDS), so the register file is there to be used.
+    // Loads are unconditional (clamped rows, never stored) so all of a step's loads are in flight together.
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int WD = 2;   // = the number of LDS stages: slot / stage index is the step's parity
+    u32x4 aring[WD][G_A_LOADS];
+    Raw wring[WD];
+    auto load_a = [&](u32x4 (&areg)[G_A_LOADS], int step) {
         const int k0 = k_begin + step * GK;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int p = tid + 256 * j, row = p >> 3, kp = p & 7;
-            areg[j] = make_uint4(0u, 0u, 0u, 0u);
-            if (m0 + row < m) areg[j] = *reinterpret_cast<const uint4*>(a + (int64_t)(m0 + row) * k + k0 + 8 * kp);
+        for (int j = 0; j < G_A_LOADS; ++j) {
+            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
+            areg[j] = *reinterpret_cast<const u32x4*>(a + (int64_t)min(m0 + row, m - 1) * k + k0 + 8 * kp);
         }
-        load_raw(wraw, wrow_ptr, k0 + 32 * wsub);
     };
-    auto store_lds = [&](int buf, int step) {
-        const int k0 = k_begin + step * GK;
+    auto store_a = [&](const u32x4 (&areg)[G_A_LOADS], int buf) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int p = tid + 256 * j, row = p >> 3, kp = p & 7;
-            *reinterpret_cast<uint4*>(a_tile(buf) + row * GSTRIDE + 8 * kp) = areg[j];
+        for (int j = 0; j < G_A_LOADS; ++j) {
+            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
+            *reinterpret_cast<u32x4*>(a_tile(buf) + row * GSTRIDE + 8 * kp) = areg[j];
         }
+    };
+    auto store_w = [&](const Raw& raw, int buf, int step) {
         float wv[32];
-        decode32(wraw, k0 + 32 * wsub, wv);
+        decode32(raw, k_begin + step * GK + 32 * wsub, wv);
         __bf16* dst = w_tile(buf) + wrow * GSTRIDE + 32 * wsub;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -183,18 +190,14 @@ __global__ __launch_bounds__(256) void dequant_gemm_kernel(const __bf16* __restr
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    if (nsteps > 0) {
-        load_global(0);
-        store_lds(0, 0);
-    }
-    __syncthreads();
-
+    // nsteps is a multiple of 4 (K chunks are whole 256-element groups) and > 0. Loads past the last step are
+    // clamped to it (a redundant load instead of a branch).
+    auto step_k = [&](int step) { return k_begin + min(step, nsteps - 1) * GK; };
     const int fr = lane & 31, fk = (lane >> 5) * 8;   // fragment row inside a 32-row tile, first k of this lane's 8
-    for (int step = 0; step < nsteps; ++step) {
-        const int buf = step & 1;
-        if (step + 1 < nsteps) load_global(step + 1);
-        const __bf16* at = a_tile(buf) + (128 * wm + fr) * GSTRIDE + fk;
-        const __bf16* wt = w_tile(buf) + (64 * wn + fr) * GSTRIDE + fk;
+    // M: this wave's 32 MFMAs on LDS stage `stage`.
+    auto phase_m = [&](int stage) {
+        const __bf16* at = a_tile(stage) + (128 * wm + fr) * GSTRIDE + fk;
+        const __bf16* wt = w_tile(stage) + (64 * wn + fr) * GSTRIDE + fk;
 #pragma unroll
         for (int kk = 0; kk < GK; kk += 16) {
             bf16x8 af[4], bf[2];
@@ -207,8 +210,33 @@ __global__ __launch_bounds__(256) void dequant_gemm_kernel(const __bf16* __restr
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
-        if (step + 1 < nsteps) store_lds(buf ^ 1, step + 1);
-        __syncthreads();
+    };
+
+    // Every wave alternates M and D; the loop body is one straight-line block (no branches), which is what lets the
+    // compiler's wait-count bookkeeping leave the newest step's loads in flight while the older ones are parked.
+    // (Measured alternatives that did not beat this: a 256 x 256 tile with 8 waves in lockstep or with the two waves
+    // of a SIMD half a step out of phase, one LDS stage with two workgroups per CU, explicit MFMA / VALU issue
+    // interleaving hints.)
+    load_a(aring[0], 0);
+    load_raw(wring[0], wrow_ptr, step_k(0) + 32 * wsub);
+    store_a(aring[0], 0);
+    store_w(wring[0], 0, 0);
+    load_a(aring[1], min(1, nsteps - 1));
+    load_raw(wring[1], wrow_ptr, step_k(1) + 32 * wsub);
+    __syncthreads();
+    for (int s0 = 0; s0 < nsteps; s0 += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int step = s0 + u;
+            // ring slot u held this step's bytes (parked one step ago): refill it with the step after next
+            load_a(aring[u], min(step + 2, nsteps - 1));
+            load_raw(wring[u], wrow_ptr, step_k(step + 2) + 32 * wsub);
+            phase_m(u);
+            // the other LDS stage was last read one step ago (a barrier since): park step + 1 there
+            store_a(aring[u ^ 1], u ^ 1);
+            store_w(wring[u ^ 1], u ^ 1, min(step + 1, nsteps - 1));
+            __syncthreads();
+        }
     }
 
     // accumulator element e of lane l sits at row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32 of its 32 x 32 tile
@@ -239,7 +267,7 @@ static int launch_gemm_enc(const __bf16* a, const uint8_t* w, float* c, int m, i
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)G_SMEM));
         attr_set = true;
     }
-    dequant_gemm_kernel<Raw, BE, BB><<<grid, dim3(256), G_SMEM, s>>>(a, w, c, m, n, k, k_chunk, atomics);
+    dequant_gemm_kernel<Raw, BE, BB><<<grid, dim3(G_THREADS), G_SMEM, s>>>(a, w, c, m, n, k, k_chunk, atomics);
     SKH_CHECK(hipGetLastError());
     return 0;
 }
@@ -270,7 +298,8 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     int ksplit = g_gemm_ksplit;
     if (ksplit <= 0) {
         ksplit = 1;
-        if (tiles < num_cus()) ksplit = (num_cus() + tiles - 1) / tiles;
+        const int want = num_cus();                             // one workgroup is resident per CU
+        if (tiles < want) ksplit = (want + tiles - 1) / tiles;
         if (ksplit > 8) ksplit = 8;
     }
     if (ksplit > kgroups) ksplit = kgroups;
