@@ -1,0 +1,28 @@
+// Pieces of the Q4_K row-streaming GEMV kernel (gemv_q4k.hip) that its launcher and callers share: the raw bytes a
+// lane holds per row, the 6-bit scale / min unpack, the epilogue selector.
+#pragma once
+#include "common.h"
+
+namespace skh {
+
+constexpr int Q4K_RMAX = 12;   // rows a wave can own per chunk (bounds the per-row accumulators)
+
+struct Q4KRow { uint4 hdr, q0, q1; };
+
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+
+// d * sc and dmin * m of the two sub-blocks (2g, 2g + 1) a lane owns. ggml get_scale_min_k4: both packings are
+// evaluated and picked with a lane-constant mask (g < 2: bytes j and j + 4; g >= 2: the split 4 + 2 bit form).
+__device__ __forceinline__ void q4k_lane_scales(const uint4& hdr, int sh, uint32_t hi_mask, float& dlo, float& dhi,
+                                                float& mlo, float& mhi) {
+    const float d = half_bits_to_float_fast(hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(hdr.x >> 16);
+    const uint32_t u = hdr.y >> sh, v = hdr.z >> sh, t = hdr.w >> sh;
+    const uint32_t sc = ((u & 0x3F3Fu) & ~hi_mask) | (((t & 0x0F0Fu) | ((u >> 2) & 0x3030u)) & hi_mask);
+    const uint32_t mn = ((v & 0x3F3Fu) & ~hi_mask) | ((((t >> 4) & 0x0F0Fu) | ((v >> 2) & 0x3030u)) & hi_mask);
+    dlo = d * ubyte0_to_float(sc); dhi = d * ubyte1_to_float(sc);
+    mlo = dmin * ubyte0_to_float(mn); mhi = dmin * ubyte1_to_float(mn);
+}
+
+int q4k_rows_waves_per_cu();
+
+}  // namespace skh

@@ -23,24 +23,16 @@
 //                         sums the squares while staging x * gain and scales its outputs at the end;
 //       epilogue residual y = residual + W . x  (residual may alias y);
 //       epilogue SwiGLU   out[j] = silu(y[2j]) * y[2j + 1] for a weight whose rows alternate gate row, up row.
-#include "common.h"
+#include "gemv_q4k.h"
 
 namespace skh {
-
-constexpr int Q4K_RMAX = 12;   // rows a wave can own (bounds the per-row accumulators)
-
-struct Q4KRow { uint4 hdr, q0, q1; };
 
 template <int B>
 __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi_mask, const float (*x)[64],
                                             const float (*xsum)[2], float* out) {
-    const float d = half_bits_to_float_fast(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(r.hdr.x >> 16);
-    // 6-bit (scale, min) pairs of sub-blocks 2g, 2g+1 (ggml get_scale_min_k4); both packings evaluated, lane-constant pick
-    const uint32_t u = r.hdr.y >> sh, v = r.hdr.z >> sh, t = r.hdr.w >> sh;
-    const uint32_t sc = ((u & 0x3F3Fu) & ~hi_mask) | (((t & 0x0F0Fu) | ((u >> 2) & 0x3030u)) & hi_mask);
-    const uint32_t mn = ((v & 0x3F3Fu) & ~hi_mask) | ((((t >> 4) & 0x0F0Fu) | ((v >> 2) & 0x3030u)) & hi_mask);
-    const float dlo = d * ubyte0_to_float(sc), dhi = d * ubyte1_to_float(sc) * 0.0625f;   // high nibbles summed as 16 * code
-    const float mlo = dmin * ubyte0_to_float(mn), mhi = dmin * ubyte1_to_float(mn);
+    float dlo, dhi, mlo, mhi;
+    q4k_lane_scales(r.hdr, sh, hi_mask, dlo, dhi, mlo, mhi);
+    dhi *= 0.0625f;                                            // high nibbles are summed as 16 * code
     const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
     float lo[B], hi[B];
 #pragma unroll
@@ -62,8 +54,6 @@ __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi
 #pragma unroll
     for (int b = 0; b < B; ++b) out[b] += dlo * lo[b] + dhi * hi[b] - (mlo * xsum[b][0] + mhi * xsum[b][1]);
 }
-
-enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 
 // Two workgroups per CU is the occupancy the register budget is cut for (the row loads in flight, the pass's
 // activations and the per-row sums all live in registers); asking for more makes the compiler spill.
@@ -217,6 +207,7 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
 
 static int g_q4k_rows_waves_per_cu = 8;
 void set_q4k_rows_waves_per_cu(int v) { if (v > 0) g_q4k_rows_waves_per_cu = v; }
+int q4k_rows_waves_per_cu() { return g_q4k_rows_waves_per_cu; }
 
 // Returns 1 when this kernel took the product, 0 when the shape is outside its range (caller falls back to the
 // slot kernel), -1 on a launch error.
@@ -245,6 +236,7 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     if (epilogue == EPI_SWIGLU) chunk_rows = (chunk_rows + 1) & ~1;
     const int waves = (n + rows_per_wave - 1) / rows_per_wave;
     const int grid = (waves + 3) / 4;
+    if (epilogue < EPI_NONE || epilogue > EPI_SWIGLU) return set_error("q4k gemv: unknown epilogue %d", epilogue);
     hipStream_t s = current_stream();
     const int variant = (gain ? 3 : 0) + epilogue;
     switch (variant) {
