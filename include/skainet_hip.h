@@ -113,6 +113,15 @@ SKAINET_HIP_API int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w,
  * Q4_K weights with m <= 2 run as one kernel; other shapes run the same arithmetic as separate launches. */
 SKAINET_HIP_API int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out,
     const float* gain, float eps, const float* residual, int32_t epilogue);
+/* One decode token's q/k/v projection with its neighbours folded in (no reference counterpart as one call: RMSNorm
+ * f32_fused.c:255-286, the product, RoPE and KvCacheStore.appendToken
+ * skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/storage/KvCacheStore.kt:125):
+ * row = W . rmsnorm(x) (gain == NULL: no norm), W's rows being [q | k | v] heads of head_dim; adjacent pairs of the q
+ * and k heads are rotated by pos * theta^(-2i/head_dim) with pos = *pos_dev; q -> q_out [heads, head_dim], k and v ->
+ * row pos of caches [kv_heads, kv_capacity, head_dim]. Q4_K weights run as one kernel. */
+SKAINET_HIP_API int32_t skainet_hip_matmul_qkv_rope_dev(const skainet_hip_weight* w, const float* x, const float* gain,
+    float eps, float* q_out, float* k_cache, float* v_cache, int32_t heads, int32_t kv_heads, int32_t head_dim,
+    int32_t kv_capacity, const int32_t* pos_dev, float theta);
 /* Measurement aid: `iters` such products back to back on this thread's stream, weight number i % nweights at
  * step i, timed with HIP events; returns the elapsed milliseconds (< 0 on failure). use_graph != 0 captures the
  * launches into a HIP graph first and times one replay, so host launch cost stays off the GPU timeline.
@@ -236,6 +245,8 @@ SKAINET_HIP_API int32_t skainet_hip_f32_rope_qkv_dev(const float* qkv, float* q_
 SKAINET_HIP_API int32_t skainet_hip_f32_heads_to_rows_dev(const float* in, float* out, int32_t heads, int32_t tokens, int32_t head_dim);
 SKAINET_HIP_API int32_t skainet_hip_i32_increment_dev(int32_t* value, int32_t delta);
 /* dst[index_dev[0] + offset] = src[0], all on the device: appends a sampled token to a log at the device-side position. */
+/* End of a greedy decode step: *pos += 1, *kv_len += 1, log[*pos] = *token (all device memory, one launch). */
+SKAINET_HIP_API int32_t skainet_hip_decode_advance_dev(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log);
 SKAINET_HIP_API int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t* index_dev, int32_t offset, const int32_t* src);
 
 /* HIP graphs (no reference counterpart; for launch-bound loops such as a decode step): graph_begin redirects this

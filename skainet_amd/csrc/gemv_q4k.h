@@ -9,7 +9,17 @@ constexpr int Q4K_RMAX = 12;   // rows a wave can own per chunk (bounds the per-
 
 struct Q4KRow { uint4 hdr, q0, q1; };
 
-enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE_QKV = 3 };
+
+// Destination of the RoPE epilogue: output rows are one token's [q | k | v] (heads, kv_heads, kv_heads heads of
+// head_dim); q goes rotated to q_out [heads, head_dim] (the kernel's y), k rotated and v raw to row *pos_dev of caches
+// laid out [kv_heads, capacity, head_dim].
+struct RopeQkvEpilogue {
+    float *k_cache, *v_cache;
+    const int32_t* pos_dev;
+    float theta;
+    int heads, kv_heads, head_dim, capacity;
+};
 
 // d * sc and dmin * m of the two sub-blocks (2g, 2g + 1) a lane owns. ggml get_scale_min_k4: both packings are
 // evaluated and picked with a lane-constant mask (g < 2: bytes j and j + 4; g >= 2: the split 4 + 2 bit form).

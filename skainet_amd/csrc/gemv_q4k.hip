@@ -22,7 +22,9 @@
 //       prologue RMSNorm  y = W . (x * gain / sqrt(mean(x^2) + eps)): every workgroup stages all of x anyway, so it
 //                         sums the squares while staging x * gain and scales its outputs at the end;
 //       epilogue residual y = residual + W . x  (residual may alias y);
-//       epilogue SwiGLU   out[j] = silu(y[2j]) * y[2j + 1] for a weight whose rows alternate gate row, up row.
+//       epilogue SwiGLU   out[j] = silu(y[2j]) * y[2j + 1] for a weight whose rows alternate gate row, up row;
+//       epilogue RoPE     the rows are one token's [q | k | v]: adjacent pairs of q and k rotated by the device-side
+//                         position, q written head-major, k and v written into their KV-cache rows.
 #include "gemv_q4k.h"
 
 namespace skh {
@@ -60,7 +62,8 @@ __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi
 template <int B, int R, int PRO, int EPI>
 __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                             float* y, int k, int n, int rows_per_wave, int chunk_rows,
-                                                            const float* __restrict__ gain, float eps, const float* residual) {
+                                                            const float* __restrict__ gain, float eps, const float* residual,
+                                                            RopeQkvEpilogue rope) {
     constexpr int NV = 16 * B;   // Q4K_RMAX rows padded to 16, times B
     constexpr int SLICE = 68;    // 64 activations + 4 floats of padding: 16-byte aligned and bank-conflict free
     __shared__ __attribute__((aligned(16))) float xlds[B][64 * SLICE];
@@ -193,7 +196,25 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
         const int idx = wave_fold_index<NV>(lane);
         const int row = idx / B, b = idx % B;
         float val = v[0] * (B == 1 ? xscale[0] : (b == 0 ? xscale[0] : xscale[B - 1]));
-        if (EPI == EPI_SWIGLU) {
+        if (EPI == EPI_ROPE_QKV) {
+            // rows 2i and 2i + 1 of a head are one rotation pair; like the SwiGLU pairs they sit NV / (2B) lanes apart
+            const float odd = __shfl_xor(val, NV / (2 * B), 64);
+            if (lane < NV && !(row & 1) && row < nrows) {
+                const int o = r0 + row, slot = o / rope.head_dim, dd = o % rope.head_dim;
+                const int p0 = rope.pos_dev[0];
+                float2 out2 = make_float2(val, odd);
+                if (slot < rope.heads + rope.kv_heads) {
+                    float sn, cs;
+                    sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
+                    out2 = make_float2(val * cs - odd * sn, val * sn + odd * cs);
+                }
+                float* dst;
+                if (slot < rope.heads) dst = y + (int64_t)slot * rope.head_dim;
+                else if (slot < rope.heads + rope.kv_heads) dst = rope.k_cache + ((int64_t)(slot - rope.heads) * rope.capacity + p0) * rope.head_dim;
+                else dst = rope.v_cache + ((int64_t)(slot - rope.heads - rope.kv_heads) * rope.capacity + p0) * rope.head_dim;
+                *reinterpret_cast<float2*>(dst + dd) = out2;
+            }
+        } else if (EPI == EPI_SWIGLU) {
             // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
             const float up = __shfl_xor(val, NV / (2 * B), 64);
             if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
@@ -213,39 +234,48 @@ int q4k_rows_waves_per_cu() { return g_q4k_rows_waves_per_cu; }
 // slot kernel), -1 on a launch error.
 template <int PRO, int EPI>
 static void launch_variant(int batch, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n,
-                           int rows_per_wave, int chunk_rows, const float* gain, float eps, const float* residual) {
+                           int rows_per_wave, int chunk_rows, const float* gain, float eps, const float* residual,
+                           const RopeQkvEpilogue& rope) {
     if (batch == 1)
-        q4k_gemv_rows_kernel<1, 4, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual);
+        q4k_gemv_rows_kernel<1, 4, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope);
     else
-        q4k_gemv_rows_kernel<2, 2, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual);
+        q4k_gemv_rows_kernel<2, 2, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope);
 }
 
 // y = epilogue(W . prologue(x)); gain != null selects the RMSNorm prologue, epilogue is one of EPI_*.
 int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k, int n, int batch, const float* gain, float eps,
-                               const float* residual, int epilogue) {
+                               const float* residual, int epilogue, const RopeQkvEpilogue* rope_in) {
     if (batch < 1 || batch > 2) return 0;
+    RopeQkvEpilogue rope{};
+    if (epilogue == EPI_ROPE_QKV) {
+        if (!rope_in || batch != 1) return 0;
+        rope = *rope_in;
+        if ((rope.head_dim & 1) || n != (rope.heads + 2 * rope.kv_heads) * rope.head_dim) return 0;
+    }
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 3)) return 0;
     if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return 0;
-    if (epilogue == EPI_SWIGLU && (n & 1)) return 0;
+    if (epilogue >= EPI_SWIGLU && (n & 1)) return 0;
     int total_waves = num_cus() * g_q4k_rows_waves_per_cu;
     int rows_per_wave = (n + total_waves - 1) / total_waves;
-    if (epilogue == EPI_SWIGLU) rows_per_wave = (rows_per_wave + 1) & ~1;   // a (gate, up) pair never straddles two waves
+    if (epilogue >= EPI_SWIGLU) rows_per_wave = (rows_per_wave + 1) & ~1;   // a (gate, up) or rotation pair never straddles two waves
     // one round of workgroups over the chip: a wave with more than Q4K_RMAX rows takes them in equal chunks
     const int nchunks = (rows_per_wave + Q4K_RMAX - 1) / Q4K_RMAX;
     int chunk_rows = (rows_per_wave + nchunks - 1) / nchunks;
-    if (epilogue == EPI_SWIGLU) chunk_rows = (chunk_rows + 1) & ~1;
+    if (epilogue >= EPI_SWIGLU) chunk_rows = (chunk_rows + 1) & ~1;
     const int waves = (n + rows_per_wave - 1) / rows_per_wave;
     const int grid = (waves + 3) / 4;
-    if (epilogue < EPI_NONE || epilogue > EPI_SWIGLU) return set_error("q4k gemv: unknown epilogue %d", epilogue);
+    if (epilogue < EPI_NONE || epilogue > EPI_ROPE_QKV) return set_error("q4k gemv: unknown epilogue %d", epilogue);
     hipStream_t s = current_stream();
-    const int variant = (gain ? 3 : 0) + epilogue;
+    const int variant = (gain ? 4 : 0) + epilogue;
     switch (variant) {
-        case 0: launch_variant<0, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
-        case 1: launch_variant<0, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
-        case 2: launch_variant<0, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
-        case 3: launch_variant<1, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
-        case 4: launch_variant<1, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
-        case 5: launch_variant<1, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual); break;
+        case 0: launch_variant<0, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
+        case 1: launch_variant<0, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
+        case 2: launch_variant<0, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
+        case 3: launch_variant<0, EPI_ROPE_QKV>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
+        case 4: launch_variant<1, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
+        case 5: launch_variant<1, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
+        case 6: launch_variant<1, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
+        case 7: launch_variant<1, EPI_ROPE_QKV>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
         default: return set_error("q4k gemv: unknown epilogue %d", epilogue);
     }
     SKH_CHECK(hipGetLastError());
@@ -253,7 +283,7 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
 }
 
 int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch) {
-    return launch_q4k_gemv_rows_fused(w, x, y, k, n, batch, nullptr, 0.f, nullptr, EPI_NONE);
+    return launch_q4k_gemv_rows_fused(w, x, y, k, n, batch, nullptr, 0.f, nullptr, EPI_NONE, nullptr);
 }
 
 }  // namespace skh

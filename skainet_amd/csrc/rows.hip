@@ -324,6 +324,22 @@ __global__ void i32_store_at_kernel(int32_t* dst, const int32_t* __restrict__ in
     if (threadIdx.x == 0 && blockIdx.x == 0) dst[index[0] + offset] = src[0];
 }
 
+// End of a greedy decode step in one launch: the position and the key count advance by one and the token just
+// sampled is appended to the log at the new position.
+__global__ void decode_advance_kernel(int32_t* pos, int32_t* kv_len, const int32_t* __restrict__ token, int32_t* log) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const int32_t p = pos[0] + 1;
+        pos[0] = p;
+        kv_len[0] += 1;
+        log[p] = token[0];
+    }
+}
+int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log) {
+    decode_advance_kernel<<<dim3(1), dim3(64), 0, current_stream()>>>(pos, kv_len, token, log);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
 int launch_rope_scatter(const float* in, int64_t in_row_pitch, float* out, int tokens, int heads, int head_dim, int pos_start,
                         const int32_t* pos_dev, float theta, int rotate, int64_t out_head_stride, int out_row_is_pos) {
     if (tokens <= 0 || heads <= 0 || head_dim <= 0) return 0;

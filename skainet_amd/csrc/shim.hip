@@ -8,6 +8,7 @@
 // resource failure
 //   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/q4k_matmul.c:326-333.
 #include "common.h"
+#include "gemv_q4k.h"
 #include "../../include/skainet_hip.h"
 
 #include <cstdarg>
@@ -32,10 +33,11 @@ int launch_rope_scatter(const float* in, int64_t in_row_pitch, float* out, int t
                         const int32_t* pos_dev, float theta, int rotate, int64_t out_head_stride, int out_row_is_pos);
 int launch_swiglu_pairs(const float* gate_up, float* out, int64_t n);
 int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k, int n, int batch, const float* gain, float eps,
-                               const float* residual, int epilogue);
+                               const float* residual, int epilogue, const RopeQkvEpilogue* rope);
 int launch_rope_qkv(const float* qkv, float* q_out, float* k_cache, float* v_cache, int tokens, int heads, int kv_heads,
                     int head_dim, int kv_capacity, int pos_start, const int32_t* pos_dev, float theta);
 int launch_i32_store_at(int32_t* dst, const int32_t* index, int32_t offset, const int32_t* src);
+int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log);
 int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim);
 int launch_i32_increment(int32_t* v, int32_t delta);
 int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink);
@@ -297,7 +299,7 @@ int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x
     if (epilogue == 1 && !residual) return set_error("matmul_fused: the residual epilogue needs a residual pointer");
     if (epilogue == 2 && (w->rows & 1)) return set_error("matmul_fused: the SwiGLU epilogue needs an even row count; got %d", w->rows);
     if (w->encoding == ENC_Q4_K && m <= 2) {
-        const int r = launch_q4k_gemv_rows_fused(w->data, x, out, w->cols, w->rows, m, gain, eps, residual, epilogue);
+        const int r = launch_q4k_gemv_rows_fused(w->data, x, out, w->cols, w->rows, m, gain, eps, residual, epilogue, nullptr);
         if (r != 0) return r < 0 ? -1 : 0;
     }
     const float* xin = x;
@@ -315,6 +317,30 @@ int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x
     if (epilogue == 1) return launch_add(residual, y, out, (int64_t)m * w->rows);
     if (epilogue == 2) return launch_swiglu_pairs(y, out, (int64_t)m * (w->rows / 2));
     return 0;
+}
+// One decode token's q/k/v projection with everything around it: out row = W . rmsnorm(x) (gain == NULL: no norm),
+// W's rows being [q | k | v] heads of head_dim; adjacent pairs of the q and k heads are rotated (RoPE, angle
+// pos * theta^(-2i / head_dim), pos read from the device), q goes to q_out [heads, head_dim], k and v to row pos of
+// caches laid out [kv_heads, kv_capacity, head_dim]. Q4_K weights: one kernel; otherwise product + rope_qkv.
+int32_t skainet_hip_matmul_qkv_rope_dev(const skainet_hip_weight* w, const float* x, const float* gain, float eps, float* q_out,
+                                        float* k_cache, float* v_cache, int32_t heads, int32_t kv_heads, int32_t head_dim,
+                                        int32_t kv_capacity, const int32_t* pos_dev, float theta) {
+    if (ensure_device() != 0) return -1;
+    if (!w || !x || !q_out || !k_cache || !v_cache || !pos_dev) return set_error("matmul_qkv_rope: null argument");
+    if (heads <= 0 || kv_heads <= 0 || head_dim <= 0 || (head_dim & 1))
+        return set_error("matmul_qkv_rope: bad head shape %d / %d x %d", heads, kv_heads, head_dim);
+    if ((int64_t)w->rows != (int64_t)(heads + 2 * kv_heads) * head_dim)
+        return set_error("matmul_qkv_rope: weight has %d rows, the head shape needs %lld", w->rows,
+                         (long long)(heads + 2 * kv_heads) * head_dim);
+    if (w->encoding == ENC_Q4_K) {
+        const RopeQkvEpilogue rope{k_cache, v_cache, pos_dev, theta, heads, kv_heads, head_dim, kv_capacity};
+        const int r = launch_q4k_gemv_rows_fused(w->data, x, q_out, w->cols, w->rows, 1, gain, eps, nullptr, EPI_ROPE_QKV, &rope);
+        if (r != 0) return r < 0 ? -1 : 0;
+    }
+    float* qkv = static_cast<float*>(scratch_get(t_fuse[1], sizeof(float) * (size_t)w->rows));
+    if (!qkv) return -1;
+    if (skainet_hip_matmul_fused_dev(w, x, 1, qkv, gain, eps, nullptr, 0) != 0) return -1;
+    return launch_rope_qkv(qkv, q_out, k_cache, v_cache, 1, heads, kv_heads, head_dim, kv_capacity, 0, pos_dev, theta);
 }
 // `iters` products back to back on this thread's stream, weight i % nweights each time (several copies of one
 // weight defeat the memory-side cache), bracketed by HIP events. With use_graph the launches are captured once
@@ -444,6 +470,11 @@ int32_t skainet_hip_f32_rope_scatter_dev(const float* in, int64_t in_row_pitch, 
     if (ensure_device() != 0) return -1;
     return launch_rope_scatter(in, in_row_pitch, out, tokens, heads, head_dim, pos_start, pos_dev, theta, rotate, out_head_stride,
                                out_row_is_pos);
+}
+int32_t skainet_hip_decode_advance_dev(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log) {
+    if (ensure_device() != 0) return -1;
+    if (!pos || !kv_len || !token || !log) return set_error("decode_advance: null argument");
+    return launch_decode_advance(pos, kv_len, token, log);
 }
 int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t* index_dev, int32_t offset, const int32_t* src) {
     if (ensure_device() != 0) return -1;

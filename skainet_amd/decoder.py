@@ -16,7 +16,9 @@ Block (standard Llama-3):  h += Wo . attn(rope(Wq n1), rope(Wk n1), Wv n1),  n1 
 q/k/v weights are stored concatenated along the output rows ([q; k; v]) and gate/up interleaved row by row
 (gate row j, up row j, gate row j + 1, ...), so each group is one pass over the activations and the SwiGLU pairs
 come out of the product side by side. The norms, the residual adds and SwiGLU ride inside the products
-(`DeviceWeight.matmul_fused`): a decode step is six launches per block.
+(`DeviceWeight.matmul_fused`): a decode step is five launches per block (q/k/v product with norm, RoPE
+and cache append; attention and its split merge; o product with residual; gate/up product with norm and SwiGLU; down
+product with residual).
 """
 from __future__ import annotations
 
@@ -218,12 +220,17 @@ class LlamaDecoder:
         c, w, L = self.cfg, self.w, self.w.layers[li]
         f = 4
         kx = kernels
-        L.wqkv.matmul_fused(self.h, rows, self.qkv, gain=L.attn_norm, eps=c.rms_eps)
         kc = self.k_cache.at(li * self.kv_layer_floats * f)
         vc = self.v_cache.at(li * self.kv_layer_floats * f)
-        # rotated queries to [heads, rows, head_dim]; rotated keys and raw values into the cache rows of these positions
-        kx.rope_qkv_dev(self.qkv, self.q, kc, vc, rows, c.heads, c.kv_heads, c.head_dim, c.ctx_max, pos_start, pos_dev,
-                        c.rope_theta)
+        if rows == 1 and pos_dev is not None:
+            # decode: norm, projection, RoPE and the cache append are one launch
+            L.wqkv.matmul_qkv_rope(self.h, self.q, kc, vc, c.heads, c.kv_heads, c.head_dim, c.ctx_max, pos_dev,
+                                   c.rope_theta, gain=L.attn_norm, eps=c.rms_eps)
+        else:
+            L.wqkv.matmul_fused(self.h, rows, self.qkv, gain=L.attn_norm, eps=c.rms_eps)
+            # rotated queries to [heads, rows, head_dim]; rotated keys and raw values into the cache rows of these positions
+            kx.rope_qkv_dev(self.qkv, self.q, kc, vc, rows, c.heads, c.kv_heads, c.head_dim, c.ctx_max, pos_start, pos_dev,
+                            c.rope_theta)
         scale = float(1.0 / np.sqrt(c.head_dim))
         kx.sdpa_cache_dev(self.q, kc, vc, self.attn, 1, c.heads, c.kv_heads, rows, seq_kv, c.ctx_max, c.head_dim, scale,
                           True, 0, 0, kv_len_dev)
@@ -271,9 +278,7 @@ class LlamaDecoder:
         for li in range(c.layers):
             self._block(li, 1, 0, self.pos, c.ctx_max, self.kv_len)
         self._head(0)
-        kernels.i32_increment_dev(self.pos, 1)
-        kernels.i32_increment_dev(self.kv_len, 1)
-        kernels.i32_store_at_dev(self.generated, self.pos, 0, self.token)
+        kernels.decode_advance_dev(self.pos, self.kv_len, self.token, self.generated)
 
     def decode(self, steps: int, use_graph: bool = True) -> np.ndarray:
         """Greedy-decode `steps` tokens after prefill(); returns them. With use_graph the step is recorded once and replayed."""

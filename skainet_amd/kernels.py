@@ -156,6 +156,13 @@ class DeviceWeight:
         check(_lib.hip().skainet_hip_matmul_fused_dev(self._h, _ptr(x), m, _ptr(out), _ptr(gain), eps, _ptr(residual), epilogue),
               "matmul_fused")
 
+    def matmul_qkv_rope(self, x, q_out, k_cache, v_cache, heads, kv_heads, head_dim, kv_capacity, pos_dev, theta,
+                        gain=None, eps: float = 0.0) -> None:
+        """One token's [q | k | v] projection + RoPE + cache append (skainet_hip_matmul_qkv_rope_dev)."""
+        check(_lib.hip().skainet_hip_matmul_qkv_rope_dev(self._h, _ptr(x), _ptr(gain), eps, _ptr(q_out), _ptr(k_cache),
+                                                         _ptr(v_cache), heads, kv_heads, head_dim, kv_capacity,
+                                                         _ptr(pos_dev), theta), "matmul_qkv_rope")
+
     def dequantize(self, out) -> None:
         check(_lib.hip().skainet_hip_dequantize_dev(self._h, _ptr(out)), "dequantize")
 
@@ -270,6 +277,10 @@ def heads_to_rows_dev(x, out, heads, tokens, head_dim) -> None:
 
 def i32_increment_dev(value, delta: int) -> None:
     check(_lib.hip().skainet_hip_i32_increment_dev(_ptr(value), delta), "i32_increment")
+
+
+def decode_advance_dev(pos, kv_len, token, log) -> None:
+    check(_lib.hip().skainet_hip_decode_advance_dev(_ptr(pos), _ptr(kv_len), _ptr(token), _ptr(log)), "decode_advance")
 
 
 def i32_store_at_dev(dst, index_dev, offset: int, src) -> None:

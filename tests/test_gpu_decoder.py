@@ -95,7 +95,11 @@ def test_heads_to_rows_and_swiglu_and_increment(hip_backend, torch_cuda):
     ctr = dev(torch, np.array([41], np.int32))
     kx.i32_increment_dev(ctr, 1)
     kx.i32_increment_dev(ctr, 3)
+    pos, klen = dev(torch, np.array([6], np.int32)), dev(torch, np.array([7], np.int32))
+    tok, log = dev(torch, np.array([99], np.int32)), dev(torch, np.zeros(10, np.int32))
+    kx.decode_advance_dev(pos, klen, tok, log)
     kx.sync()
+    assert int(pos.cpu()[0]) == 7 and int(klen.cpu()[0]) == 8 and log.cpu().tolist() == [0] * 7 + [99, 0, 0]
     assert np.array_equal(out.cpu().numpy().reshape(tokens, heads, hd), a.transpose(1, 0, 2))
     g, u = gu[:, 0::2].astype(np.float64), gu[:, 1::2].astype(np.float64)
     assert max_norm_err(act.cpu().numpy().reshape(rows, ffn), g / (1 + np.exp(-g)) * u) < 1e-6
@@ -164,6 +168,37 @@ def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
         w.matmul_fused(d_x, m, out, epilogue=kx.EPI_RESIDUAL)          # residual epilogue without a residual
     with pytest.raises(HipError):
         w.matmul_fused(d_x, m, out, epilogue=7)
+
+
+@pytest.mark.parametrize("enc,heads,kvh,hd,k", [("Q4_K", 8, 2, 64, 512), ("Q4_K", 32, 8, 128, 4096), ("Q4_K", 3, 1, 64, 256),
+                                                ("Q6_K", 4, 2, 64, 512)])
+def test_matmul_qkv_rope_equals_product_then_rope(hip_backend, torch_cuda, enc, heads, kvh, hd, k):
+    """The one-launch decode projection (norm + product + RoPE + cache append) against the separate entries, with and
+    without the norm, at a device-side position; rows of the caches other than the position stay untouched."""
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(heads * hd + k)
+    n, cap, pos, theta, eps = (heads + 2 * kvh) * hd, 24, 13, 500000.0, 1e-5
+    w = kx.DeviceWeight.upload(enc, kx.quantize(enc, (rng.standard_normal((n, k)) * 0.05).astype(np.float32)), n, k)
+    x = dev(torch, rng.standard_normal(k).astype(np.float32))
+    gain = dev(torch, (1 + 0.1 * rng.standard_normal(k)).astype(np.float32))
+    pos_dev = dev(torch, np.array([pos], np.int32))
+    for g in (None, gain):
+        q1 = torch.zeros(heads * hd, device="cuda")
+        k1 = torch.full((kvh * cap * hd,), 5.0, device="cuda")
+        v1 = torch.full((kvh * cap * hd,), 5.0, device="cuda")
+        q2, k2, v2 = torch.zeros_like(q1), torch.full_like(k1, 5.0), torch.full_like(v1, 5.0)
+        w.matmul_qkv_rope(x, q1, k1, v1, heads, kvh, hd, cap, pos_dev, theta, gain=g, eps=eps)
+        qkv = torch.empty(n, device="cuda")
+        w.matmul_fused(x, 1, qkv, gain=g, eps=eps)
+        kx.rope_qkv_dev(qkv, q2, k2, v2, 1, heads, kvh, hd, cap, 0, pos_dev, theta)
+        kx.sync()
+        for a, b in ((q1, q2), (k1, k2), (v1, v2)):
+            a, b = a.cpu().numpy(), b.cpu().numpy()
+            assert np.abs(a - b).max() <= 1e-5 * max(np.abs(b).max(), 1.0)
+            assert np.array_equal(a == 5.0, b == 5.0)
+    from skainet_amd._lib import HipError
+    with pytest.raises(HipError):
+        w.matmul_qkv_rope(x, q1, k1, v1, heads + 1, kvh, hd, cap, pos_dev, theta)     # head shape does not match the rows
 
 
 def test_sdpa_cache_layout_matches_contiguous(hip_backend, torch_cuda):
