@@ -173,6 +173,130 @@ class LlamaWeights:
         self.out_norm = gain("out_norm")
         self.head = packed("head", cfg.head_encoding, cfg.vocab, cfg.hidden)
 
+    # ------------------------------------------------------------------ GGUF files
+    @classmethod
+    def from_gguf(cls, path: str, ctx_max: Optional[int] = None, keep_host: bool = False) -> "LlamaWeights":
+        """Load a llama-architecture GGUF file (llama.cpp tensor names): packed tensors go from the file mapping to the
+        device; q/k/v are concatenated and gate/up interleaved row by row on the way (they must share an encoding).
+        `output.weight` may be absent (tied embeddings): the token embedding is used."""
+        from . import gguf
+        kernels._require_available()
+        with gguf.GGUFReader(path) as r:
+            f = r.fields
+            arch = f.get("general.architecture", "llama")
+
+            def meta(key, default=None):
+                v = f.get(f"{arch}.{key}", default)
+                if v is None:
+                    raise gguf.GGUFError(f"{path}: metadata key {arch}.{key} is missing")
+                return v
+
+            hidden, heads = int(meta("embedding_length")), int(meta("attention.head_count"))
+            emb = r.info("token_embd.weight")
+            cfg = LlamaConfig(
+                layers=int(meta("block_count")), hidden=hidden, heads=heads,
+                kv_heads=int(meta("attention.head_count_kv", heads)),
+                head_dim=int(meta("attention.key_length", hidden // heads)), ffn=int(meta("feed_forward_length")),
+                vocab=emb.rows, rms_eps=float(meta("attention.layer_norm_rms_epsilon", 1e-5)),
+                rope_theta=float(meta("rope.freq_base", 10000.0)),
+                ctx_max=int(ctx_max if ctx_max is not None else meta("context_length", 2048)),
+                linear_encoding=r.info("blk.0.attn_q.weight").type_name,
+                head_encoding=(r.info("output.weight") if "output.weight" in r.names() else emb).type_name)
+            self = object.__new__(cls)
+            self.cfg = cfg
+            self.host = {} if keep_host else None
+
+            def keep(name, a):
+                if self.host is not None:
+                    self.host[name] = np.array(a)
+                return a
+
+            def packed_rows(name, rows_expected, cols_expected):
+                t = r.info(name)
+                if t.type_name not in gguf.DEVICE_ENCODINGS:
+                    raise gguf.GGUFError(f"{path}: {name} is {t.type_name}; the device kernels take {gguf.DEVICE_ENCODINGS}")
+                if (t.rows, t.cols) != (rows_expected, cols_expected):
+                    raise gguf.GGUFError(f"{path}: {name} is {t.rows} x {t.cols}, expected {rows_expected} x {cols_expected}")
+                return t.type_name, r.tensor_bytes(name).reshape(t.rows, -1)
+
+            def fused(name, parts, interleave=False):
+                encs = {e for e, _ in parts}
+                if len(encs) != 1:
+                    raise gguf.GGUFError(f"{path}: {name}: tensors fused into one product must share an encoding, got {sorted(encs)}")
+                mats = [m for _, m in parts]
+                if interleave:
+                    out = np.empty((2 * mats[0].shape[0], mats[0].shape[1]), np.uint8)
+                    out[0::2], out[1::2] = mats
+                else:
+                    out = np.concatenate(mats, axis=0)
+                out = keep(name, out.reshape(-1))
+                return kernels.DeviceWeight.upload(encs.pop(), out, sum(m.shape[0] for m in mats), cfg_cols[name.split(".")[-1]])
+
+            def single(name, host_name, rows, cols):
+                enc, m = packed_rows(name, rows, cols)
+                return kernels.DeviceWeight.upload(enc, keep(host_name, m.reshape(-1)), rows, cols)
+
+            def gain(name, host_name):
+                g = np.ascontiguousarray(r.tensor_f32(name), dtype=np.float32).reshape(-1)
+                if g.size != hidden:
+                    raise gguf.GGUFError(f"{path}: {name} has {g.size} elements, expected {hidden}")
+                return DeviceBuffer(g.nbytes).upload(keep(host_name, g))
+
+            cfg_cols = {"wqkv": hidden, "w_gate_up": hidden}
+            self.tok_embd = single("token_embd.weight", "tok_embd", cfg.vocab, hidden)
+            self.layers = []
+            for i in range(cfg.layers):
+                b = f"blk.{i}."
+                self.layers.append(LayerWeights(
+                    attn_norm=gain(b + "attn_norm.weight", f"l{i}.attn_norm"),
+                    wqkv=fused(f"l{i}.wqkv", [packed_rows(b + "attn_q.weight", cfg.q_dim, hidden),
+                                              packed_rows(b + "attn_k.weight", cfg.kv_dim, hidden),
+                                              packed_rows(b + "attn_v.weight", cfg.kv_dim, hidden)]),
+                    wo=single(b + "attn_output.weight", f"l{i}.wo", hidden, cfg.q_dim),
+                    ffn_norm=gain(b + "ffn_norm.weight", f"l{i}.ffn_norm"),
+                    w_gate_up=fused(f"l{i}.w_gate_up", [packed_rows(b + "ffn_gate.weight", cfg.ffn, hidden),
+                                                        packed_rows(b + "ffn_up.weight", cfg.ffn, hidden)], interleave=True),
+                    w_down=single(b + "ffn_down.weight", f"l{i}.w_down", hidden, cfg.ffn)))
+            self.out_norm = gain("output_norm.weight", "out_norm")
+            head_name = "output.weight" if "output.weight" in r.names() else "token_embd.weight"
+            self.head = single(head_name, "head", cfg.vocab, hidden)
+        return self
+
+    def to_gguf(self, path: str) -> None:
+        """Write this model as a llama-architecture GGUF file with llama.cpp tensor names (needs keep_host=True)."""
+        from . import gguf
+        if self.host is None:
+            raise ValueError("to_gguf needs the host copies: build the weights with keep_host=True")
+        c, h = self.cfg, self.host
+        w = gguf.GGUFWriter()
+        w.add_string("general.architecture", "llama")
+        for key, v in (("block_count", c.layers), ("embedding_length", c.hidden), ("attention.head_count", c.heads),
+                       ("attention.head_count_kv", c.kv_heads), ("attention.key_length", c.head_dim),
+                       ("feed_forward_length", c.ffn), ("context_length", c.ctx_max), ("vocab_size", c.vocab)):
+            w.add_u32("llama." + key, v)
+        w.add_f32("llama.attention.layer_norm_rms_epsilon", c.rms_eps)
+        w.add_f32("llama.rope.freq_base", c.rope_theta)
+        le, he = c.linear_encoding, c.head_encoding
+        _, bs, nb = kernels.ENCODINGS[le]
+        row_bytes = c.hidden // bs * nb
+        w.add_tensor("token_embd.weight", le, (c.vocab, c.hidden), h["tok_embd"])
+        for i in range(c.layers):
+            b = f"blk.{i}."
+            qkv = h[f"l{i}.wqkv"].reshape(-1, row_bytes)
+            gu = h[f"l{i}.w_gate_up"].reshape(-1, row_bytes)
+            w.add_tensor(b + "attn_norm.weight", "F32", (c.hidden,), h[f"l{i}.attn_norm"])
+            w.add_tensor(b + "attn_q.weight", le, (c.q_dim, c.hidden), qkv[:c.q_dim])
+            w.add_tensor(b + "attn_k.weight", le, (c.kv_dim, c.hidden), qkv[c.q_dim:c.q_dim + c.kv_dim])
+            w.add_tensor(b + "attn_v.weight", le, (c.kv_dim, c.hidden), qkv[c.q_dim + c.kv_dim:])
+            w.add_tensor(b + "attn_output.weight", le, (c.hidden, c.q_dim), h[f"l{i}.wo"])
+            w.add_tensor(b + "ffn_norm.weight", "F32", (c.hidden,), h[f"l{i}.ffn_norm"])
+            w.add_tensor(b + "ffn_gate.weight", le, (c.ffn, c.hidden), gu[0::2])
+            w.add_tensor(b + "ffn_up.weight", le, (c.ffn, c.hidden), gu[1::2])
+            w.add_tensor(b + "ffn_down.weight", le, (c.hidden, c.ffn), h[f"l{i}.w_down"])
+        w.add_tensor("output_norm.weight", "F32", (c.hidden,), h["out_norm"])
+        w.add_tensor("output.weight", he, (c.vocab, c.hidden), h["head"])
+        w.write(path)
+
     def packed_bytes(self) -> int:
         n = self.tok_embd.nbytes + self.head.nbytes
         for l in self.layers:

@@ -336,3 +336,40 @@ def test_prefill_rejects_oversized_prompt(small_model):
     dec.prefill(np.zeros(4, np.int32))
     with pytest.raises(ValueError):
         dec.decode(cfg.ctx_max, use_graph=False)
+
+
+def test_gguf_round_trip_gives_the_same_model(small_model, tmp_path):
+    """Export the synthetic model as a llama-architecture GGUF file (separate q / k / v and gate / up tensors, llama.cpp
+    names), load it back through the memory-mapped reader (which re-fuses them) and decode: same bytes on the device,
+    so the tokens and logits are identical; a packed tensor uploaded straight from the mapping multiplies like the
+    original."""
+    from skainet_amd import gguf
+    from skainet_amd.decoder import LlamaDecoder, LlamaWeights
+    cfg, w = small_model
+    path = str(tmp_path / "model.gguf")
+    w.to_gguf(path)
+    w2 = LlamaWeights.from_gguf(path, keep_host=True)
+    from dataclasses import replace
+    assert w2.cfg.rms_eps == pytest.approx(cfg.rms_eps, rel=1e-6)            # stored as float32 in the file
+    assert replace(w2.cfg, rms_eps=cfg.rms_eps) == cfg
+    for name, a in w.host.items():
+        assert np.array_equal(np.asarray(a).reshape(-1), np.asarray(w2.host[name]).reshape(-1)), name
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 6)
+    outs = []
+    for weights in (w, w2):
+        dec = LlamaDecoder(weights, max_prefill=8)
+        first = dec.prefill(prompt)
+        outs.append((first, dec.decode(6, use_graph=False), dec.last_logits()))
+    assert outs[0][0] == outs[1][0] and np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][2], outs[1][2])
+    with gguf.GGUFReader(path) as r:
+        assert r.fields["llama.block_count"] == cfg.layers
+        dw = r.upload("blk.1.ffn_down.weight")
+        assert (dw.rows, dw.cols, dw.encoding) == (cfg.hidden, cfg.ffn, "Q4_K")
+    from skainet_amd import kernels as kx
+    import torch
+    x = torch.randn(cfg.ffn, device="cuda")
+    y1, y2 = torch.empty(cfg.hidden, device="cuda"), torch.empty(cfg.hidden, device="cuda")
+    dw.matmul(x, 1, y1)
+    w.layers[1].w_down.matmul(x, 1, y2)
+    kx.sync()
+    assert torch.equal(y1, y2)
