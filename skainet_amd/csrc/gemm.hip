@@ -60,7 +60,10 @@ __device__ __forceinline__ void load_raw(RawQ4K& r, const uint8_t* row, int e) {
     r.q0 = *reinterpret_cast<const uint4*>(blk + 16 + g * 32);
     r.q1 = *reinterpret_cast<const uint4*>(blk + 32 + g * 32);
 }
-__device__ __forceinline__ void decode32(const RawQ4K& r, int e, float* w) {
+// The decode of a thread's 32 weights is split into a header part and eight 4-weight parts (one per dword of
+// codes) so the main loop can place the parts between its MFMAs.
+struct DecQ4K { float scale, offset; int shift; };
+__device__ __forceinline__ void decode_prepare(const RawQ4K& r, int e, DecQ4K& c) {
     const int sb = (e & 255) >> 5;
     const float d = half_bits_to_float_fast(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(r.hdr.x >> 16);
     // ggml get_scale_min_k4 on the 12 scale bytes s[0..11] (hdr.y = s[0..3], hdr.z = s[4..7], hdr.w = s[8..11])
@@ -68,17 +71,19 @@ __device__ __forceinline__ void decode32(const RawQ4K& r, int e, float* w) {
     const uint32_t sa = (r.hdr.y >> sh) & 0xFFu, sbm = (r.hdr.z >> sh) & 0xFFu, st = (r.hdr.w >> sh) & 0xFFu;
     const uint32_t sc = sb < 4 ? (sa & 63u) : ((st & 0xFu) | ((sa >> 6) << 4));
     const uint32_t mn = sb < 4 ? (sbm & 63u) : ((st >> 4) | ((sbm >> 6) << 4));
-    const float scale = d * (float)sc, offset = dmin * (float)mn;
-    const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-    const int shift = (sb & 1) * 4;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t v = (q[i] >> shift) & 0x0F0F0F0Fu;
-        w[4 * i + 0] = fmaf(ubyte0_to_float(v), scale, -offset);
-        w[4 * i + 1] = fmaf(ubyte1_to_float(v), scale, -offset);
-        w[4 * i + 2] = fmaf(ubyte2_to_float(v), scale, -offset);
-        w[4 * i + 3] = fmaf(ubyte3_to_float(v), scale, -offset);
-    }
+    c.scale = d * (float)sc;
+    c.offset = dmin * (float)mn;
+    c.shift = (sb & 1) * 4;
+}
+template <int I>
+__device__ __forceinline__ void decode_dword(const RawQ4K& r, const DecQ4K& c, float* w4) {
+    const uint32_t q = I == 0 ? r.q0.x : I == 1 ? r.q0.y : I == 2 ? r.q0.z : I == 3 ? r.q0.w
+                     : I == 4 ? r.q1.x : I == 5 ? r.q1.y : I == 6 ? r.q1.z : r.q1.w;
+    const uint32_t v = (q >> c.shift) & 0x0F0F0F0Fu;
+    w4[0] = fmaf(ubyte0_to_float(v), c.scale, -c.offset);
+    w4[1] = fmaf(ubyte1_to_float(v), c.scale, -c.offset);
+    w4[2] = fmaf(ubyte2_to_float(v), c.scale, -c.offset);
+    w4[3] = fmaf(ubyte3_to_float(v), c.scale, -c.offset);
 }
 
 __device__ __forceinline__ void load_raw(RawQ6K& r, const uint8_t* row, int e) {
@@ -92,22 +97,25 @@ __device__ __forceinline__ void load_raw(RawQ6K& r, const uint8_t* row, int e) {
     r.sc = load_u16(blk + 192 + half * 8 + 2 * kq);
     r.d = load_u16(blk + 208);
 }
-__device__ __forceinline__ void decode32(const RawQ6K& r, int e, float* w) {
+struct DecQ6K { float s0, s1; int nib, hs; };
+__device__ __forceinline__ void decode_prepare(const RawQ6K& r, int e, DecQ6K& c) {
     const int kq = (e & 127) >> 5;
     const float d = half_bits_to_float_fast(r.d);
-    const float s0 = d * (float)(int8_t)(r.sc & 0xFF), s1 = d * (float)(int8_t)(r.sc >> 8);
-    const int nib = (kq >> 1) * 4, hs = 2 * kq;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t lo = (r.ql[i] >> nib) & 0x0F0F0F0Fu;
-        const uint32_t hi = ((r.qh[i] >> hs) & 0x03030303u) << 4;
-        const uint32_t c = lo | hi;                          // four 6-bit codes, one per byte
-        const float sc = i < 4 ? s0 : s1;
-        w[4 * i + 0] = sc * (ubyte0_to_float(c) - 32.f);
-        w[4 * i + 1] = sc * (ubyte1_to_float(c) - 32.f);
-        w[4 * i + 2] = sc * (ubyte2_to_float(c) - 32.f);
-        w[4 * i + 3] = sc * (ubyte3_to_float(c) - 32.f);
-    }
+    c.s0 = d * (float)(int8_t)(r.sc & 0xFF);
+    c.s1 = d * (float)(int8_t)(r.sc >> 8);
+    c.nib = (kq >> 1) * 4;
+    c.hs = 2 * kq;
+}
+template <int I>
+__device__ __forceinline__ void decode_dword(const RawQ6K& r, const DecQ6K& c, float* w4) {
+    const uint32_t lo = (r.ql[I] >> c.nib) & 0x0F0F0F0Fu;
+    const uint32_t hi = ((r.qh[I] >> c.hs) & 0x03030303u) << 4;
+    const uint32_t q = lo | hi;                              // four 6-bit codes, one per byte
+    const float sc = I < 4 ? c.s0 : c.s1;
+    w4[0] = sc * (ubyte0_to_float(q) - 32.f);
+    w4[1] = sc * (ubyte1_to_float(q) - 32.f);
+    w4[2] = sc * (ubyte2_to_float(q) - 32.f);
+    w4[3] = sc * (ubyte3_to_float(q) - 32.f);
 }
 
 __device__ __forceinline__ void load_raw(RawQ80& r, const uint8_t* row, int e) {
@@ -116,13 +124,26 @@ __device__ __forceinline__ void load_raw(RawQ80& r, const uint8_t* row, int e) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) r.q[i] = load_u32_a2(blk + 2 + 4 * i);
 }
-__device__ __forceinline__ void decode32(const RawQ80& r, int, float* w) {
-    const float d = half_bits_to_float_fast(r.d);
+struct DecQ80 { float d; };
+__device__ __forceinline__ void decode_prepare(const RawQ80& r, int, DecQ80& c) { c.d = half_bits_to_float_fast(r.d); }
+template <int I>
+__device__ __forceinline__ void decode_dword(const RawQ80& r, const DecQ80& c, float* w4) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) w[4 * i + j] = (float)(int8_t)(r.q[i] >> (8 * j)) * d;
-    }
+    for (int j = 0; j < 4; ++j) w4[j] = (float)(int8_t)(r.q[I] >> (8 * j)) * c.d;
+}
+
+template <class Raw> struct DecOf;
+template <> struct DecOf<RawQ4K> { typedef DecQ4K type; };
+template <> struct DecOf<RawQ6K> { typedef DecQ6K type; };
+template <> struct DecOf<RawQ80> { typedef DecQ80 type; };
+
+typedef __bf16 gemm_bf16x4 __attribute__((ext_vector_type(4)));
+// part I (0..7) of a thread's 32 weights -> 4 bf16 values
+template <int I, class Raw, class Dec>
+__device__ __forceinline__ gemm_bf16x4 decode_part(const Raw& r, const Dec& c) {
+    float w4[4];
+    decode_dword<I>(r, c, w4);
+    return gemm_bf16x4{(__bf16)w4[0], (__bf16)w4[1], (__bf16)w4[2], (__bf16)w4[3]};
 }
 
 template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES>
@@ -169,17 +190,18 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
             *reinterpret_cast<u32x4*>(a_tile(buf) + row * GSTRIDE + 8 * kp) = areg[j];
         }
     };
-    auto store_w = [&](const Raw& raw, int buf, int step) {
-        float wv[32];
-        decode32(raw, k_begin + step * GK + 32 * wsub, wv);
+    typedef typename DecOf<Raw>::type Dec;
+    auto write_w = [&](const gemm_bf16x4 (&wp)[8], int buf) {
         __bf16* dst = w_tile(buf) + wrow * GSTRIDE + 32 * wsub;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            bf16x8 o;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) o[j] = (__bf16)wv[8 * i + j];
-            *reinterpret_cast<bf16x8*>(dst + 8 * i) = o;
-        }
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<bf16x8*>(dst + 8 * i) = __builtin_shufflevector(wp[2 * i], wp[2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    auto decode_all = [&](const Raw& raw, int step, gemm_bf16x4 (&wp)[8]) {
+        Dec c;
+        decode_prepare(raw, k_begin + step * GK + 32 * wsub, c);
+        wp[0] = decode_part<0>(raw, c); wp[1] = decode_part<1>(raw, c); wp[2] = decode_part<2>(raw, c); wp[3] = decode_part<3>(raw, c);
+        wp[4] = decode_part<4>(raw, c); wp[5] = decode_part<5>(raw, c); wp[6] = decode_part<6>(raw, c); wp[7] = decode_part<7>(raw, c);
     };
 
     f32x16 acc[4][2];
@@ -194,33 +216,74 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     // clamped to it (a redundant load instead of a branch).
     auto step_k = [&](int step) { return k_begin + min(step, nsteps - 1) * GK; };
     const int fr = lane & 31, fk = (lane >> 5) * 8;   // fragment row inside a 32-row tile, first k of this lane's 8
-    // M: this wave's 32 MFMAs on LDS stage `stage`.
-    auto phase_m = [&](int stage) {
+    // One K step of a wave: its 32 MFMAs on LDS stage `stage`, with the decode of the NEXT step's weights (header part,
+    // then one 4-weight part after every fourth MFMA) and the fragment reads of the next 16-wide slice placed between
+    // them. A wave issues in order and an MFMA occupies the matrix core for 32 cycles: whatever sits between two MFMAs
+    // in program order runs for free, whatever sits after the last one is paid for. sched_barrier(0) pins the order.
+    auto step_body = [&](int stage, const Raw& raw_next, int step_next, const u32x4 (&a_next)[G_A_LOADS]) {
         const __bf16* at = a_tile(stage) + (128 * wm + fr) * GSTRIDE + fk;
         const __bf16* wt = w_tile(stage) + (64 * wn + fr) * GSTRIDE + fk;
+        __bf16* a_dst = a_tile(stage ^ 1);
+        __bf16* w_dst = w_tile(stage ^ 1) + wrow * GSTRIDE + 32 * wsub;
+        bf16x8 af[2][4], bf[2][2];
+        gemm_bf16x4 wp[8];
+        auto frags = [&](int set, int kk) {
 #pragma unroll
-        for (int kk = 0; kk < GK; kk += 16) {
-            bf16x8 af[4], bf[2];
+            for (int i = 0; i < 4; ++i) af[set][i] = *reinterpret_cast<const bf16x8*>(at + 32 * i * GSTRIDE + kk);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(at + 32 * i * GSTRIDE + kk);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(wt + 32 * j * GSTRIDE + kk);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
+            for (int j = 0; j < 2; ++j) bf[set][j] = *reinterpret_cast<const bf16x8*>(wt + 32 * j * GSTRIDE + kk);
+        };
+        auto park_a = [&](int j) {               // chunk j of the next step's activation tile -> the other LDS stage
+            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
+            *reinterpret_cast<u32x4*>(a_dst + row * GSTRIDE + 8 * kp) = a_next[j];
+        };
+        auto park_w = [&](int i) {               // weights 8 i .. 8 i + 7 of this thread's 32
+            *reinterpret_cast<bf16x8*>(w_dst + 8 * i) = __builtin_shufflevector(wp[2 * i], wp[2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        Dec c;
+        frags(0, 0);
+        decode_prepare(raw_next, k_begin + step_next * GK + 32 * wsub, c);
+        __builtin_amdgcn_sched_barrier(0);
+#define SKH_MFMA(set, i, j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0); \
+                            __builtin_amdgcn_sched_barrier(0);
+        // slice kk: MFMAs on fragment set `set`; between them the reads of the next slice, two decode parts (P0, P1) and
+        // the LDS stores S0.. of the next stage (the other stage: nobody reads it during this step)
+#define SKH_SLICE(set, kk, P0, P1, STORES0, STORES1)                                                 \
+        if (kk + 16 < GK) frags(set ^ 1, kk + 16);                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        SKH_MFMA(set, 0, 0) SKH_MFMA(set, 0, 1)                                                      \
+        wp[P0] = decode_part<P0>(raw_next, c);                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        SKH_MFMA(set, 1, 0) SKH_MFMA(set, 1, 1)                                                      \
+        STORES0                                                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        SKH_MFMA(set, 2, 0) SKH_MFMA(set, 2, 1)                                                      \
+        wp[P1] = decode_part<P1>(raw_next, c);                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        SKH_MFMA(set, 3, 0) SKH_MFMA(set, 3, 1)                                                      \
+        STORES1                                                                                      \
+        __builtin_amdgcn_sched_barrier(0);
+        static_assert(G_A_LOADS == 8, "the store schedule below places eight activation chunks");
+        SKH_SLICE(0, 0, 0, 1, , park_w(0);)
+        SKH_SLICE(1, 16, 2, 3, park_a(0);, park_a(1); park_w(1);)
+        SKH_SLICE(0, 32, 4, 5, park_a(2); park_a(3);, park_a(4); park_w(2);)
+        SKH_SLICE(1, 48, 6, 7, park_a(5); park_a(6);, park_a(7); park_w(3);)
+#undef SKH_SLICE
+#undef SKH_MFMA
     };
 
-    // Every wave alternates M and D; the loop body is one straight-line block (no branches), which is what lets the
-    // compiler's wait-count bookkeeping leave the newest step's loads in flight while the older ones are parked.
+    // The loop body is one straight-line block (no branches), which is what lets the compiler's wait-count
+    // bookkeeping leave the newest step's loads in flight while the older ones are parked.
     // (Measured alternatives that did not beat this: a 256 x 256 tile with 8 waves in lockstep or with the two waves
-    // of a SIMD half a step out of phase, one LDS stage with two workgroups per CU, explicit MFMA / VALU issue
-    // interleaving hints.)
-    load_a(aring[0], 0);
-    load_raw(wring[0], wrow_ptr, step_k(0) + 32 * wsub);
-    store_a(aring[0], 0);
-    store_w(wring[0], 0, 0);
+    // of a SIMD half a step out of phase, one LDS stage with two workgroups per CU.)
+    {
+        gemm_bf16x4 wp0[8];
+        load_a(aring[0], 0);
+        load_raw(wring[0], wrow_ptr, step_k(0) + 32 * wsub);
+        store_a(aring[0], 0);
+        decode_all(wring[0], 0, wp0);
+        write_w(wp0, 0);
+    }
     load_a(aring[1], min(1, nsteps - 1));
     load_raw(wring[1], wrow_ptr, step_k(1) + 32 * wsub);
     __syncthreads();
@@ -231,10 +294,8 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
             // ring slot u held this step's bytes (parked one step ago): refill it with the step after next
             load_a(aring[u], min(step + 2, nsteps - 1));
             load_raw(wring[u], wrow_ptr, step_k(step + 2) + 32 * wsub);
-            phase_m(u);
-            // the other LDS stage was last read one step ago (a barrier since): park step + 1 there
-            store_a(aring[u ^ 1], u ^ 1);
-            store_w(wring[u ^ 1], u ^ 1, min(step + 1, nsteps - 1));
+            // MFMAs of this step on stage u; step + 1 (ring slot u ^ 1) is decoded and parked in stage u ^ 1 meanwhile
+            step_body(u, wring[u ^ 1], min(step + 1, nsteps - 1), aring[u ^ 1]);
             __syncthreads();
         }
     }
