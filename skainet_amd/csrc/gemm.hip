@@ -23,9 +23,12 @@ namespace skh {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int GM = 256, GN = 128, GK = 64;
-constexpr int G_THREADS = (GM / 128) * (GN / 64) * 64;        // one wave per 128 x 64 patch
+constexpr int G_WTN = 2;                                      // 32-column MFMA tiles per wave along N (rows: always 4)
+constexpr int G_WAVES_M = 2, G_WAVES_N = 2;
+constexpr int GM = 128 * G_WAVES_M, GN = 32 * G_WTN * G_WAVES_N, GK = 64;
+constexpr int G_THREADS = G_WAVES_M * G_WAVES_N * 64;
 constexpr int G_A_LOADS = GM * (GK / 8) / G_THREADS;          // 16-byte chunks of the activation tile per thread
+constexpr int G_W_TASKS = GN * 2 / G_THREADS;                 // 32-weight decode tasks per thread and step
 constexpr int GSTRIDE = GK + 8;                               // bf16 elements per LDS row (144 bytes)
 constexpr int G_A_ELEMS = GM * GSTRIDE, G_W_ELEMS = GN * GSTRIDE;
 constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16);   // two stages
@@ -146,6 +149,21 @@ __device__ __forceinline__ gemm_bf16x4 decode_part(const Raw& r, const Dec& c) {
     return gemm_bf16x4{(__bf16)w4[0], (__bf16)w4[1], (__bf16)w4[2], (__bf16)w4[3]};
 }
 
+// part I of a thread's 32 weights with I a (constant-folded) loop variable
+template <class Raw, class Dec>
+__device__ __forceinline__ gemm_bf16x4 decode_part_at(int i, const Raw& r, const Dec& c) {
+    switch (i) {
+        case 0: return decode_part<0>(r, c);
+        case 1: return decode_part<1>(r, c);
+        case 2: return decode_part<2>(r, c);
+        case 3: return decode_part<3>(r, c);
+        case 4: return decode_part<4>(r, c);
+        case 5: return decode_part<5>(r, c);
+        case 6: return decode_part<6>(r, c);
+        default: return decode_part<7>(r, c);
+    }
+}
+
 template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES>
 __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
                                                            float* __restrict__ c, int m, int n, int k, int k_chunk,
@@ -156,146 +174,134 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     auto w_tile = [&](int buf) { return smem + buf * (G_A_ELEMS + G_W_ELEMS) + G_A_ELEMS; };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / (GN / 64), wn = wave % (GN / 64);
+    const int wm = wave / G_WAVES_N, wn = wave % G_WAVES_N;
     const int m0 = blockIdx.y * GM, n0 = blockIdx.x * GN;
     const int k_begin = blockIdx.z * k_chunk;
     const int k_end = min(k, k_begin + k_chunk);
     const int nsteps = (k_end - k_begin) / GK;
     const int64_t row_bytes = (int64_t)(k / BLOCK_ELEMS) * BLOCK_BYTES;
 
-    // this thread's share of the weight tile: 32 consecutive elements of one row per K step
+    // this thread's share of the weight tile: G_W_TASKS times 32 consecutive elements of one row per K step
     const int wrow = tid >> 1, wsub = tid & 1;
-    const uint8_t* wrow_ptr = w + (int64_t)min(n0 + wrow, n - 1) * row_bytes;   // rows past N decode a valid row, never stored
+    const uint8_t* wrow_ptr[G_W_TASKS];
+#pragma unroll
+    for (int t = 0; t < G_W_TASKS; ++t)   // rows past N decode a valid row, never stored
+        wrow_ptr[t] = w + (int64_t)min(n0 + wrow + (G_THREADS / 2) * t, n - 1) * row_bytes;
 
-    // Staging registers: rings three steps deep of the activation tile (8 x 16 bytes per thread and step) and of the
-    // raw weight bytes, so a load has two full steps of MFMA work to arrive before it is written to LDS. One
-    // workgroup owns a CU (the double-buffered tiles fill its LDS), so the register file is there to be used.
-    // Loads are unconditional (clamped rows, never stored) so all of a step's loads are in flight together.
+    // Staging registers: a two-slot ring of the activation tile chunks and of the raw weight bytes, requested two
+    // steps ahead. One workgroup owns a CU (the double-buffered tiles fill its LDS), so the register file is there
+    // to be used. Loads are unconditional (clamped rows, never stored) so a step's loads are in flight together.
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    constexpr int WD = 2;   // = the number of LDS stages: slot / stage index is the step's parity
-    u32x4 aring[WD][G_A_LOADS];
-    Raw wring[WD];
-    auto load_a = [&](u32x4 (&areg)[G_A_LOADS], int step) {
-        const int k0 = k_begin + step * GK;
-#pragma unroll
-        for (int j = 0; j < G_A_LOADS; ++j) {
-            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
-            areg[j] = *reinterpret_cast<const u32x4*>(a + (int64_t)min(m0 + row, m - 1) * k + k0 + 8 * kp);
-        }
-    };
-    auto store_a = [&](const u32x4 (&areg)[G_A_LOADS], int buf) {
-#pragma unroll
-        for (int j = 0; j < G_A_LOADS; ++j) {
-            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
-            *reinterpret_cast<u32x4*>(a_tile(buf) + row * GSTRIDE + 8 * kp) = areg[j];
-        }
-    };
     typedef typename DecOf<Raw>::type Dec;
-    auto write_w = [&](const gemm_bf16x4 (&wp)[8], int buf) {
-        __bf16* dst = w_tile(buf) + wrow * GSTRIDE + 32 * wsub;
+    u32x4 aring[2][G_A_LOADS];
+    Raw wring[2][G_W_TASKS];
+    auto step_k = [&](int step) { return k_begin + min(step, nsteps - 1) * GK; };   // loads past the end re-read the last step
+    auto load_step = [&](int slot, int step) __attribute__((always_inline)) {
+        const int k0 = step_k(step);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<bf16x8*>(dst + 8 * i) = __builtin_shufflevector(wp[2 * i], wp[2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int j = 0; j < G_A_LOADS; ++j) {
+            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
+            aring[slot][j] = *reinterpret_cast<const u32x4*>(a + (int64_t)min(m0 + row, m - 1) * k + k0 + 8 * kp);
+        }
+#pragma unroll
+        for (int t = 0; t < G_W_TASKS; ++t) load_raw(wring[slot][t], wrow_ptr[t], k0 + 32 * wsub);
     };
-    auto decode_all = [&](const Raw& raw, int step, gemm_bf16x4 (&wp)[8]) {
-        Dec c;
-        decode_prepare(raw, k_begin + step * GK + 32 * wsub, c);
-        wp[0] = decode_part<0>(raw, c); wp[1] = decode_part<1>(raw, c); wp[2] = decode_part<2>(raw, c); wp[3] = decode_part<3>(raw, c);
-        wp[4] = decode_part<4>(raw, c); wp[5] = decode_part<5>(raw, c); wp[6] = decode_part<6>(raw, c); wp[7] = decode_part<7>(raw, c);
+    auto park_a = [&](int slot, int stage, int j) __attribute__((always_inline)) {      // chunk j of a step's activation tile -> LDS stage
+        const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
+        *reinterpret_cast<u32x4*>(a_tile(stage) + row * GSTRIDE + 8 * kp) = aring[slot][j];
+    };
+    gemm_bf16x4 wp[G_W_TASKS][8];
+    auto park_w = [&](int stage, int t, int i) __attribute__((always_inline)) {         // weights 8 i .. 8 i + 7 of task t's 32
+        __bf16* dst = w_tile(stage) + (wrow + (G_THREADS / 2) * t) * GSTRIDE + 32 * wsub;
+        *reinterpret_cast<bf16x8*>(dst + 8 * i) = __builtin_shufflevector(wp[t][2 * i], wp[t][2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
     };
 
-    f32x16 acc[4][2];
+    f32x16 acc[4][G_WTN];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < G_WTN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    // nsteps is a multiple of 4 (K chunks are whole 256-element groups) and > 0. Loads past the last step are
-    // clamped to it (a redundant load instead of a branch).
-    auto step_k = [&](int step) { return k_begin + min(step, nsteps - 1) * GK; };
     const int fr = lane & 31, fk = (lane >> 5) * 8;   // fragment row inside a 32-row tile, first k of this lane's 8
-    // One K step of a wave: its 32 MFMAs on LDS stage `stage`, with the decode of the NEXT step's weights (header part,
-    // then one 4-weight part after every fourth MFMA) and the fragment reads of the next 16-wide slice placed between
-    // them. A wave issues in order and an MFMA occupies the matrix core for 32 cycles: whatever sits between two MFMAs
-    // in program order runs for free, whatever sits after the last one is paid for. sched_barrier(0) pins the order.
-    auto step_body = [&](int stage, const Raw& raw_next, int step_next, const u32x4 (&a_next)[G_A_LOADS]) {
+
+    // One K step of a wave: its MFMAs on LDS stage `stage`, with everything that prepares the NEXT step placed between
+    // them in program order -- the fragment reads of the next 16-wide slice, the decode of the next step's weights in
+    // 4-weight parts, the LDS stores into the other stage. A wave issues in order and an MFMA occupies the matrix core
+    // for 32 cycles: what sits between two MFMAs runs for free, what sits after the last one is paid for.
+    // sched_barrier(0) pins the order. The decode parts are spread over the first MFMAs, the LDS stores take one slot
+    // each behind the last N_STORES MFMAs (every weight chunk after its parts, the activation chunks as late as possible).
+    auto step_body = [&](int stage, int slot_next, int step_next) __attribute__((always_inline)) {
+        constexpr int N_MFMA = 4 * G_WTN * (GK / 16), N_PARTS = 8 * G_W_TASKS, N_STORES = G_A_LOADS + 4 * G_W_TASKS;
+        constexpr int PSTRIDE = (N_MFMA - N_STORES) / N_PARTS;      // a decode part after every PSTRIDE-th MFMA
+        static_assert(PSTRIDE >= 1, "more work items than slots between the MFMAs");
         const __bf16* at = a_tile(stage) + (128 * wm + fr) * GSTRIDE + fk;
-        const __bf16* wt = w_tile(stage) + (64 * wn + fr) * GSTRIDE + fk;
-        __bf16* a_dst = a_tile(stage ^ 1);
-        __bf16* w_dst = w_tile(stage ^ 1) + wrow * GSTRIDE + 32 * wsub;
-        bf16x8 af[2][4], bf[2][2];
-        gemm_bf16x4 wp[8];
-        auto frags = [&](int set, int kk) {
+        const __bf16* wt = w_tile(stage) + (32 * G_WTN * wn + fr) * GSTRIDE + fk;
+        bf16x8 af[2][4], bf[2][G_WTN];
+        auto frags = [&](int set, int kk) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) af[set][i] = *reinterpret_cast<const bf16x8*>(at + 32 * i * GSTRIDE + kk);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) bf[set][j] = *reinterpret_cast<const bf16x8*>(wt + 32 * j * GSTRIDE + kk);
+            for (int j = 0; j < G_WTN; ++j) bf[set][j] = *reinterpret_cast<const bf16x8*>(wt + 32 * j * GSTRIDE + kk);
         };
-        auto park_a = [&](int j) {               // chunk j of the next step's activation tile -> the other LDS stage
-            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
-            *reinterpret_cast<u32x4*>(a_dst + row * GSTRIDE + 8 * kp) = a_next[j];
-        };
-        auto park_w = [&](int i) {               // weights 8 i .. 8 i + 7 of this thread's 32
-            *reinterpret_cast<bf16x8*>(w_dst + 8 * i) = __builtin_shufflevector(wp[2 * i], wp[2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-        };
-        Dec c;
+        Dec dc[G_W_TASKS];
         frags(0, 0);
-        decode_prepare(raw_next, k_begin + step_next * GK + 32 * wsub, c);
+#pragma unroll
+        for (int t = 0; t < G_W_TASKS; ++t) decode_prepare(wring[slot_next][t], step_k(step_next) + 32 * wsub, dc[t]);
         __builtin_amdgcn_sched_barrier(0);
-#define SKH_MFMA(set, i, j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0); \
-                            __builtin_amdgcn_sched_barrier(0);
-        // slice kk: MFMAs on fragment set `set`; between them the reads of the next slice, two decode parts (P0, P1) and
-        // the LDS stores S0.. of the next stage (the other stage: nobody reads it during this step)
-#define SKH_SLICE(set, kk, P0, P1, STORES0, STORES1)                                                 \
-        if (kk + 16 < GK) frags(set ^ 1, kk + 16);                                                   \
-        __builtin_amdgcn_sched_barrier(0);                                                           \
-        SKH_MFMA(set, 0, 0) SKH_MFMA(set, 0, 1)                                                      \
-        wp[P0] = decode_part<P0>(raw_next, c);                                                       \
-        __builtin_amdgcn_sched_barrier(0);                                                           \
-        SKH_MFMA(set, 1, 0) SKH_MFMA(set, 1, 1)                                                      \
-        STORES0                                                                                      \
-        __builtin_amdgcn_sched_barrier(0);                                                           \
-        SKH_MFMA(set, 2, 0) SKH_MFMA(set, 2, 1)                                                      \
-        wp[P1] = decode_part<P1>(raw_next, c);                                                       \
-        __builtin_amdgcn_sched_barrier(0);                                                           \
-        SKH_MFMA(set, 3, 0) SKH_MFMA(set, 3, 1)                                                      \
-        STORES1                                                                                      \
-        __builtin_amdgcn_sched_barrier(0);
-        static_assert(G_A_LOADS == 8, "the store schedule below places eight activation chunks");
-        SKH_SLICE(0, 0, 0, 1, , park_w(0);)
-        SKH_SLICE(1, 16, 2, 3, park_a(0);, park_a(1); park_w(1);)
-        SKH_SLICE(0, 32, 4, 5, park_a(2); park_a(3);, park_a(4); park_w(2);)
-        SKH_SLICE(1, 48, 6, 7, park_a(5); park_a(6);, park_a(7); park_w(3);)
-#undef SKH_SLICE
-#undef SKH_MFMA
+#pragma clang loop unroll(full)
+        for (int q = 0; q < N_MFMA; ++q) {
+            const int kk = q / (4 * G_WTN), r = q % (4 * G_WTN), i = r / G_WTN, j = r % G_WTN, set = kk & 1;
+            if (r == 0 && kk + 1 < GK / 16) {
+                frags(set ^ 1, 16 * (kk + 1));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (q < N_PARTS * PSTRIDE && q % PSTRIDE == PSTRIDE - 1) {
+                const int item = q / PSTRIDE;
+                wp[item / 8][item % 8] = decode_part_at(item % 8, wring[slot_next][item / 8], dc[item / 8]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (q >= N_MFMA - N_STORES) {
+                // first the weight chunks of all but the last task, then the activation chunks (their loads are the
+                // youngest), then the last task's weight chunks
+                const int sidx = q - (N_MFMA - N_STORES);
+                constexpr int W_FIRST = 4 * (G_W_TASKS - 1);
+                if (sidx < W_FIRST) park_w(stage ^ 1, sidx / 4, sidx % 4);
+                else if (sidx < W_FIRST + G_A_LOADS) park_a(slot_next, stage ^ 1, sidx - W_FIRST);
+                else park_w(stage ^ 1, G_W_TASKS - 1, sidx - W_FIRST - G_A_LOADS);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
     };
 
-    // The loop body is one straight-line block (no branches), which is what lets the compiler's wait-count
-    // bookkeeping leave the newest step's loads in flight while the older ones are parked.
-    // (Measured alternatives that did not beat this: a 256 x 256 tile with 8 waves in lockstep or with the two waves
-    // of a SIMD half a step out of phase, one LDS stage with two workgroups per CU.)
-    {
-        gemm_bf16x4 wp0[8];
-        load_a(aring[0], 0);
-        load_raw(wring[0], wrow_ptr, step_k(0) + 32 * wsub);
-        store_a(aring[0], 0);
-        decode_all(wring[0], 0, wp0);
-        write_w(wp0, 0);
+    // nsteps is a multiple of 4 (K chunks are whole 256-element groups) and > 0. The loop body is one straight-line
+    // block (no branches), which is what lets the compiler's wait-count bookkeeping leave the newest step's loads in
+    // flight while the older ones are parked.
+    load_step(0, 0);
+#pragma unroll
+    for (int j = 0; j < G_A_LOADS; ++j) park_a(0, 0, j);
+#pragma unroll
+    for (int t = 0; t < G_W_TASKS; ++t) {
+        Dec d0;
+        decode_prepare(wring[0][t], step_k(0) + 32 * wsub, d0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wp[t][i] = decode_part_at(i, wring[0][t], d0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) park_w(0, t, i);
     }
-    load_a(aring[1], min(1, nsteps - 1));
-    load_raw(wring[1], wrow_ptr, step_k(1) + 32 * wsub);
+    load_step(1, 1);
     __syncthreads();
     for (int s0 = 0; s0 < nsteps; s0 += 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int step = s0 + u;
             // ring slot u held this step's bytes (parked one step ago): refill it with the step after next
-            load_a(aring[u], min(step + 2, nsteps - 1));
-            load_raw(wring[u], wrow_ptr, step_k(step + 2) + 32 * wsub);
+            load_step(u, step + 2);
             // MFMAs of this step on stage u; step + 1 (ring slot u ^ 1) is decoded and parked in stage u ^ 1 meanwhile
-            step_body(u, wring[u ^ 1], min(step + 1, nsteps - 1), aring[u ^ 1]);
+            step_body(u, u ^ 1, step + 1);
             __syncthreads();
         }
     }
@@ -304,8 +310,8 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = n0 + 64 * wn + 32 * j + (lane & 31);
+        for (int j = 0; j < G_WTN; ++j) {
+            const int col = n0 + 32 * G_WTN * wn + 32 * j + (lane & 31);
             if (col >= n) continue;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
