@@ -36,18 +36,19 @@ constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16); 
 void* kernel_workspace(size_t bytes);   // shim.hip
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);   // gemv.hip
 
-__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, __bf16* __restrict__ out, int64_t n4) {
+// The pass in front of the GEMM, one launch: activations fp32 -> bf16 (nearest even), and, when K is split, C zeroed
+// for the atomic accumulation. Thread i handles float4 number i of each.
+__global__ __launch_bounds__(256) void gemm_prepass_kernel(const float* __restrict__ in, __bf16* __restrict__ out, int64_t n4,
+                                                           float* __restrict__ c, int64_t c4, int64_t c_tail, int64_t c_total) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n4) return;
-    const float4 v = reinterpret_cast<const float4*>(in)[i];
-    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-    bf16x4 o = {(__bf16)v.x, (__bf16)v.y, (__bf16)v.z, (__bf16)v.w};
-    reinterpret_cast<bf16x4*>(out)[i] = o;
-}
-
-__global__ __launch_bounds__(256) void zero_f32_kernel(float* out, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = 0.f;
+    if (i < n4) {
+        const float4 v = reinterpret_cast<const float4*>(in)[i];
+        typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+        bf16x4 o = {(__bf16)v.x, (__bf16)v.y, (__bf16)v.z, (__bf16)v.w};
+        reinterpret_cast<bf16x4*>(out)[i] = o;
+    }
+    if (i < c4) reinterpret_cast<float4*>(c)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < c_tail) c[c_total - 1 - i] = 0.f;      // what a float4 sweep leaves over (everything, if C is not 16-byte aligned)
 }
 
 // ---- raw bytes a thread needs to decode 32 consecutive weights of one row, per encoding ----
@@ -354,10 +355,6 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     hipStream_t s = current_stream();
     __bf16* a = static_cast<__bf16*>(kernel_workspace((size_t)m * k * sizeof(__bf16)));
     if (!a) return -1;
-    const int64_t n4 = (int64_t)m * k / 4;
-    f32_to_bf16_kernel<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s>>>(x, a, n4);
-    SKH_CHECK(hipGetLastError());
-
     const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;
     const int tiles = tiles_m * tiles_n;
     // K chunks are whole 256-element groups so every encoding's blocks stay intact
@@ -372,9 +369,13 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (ksplit > kgroups) ksplit = kgroups;
     const int k_chunk = ((kgroups + ksplit - 1) / ksplit) * 256;
     ksplit = (k + k_chunk - 1) / k_chunk;
-    if (ksplit > 1) {
-        const int64_t cn = (int64_t)m * n;
-        zero_f32_kernel<<<dim3((unsigned)((cn + 255) / 256)), dim3(256), 0, s>>>(y, cn);
+    {
+        const int64_t n4 = (int64_t)m * k / 4;                      // k is a multiple of 64
+        const int64_t cn = ksplit > 1 ? (int64_t)m * n : 0;
+        const bool c_aligned = (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+        const int64_t c4 = c_aligned ? cn / 4 : 0, c_tail = cn - 4 * c4;   // an unaligned C is zeroed element by element
+        const int64_t threads = n4 > c4 ? (n4 > c_tail ? n4 : c_tail) : (c4 > c_tail ? c4 : c_tail);
+        gemm_prepass_kernel<<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s>>>(x, a, n4, y, c4, c_tail, cn);
         SKH_CHECK(hipGetLastError());
     }
     const dim3 grid(tiles_n, tiles_m, ksplit);
