@@ -118,10 +118,13 @@ SKAINET_HIP_API int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w
  * skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/storage/KvCacheStore.kt:125):
  * row = W . rmsnorm(x) (gain == NULL: no norm), W's rows being [q | k | v] heads of head_dim; adjacent pairs of the q
  * and k heads are rotated by pos * theta^(-2i/head_dim) with pos = *pos_dev; q -> q_out [heads, head_dim], k and v ->
- * row pos of caches [kv_heads, kv_capacity, head_dim]. Q4_K weights run as one kernel. */
+ * row pos of caches [kv_heads, kv_capacity, head_dim]. Q4_K weights run as one kernel. rope_table (may be NULL) is
+ * the (cos, sin) table of that position from skainet_hip_f32_rope_table_dev: every layer of a token shares it. */
 SKAINET_HIP_API int32_t skainet_hip_matmul_qkv_rope_dev(const skainet_hip_weight* w, const float* x, const float* gain,
     float eps, float* q_out, float* k_cache, float* v_cache, int32_t heads, int32_t kv_heads, int32_t head_dim,
-    int32_t kv_capacity, const int32_t* pos_dev, float theta);
+    int32_t kv_capacity, const int32_t* pos_dev, float theta, const float* rope_table);
+/* table[2i], table[2i+1] = cos, sin of (*pos_dev) * theta^(-2i/head_dim), i < head_dim/2 (head_dim floats). */
+SKAINET_HIP_API int32_t skainet_hip_f32_rope_table_dev(const int32_t* pos_dev, float theta, int32_t head_dim, float* table);
 /* Measurement aid: `iters` such products back to back on this thread's stream, weight number i % nweights at
  * step i, timed with HIP events; returns the elapsed milliseconds (< 0 on failure). use_graph != 0 captures the
  * launches into a HIP graph first and times one replay, so host launch cost stays off the GPU timeline.

@@ -42,7 +42,8 @@ SIGNATURES = {
     "skainet_hip_matmul_dev": (_i32, [_vp, _vp, _i32, _vp]),
     "skainet_hip_matmul_kind_dev": (_i32, [_vp, _vp, _i32, _vp, _i32]),
     "skainet_hip_matmul_fused_dev": (_i32, [_vp, _vp, _i32, _vp, _vp, _f32, _vp, _i32]),
-    "skainet_hip_matmul_qkv_rope_dev": (_i32, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _f32]),
+    "skainet_hip_matmul_qkv_rope_dev": (_i32, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _vp]),
+    "skainet_hip_f32_rope_table_dev": (_i32, [_vp, _f32, _i32, _vp]),
     "skainet_hip_matmul_repeat_dev": (_f32, [_vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32]),
     "skainet_hip_read_probe_dev": (_f32, [_vp, _i32, _i64, _i32, _i32]),
     "skainet_hip_dequantize_dev": (_i32, [_vp, _vp]),

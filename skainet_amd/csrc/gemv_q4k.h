@@ -17,6 +17,7 @@ enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE_QKV = 3 };
 struct RopeQkvEpilogue {
     float *k_cache, *v_cache;
     const int32_t* pos_dev;
+    const float2* table;   // (cos, sin) of pos * theta^(-2i / head_dim), i < head_dim / 2, for the position in *pos_dev; or null
     float theta;
     int heads, kv_heads, head_dim, capacity;
 };

@@ -205,7 +205,8 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
                 float2 out2 = make_float2(val, odd);
                 if (slot < rope.heads + rope.kv_heads) {
                     float sn, cs;
-                    sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
+                    if (rope.table) { const float2 t = rope.table[dd >> 1]; cs = t.x; sn = t.y; }
+                    else sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
                     out2 = make_float2(val * cs - odd * sn, val * sn + odd * cs);
                 }
                 float* dst;

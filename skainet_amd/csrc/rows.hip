@@ -324,6 +324,22 @@ __global__ void i32_store_at_kernel(int32_t* dst, const int32_t* __restrict__ in
     if (threadIdx.x == 0 && blockIdx.x == 0) dst[index[0] + offset] = src[0];
 }
 
+// (cos, sin) of (*pos) * theta^(-2i / head_dim) for i < head_dim / 2: the rotation table of one decode position, computed
+// once per token and read by every layer's q/k/v epilogue (same expressions as rope_qkv_kernel, so the same bits).
+__global__ void rope_table_kernel(const int32_t* __restrict__ pos, float theta, int head_dim, float2* __restrict__ table) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= head_dim / 2) return;
+    float sn, cs;
+    sincosf((float)pos[0] * powf(theta, -2.0f * (float)i / (float)head_dim), &sn, &cs);
+    table[i] = make_float2(cs, sn);
+}
+int launch_rope_table(const int32_t* pos, float theta, int head_dim, float* table) {
+    if (head_dim <= 0 || (head_dim & 1)) return set_error("rope_table: head_dim must be positive and even; got %d", head_dim);
+    rope_table_kernel<<<dim3((head_dim / 2 + 63) / 64), dim3(64), 0, current_stream()>>>(pos, theta, head_dim, reinterpret_cast<float2*>(table));
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
 // End of a greedy decode step in one launch: the position and the key count advance by one and the token just
 // sampled is appended to the log at the new position.
 __global__ void decode_advance_kernel(int32_t* pos, int32_t* kv_len, const int32_t* __restrict__ token, int32_t* log) {

@@ -37,6 +37,7 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
 int launch_rope_qkv(const float* qkv, float* q_out, float* k_cache, float* v_cache, int tokens, int heads, int kv_heads,
                     int head_dim, int kv_capacity, int pos_start, const int32_t* pos_dev, float theta);
 int launch_i32_store_at(int32_t* dst, const int32_t* index, int32_t offset, const int32_t* src);
+int launch_rope_table(const int32_t* pos, float theta, int head_dim, float* table);
 int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log);
 int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim);
 int launch_i32_increment(int32_t* v, int32_t delta);
@@ -324,16 +325,18 @@ int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x
 // caches laid out [kv_heads, kv_capacity, head_dim]. Q4_K weights: one kernel; otherwise product + rope_qkv.
 int32_t skainet_hip_matmul_qkv_rope_dev(const skainet_hip_weight* w, const float* x, const float* gain, float eps, float* q_out,
                                         float* k_cache, float* v_cache, int32_t heads, int32_t kv_heads, int32_t head_dim,
-                                        int32_t kv_capacity, const int32_t* pos_dev, float theta) {
+                                        int32_t kv_capacity, const int32_t* pos_dev, float theta, const float* rope_table) {
     if (ensure_device() != 0) return -1;
     if (!w || !x || !q_out || !k_cache || !v_cache || !pos_dev) return set_error("matmul_qkv_rope: null argument");
+    if (rope_table && (reinterpret_cast<uintptr_t>(rope_table) & 7)) return set_error("matmul_qkv_rope: the rotation table must be 8-byte aligned");
     if (heads <= 0 || kv_heads <= 0 || head_dim <= 0 || (head_dim & 1))
         return set_error("matmul_qkv_rope: bad head shape %d / %d x %d", heads, kv_heads, head_dim);
     if ((int64_t)w->rows != (int64_t)(heads + 2 * kv_heads) * head_dim)
         return set_error("matmul_qkv_rope: weight has %d rows, the head shape needs %lld", w->rows,
                          (long long)(heads + 2 * kv_heads) * head_dim);
     if (w->encoding == ENC_Q4_K) {
-        const RopeQkvEpilogue rope{k_cache, v_cache, pos_dev, theta, heads, kv_heads, head_dim, kv_capacity};
+        const RopeQkvEpilogue rope{k_cache, v_cache, pos_dev, reinterpret_cast<const float2*>(rope_table), theta, heads, kv_heads,
+                                   head_dim, kv_capacity};
         const int r = launch_q4k_gemv_rows_fused(w->data, x, q_out, w->cols, w->rows, 1, gain, eps, nullptr, EPI_ROPE_QKV, &rope);
         if (r != 0) return r < 0 ? -1 : 0;
     }
@@ -470,6 +473,11 @@ int32_t skainet_hip_f32_rope_scatter_dev(const float* in, int64_t in_row_pitch, 
     if (ensure_device() != 0) return -1;
     return launch_rope_scatter(in, in_row_pitch, out, tokens, heads, head_dim, pos_start, pos_dev, theta, rotate, out_head_stride,
                                out_row_is_pos);
+}
+int32_t skainet_hip_f32_rope_table_dev(const int32_t* pos_dev, float theta, int32_t head_dim, float* table) {
+    if (ensure_device() != 0) return -1;
+    if (!pos_dev || !table) return set_error("rope_table: null argument");
+    return launch_rope_table(pos_dev, theta, head_dim, table);
 }
 int32_t skainet_hip_decode_advance_dev(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log) {
     if (ensure_device() != 0) return -1;

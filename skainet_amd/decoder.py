@@ -332,6 +332,7 @@ class LlamaDecoder:
         self.pos = DeviceBuffer(4).upload(np.zeros(1, np.int32))        # tokens already in the cache
         self.kv_len = DeviceBuffer(4).upload(np.zeros(1, np.int32))     # = pos + 1 during a decode step
         self.token = DeviceBuffer(4).upload(np.zeros(1, np.int32))
+        self.rope_table = DeviceBuffer(4 * c.head_dim)      # (cos, sin) per rotation pair of the current decode position
         self.generated = DeviceBuffer(4 * (c.ctx_max + 1))   # generated[p] = the token predicted for position p
         self.prompt_len = 0
         self._graph: Optional[kernels.Graph] = None
@@ -349,7 +350,7 @@ class LlamaDecoder:
         if rows == 1 and pos_dev is not None:
             # decode: norm, projection, RoPE and the cache append are one launch
             L.wqkv.matmul_qkv_rope(self.h, self.q, kc, vc, c.heads, c.kv_heads, c.head_dim, c.ctx_max, pos_dev,
-                                   c.rope_theta, gain=L.attn_norm, eps=c.rms_eps)
+                                   c.rope_theta, gain=L.attn_norm, eps=c.rms_eps, rope_table=self.rope_table)
         else:
             L.wqkv.matmul_fused(self.h, rows, self.qkv, gain=L.attn_norm, eps=c.rms_eps)
             # rotated queries to [heads, rows, head_dim]; rotated keys and raw values into the cache rows of these positions
@@ -399,6 +400,7 @@ class LlamaDecoder:
         """Consumes self.token at device position self.pos, leaves the next token in self.token, advances the position."""
         c = self.cfg
         self.w.tok_embd.dequantize_rows(self.token, 1, self.h)
+        kernels.rope_table_dev(self.pos, c.rope_theta, c.head_dim, self.rope_table)     # once per token, shared by all layers
         for li in range(c.layers):
             self._block(li, 1, 0, self.pos, c.ctx_max, self.kv_len)
         self._head(0)

@@ -157,11 +157,11 @@ class DeviceWeight:
               "matmul_fused")
 
     def matmul_qkv_rope(self, x, q_out, k_cache, v_cache, heads, kv_heads, head_dim, kv_capacity, pos_dev, theta,
-                        gain=None, eps: float = 0.0) -> None:
+                        gain=None, eps: float = 0.0, rope_table=None) -> None:
         """One token's [q | k | v] projection + RoPE + cache append (skainet_hip_matmul_qkv_rope_dev)."""
         check(_lib.hip().skainet_hip_matmul_qkv_rope_dev(self._h, _ptr(x), _ptr(gain), eps, _ptr(q_out), _ptr(k_cache),
                                                          _ptr(v_cache), heads, kv_heads, head_dim, kv_capacity,
-                                                         _ptr(pos_dev), theta), "matmul_qkv_rope")
+                                                         _ptr(pos_dev), theta, _ptr(rope_table)), "matmul_qkv_rope")
 
     def dequantize(self, out) -> None:
         check(_lib.hip().skainet_hip_dequantize_dev(self._h, _ptr(out)), "dequantize")
@@ -277,6 +277,11 @@ def heads_to_rows_dev(x, out, heads, tokens, head_dim) -> None:
 
 def i32_increment_dev(value, delta: int) -> None:
     check(_lib.hip().skainet_hip_i32_increment_dev(_ptr(value), delta), "i32_increment")
+
+
+def rope_table_dev(pos_dev, theta: float, head_dim: int, table) -> None:
+    """table[2i], table[2i + 1] = cos, sin of (*pos_dev) * theta^(-2i / head_dim)."""
+    check(_lib.hip().skainet_hip_f32_rope_table_dev(_ptr(pos_dev), theta, head_dim, _ptr(table)), "rope_table")
 
 
 def decode_advance_dev(pos, kv_len, token, log) -> None:

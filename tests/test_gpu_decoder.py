@@ -188,6 +188,13 @@ def test_matmul_qkv_rope_equals_product_then_rope(hip_backend, torch_cuda, enc, 
         v1 = torch.full((kvh * cap * hd,), 5.0, device="cuda")
         q2, k2, v2 = torch.zeros_like(q1), torch.full_like(k1, 5.0), torch.full_like(v1, 5.0)
         w.matmul_qkv_rope(x, q1, k1, v1, heads, kvh, hd, cap, pos_dev, theta, gain=g, eps=eps)
+        # the same call with the per-token rotation table: identical bits
+        table = torch.empty(hd, device="cuda")
+        kx.rope_table_dev(pos_dev, theta, hd, table)
+        q3, k3, v3 = torch.zeros_like(q1), torch.full_like(k1, 5.0), torch.full_like(v1, 5.0)
+        w.matmul_qkv_rope(x, q3, k3, v3, heads, kvh, hd, cap, pos_dev, theta, gain=g, eps=eps, rope_table=table)
+        kx.sync()
+        assert torch.equal(q1, q3) and torch.equal(k1, k3) and torch.equal(v1, v3)
         qkv = torch.empty(n, device="cuda")
         w.matmul_fused(x, 1, qkv, gain=g, eps=eps)
         kx.rope_qkv_dev(qkv, q2, k2, v2, 1, heads, kvh, hd, cap, 0, pos_dev, theta)
