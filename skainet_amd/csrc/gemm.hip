@@ -15,7 +15,8 @@
 // 8 x 16 bytes of the bf16 activation tile; LDS rows are padded to 144 bytes so the 16-byte fragment reads of 32
 // consecutive rows fall on distinct banks. Two LDS stages (108 KB: one workgroup per CU); global loads run two
 // steps ahead in a two-slot register ring, one barrier per step. When the tile grid is smaller than the chip, K is split across gridDim.z and
-// the partial tiles are combined with fp32 atomic adds into a zeroed C.
+// each split parks its partial tile in a workspace with plain stores and a second launch sums the splits in split order
+// (fp32 atomic adds into C cost more than the K loop at these sizes, and their order is not reproducible).
 #include "common.h"
 
 namespace skh {
@@ -36,10 +37,8 @@ constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16); 
 void* kernel_workspace(size_t bytes);   // shim.hip
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);   // gemv.hip
 
-// The pass in front of the GEMM, one launch: activations fp32 -> bf16 (nearest even), and, when K is split, C zeroed
-// for the atomic accumulation. Thread i handles float4 number i of each.
-__global__ __launch_bounds__(256) void gemm_prepass_kernel(const float* __restrict__ in, __bf16* __restrict__ out, int64_t n4,
-                                                           float* __restrict__ c, int64_t c4, int64_t c_tail, int64_t c_total) {
+// The pass in front of the GEMM: activations fp32 -> bf16 (nearest even). Thread i handles float4 number i.
+__global__ __launch_bounds__(256) void gemm_prepass_kernel(const float* __restrict__ in, __bf16* __restrict__ out, int64_t n4) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n4) {
         const float4 v = reinterpret_cast<const float4*>(in)[i];
@@ -47,8 +46,22 @@ __global__ __launch_bounds__(256) void gemm_prepass_kernel(const float* __restri
         bf16x4 o = {(__bf16)v.x, (__bf16)v.y, (__bf16)v.z, (__bf16)v.w};
         reinterpret_cast<bf16x4*>(out)[i] = o;
     }
-    if (i < c4) reinterpret_cast<float4*>(c)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (i < c_tail) c[c_total - 1 - i] = 0.f;      // what a float4 sweep leaves over (everything, if C is not 16-byte aligned)
+}
+
+// Split K: C = sum over the splits, in split order, of the partial products parked `stride` floats apart (stride a
+// multiple of 4, the buffer 16-byte aligned). Thread i owns elements 4i .. 4i + 3.
+__global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float* __restrict__ part, int64_t stride, int splits,
+                                                              float* __restrict__ c, int64_t total, int c_aligned) {
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= total) return;
+    float4 acc = *reinterpret_cast<const float4*>(part + i);
+    for (int z = 1; z < splits; ++z) {
+        const float4 v = *reinterpret_cast<const float4*>(part + z * stride + i);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    if (c_aligned && i + 4 <= total) { *reinterpret_cast<float4*>(c + i) = acc; return; }
+    const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+    for (int j = 0; j < 4 && i + j < total; ++j) c[i + j] = v[j];
 }
 
 // ---- raw bytes a thread needs to decode 32 consecutive weights of one row, per encoding ----
@@ -168,7 +181,7 @@ __device__ __forceinline__ gemm_bf16x4 decode_part_at(int i, const Raw& r, const
 template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES>
 __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
                                                            float* __restrict__ c, int m, int n, int k, int k_chunk,
-                                                           int use_atomics) {
+                                                           int64_t split_stride) {
     extern __shared__ __attribute__((aligned(16))) __bf16 smem[];
     // stage `buf` (0 / 1): activation tile, then weight tile
     auto a_tile = [&](int buf) { return smem + buf * (G_A_ELEMS + G_W_ELEMS); };
@@ -307,6 +320,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
         }
     }
 
+    float* cz = c + (int64_t)blockIdx.z * split_stride;      // split K: this split's partial product
     // accumulator element e of lane l sits at row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32 of its 32 x 32 tile
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -318,24 +332,22 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
             for (int e = 0; e < 16; ++e) {
                 const int row = m0 + 128 * wm + 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (row < m) {
-                    float* dst = c + (int64_t)row * n + col;
-                    if (use_atomics) atomicAdd(dst, acc[i][j][e]);
-                    else *dst = acc[i][j][e];
+                    cz[(int64_t)row * n + col] = acc[i][j][e];
                 }
             }
         }
 }
 
 template <class Raw, int BE, int BB>
-static int launch_gemm_enc(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk, int atomics,
-                           hipStream_t s) {
+static int launch_gemm_enc(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
+                           int64_t split_stride, hipStream_t s) {
     static bool attr_set = false;
     if (!attr_set) {
         SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&dequant_gemm_kernel<Raw, BE, BB>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)G_SMEM));
         attr_set = true;
     }
-    dequant_gemm_kernel<Raw, BE, BB><<<grid, dim3(G_THREADS), G_SMEM, s>>>(a, w, c, m, n, k, k_chunk, atomics);
+    dequant_gemm_kernel<Raw, BE, BB><<<grid, dim3(G_THREADS), G_SMEM, s>>>(a, w, c, m, n, k, k_chunk, split_stride);
     SKH_CHECK(hipGetLastError());
     return 0;
 }
@@ -353,8 +365,6 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (k % GK != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15))
         return launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
-    __bf16* a = static_cast<__bf16*>(kernel_workspace((size_t)m * k * sizeof(__bf16)));
-    if (!a) return -1;
     const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;
     const int tiles = tiles_m * tiles_n;
     // K chunks are whole 256-element groups so every encoding's blocks stay intact
@@ -369,19 +379,28 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (ksplit > kgroups) ksplit = kgroups;
     const int k_chunk = ((kgroups + ksplit - 1) / ksplit) * 256;
     ksplit = (k + k_chunk - 1) / k_chunk;
-    {
-        const int64_t n4 = (int64_t)m * k / 4;                      // k is a multiple of 64
-        const int64_t cn = ksplit > 1 ? (int64_t)m * n : 0;
-        const bool c_aligned = (reinterpret_cast<uintptr_t>(y) & 15) == 0;
-        const int64_t c4 = c_aligned ? cn / 4 : 0, c_tail = cn - 4 * c4;   // an unaligned C is zeroed element by element
-        const int64_t threads = n4 > c4 ? (n4 > c_tail ? n4 : c_tail) : (c4 > c_tail ? c4 : c_tail);
-        gemm_prepass_kernel<<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s>>>(x, a, n4, y, c4, c_tail, cn);
-        SKH_CHECK(hipGetLastError());
-    }
+    // workspace: the bf16 activations, then (split K) one partial product per split
+    const size_t a_bytes = (((size_t)m * k * sizeof(__bf16)) + 255) & ~(size_t)255;
+    const int64_t split_stride = ksplit > 1 ? (((int64_t)m * n + 3) & ~(int64_t)3) : 0;
+    char* ws = static_cast<char*>(kernel_workspace(a_bytes + (size_t)split_stride * ksplit * sizeof(float)));
+    if (!ws) return -1;
+    __bf16* a = reinterpret_cast<__bf16*>(ws);
+    float* part = reinterpret_cast<float*>(ws + a_bytes);
+    const int64_t n4 = (int64_t)m * k / 4;                      // k is a multiple of 64
+    gemm_prepass_kernel<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s>>>(x, a, n4);
+    SKH_CHECK(hipGetLastError());
     const dim3 grid(tiles_n, tiles_m, ksplit);
-    if (enc == ENC_Q4_K) return launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(a, w, y, m, n, k, grid, k_chunk, ksplit > 1, s);
-    if (enc == ENC_Q6_K) return launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(a, w, y, m, n, k, grid, k_chunk, ksplit > 1, s);
-    return launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(a, w, y, m, n, k, grid, k_chunk, ksplit > 1, s);
+    float* c = ksplit > 1 ? part : y;
+    int rc;
+    if (enc == ENC_Q4_K) rc = launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q6_K) rc = launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    if (rc != 0 || ksplit == 1) return rc;
+    const int64_t total = (int64_t)m * n;
+    gemm_splitk_sum_kernel<<<dim3((unsigned)((total / 4 + 256) / 256)), dim3(256), 0, s>>>(
+        part, split_stride, ksplit, y, total, (reinterpret_cast<uintptr_t>(y) & 15) == 0);
+    SKH_CHECK(hipGetLastError());
+    return 0;
 }
 
 }  // namespace skh
