@@ -83,6 +83,10 @@ template <int J> __device__ __forceinline__ float ubyte_to_float(uint32_t v) {
 struct __attribute__((packed, aligned(2))) u32_a2 { uint32_t v; };
 __device__ __forceinline__ uint32_t load_u32_a2(const uint8_t* p) { return reinterpret_cast<const u32_a2*>(p)->v; }
 __device__ __forceinline__ uint32_t load_u16(const uint8_t* p) { return *reinterpret_cast<const uint16_t*>(p); }
+// 16 bytes from a 4-byte aligned address as one load (global dwordx4 loads need dword alignment only).
+typedef uint32_t u32x4_vec __attribute__((ext_vector_type(4)));
+struct __attribute__((packed, aligned(4))) u32x4_a4 { u32x4_vec v; };
+__device__ __forceinline__ u32x4_vec load_u32x4_a4(const uint8_t* p) { return reinterpret_cast<const u32x4_a4*>(p)->v; }
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

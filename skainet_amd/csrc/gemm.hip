@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float* __res
 // ---- raw bytes a thread needs to decode 32 consecutive weights of one row, per encoding ----
 struct RawQ4K { uint4 hdr, q0, q1; };
 struct RawQ6K { uint32_t ql[8], qh[8]; uint32_t sc, d; };
-struct RawQ80 { uint32_t d; uint32_t q[8]; };
+struct RawQ80 { u32x4_vec lo, hi; uint32_t edge, odd; };   // aligned 32-byte body, the 2 bytes outside it, start parity
 
 // `e` = element offset inside the row, a multiple of 32.
 __device__ __forceinline__ void load_raw(RawQ4K& r, const uint8_t* row, int e) {
@@ -136,17 +136,26 @@ __device__ __forceinline__ void decode_dword(const RawQ6K& r, const DecQ6K& c, f
 }
 
 __device__ __forceinline__ void load_raw(RawQ80& r, const uint8_t* row, int e) {
+    // a 34-byte block starts 0 or 2 bytes past a dword boundary: two 16-byte loads of its dword-aligned body and one
+    // 2-byte load of what the body leaves out (the last code pair, or the scale)
     const uint8_t* blk = row + (e >> 5) * Q80_BYTES;
-    r.d = load_u16(blk);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) r.q[i] = load_u32_a2(blk + 2 + 4 * i);
+    r.odd = (uint32_t)(reinterpret_cast<uintptr_t>(blk) >> 1) & 1u;
+    const uint8_t* body = blk + 2 * r.odd;
+    r.lo = load_u32x4_a4(body);
+    r.hi = load_u32x4_a4(body + 16);
+    r.edge = load_u16(blk + (r.odd ? 0 : 32));
 }
-struct DecQ80 { float d; };
-__device__ __forceinline__ void decode_prepare(const RawQ80& r, int, DecQ80& c) { c.d = half_bits_to_float_fast(r.d); }
+struct DecQ80 { float d; uint32_t drop; };
+__device__ __forceinline__ void decode_prepare(const RawQ80& r, int, DecQ80& c) {
+    c.d = half_bits_to_float_fast(r.odd ? r.edge : (r.lo.x & 0xFFFFu));
+    c.drop = r.odd ? 0u : 2u;                        // bytes in front of the codes in the loaded dwords
+}
 template <int I>
 __device__ __forceinline__ void decode_dword(const RawQ80& r, const DecQ80& c, float* w4) {
+    const uint32_t v[9] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w, r.edge};
+    const uint32_t q = __builtin_amdgcn_alignbyte(v[I + 1], v[I], c.drop);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) w4[j] = (float)(int8_t)(r.q[I] >> (8 * j)) * c.d;
+    for (int j = 0; j < 4; ++j) w4[j] = (float)(int8_t)(q >> (8 * j)) * c.d;
 }
 
 template <class Raw> struct DecOf;

@@ -168,20 +168,35 @@ struct Q6KSlot {
 // ---------------------------------------------------------------------------------------------- Q8_0
 struct Q80Slot {
     static constexpr int BLOCK_BYTES = Q80_BYTES, SLOTS_PER_BLOCK = 1, SLOT_ELEMS = 32, NX = 32;
-    struct Raw { uint32_t d; uint32_t q[8]; };
+    // A 34-byte block starts 0 or 2 bytes past a dword boundary. Its aligned 32-byte body (bytes 0..31 of the block
+    // when it starts on a boundary, bytes 2..33 otherwise) comes in as two 16-byte loads, the two bytes outside the
+    // body (the last code pair, or the scale) as one 2-byte load: three loads per block, none outside the block.
+    struct Raw { u32x4_vec lo, hi; uint32_t edge; uint32_t odd; };
     struct Lane { int blk_off; };
     __device__ static void init(Lane& ln, int slot) { ln.blk_off = slot * BLOCK_BYTES; }
     __device__ static int x_index(int slot, int i) { return slot * 32 + i; }
     __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
         const uint8_t* p = row + ln.blk_off;
-        r.d = load_u16(p);
+        const uint32_t odd = (uint32_t)(reinterpret_cast<uintptr_t>(p) >> 1) & 1u;   // 1: the block starts 2 bytes past a boundary
+        const uint8_t* body = p + 2 * odd;
+        r.lo = load_u32x4_a4(body);
+        r.hi = load_u32x4_a4(body + 16);
+        r.edge = load_u16(p + (odd ? 0 : 32));
+        r.odd = odd;
+    }
+    // The block's scale bits and its eight code dwords from the three loads.
+    __device__ static uint32_t unpack(const Raw& r, uint32_t* q) {
+        const uint32_t v[9] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w, r.edge};
+        const uint32_t sh = r.odd ? 0u : 2u;                 // bytes to drop in front of the codes
 #pragma unroll
-        for (int i = 0; i < 8; ++i) r.q[i] = load_u32_a2(p + 2 + 4 * i);
+        for (int i = 0; i < 8; ++i) q[i] = __builtin_amdgcn_alignbyte(v[i + 1], v[i], sh);
+        return r.odd ? r.edge : (r.lo.x & 0xFFFFu);
     }
     __device__ static void prep(const float*, float*) {}
     template <int B>
     __device__ static void dot(const Raw& r, const Lane&, const float (*x)[NX], const float (*)[1], float* acc) {
-        const float d = half_bits_to_float_fast(r.d);
+        uint32_t q[8];
+        const float d = half_bits_to_float_fast(unpack(r, q));
         float s[B];
 #pragma unroll
         for (int b = 0; b < B; ++b) s[b] = 0.f;
@@ -189,7 +204,7 @@ struct Q80Slot {
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float cf = (float)(int8_t)(r.q[i] >> (8 * j));
+                const float cf = (float)(int8_t)(q[i] >> (8 * j));
 #pragma unroll
                 for (int b = 0; b < B; ++b) s[b] = fmaf(x[b][i * 4 + j], cf, s[b]);
             }
@@ -304,7 +319,7 @@ static int launch_format(const uint8_t* w, const float* x, float* y, int k, int 
     return launch_one<F, 4, 2>(w, x, y, k, n, batch, waves_per_cu);
 }
 
-static int g_gemv_waves_per_cu = 8;
+static int g_gemv_waves_per_cu = 0;   // 0: per encoding (measured best: Q8_0 4, Q4_K / Q6_K 8)
 static int g_q4k_rows_enable = 1;
 void set_q4k_rows_waves_per_cu(int v);
 void set_gemm_ksplit(int v);
@@ -313,7 +328,7 @@ int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int 
 
 // Experiment knobs (defaults are the measured best): returns 0 when the key is known.
 int set_tuning(const char* key, int value) {
-    if (!strcmp(key, "gemv_waves_per_cu")) { if (value > 0) g_gemv_waves_per_cu = value; return 0; }
+    if (!strcmp(key, "gemv_waves_per_cu")) { if (value >= 0) g_gemv_waves_per_cu = value; return 0; }
     if (!strcmp(key, "q4k_rows_waves_per_cu")) { set_q4k_rows_waves_per_cu(value); return 0; }
     if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }
     if (!strcmp(key, "gemm_ksplit")) { set_gemm_ksplit(value); return 0; }
@@ -327,6 +342,7 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (!is_packed(enc)) return set_error("gemv: unsupported encoding %d", enc);
     if (k <= 0 || k % block_elems(enc) != 0)
         return set_error("gemv: inputDim must be a positive multiple of %d; got %d", block_elems(enc), k);
+    const int waves_per_cu = g_gemv_waves_per_cu > 0 ? g_gemv_waves_per_cu : (enc == ENC_Q8_0 ? 4 : 8);
     for (int b0 = 0; b0 < m; b0 += 4) {
         const int nb = m - b0 < 4 ? m - b0 : 4;
         const float* xb = x + (int64_t)b0 * k;
@@ -337,9 +353,9 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
             if (rc < 0) return rc;
             if (rc == 1) continue;
         }
-        if (enc == ENC_Q4_K) rc = launch_format<Q4KSlot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
-        else if (enc == ENC_Q6_K) rc = launch_format<Q6KSlot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
-        else rc = launch_format<Q80Slot>(w, xb, yb, k, n, nb, g_gemv_waves_per_cu);
+        if (enc == ENC_Q4_K) rc = launch_format<Q4KSlot>(w, xb, yb, k, n, nb, waves_per_cu);
+        else if (enc == ENC_Q6_K) rc = launch_format<Q6KSlot>(w, xb, yb, k, n, nb, waves_per_cu);
+        else rc = launch_format<Q80Slot>(w, xb, yb, k, n, nb, waves_per_cu);
         if (rc != 0) return rc;
     }
     return 0;
