@@ -325,6 +325,7 @@ void set_q4k_rows_waves_per_cu(int v);
 void set_gemm_ksplit(int v);
 void set_sdpa_prefill_mfma(int v);
 int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch);   // gemv_q4k.hip
+int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int n, int batch);  // gemv_q4k_quads.hip
 
 // Experiment knobs (defaults are the measured best): returns 0 when the key is known.
 int set_tuning(const char* key, int value) {
@@ -343,20 +344,24 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (k <= 0 || k % block_elems(enc) != 0)
         return set_error("gemv: inputDim must be a positive multiple of %d; got %d", block_elems(enc), k);
     const int waves_per_cu = g_gemv_waves_per_cu > 0 ? g_gemv_waves_per_cu : (enc == ENC_Q8_0 ? 4 : 8);
-    for (int b0 = 0; b0 < m; b0 += 4) {
-        const int nb = m - b0 < 4 ? m - b0 : 4;
+    for (int b0 = 0; b0 < m;) {
+        const int left = m - b0;
         const float* xb = x + (int64_t)b0 * k;
         float* yb = y + (int64_t)b0 * n;
         int rc;
         if (enc == ENC_Q4_K && g_q4k_rows_enable) {
-            rc = launch_q4k_gemv_rows(w, xb, yb, k, n, nb);
+            // 3 to 8 rows: the fp32 matrix-instruction kernel; 1 or 2: the row-streaming kernel
+            const int nq = left < 8 ? left : 8;
+            rc = left >= 3 ? launch_q4k_gemv_quads(w, xb, yb, k, n, nq) : launch_q4k_gemv_rows(w, xb, yb, k, n, left);
             if (rc < 0) return rc;
-            if (rc == 1) continue;
+            if (rc == 1) { b0 += left >= 3 ? nq : left; continue; }
         }
+        const int nb = left < 4 ? left : 4;
         if (enc == ENC_Q4_K) rc = launch_format<Q4KSlot>(w, xb, yb, k, n, nb, waves_per_cu);
         else if (enc == ENC_Q6_K) rc = launch_format<Q6KSlot>(w, xb, yb, k, n, nb, waves_per_cu);
         else rc = launch_format<Q80Slot>(w, xb, yb, k, n, nb, waves_per_cu);
         if (rc != 0) return rc;
+        b0 += nb;
     }
     return 0;
 }

@@ -133,6 +133,22 @@ def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cud
         hip_backend.set_tuning("q4k_rows_enable", 1)
 
 
+@pytest.mark.parametrize("n,k,m", [(5, 256, 3), (25, 1280, 8), (77, 2304, 7), (1000, 11008, 4), (11008, 4096, 6), (4096, 14336, 8),
+                                   (130, 4096, 9), (64, 1024, 11)])
+def test_q4k_three_to_eight_rows_on_the_fp32_matrix_instruction(hip_backend, torch_cuda, n, k, m):
+    """3 to 8 activation rows take the 4x4x1 fp32 MFMA kernel (9 and 11 rows: 8 + the rest): exact fp32 products, so
+    the one-row bound holds; every batch row must also equal that row run alone to fp32 rounding."""
+    for packed in (gaussian_weight(hip_backend, "Q4_K", n, k, 81), random_valid_blocks("Q4_K", n * k // 256, 82)):
+        x = np.random.default_rng(83 + m).standard_normal((m, k)).astype(np.float32)
+        x[1, :64] = 0.0
+        x[m - 1, 100] = -41.0
+        got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert got.shape == (m, n) and not np.isnan(got).any()
+        assert normalized_err(got, L.gemv("Q4_K", x, packed, n)) <= GEMV_TOL
+        alone = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x[m - 1:m])
+        assert normalized_err(got[m - 1], alone[0]) <= 1e-4
+
+
 def test_gemv_is_linear_and_deterministic_at_full_size(hip_backend, torch_cuda):
     """Size-independent properties at the benchmark shape: y(a*x1 + x2) == a*y(x1) + y(x2) within rounding; two runs agree bit for bit."""
     n, k = 11008, 4096
