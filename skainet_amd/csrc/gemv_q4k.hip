@@ -29,28 +29,39 @@
 
 namespace skh {
 
+// One row's 64 weights of a lane against its 64 activations. The 4-bit codes are never converted: a dword of codes is
+// masked into pairs of 16-bit fields whose low mantissa bits hold a code (0x000F000F: the low nibbles of bytes 0 and 2;
+// 0x00F000F0: their high nibbles, i.e. 16 * code; the same on the dword shifted right by 8 for bytes 1 and 3). Read as
+// fp16 such a field is the subnormal code * 2^-24 (or 16 * code * 2^-24), which v_fma_mix_f32 widens to fp32 exactly on
+// its way into an fp32 FMA -- five mask / shift operations per eight weights instead of eight conversions, and the
+// products and sums are the same fp32 values as with converted codes (the powers of two go into the block scales).
+typedef _Float16 q4k_h2 __attribute__((ext_vector_type(2)));
 template <int B>
 __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi_mask, const float (*x)[64],
                                             const float (*xsum)[2], float* out) {
     float dlo, dhi, mlo, mhi;
     q4k_lane_scales(r.hdr, sh, hi_mask, dlo, dhi, mlo, mhi);
-    dhi *= 0.0625f;                                            // high nibbles are summed as 16 * code
+    dlo *= 16777216.0f;                                        // codes enter as code * 2^-24
+    dhi *= 1048576.0f;                                         // high nibbles as 16 * code * 2^-24
     const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
     float lo[B], hi[B];
 #pragma unroll
     for (int b = 0; b < B; ++b) lo[b] = hi[b] = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const uint32_t l4 = q[i] & 0x0F0F0F0Fu, h4 = q[i] & 0xF0F0F0F0u;
-        const float cl[4] = {ubyte0_to_float(l4), ubyte1_to_float(l4), ubyte2_to_float(l4), ubyte3_to_float(l4)};
-        const float ch[4] = {ubyte0_to_float(h4), ubyte1_to_float(h4), ubyte2_to_float(h4), ubyte3_to_float(h4)};
+        const uint32_t q8 = q[i] >> 8;
+        const q4k_h2 l02 = __builtin_bit_cast(q4k_h2, q[i] & 0x000F000Fu), h02 = __builtin_bit_cast(q4k_h2, q[i] & 0x00F000F0u);
+        const q4k_h2 l13 = __builtin_bit_cast(q4k_h2, q8 & 0x000F000Fu), h13 = __builtin_bit_cast(q4k_h2, q8 & 0x00F000F0u);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-            for (int b = 0; b < B; ++b) {
-                lo[b] = fmaf(x[b][i * 4 + j], cl[j], lo[b]);
-                hi[b] = fmaf(x[b][32 + i * 4 + j], ch[j], hi[b]);
-            }
+        for (int b = 0; b < B; ++b) {
+            lo[b] = fmaf((float)l02.x, x[b][i * 4 + 0], lo[b]);
+            hi[b] = fmaf((float)h02.x, x[b][32 + i * 4 + 0], hi[b]);
+            lo[b] = fmaf((float)l13.x, x[b][i * 4 + 1], lo[b]);
+            hi[b] = fmaf((float)h13.x, x[b][32 + i * 4 + 1], hi[b]);
+            lo[b] = fmaf((float)l02.y, x[b][i * 4 + 2], lo[b]);
+            hi[b] = fmaf((float)h02.y, x[b][32 + i * 4 + 2], hi[b]);
+            lo[b] = fmaf((float)l13.y, x[b][i * 4 + 3], lo[b]);
+            hi[b] = fmaf((float)h13.y, x[b][32 + i * 4 + 3], hi[b]);
         }
     }
 #pragma unroll
@@ -59,19 +70,25 @@ __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi
 
 // Two workgroups per CU is the occupancy the register budget is cut for (the row loads in flight, the pass's
 // activations and the per-row sums all live in registers); asking for more makes the compiler spill.
-template <int B, int R, int PRO, int EPI>
+//
+// NR, the rows a wave owns per chunk, is a template parameter and every wave computes exactly NR rows per chunk (rows
+// past N are clamped to the last row and never stored): a pass is then one straight-line block without a guard
+// around any load. With a run-time row count every load sits behind a (uniform) branch, and at the join after a
+// branch the compiler's wait-count bookkeeping makes the wave wait for loads it has only just issued -- the rows meant
+// to be in flight together were fetched one round trip after the other.
+template <int B, int R, int NR, int PRO>
 __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                                            float* y, int k, int n, int rows_per_wave, int chunk_rows,
+                                                            float* y, int k, int n, int nchunks,
                                                             const float* __restrict__ gain, float eps, const float* residual,
-                                                            RopeQkvEpilogue rope) {
+                                                            int epilogue, RopeQkvEpilogue rope) {
     constexpr int NV = 16 * B;   // Q4K_RMAX rows padded to 16, times B
     constexpr int SLICE = 68;    // 64 activations + 4 floats of padding: 16-byte aligned and bank-conflict free
+    static_assert(NR >= 1 && NR <= Q4K_RMAX, "rows per chunk");
     __shared__ __attribute__((aligned(16))) float xlds[B][64 * SLICE];
     const int lane = threadIdx.x & 63;
-    // readfirstlane: the wave index is uniform across a wave, and saying so keeps every row guard a scalar branch
+    // readfirstlane: the wave index is uniform across a wave, and saying so keeps the row addresses scalar
     const int gw = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
-    const int wave_r0 = gw * rows_per_wave;
-    const int wave_end = min(n, wave_r0 + rows_per_wave);
+    const int wave_r0 = gw * (NR * nchunks);
     const int bpr = k >> 8;
     const int64_t row_bytes = (int64_t)bpr * Q4K_BYTES;
     const int g = lane & 3;
@@ -83,12 +100,10 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
 #pragma unroll
     for (int b = 0; b < B; ++b) { ssq[b] = 0.f; xscale[b] = 1.0f; }
 
-    // A wave's rows are taken in chunks of at most Q4K_RMAX (the per-row accumulators live in registers); every
-    // wave of the grid runs the same number of chunks and passes, so the barriers below are uniform.
-    for (int c0 = 0; c0 < rows_per_wave; c0 += chunk_rows) {
-        const int r0 = wave_r0 + c0;
-        const int nrows = max(0, min(wave_end, r0 + chunk_rows) - r0);   // a wave without rows still helps stage activations
-        const uint8_t* wbase = w + (int64_t)r0 * row_bytes;
+    for (int c0 = 0; c0 < nchunks; ++c0) {
+        const int r0 = wave_r0 + c0 * NR;
+        const int nrows = max(0, min(n - r0, NR));               // rows of this chunk that exist (the rest are clamped copies)
+        const float first = c0 == 0 ? 1.0f : 0.0f;               // the squares are summed during the first chunk only
 
         float acc[16][B];
 #pragma unroll
@@ -99,22 +114,13 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
         for (int blk0 = 0; blk0 < bpr; blk0 += 16) {
             const int blk = blk0 + (lane >> 2);
             const int blk_c = min(blk, bpr - 1);            // lanes past K re-read a valid block and multiply it by zero activations
-            const uint8_t* lane_base = wbase + blk_c * Q4K_BYTES;
+            auto row_ptr = [&](int i) { return w + (int64_t)min(r0 + i, n - 1) * row_bytes + (int64_t)blk_c * Q4K_BYTES; };
 
-            // the first rows' weight loads go out before anything else
-            Q4KRow raw[R];
-#pragma unroll
-            for (int i = 0; i < R; ++i) {
-                if (i < nrows) {                                // wave-uniform
-                    const uint8_t* p = lane_base + (int64_t)i * row_bytes;
-                    raw[i].hdr = *reinterpret_cast<const uint4*>(p);
-                    raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
-                    raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
-                }
-            }
-
-            // stage this pass's activations: float4 number f of the pass goes to slice f / 16, position f % 16.
-            // All loads are issued unconditionally (clamped address, zeroed afterwards) so they overlap.
+            // This pass's activations are requested first, the first R rows of weights right behind them: loads return in
+            // the order they were issued, so the (L2-resident) activations must not queue behind the weight stream --
+            // the arithmetic can then start on the first row while the later rows are still arriving.
+            // float4 number f of the pass goes to LDS slice f / 16, position f % 16. All loads are issued unconditionally
+            // (clamped address, zeroed afterwards) so they overlap.
             float4 xv[B][4], gv[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -123,17 +129,27 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
                 for (int b = 0; b < B; ++b) xv[b][j] = *reinterpret_cast<const float4*>(x + (int64_t)b * k + e);
                 if (PRO) gv[j] = *reinterpret_cast<const float4*>(gain + e);
             }
-            if (blk0 > 0 || c0 > 0) __syncthreads();   // the previous pass's slices have been read
+            __builtin_amdgcn_sched_barrier(0);
+            Q4KRow raw[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const uint8_t* p = row_ptr(i < NR ? i : NR - 1);
+                raw[i].hdr = *reinterpret_cast<const uint4*>(p);
+                raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();                                // the previous pass's slices have been read
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int f = threadIdx.x + 256 * j;
-                const bool inside = blk0 * 256 + f * 4 < k;
+                const float inside = blk0 * 256 + f * 4 < k ? 1.0f : 0.0f;
 #pragma unroll
                 for (int b = 0; b < B; ++b) {
                     float4 v4 = xv[b][j];
-                    if (!inside) v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                    v4.x *= inside; v4.y *= inside; v4.z *= inside; v4.w *= inside;
                     if (PRO) {
-                        if (c0 == 0) ssq[b] = fmaf(v4.x, v4.x, fmaf(v4.y, v4.y, fmaf(v4.z, v4.z, fmaf(v4.w, v4.w, ssq[b]))));
+                        ssq[b] = fmaf(first, fmaf(v4.x, v4.x, fmaf(v4.y, v4.y, fmaf(v4.z, v4.z, v4.w * v4.w))), ssq[b]);
                         v4.x *= gv[j].x; v4.y *= gv[j].y; v4.z *= gv[j].z; v4.w *= gv[j].w;
                     }
                     *reinterpret_cast<float4*>(&xlds[b][(f >> 4) * SLICE + (f & 15) * 4]) = v4;
@@ -156,19 +172,15 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
             }
 
 #pragma unroll
-            for (int c = 0; c < Q4K_RMAX; c += R) {
-                if (c < nrows) {                                  // wave-uniform
-#pragma unroll
-                    for (int i = 0; i < R; ++i) {
-                        if (c + i < nrows) q4k_row_dot<B>(raw[i], sh, hi_mask, xs, xsum, acc[c + i]);
-                        if (c + R + i < nrows) {                  // refill with the row R ahead
-                            const uint8_t* p = lane_base + (int64_t)(c + R + i) * row_bytes;
-                            raw[i].hdr = *reinterpret_cast<const uint4*>(p);
-                            raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
-                            raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
-                        }
-                    }
+            for (int c = 0; c < NR; ++c) {
+                q4k_row_dot<B>(raw[c % R], sh, hi_mask, xs, xsum, acc[c]);
+                if (c + R < NR) {                               // compile-time: refill with the row R ahead
+                    const uint8_t* p = row_ptr(c + R);
+                    raw[c % R].hdr = *reinterpret_cast<const uint4*>(p);
+                    raw[c % R].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                    raw[c % R].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
                 }
+                __builtin_amdgcn_sched_barrier(0);              // a refill is issued where it is written, not later
             }
         }
 
@@ -196,7 +208,7 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
         const int idx = wave_fold_index<NV>(lane);
         const int row = idx / B, b = idx % B;
         float val = v[0] * (B == 1 ? xscale[0] : (b == 0 ? xscale[0] : xscale[B - 1]));
-        if (EPI == EPI_ROPE_QKV) {
+        if (epilogue == EPI_ROPE_QKV) {
             // rows 2i and 2i + 1 of a head are one rotation pair; like the SwiGLU pairs they sit NV / (2B) lanes apart
             const float odd = __shfl_xor(val, NV / (2 * B), 64);
             if (lane < NV && !(row & 1) && row < nrows) {
@@ -215,13 +227,13 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
                 else dst = rope.v_cache + ((int64_t)(slot - rope.heads - rope.kv_heads) * rope.capacity + p0) * rope.head_dim;
                 *reinterpret_cast<float2*>(dst + dd) = out2;
             }
-        } else if (EPI == EPI_SWIGLU) {
+        } else if (epilogue == EPI_SWIGLU) {
             // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
             const float up = __shfl_xor(val, NV / (2 * B), 64);
             if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
         } else if (lane < NV && row < nrows) {
             const int64_t o = (int64_t)b * n + r0 + row;
-            if (EPI == EPI_RESIDUAL) val += residual[o];
+            if (epilogue == EPI_RESIDUAL) val += residual[o];
             y[o] = val;
         }
     }
@@ -231,22 +243,30 @@ static int g_q4k_rows_waves_per_cu = 8;
 void set_q4k_rows_waves_per_cu(int v) { if (v > 0) g_q4k_rows_waves_per_cu = v; }
 int q4k_rows_waves_per_cu() { return g_q4k_rows_waves_per_cu; }
 
-// Returns 1 when this kernel took the product, 0 when the shape is outside its range (caller falls back to the
-// slot kernel), -1 on a launch error.
-template <int PRO, int EPI>
-static void launch_variant(int batch, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n,
-                           int rows_per_wave, int chunk_rows, const float* gain, float eps, const float* residual,
-                           const RopeQkvEpilogue& rope) {
-    if (batch == 1)
-        q4k_gemv_rows_kernel<1, 4, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope);
-    else
-        q4k_gemv_rows_kernel<2, 2, PRO, EPI><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope);
+template <int B, int R, int NR>
+static void launch_rows(bool pro, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int nchunks,
+                        const float* gain, float eps, const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+    if (pro) q4k_gemv_rows_kernel<B, R, NR, 1><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, nchunks, gain, eps, residual, epilogue, rope);
+    else q4k_gemv_rows_kernel<B, R, NR, 0><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, nchunks, gain, eps, residual, epilogue, rope);
+}
+template <int B, int R>
+static void launch_rows_nr(int nr, bool pro, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n,
+                           int nchunks, const float* gain, float eps, const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+#define SKH_NR_CASE(N) case N: launch_rows<B, (R < N ? R : N), N>(pro, grid, s, w, x, y, k, n, nchunks, gain, eps, residual, epilogue, rope); break;
+    switch (nr) {
+        SKH_NR_CASE(1) SKH_NR_CASE(2) SKH_NR_CASE(3) SKH_NR_CASE(4) SKH_NR_CASE(5) SKH_NR_CASE(6)
+        SKH_NR_CASE(7) SKH_NR_CASE(8) SKH_NR_CASE(9) SKH_NR_CASE(10) SKH_NR_CASE(11) SKH_NR_CASE(12)
+    }
+#undef SKH_NR_CASE
 }
 
+// Returns 1 when this kernel took the product, 0 when the shape is outside its range (caller falls back to the
+// slot kernel), -1 on a launch error.
 // y = epilogue(W . prologue(x)); gain != null selects the RMSNorm prologue, epilogue is one of EPI_*.
 int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k, int n, int batch, const float* gain, float eps,
                                const float* residual, int epilogue, const RopeQkvEpilogue* rope_in) {
     if (batch < 1 || batch > 2) return 0;
+    if (epilogue < EPI_NONE || epilogue > EPI_ROPE_QKV) return set_error("q4k gemv: unknown epilogue %d", epilogue);
     RopeQkvEpilogue rope{};
     if (epilogue == EPI_ROPE_QKV) {
         if (!rope_in || batch != 1) return 0;
@@ -255,30 +275,21 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     }
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 3)) return 0;
     if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return 0;
-    if (epilogue >= EPI_SWIGLU && (n & 1)) return 0;
-    int total_waves = num_cus() * g_q4k_rows_waves_per_cu;
-    int rows_per_wave = (n + total_waves - 1) / total_waves;
-    if (epilogue >= EPI_SWIGLU) rows_per_wave = (rows_per_wave + 1) & ~1;   // a (gate, up) or rotation pair never straddles two waves
-    // one round of workgroups over the chip: a wave with more than Q4K_RMAX rows takes them in equal chunks
-    const int nchunks = (rows_per_wave + Q4K_RMAX - 1) / Q4K_RMAX;
-    int chunk_rows = (rows_per_wave + nchunks - 1) / nchunks;
-    if (epilogue >= EPI_SWIGLU) chunk_rows = (chunk_rows + 1) & ~1;
+    const bool pairs = epilogue >= EPI_SWIGLU;                   // a (gate, up) or rotation pair never straddles two waves
+    if (pairs && (n & 1)) return 0;
+    // one round of workgroups over the chip: a wave's rows, taken in equal chunks of at most Q4K_RMAX (the chunk size
+    // is a template parameter, so the share is rounded up to a whole number of chunks)
+    const int total_waves = num_cus() * g_q4k_rows_waves_per_cu;
+    const int share = (n + total_waves - 1) / total_waves;
+    const int nchunks = (share + Q4K_RMAX - 1) / Q4K_RMAX;
+    int nr = (share + nchunks - 1) / nchunks;
+    if (pairs) nr = (nr + 1) & ~1;
+    const int rows_per_wave = nr * nchunks;
     const int waves = (n + rows_per_wave - 1) / rows_per_wave;
     const int grid = (waves + 3) / 4;
-    if (epilogue < EPI_NONE || epilogue > EPI_ROPE_QKV) return set_error("q4k gemv: unknown epilogue %d", epilogue);
     hipStream_t s = current_stream();
-    const int variant = (gain ? 4 : 0) + epilogue;
-    switch (variant) {
-        case 0: launch_variant<0, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        case 1: launch_variant<0, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        case 2: launch_variant<0, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        case 3: launch_variant<0, EPI_ROPE_QKV>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        case 4: launch_variant<1, EPI_NONE>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        case 5: launch_variant<1, EPI_RESIDUAL>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        case 6: launch_variant<1, EPI_SWIGLU>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        case 7: launch_variant<1, EPI_ROPE_QKV>(batch, grid, s, w, x, y, k, n, rows_per_wave, chunk_rows, gain, eps, residual, rope); break;
-        default: return set_error("q4k gemv: unknown epilogue %d", epilogue);
-    }
+    if (batch == 1) launch_rows_nr<1, 6>(nr, gain != nullptr, grid, s, w, x, y, k, n, nchunks, gain, eps, residual, epilogue, rope);
+    else launch_rows_nr<2, 2>(nr, gain != nullptr, grid, s, w, x, y, k, n, nchunks, gain, eps, residual, epilogue, rope);
     SKH_CHECK(hipGetLastError());
     return 1;
 }
