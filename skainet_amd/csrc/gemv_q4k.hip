@@ -279,7 +279,10 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     if (pairs && (n & 1)) return 0;
     // one round of workgroups over the chip: a wave's rows, taken in equal chunks of at most Q4K_RMAX (the chunk size
     // is a template parameter, so the share is rounded up to a whole number of chunks)
-    const int total_waves = num_cus() * g_q4k_rows_waves_per_cu;
+    // (more waves per CU when that keeps a wave's share in one chunk: a second chunk stages the activations again)
+    int waves_per_cu = g_q4k_rows_waves_per_cu;
+    while (waves_per_cu < 32 && (n + num_cus() * waves_per_cu - 1) / (num_cus() * waves_per_cu) > Q4K_RMAX) waves_per_cu += 4;
+    const int total_waves = num_cus() * waves_per_cu;
     const int share = (n + total_waves - 1) / total_waves;
     const int nchunks = (share + Q4K_RMAX - 1) / Q4K_RMAX;
     int nr = (share + nchunks - 1) / nchunks;

@@ -87,17 +87,10 @@ __global__ __launch_bounds__(256, OCC) void q4k_gemv_quads_kernel(const uint8_t*
         // this lane's weight row of quad q: r0 + 4 q + j, clamped (rows past N are computed and never stored)
         auto row_ptr = [&](int q) { return w + (int64_t)min(r0 + 4 * q + j, n - 1) * row_bytes + (int64_t)sb_c * Q4K_BYTES; };
 
-        // the first quads' weight loads go out before anything else
+        // The round's activations are requested first and the first quads' weights right behind them: loads return in
+        // issue order, and the (L2-resident) activations must not queue behind the weight stream.
+        // float4 number f (of 1024) of batch row b goes to slice f / 16 of that row, position f % 16.
         Q4KRow raw[R];
-#pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const uint8_t* p = row_ptr(i < Q ? i : Q - 1);
-            raw[i].hdr = *reinterpret_cast<const uint4*>(p);
-            raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
-            raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
-        }
-
-        // stage the round: float4 number f (of 1024) of batch row b goes to slice f / 16 of that row, position f % 16
         {
             float4 xv[4 * NB][4];
 #pragma unroll
@@ -107,7 +100,16 @@ __global__ __launch_bounds__(256, OCC) void q4k_gemv_quads_kernel(const uint8_t*
                     const int e = min(round * 4096 + (threadIdx.x + 256 * u) * 4, k - 4);
                     xv[b][u] = *reinterpret_cast<const float4*>(x + (int64_t)min(b, batch - 1) * k + e);
                 }
-            if (round > 0) __syncthreads();                // the previous round's slices have been read
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const uint8_t* p = row_ptr(i < Q ? i : Q - 1);
+                raw[i].hdr = *reinterpret_cast<const uint4*>(p);
+                raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();                               // the previous round's slices have been read
 #pragma unroll
             for (int b = 0; b < 4 * NB; ++b)
 #pragma unroll
