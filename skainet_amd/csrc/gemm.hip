@@ -369,9 +369,10 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (!is_packed(enc)) return set_error("gemm: unsupported encoding %d", enc);
     if (k <= 0 || k % block_elems(enc) != 0)
         return set_error("gemm: inputDim must be a positive multiple of %d; got %d", block_elems(enc), k);
-    // shapes the tile loader cannot take (a Q8_0 row that is not a whole number of 64-element steps, unaligned
-    // operands) go through the row kernels: same result to fp32 rounding, the weight streamed once per 4 rows
-    if (k % GK != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15))
+    // shapes the tile loader cannot take (a Q8_0 row that is not a whole number of 256-element groups: the K loop
+    // runs pairs of 64-element steps over whole groups; unaligned operands) go through the row kernels: same result
+    // to fp32 rounding, the weight streamed once per 4 rows
+    if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15))
         return launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
     const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;

@@ -242,21 +242,30 @@ __global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
         typename F::Lane ln;
         F::init(ln, active ? slot : 0);
 
-        // First rows' weight loads are issued before the activation slice is fetched.
+        // The activation slice is requested first and unconditionally (clamped address, zeroed afterwards), the first
+        // R rows of weights right behind it: loads return in issue order, so the L2-resident activations must not
+        // queue behind the weight stream, and a branch around a load would make the wave wait for every load in flight.
+        float xs[B][NX], xsum[B][NS];
+        const int xslot = active ? slot : 0;
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const float* xb = x + (int64_t)(b < batch ? b : 0) * k;
+#pragma unroll
+            for (int i = 0; i < NX; i += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(xb + F::x_index(xslot, i));
+                xs[b][i] = v.x; xs[b][i + 1] = v.y; xs[b][i + 2] = v.z; xs[b][i + 3] = v.w;
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         typename F::Raw raw[R];
 #pragma unroll
         for (int i = 0; i < R; ++i) F::load(raw[i], wbase + (int64_t)min(i, nrows - 1) * row_bytes, ln);
-
-        float xs[B][NX], xsum[B][NS];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int b = 0; b < B; ++b) {
-            const bool have = active && b < batch;
+            const float keep = (active && b < batch) ? 1.0f : 0.0f;
 #pragma unroll
-            for (int i = 0; i < NX; i += 4) {
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (have) v = *reinterpret_cast<const float4*>(x + (int64_t)b * k + F::x_index(slot, i));
-                xs[b][i] = v.x; xs[b][i + 1] = v.y; xs[b][i + 2] = v.z; xs[b][i + 3] = v.w;
-            }
+            for (int i = 0; i < NX; ++i) xs[b][i] *= keep;
             F::prep(xs[b], xsum[b]);
         }
 

@@ -68,6 +68,43 @@ __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi
     for (int b = 0; b < B; ++b) out[b] += dlo * lo[b] + dhi * hi[b] - (mlo * xsum[b][0] + mhi * xsum[b][1]);
 }
 
+// Epilogue of a chunk: after the fold lane l < 16 B holds the total of row `row` (of the chunk that starts at output
+// row r0) for activation row b. Plain store, `+ residual`, SwiGLU over adjacent (gate, up) rows, or RoPE + scatter of
+// one token's [q | k | v] rows.
+template <int B>
+__device__ __forceinline__ void q4k_rows_epilogue(float val, int lane, int row, int b, int r0, int nrows, int n, float* y,
+                                                  const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+    constexpr int NV = 16 * B;
+    if (epilogue == EPI_ROPE_QKV) {
+        // rows 2i and 2i + 1 of a head are one rotation pair; like the SwiGLU pairs they sit NV / (2B) lanes apart
+        const float odd = __shfl_xor(val, NV / (2 * B), 64);
+        if (lane < NV && !(row & 1) && row < nrows) {
+            const int o = r0 + row, slot = o / rope.head_dim, dd = o % rope.head_dim;
+            const int p0 = rope.pos_dev[0];
+            float2 out2 = make_float2(val, odd);
+            if (slot < rope.heads + rope.kv_heads) {
+                float sn, cs;
+                if (rope.table) { const float2 t = rope.table[dd >> 1]; cs = t.x; sn = t.y; }
+                else sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
+                out2 = make_float2(val * cs - odd * sn, val * sn + odd * cs);
+            }
+            float* dst;
+            if (slot < rope.heads) dst = y + (int64_t)slot * rope.head_dim;
+            else if (slot < rope.heads + rope.kv_heads) dst = rope.k_cache + ((int64_t)(slot - rope.heads) * rope.capacity + p0) * rope.head_dim;
+            else dst = rope.v_cache + ((int64_t)(slot - rope.heads - rope.kv_heads) * rope.capacity + p0) * rope.head_dim;
+            *reinterpret_cast<float2*>(dst + dd) = out2;
+        }
+    } else if (epilogue == EPI_SWIGLU) {
+        // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
+        const float up = __shfl_xor(val, NV / (2 * B), 64);
+        if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
+    } else if (lane < NV && row < nrows) {
+        const int64_t o = (int64_t)b * n + r0 + row;
+        if (epilogue == EPI_RESIDUAL) val += residual[o];
+        y[o] = val;
+    }
+}
+
 // Two workgroups per CU is the occupancy the register budget is cut for (the row loads in flight, the pass's
 // activations and the per-row sums all live in registers); asking for more makes the compiler spill.
 //
@@ -208,34 +245,7 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
         const int idx = wave_fold_index<NV>(lane);
         const int row = idx / B, b = idx % B;
         float val = v[0] * (B == 1 ? xscale[0] : (b == 0 ? xscale[0] : xscale[B - 1]));
-        if (epilogue == EPI_ROPE_QKV) {
-            // rows 2i and 2i + 1 of a head are one rotation pair; like the SwiGLU pairs they sit NV / (2B) lanes apart
-            const float odd = __shfl_xor(val, NV / (2 * B), 64);
-            if (lane < NV && !(row & 1) && row < nrows) {
-                const int o = r0 + row, slot = o / rope.head_dim, dd = o % rope.head_dim;
-                const int p0 = rope.pos_dev[0];
-                float2 out2 = make_float2(val, odd);
-                if (slot < rope.heads + rope.kv_heads) {
-                    float sn, cs;
-                    if (rope.table) { const float2 t = rope.table[dd >> 1]; cs = t.x; sn = t.y; }
-                    else sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
-                    out2 = make_float2(val * cs - odd * sn, val * sn + odd * cs);
-                }
-                float* dst;
-                if (slot < rope.heads) dst = y + (int64_t)slot * rope.head_dim;
-                else if (slot < rope.heads + rope.kv_heads) dst = rope.k_cache + ((int64_t)(slot - rope.heads) * rope.capacity + p0) * rope.head_dim;
-                else dst = rope.v_cache + ((int64_t)(slot - rope.heads - rope.kv_heads) * rope.capacity + p0) * rope.head_dim;
-                *reinterpret_cast<float2*>(dst + dd) = out2;
-            }
-        } else if (epilogue == EPI_SWIGLU) {
-            // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
-            const float up = __shfl_xor(val, NV / (2 * B), 64);
-            if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
-        } else if (lane < NV && row < nrows) {
-            const int64_t o = (int64_t)b * n + r0 + row;
-            if (epilogue == EPI_RESIDUAL) val += residual[o];
-            y[o] = val;
-        }
+        q4k_rows_epilogue<B>(val, lane, row, b, r0, nrows, n, y, residual, epilogue, rope);
     }
 }
 

@@ -135,10 +135,12 @@ def test_rope_qkv_equals_three_scatters(hip_backend, torch_cuda):
 
 
 @pytest.mark.parametrize("enc,n,k,m", [("Q4_K", 1536, 1024, 1), ("Q4_K", 1030, 512, 2), ("Q4_K", 24, 4096 + 256, 1),
-                                        ("Q4_K", 640, 512, 5), ("Q6_K", 512, 512, 1), ("Q4_K", 768, 1024, 24)])
+                                        ("Q4_K", 640, 512, 5), ("Q6_K", 512, 512, 1), ("Q4_K", 768, 1024, 24),
+                                        ("Q4_K", 1030, 14336, 1), ("Q4_K", 26, 16640, 1), ("Q4_K", 4096, 12288, 1)])
 def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
     """Every prologue / epilogue combination against float64 arithmetic on the oracle-decoded weight; the decode
-    shapes of Q4_K run the one-kernel route, the other cases the composed route of the same entry."""
+    shapes of Q4_K run the one-kernel route (also with K of several passes), the other cases the composed route of the
+    same entry."""
     from oracle import lib as O
     torch, kx = torch_cuda, hip_backend
     rng = np.random.default_rng(n + k + m)

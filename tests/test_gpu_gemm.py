@@ -79,8 +79,11 @@ def test_gemm_on_random_valid_blocks_and_forced_k_splits(hip_backend, torch_cuda
         hip_backend.set_tuning("gemm_ksplit", 0)
 
 
-def test_gemm_q8_0_rows_that_do_not_fill_a_k_step_fall_back_to_the_row_kernels(hip_backend, torch_cuda):
-    m, n, k = 20, 50, 96          # 3 Q8_0 blocks: not a multiple of the 64-element K step
+@pytest.mark.parametrize("k", [96, 192, 320, 448])
+def test_gemm_q8_0_rows_that_are_not_whole_256_element_groups_fall_back_to_the_row_kernels(hip_backend, torch_cuda, k):
+    """The tile kernel's K loop runs over whole 256-element groups; a Q8_0 row of 3, 6, 10 or 14 blocks takes the
+    row kernels instead (exact fp32 products, so the one-row bound applies)."""
+    m, n = 20, 50
     packed = gaussian_weight(hip_backend, "Q8_0", n, k, 7)
     x = np.random.default_rng(8).standard_normal((m, k)).astype(np.float32)
     got = gpu_gemm(hip_backend, torch_cuda, "Q8_0", packed, n, k, x)
