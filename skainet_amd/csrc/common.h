@@ -67,7 +67,10 @@ __device__ __forceinline__ float half_bits_to_float_fast(uint32_t h) {
 }
 
 // Byte N of a dword as float (v_cvt_f32_ubyteN). Written as asm so the compiler keeps one pre-masked dword
-// and four conversions instead of re-deriving a shift/mask per byte.
+// and four conversions instead of re-deriving a shift/mask per byte. The result must pass through another vector-ALU
+// instruction before a matrix instruction reads it: an MFMA operand written by the VALU instruction just before needs
+// wait states that the compiler only inserts for writes it can see, not for inline assembly (kernels that feed
+// conversions straight into an MFMA write them in plain C instead).
 __device__ __forceinline__ float ubyte0_to_float(uint32_t v) { float f; asm("v_cvt_f32_ubyte0_e32 %0, %1" : "=v"(f) : "v"(v)); return f; }
 __device__ __forceinline__ float ubyte1_to_float(uint32_t v) { float f; asm("v_cvt_f32_ubyte1_e32 %0, %1" : "=v"(f) : "v"(v)); return f; }
 __device__ __forceinline__ float ubyte2_to_float(uint32_t v) { float f; asm("v_cvt_f32_ubyte2_e32 %0, %1" : "=v"(f) : "v"(v)); return f; }

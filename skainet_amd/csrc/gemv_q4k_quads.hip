@@ -159,12 +159,13 @@ __global__ __launch_bounds__(256, OCC) void q4k_gemv_quads_kernel(const uint8_t*
                 for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                     for (int c = 0; c < NCH; ++c) { dlc[nb][c] = f32x4_q{0.f, 0.f, 0.f, 0.f}; dhc[nb][c] = f32x4_q{0.f, 0.f, 0.f, 0.f}; }
-                // The conversions are plain C so the compiler sees every vector-ALU write near the matrix instructions (an
-                // operand written by the instruction just before costs wait states, and inline assembly would hide the
-                // write from that bookkeeping altogether). The empty asm emits nothing: it hides the nibble masks from
-                // the optimiser, which otherwise turns each byte conversion into a bit-field extract plus a conversion
-                // instead of one v_cvt_f32_ubyteN. Program order is pinned so that the conversions of code dword i + 1
-                // sit between the matrix instructions of dword i: each operand is written a dword ahead of its use.
+                // The conversions are plain C so the compiler sees the vector-ALU write of every matrix-instruction
+                // operand (an operand written by the instruction just before needs wait states, which the compiler
+                // cannot insert for inline assembly: the matrix instruction then reads the register's old value).
+                // The empty asm emits nothing: it hides the nibble masks from the optimiser, which otherwise turns
+                // each byte conversion into a bit-field extract plus a conversion instead of one v_cvt_f32_ubyteN.
+                // Program order is pinned so that the conversions of code dword i + 1 sit between the matrix
+                // instructions of dword i: each operand is written a dword ahead of its use.
                 float cl[2][4], ch[2][4];
                 auto convert = [&](int set, int t, uint32_t l4, uint32_t h4) __attribute__((always_inline)) {
                     cl[set][t] = t == 0 ? (float)(l4 & 0xFFu) : t == 1 ? (float)((l4 >> 8) & 0xFFu) : t == 2 ? (float)((l4 >> 16) & 0xFFu) : (float)(l4 >> 24);
