@@ -276,12 +276,13 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
 #pragma clang loop unroll(full)
         for (int q = 0; q < N_MFMA; ++q) {
             const int kk = q / (4 * G_WTN), r = q % (4 * G_WTN), i = r / G_WTN, j = r % G_WTN, set = kk & 1;
-            if (r == 0 && kk + 1 < GK / 16) {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (r == 0 && kk + 1 < GK / 16) {                   // behind the slice's first MFMA: its wait covers only its own reads
                 frags(set ^ 1, 16 * (kk + 1));
                 __builtin_amdgcn_sched_barrier(0);
             }
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+
             if (q < N_PARTS * PSTRIDE && q % PSTRIDE == PSTRIDE - 1) {
                 const int item = q / PSTRIDE;
                 wp[item / 8][item % 8] = decode_part_at(item % 8, wring[slot_next][item / 8], dc[item / 8]);
