@@ -15,10 +15,15 @@ import numpy as np
 
 MASK64 = (1 << 64) - 1
 
-# (block_size, bytes_per_block, byte offset of the fp16 `d`, byte offset of a second fp16 or None)
+# (block_size, bytes_per_block, byte offset of the fp16 `d`, byte offset of a second fp16 or None); the second fp16 is
+# `dMin` for the K-quants and `m` for Q5_1 (GoldenSupport.kt:50, :61-66)
 PACKED = {
+    "Q4_0": (32, 18, 0, None),
+    "Q5_0": (32, 22, 0, None),
+    "Q5_1": (32, 24, 0, 2),
     "Q8_0": (32, 34, 0, None),
     "Q4_K": (256, 144, 0, 2),
+    "Q5_K": (256, 176, 0, 2),
     "Q6_K": (256, 210, 208, None),
 }
 
@@ -66,10 +71,10 @@ def block(enc: str, rng: Rng) -> bytes:
     b = bytearray(rng.next_byte() for _ in range(nbytes))
     d = np.float32(rng.next_float() * np.float32(0.045) + np.float32(0.005))
     d_min = np.float32(rng.next_float() * np.float32(0.02) + np.float32(0.005))
-    rng.next_signed()  # `m`, drawn for every encoding, used only by Q5_1
+    m = np.float32(rng.next_signed() * np.float32(0.5))  # drawn for every encoding, used only by Q5_1
     b[d_off:d_off + 2] = struct.pack("<H", half_trunc(d))
     if d2_off is not None:
-        b[d2_off:d2_off + 2] = struct.pack("<H", half_trunc(d_min))
+        b[d2_off:d2_off + 2] = struct.pack("<H", half_trunc(m if enc == "Q5_1" else d_min))
     return bytes(b)
 
 

@@ -52,13 +52,14 @@ def oracle(fast: bool = False) -> C.CDLL:
     lib.orc_half_to_float.restype = C.c_float
     lib.orc_float_to_half.argtypes = [C.c_float]
     lib.orc_float_to_half.restype = C.c_uint32
-    for n in ("q8_0", "q4k", "q6k"):
+    for n in ("q8_0", "q4k", "q6k", "q4_0", "q5_0", "q5_1", "q5k"):
         f = getattr(lib, f"orc_dequant_{n}")
         f.argtypes = [_u8p, C.c_int64, _f32p]
         f.restype = None
         f = getattr(lib, f"orc_{n}_matmul")
         f.argtypes = _GEMV_ARGS + [C.c_int32]
         f.restype = None
+    for n in ("q8_0", "q4k", "q6k"):
         f = getattr(lib, f"orc_native_{n}_matmul_rm")
         f.argtypes = _GEMV_ARGS
         f.restype = None
@@ -111,8 +112,9 @@ def ref():
 
 # ---------------------------------------------------------------- numpy-level helpers
 
-BLOCK = {"Q8_0": (32, 34), "Q4_K": (256, 144), "Q6_K": (256, 210)}
-_SHORT = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k"}
+BLOCK = {"Q8_0": (32, 34), "Q4_K": (256, 144), "Q6_K": (256, 210), "Q4_0": (32, 18), "Q5_0": (32, 22), "Q5_1": (32, 24),
+         "Q5_K": (256, 176)}
+_SHORT = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k", "Q4_0": "q4_0", "Q5_0": "q5_0", "Q5_1": "q5_1", "Q5_K": "q5k"}
 
 
 def dequant(enc: str, w: np.ndarray) -> np.ndarray:

@@ -17,6 +17,10 @@
  *   [Q80M]   skainet-backends/skainet-backend-cpu/src/commonMain/kotlin/sk/ainet/exec/kernel/ScalarQ8_0MatmulKernel.kt:27-66
  *   [Q4KM]   .../exec/kernel/ScalarQ4_KMatmulKernel.kt:21-80
  *   [Q6KM]   .../exec/kernel/ScalarQ6_KMatmulKernel.kt:21-86
+ *   [Q40D]   .../lang/tensor/data/Q4_0TensorData.kt:93-107, [Q50D] Q5_0TensorData.kt:68-86, [Q51D] Q5_1TensorData.kt:73-92,
+ *   [Q5KD]   Q5_KTensorData.kt:126-142 (decode), :190-219 (scale/min index), :221-236 (code)
+ *   [Q40M]   .../exec/kernel/ScalarQ4_0MatmulKernel.kt:29-63, [Q50M] ScalarQ5_0MatmulKernel.kt, [Q51M] ScalarQ5_1MatmulKernel.kt,
+ *   [Q5KM]   ScalarQ5_KMatmulKernel.kt (all: one `override fun matmul`)
  *   [Q80Q]   skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/data/Q8_0Quantizer.kt:28-53
  *   [FP16E]  skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/types/NarrowFloatCodec.kt:87-130
  *   [SDPA]   skainet-backends/skainet-backend-native-cpu/native/src/f32_fused.c:304-396 and
@@ -32,6 +36,9 @@
  *   orc_half_to_float          all 65536 patterns vs numpy float16 (finite + inf), pinned
  *   orc_dequant_{q8_0,q4k,q6k} reference golden digests decode/Q8_0, decode/Q4_K, decode/Q6_K, pinned
  *   orc_{q8_0,q4k,q6k}_matmul  reference golden digests scalar-matmul and dispatch-bridge, pinned
+ *   orc_dequant_{q4_0,q5_0,q5_1,q5k} and orc_{q4_0,q5_0,q5_1,q5k}_matmul
+ *                              reference golden digests decode/, transpose/, scalar-matmul/, dispatch-bridge/ of
+ *                              Q4_0, Q5_0, Q5_1, Q5_K, pinned
  *   orc_q8_0_quantize          known answers of the reference's Q8_0QuantizerTest + numpy fp16 RNE, pinned
  *   orc_f32_sdpa, rms_norm,    the reference C library compiled from its own sources (oracle/_ref),
  *   softmax, fp32 matmuls      fp64 closed forms and mask-rule invariants, pinned
@@ -101,6 +108,10 @@ ORC_API uint32_t orc_float_to_half(float value) {
 #define QK_BS 256
 #define Q4K_BYTES 144
 #define Q6K_BYTES 210
+#define Q40_BYTES 18
+#define Q50_BYTES 22
+#define Q51_BYTES 24
+#define Q5K_BYTES 176
 
 static inline uint32_t le16(const uint8_t* p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8); }
 
@@ -161,6 +172,71 @@ static void q6k_block(const uint8_t* b, float* out) {
     }
 }
 
+/* [Q40D] low nibbles are elements 0..15, high nibbles 16..31; w = (float)(code - 8) * d */
+static void q4_0_block(const uint8_t* b, float* out) {
+    const float d = orc_half_to_float(le16(b));
+    for (int j = 0; j < 16; ++j) {
+        out[j] = (float)((b[2 + j] & 0x0F) - 8) * d;
+        out[16 + j] = (float)((b[2 + j] >> 4) - 8) * d;
+    }
+}
+
+/* bit j of the 32-bit little-endian high-bit plane at qh */
+static inline int q5_bit(const uint8_t* qh, int j) { return (qh[j >> 3] >> (j & 7)) & 1; }
+
+/* [Q50D] w = d * (float)(code5 - 16) */
+static void q5_0_block(const uint8_t* b, float* out) {
+    const float d = orc_half_to_float(le16(b));
+    const uint8_t *qh = b + 2, *qs = b + 6;
+    for (int j = 0; j < 16; ++j) {
+        out[j] = d * (float)((qs[j] & 0x0F) + (q5_bit(qh, j) << 4) - 16);
+        out[16 + j] = d * (float)((qs[j] >> 4) + (q5_bit(qh, j + 16) << 4) - 16);
+    }
+}
+
+/* [Q51D] w = d * (float)code5 + m: product rounded, then the add */
+static void q5_1_block(const uint8_t* b, float* out) {
+    const float d = orc_half_to_float(le16(b)), m = orc_half_to_float(le16(b + 2));
+    const uint8_t *qh = b + 4, *qs = b + 8;
+    for (int j = 0; j < 16; ++j) {
+        const float lo = d * (float)((qs[j] & 0x0F) + (q5_bit(qh, j) << 4));
+        const float hi = d * (float)((qs[j] >> 4) + (q5_bit(qh, j + 16) << 4));
+        out[j] = lo + m;
+        out[16 + j] = hi + m;
+    }
+}
+
+/* [Q5KD] the Q4_K scale/min packing; element e of 64-element group g: low nibble (e < 32) or high nibble of
+ * qs[g*32 + e%32], fifth bit = bit (2g or 2g+1) of qh[e%32]; w = (float)code * (d*sc) - (dmin*m) */
+static inline int q5k_code(const uint8_t* b, int g, int half, int l) {
+    const int byte = b[48 + g * 32 + l];
+    const int low = half ? (byte >> 4) : (byte & 0x0F);
+    return low | (((b[16 + l] >> (2 * g + half)) & 1) << 4);
+}
+static void q5k_block(const uint8_t* b, float* out) {
+    const float d = orc_half_to_float(le16(b));
+    const float dmin = orc_half_to_float(le16(b + 2));
+    int sc[8], mn[8];
+    q4k_scale_min(b + 4, sc, mn);
+    for (int sb = 0; sb < 8; ++sb) {
+        const float scale = d * (float)sc[sb];
+        const float offset = dmin * (float)mn[sb];
+        for (int j = 0; j < 32; ++j) out[sb * 32 + j] = (float)q5k_code(b, sb >> 1, sb & 1, j) * scale - offset;
+    }
+}
+
+ORC_API void orc_dequant_q4_0(const uint8_t* w, int64_t nblocks, float* out) {
+    for (int64_t b = 0; b < nblocks; ++b) q4_0_block(w + b * Q40_BYTES, out + b * 32);
+}
+ORC_API void orc_dequant_q5_0(const uint8_t* w, int64_t nblocks, float* out) {
+    for (int64_t b = 0; b < nblocks; ++b) q5_0_block(w + b * Q50_BYTES, out + b * 32);
+}
+ORC_API void orc_dequant_q5_1(const uint8_t* w, int64_t nblocks, float* out) {
+    for (int64_t b = 0; b < nblocks; ++b) q5_1_block(w + b * Q51_BYTES, out + b * 32);
+}
+ORC_API void orc_dequant_q5k(const uint8_t* w, int64_t nblocks, float* out) {
+    for (int64_t b = 0; b < nblocks; ++b) q5k_block(w + b * Q5K_BYTES, out + b * QK_BS);
+}
 ORC_API void orc_dequant_q8_0(const uint8_t* w, int64_t nblocks, float* out) {
     for (int64_t b = 0; b < nblocks; ++b) q8_0_block(w + b * Q80_BYTES, out + b * Q80_BS);
 }
@@ -199,6 +275,101 @@ ORC_API void orc_q8_0_matmul(const float* input, int32_t input_offset, const uin
             for (int k = 0; k < Q80_BS; ++k) {
                 const float t = x[k] * (float)codes[k];
                 acc += t * d;
+            }
+        }
+        output[output_offset + o] = acc;
+    }
+}
+
+/* [Q40M] per byte j: acc += (x[j] * lo) * d, then acc += (x[16+j] * hi) * d */
+ORC_API void orc_q4_0_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+                             int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim,
+                             float* output, int32_t output_offset, int32_t row_major) {
+    if (output_dim <= 0) return;
+    const int64_t bpr = input_dim / 32;
+    const uint8_t* w = weight + weight_byte_offset;
+    for (int64_t o = 0; o < output_dim; ++o) {
+        float acc = 0.0f;
+        for (int64_t b = 0; b < bpr; ++b) {
+            const uint8_t* p = blk(w, row_major, b, o, bpr, output_dim, Q40_BYTES);
+            const float d = orc_half_to_float(le16(p));
+            const float* x = input + input_offset + b * 32;
+            for (int j = 0; j < 16; ++j) {
+                const float lo = (float)((p[2 + j] & 0x0F) - 8), hi = (float)((p[2 + j] >> 4) - 8);
+                const float t0 = x[j] * lo;
+                acc += t0 * d;
+                const float t1 = x[16 + j] * hi;
+                acc += t1 * d;
+            }
+        }
+        output[output_offset + o] = acc;
+    }
+}
+
+/* [Q50M] / [Q51M] per byte j: wLo, wHi decoded as in the block decoders; acc += (x[j]*wLo + x[16+j]*wHi) */
+static void q5_01_matmul(const float* input, int32_t input_offset, const uint8_t* weight, int32_t weight_byte_offset,
+                         int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset, int32_t row_major,
+                         int is_q5_1) {
+    if (output_dim <= 0) return;
+    const int bytes = is_q5_1 ? Q51_BYTES : Q50_BYTES;
+    const int64_t bpr = input_dim / 32;
+    const uint8_t* w = weight + weight_byte_offset;
+    float dec[32];
+    for (int64_t o = 0; o < output_dim; ++o) {
+        float acc = 0.0f;
+        for (int64_t b = 0; b < bpr; ++b) {
+            const uint8_t* p = blk(w, row_major, b, o, bpr, output_dim, bytes);
+            if (is_q5_1) q5_1_block(p, dec); else q5_0_block(p, dec);
+            const float* x = input + input_offset + b * 32;
+            for (int j = 0; j < 16; ++j) {
+                const float a = x[j] * dec[j];
+                const float c = x[16 + j] * dec[16 + j];
+                acc += a + c;
+            }
+        }
+        output[output_offset + o] = acc;
+    }
+}
+ORC_API void orc_q5_0_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+                             int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim,
+                             float* output, int32_t output_offset, int32_t row_major) {
+    q5_01_matmul(input, input_offset, weight, weight_byte_offset, input_dim, output_dim, output, output_offset, row_major, 0);
+}
+ORC_API void orc_q5_1_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+                             int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim,
+                             float* output, int32_t output_offset, int32_t row_major) {
+    q5_01_matmul(input, input_offset, weight, weight_byte_offset, input_dim, output_dim, output, output_offset, row_major, 1);
+}
+
+/* [Q5KM] the Q4_K kernel's shape with 5-bit codes: per sub-block codeSum, inputSum; acc += codeSum*(d*sc) - inputSum*(dmin*m) */
+ORC_API void orc_q5k_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+                            int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim,
+                            float* output, int32_t output_offset, int32_t row_major) {
+    if (output_dim <= 0) return;
+    const int64_t bpr = input_dim / QK_BS;
+    const uint8_t* w = weight + weight_byte_offset;
+    for (int64_t o = 0; o < output_dim; ++o) {
+        float acc = 0.0f;
+        for (int64_t b = 0; b < bpr; ++b) {
+            const uint8_t* p = blk(w, row_major, b, o, bpr, output_dim, Q5K_BYTES);
+            const float d = orc_half_to_float(le16(p));
+            const float dmin = orc_half_to_float(le16(p + 2));
+            int sc[8], mn[8];
+            q4k_scale_min(p + 4, sc, mn);
+            const float* x = input + input_offset + b * QK_BS;
+            for (int g = 0; g < 4; ++g) {
+                for (int half = 0; half < 2; ++half) {
+                    const int sb = 2 * g + half;
+                    float code_sum = 0.0f, input_sum = 0.0f;
+                    for (int i = 0; i < 32; ++i) {
+                        const float v = x[sb * 32 + i];
+                        code_sum += v * (float)q5k_code(p, g, half, i);
+                        input_sum += v;
+                    }
+                    const float a = code_sum * (d * (float)sc[sb]);
+                    const float c = input_sum * (dmin * (float)mn[sb]);
+                    acc += a - c;
+                }
             }
         }
         output[output_offset + o] = acc;

@@ -15,7 +15,8 @@ from oracle import lib as L
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDENS = json.load(open(os.path.join(HERE, "golden", "reference_goldens.json")))
-ENCS = ["Q8_0", "Q4_K", "Q6_K"]
+ENCS = ["Q8_0", "Q4_K", "Q6_K", "Q4_0", "Q5_0", "Q5_1", "Q5_K"]
+NATIVE_ENCS = ["Q8_0", "Q4_K", "Q6_K"]          # the formats the reference's native C library covers
 
 
 # ---- fp16 ----------------------------------------------------------------------------------------------
@@ -232,7 +233,7 @@ def test_softmax_and_dense_matmuls_against_numpy():
 
 
 # ---- the int8-activation port against the reference-built library -----------------------------------------
-@pytest.mark.parametrize("enc", ENCS)
+@pytest.mark.parametrize("enc", NATIVE_ENCS)
 def test_native_port_is_bit_identical_to_the_reference_library(enc):
     ref = L.ref()
     vec_path = os.path.join(HERE, "golden", "ref_vectors.npz")
