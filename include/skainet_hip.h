@@ -38,8 +38,12 @@ extern "C" {
 
 /* Weight encodings: the GGML tensor-type ids StreamingGGUFReader maps to TensorEncoding
  * (REF/../skainet-io/skainet-io-gguf/src/commonMain/kotlin/sk/ainet/io/gguf/StreamingGGUFReader.kt:190-211). */
+#define SKAINET_HIP_ENC_Q4_0 2
+#define SKAINET_HIP_ENC_Q5_0 6
+#define SKAINET_HIP_ENC_Q5_1 7
 #define SKAINET_HIP_ENC_Q8_0 8
 #define SKAINET_HIP_ENC_Q4_K 12
+#define SKAINET_HIP_ENC_Q5_K 13
 #define SKAINET_HIP_ENC_Q6_K 14
 
 /* Block orders of a packed weight (REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/memory/Layout.kt:21-27). */
@@ -139,7 +143,8 @@ SKAINET_HIP_API float skainet_hip_read_probe_dev(const void* const* buffers, int
     int32_t iters, int32_t grid);
 /* Bit-exact decode of the whole weight to fp32 [rows, cols] (the TensorData.dequantizeBlock semantics,
  * REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/data/Q4_KTensorData.kt:120,
- * Q6_KTensorData.kt:112, Q8_0TensorData.kt:80). */
+ * Q6_KTensorData.kt:112, Q8_0TensorData.kt:80, Q4_0TensorData.kt:93, Q5_0TensorData.kt:68, Q5_1TensorData.kt:73,
+ * Q5_KTensorData.kt:126). */
 SKAINET_HIP_API int32_t skainet_hip_dequantize_dev(const skainet_hip_weight* w, float* out);
 /* Decode `count` rows picked by `row_ids` (device int32) into out[count, cols]: the packed embedding
  * lookup (RowDequantSource.dequantRow, .../tensor/data/Q8_0TensorData.kt:91-100). */
@@ -164,6 +169,26 @@ SKAINET_HIP_API void skainet_hip_q6k_matmul_rm(const float* input, int32_t input
 SKAINET_HIP_API void skainet_hip_q8_0_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
 SKAINET_HIP_API void skainet_hip_q8_0_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+/* The remaining packed formats of the provider SPI (API/KernelProvider.kt:74-104): Q4_0MatmulKernel.matmul
+ * (API/Q4_0MatmulKernel.kt:40), Q5_0MatmulKernel.matmul (API/Q5_0MatmulKernel.kt:37), Q5_1MatmulKernel.matmul
+ * (API/Q5_1MatmulKernel.kt:47), Q5KMatmulKernel.matmul (API/Q5KMatmulKernel.kt:53). The reference has no native C
+ * twin for these; the signatures follow the ones above. Plain name: input-block-major weight, `_rm`: canonical order. */
+SKAINET_HIP_API void skainet_hip_q4_0_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q4_0_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q5_0_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q5_0_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q5_1_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q5_1_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q5k_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
+    int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+SKAINET_HIP_API void skainet_hip_q5k_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
 
 /* NAT:271 skainet_fp32_matmul (Fp32MatmulKernel.matmul, API/Fp32MatmulKernel.kt:25-50): C(m,n) = A(m,k) B(k,n),

@@ -54,6 +54,14 @@ SIGNATURES = {
     "skainet_hip_q6k_matmul_rm": (None, _GEMV),
     "skainet_hip_q8_0_matmul": (None, _GEMV),
     "skainet_hip_q8_0_matmul_rm": (None, _GEMV),
+    "skainet_hip_q4_0_matmul": (None, _GEMV),
+    "skainet_hip_q4_0_matmul_rm": (None, _GEMV),
+    "skainet_hip_q5_0_matmul": (None, _GEMV),
+    "skainet_hip_q5_0_matmul_rm": (None, _GEMV),
+    "skainet_hip_q5_1_matmul": (None, _GEMV),
+    "skainet_hip_q5_1_matmul_rm": (None, _GEMV),
+    "skainet_hip_q5k_matmul": (None, _GEMV),
+    "skainet_hip_q5k_matmul_rm": (None, _GEMV),
     "skainet_hip_fp32_matmul": (None, _SGEMM),
     "skainet_hip_fp32_matmul_wt": (None, _SGEMM_WT),
     "skainet_hip_f32_rms_norm": (None, [_vp, _vp, _vp, _i32, _i32, _f32]),

@@ -10,14 +10,27 @@ namespace skh {
 // /root/reference/skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/memory/BlockSpec.kt:84-87
 constexpr int Q80_ELEMS = 32, Q80_BYTES = 34;
 constexpr int QK_ELEMS = 256, Q4K_BYTES = 144, Q6K_BYTES = 210;
+constexpr int Q40_BYTES = 18, Q50_BYTES = 22, Q51_BYTES = 24, Q5K_BYTES = 176;   // Q4_0 / Q5_0 / Q5_1: 32 elements; Q5_K: 256
 
 // Encoding ids are the GGML tensor-type numbers the GGUF reader maps from
 // (/root/reference/skainet-io/skainet-io-gguf/src/commonMain/kotlin/sk/ainet/io/gguf/StreamingGGUFReader.kt:190-211).
-enum Encoding : int32_t { ENC_F32 = 0, ENC_Q8_0 = 8, ENC_Q4_K = 12, ENC_Q6_K = 14 };
+enum Encoding : int32_t { ENC_F32 = 0, ENC_Q4_0 = 2, ENC_Q5_0 = 6, ENC_Q5_1 = 7, ENC_Q8_0 = 8, ENC_Q4_K = 12, ENC_Q5_K = 13, ENC_Q6_K = 14 };
 
-inline int block_elems(int enc) { return enc == ENC_Q8_0 ? Q80_ELEMS : QK_ELEMS; }
-inline int block_bytes(int enc) { return enc == ENC_Q8_0 ? Q80_BYTES : (enc == ENC_Q4_K ? Q4K_BYTES : Q6K_BYTES); }
-inline bool is_packed(int enc) { return enc == ENC_Q8_0 || enc == ENC_Q4_K || enc == ENC_Q6_K; }
+inline bool is_packed(int enc) {
+    return enc == ENC_Q8_0 || enc == ENC_Q4_K || enc == ENC_Q6_K || enc == ENC_Q4_0 || enc == ENC_Q5_0 || enc == ENC_Q5_1 || enc == ENC_Q5_K;
+}
+inline int block_elems(int enc) { return (enc == ENC_Q4_K || enc == ENC_Q5_K || enc == ENC_Q6_K) ? QK_ELEMS : Q80_ELEMS; }
+inline int block_bytes(int enc) {
+    switch (enc) {
+        case ENC_Q4_0: return Q40_BYTES;
+        case ENC_Q5_0: return Q50_BYTES;
+        case ENC_Q5_1: return Q51_BYTES;
+        case ENC_Q8_0: return Q80_BYTES;
+        case ENC_Q4_K: return Q4K_BYTES;
+        case ENC_Q5_K: return Q5K_BYTES;
+        default: return Q6K_BYTES;
+    }
+}
 
 // ---- error plumbing (shim.hip owns the storage) ----
 int set_error(const char* fmt, ...);          // records a thread-local message, returns -1

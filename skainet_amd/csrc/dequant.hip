@@ -1,10 +1,14 @@
-// Bit-exact GGUF block decode on the device: packed Q8_0 / Q4_K / Q6_K bytes -> fp32.
+// Bit-exact GGUF block decode on the device: packed Q8_0 / Q4_K / Q6_K (and Q4_0 / Q5_0 / Q5_1 / Q5_K) bytes -> fp32.
 //
 // Every product and difference is rounded exactly where the reference decoders round
 // (explicit __fmul_rn / __fsub_rn, never an FMA), so the output bits equal
 //   Q8_0: (float)code * d                         Q8_0TensorData.kt:80-89
 //   Q4_K: code * (d * scaleIdx) - (dmin * minIdx)  Q4_KTensorData.kt:120-136, :184-206, :215-226
 //   Q6_K: (d * sc) * q,  q = 6-bit code - 32       Q6_KTensorData.kt:112-165
+//   Q4_0: (float)(code - 8) * d                    Q4_0TensorData.kt:93-107 (low nibbles: elements 0..15, high: 16..31)
+//   Q5_0: d * (float)(code5 - 16)                  Q5_0TensorData.kt:68-86  (fifth bit j of the 32-bit plane `qh`)
+//   Q5_1: d * (float)code5 + m                     Q5_1TensorData.kt:73-92
+//   Q5_K: code5 * (d * scaleIdx) - (dmin * minIdx)  Q5_KTensorData.kt:126-142, :190-236
 // (paths under /root/reference/skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/data/).
 //
 // HBM-bound: one thread decodes 8 (Q8_0: all 32 of a block per 4 threads) consecutive outputs and
@@ -111,17 +115,85 @@ __global__ __launch_bounds__(256) void dequant_q6k_kernel(const uint8_t* __restr
     o[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
 
+// Q4_0 / Q5_0 / Q5_1: 32-element blocks of 18 / 22 / 24 bytes (fp16 d [, fp16 m] [, 4 bytes of fifth bits], 16 bytes of
+// nibbles). One thread per 8 output elements, 4 threads per block: part p < 2 decodes the low nibbles of bytes
+// 8p .. 8p+7, part p >= 2 the high nibbles of bytes 8(p-2) .. 8(p-2)+7. FMT: 0 = Q4_0, 1 = Q5_0, 2 = Q5_1.
+template <int FMT>
+__global__ __launch_bounds__(256) void dequant_q45_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
+                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr) {
+    constexpr int BYTES = FMT == 0 ? Q40_BYTES : (FMT == 1 ? Q50_BYTES : Q51_BYTES);
+    constexpr int QH = FMT == 2 ? 4 : 2, QS = FMT == 0 ? 2 : QH + 4;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t b = t >> 2;
+    if (b >= nblocks) return;
+    const int part = (int)(t & 3), byte0 = (part & 1) * 8, shift = (part >> 1) * 4;
+    const uint8_t* p = w + source_block(b, row_ids, bpr) * BYTES;
+    const float d = half_bits_to_float(load_u16(p));
+    float m = 0.f;
+    uint32_t qh = 0;
+    if (FMT == 2) m = half_bits_to_float(load_u16(p + 2));
+    if (FMT != 0) qh = load_u16(p + QH) | (load_u16(p + QH + 2) << 16);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int j = byte0 + i;                                  // byte of the block's nibble plane; element j or 16 + j
+        int code = (p[QS + j] >> shift) & 0xF;
+        if (FMT != 0) code |= (int)((qh >> (part * 8 + i)) & 1u) << 4;
+        if (FMT == 0) v[i] = __fmul_rn((float)(code - 8), d);
+        else if (FMT == 1) v[i] = __fmul_rn(d, (float)(code - 16));
+        else v[i] = __fadd_rn(__fmul_rn(d, (float)code), m);
+    }
+    float4* o = reinterpret_cast<float4*>(out + b * Q80_ELEMS + part * 8);
+    o[0] = make_float4(v[0], v[1], v[2], v[3]);
+    o[1] = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+// Q5_K: the Q4_K layout with a 32-byte plane of fifth bits at byte 16 and the nibbles at byte 48 (176 bytes). Thread
+// u of 32: sub-block sb = u / 4, elements [8 * (u % 4), +8): bytes e0 .. e0+7 of nibble group sb / 2, bit sb of qh[e0 ..].
+__global__ __launch_bounds__(256) void dequant_q5k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
+                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t b = t >> 5;
+    if (b >= nblocks) return;
+    const int u = (int)(t & 31), sb = u >> 2, e0 = (u & 3) * 8;
+    const uint8_t* p = w + source_block(b, row_ids, bpr) * Q5K_BYTES;
+    const uint32_t dd = *reinterpret_cast<const uint32_t*>(p);
+    const float d = half_bits_to_float(dd & 0xFFFFu), dmin = half_bits_to_float(dd >> 16);
+    int sc, mn;
+    q4k_scale_min(p + 4, sb, sc, mn);
+    const float scale = __fmul_rn(d, (float)sc);
+    const float offset = __fmul_rn(dmin, (float)mn);
+    const uint2 q = *reinterpret_cast<const uint2*>(p + 48 + (sb >> 1) * 32 + e0);
+    const uint2 h = *reinterpret_cast<const uint2*>(p + 16 + e0);
+    const int shift = (sb & 1) * 4;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t c0 = ((q.x >> (8 * i + shift)) & 0xF) | (((h.x >> (8 * i + sb)) & 1u) << 4);
+        const uint32_t c1 = ((q.y >> (8 * i + shift)) & 0xF) | (((h.y >> (8 * i + sb)) & 1u) << 4);
+        v[i] = __fsub_rn(__fmul_rn((float)c0, scale), offset);
+        v[4 + i] = __fsub_rn(__fmul_rn((float)c1, scale), offset);
+    }
+    float4* o = reinterpret_cast<float4*>(out + b * QK_ELEMS + sb * 32 + e0);
+    o[0] = make_float4(v[0], v[1], v[2], v[3]);
+    o[1] = make_float4(v[4], v[5], v[6], v[7]);
+}
+
 // Decodes `nblocks` consecutive output blocks; with `row_ids` (device int32) output row r is source row row_ids[r]
 // of a weight with `bpr` blocks per row.
 int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr) {
     if (nblocks <= 0) return 0;
     if (!is_packed(enc)) return set_error("dequantize: unsupported encoding %d", enc);
     hipStream_t s = current_stream();
-    const int64_t threads = nblocks * (enc == ENC_Q8_0 ? 4 : 32);
+    const int64_t threads = nblocks * (block_elems(enc) / 8);
     const int64_t grid = (threads + 255) / 256;
     if (grid > 0x7FFFFFFFLL) return set_error("dequantize: %lld blocks exceed one launch", (long long)nblocks);
     if (enc == ENC_Q8_0) dequant_q8_0_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
     else if (enc == ENC_Q4_K) dequant_q4k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
+    else if (enc == ENC_Q5_K) dequant_q5k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
+    else if (enc == ENC_Q4_0) dequant_q45_kernel<0><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
+    else if (enc == ENC_Q5_0) dequant_q45_kernel<1><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
+    else if (enc == ENC_Q5_1) dequant_q45_kernel<2><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
     else dequant_q6k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
     SKH_CHECK(hipGetLastError());
     return 0;

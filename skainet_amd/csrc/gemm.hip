@@ -373,7 +373,9 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     // shapes the tile loader cannot take (a Q8_0 row that is not a whole number of 256-element groups: the K loop
     // runs pairs of 64-element steps over whole groups; unaligned operands) go through the row kernels: same result
     // to fp32 rounding, the weight streamed once per 4 rows
-    if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15))
+    // (so do the formats the tile loader has no decoder for: Q4_0, Q5_0, Q5_1, Q5_K)
+    if ((enc != ENC_Q4_K && enc != ENC_Q6_K && enc != ENC_Q8_0) || k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) ||
+        (reinterpret_cast<uintptr_t>(x) & 15))
         return launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
     const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;

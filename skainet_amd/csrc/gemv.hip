@@ -214,9 +214,129 @@ struct Q80Slot {
     }
 };
 
+// ------------------------------------------------------------------------------- Q4_0 / Q5_0 / Q5_1
+// 32-element blocks: fp16 d [fp16 m] [32 fifth bits] 16 bytes of nibbles (low nibbles: elements 0..15, high: 16..31).
+// Semantics of ScalarQ4_0MatmulKernel.kt:29-63, ScalarQ5_0MatmulKernel.kt, ScalarQ5_1MatmulKernel.kt (same directory as
+// the kernels cited at the top) with the code bias and the Q5_1 minimum taken out of the inner loop:
+//   Q4_0  d * (sum code x - 8 sum x)     Q5_0  d * (sum code5 x - 16 sum x)     Q5_1  d * sum code5 x + m * sum x
+// The fifth bits of four adjacent elements are spread into bit 4 of the four code bytes with one multiply.
+template <int FMT>   // 0 = Q4_0, 1 = Q5_0, 2 = Q5_1
+struct Q45Slot {
+    static constexpr int BLOCK_BYTES = FMT == 0 ? Q40_BYTES : (FMT == 1 ? Q50_BYTES : Q51_BYTES);
+    static constexpr int SLOTS_PER_BLOCK = 1, SLOT_ELEMS = 32, NX = 32;
+    static constexpr int QH = FMT == 2 ? 4 : 2, QS = FMT == 0 ? 2 : QH + 4;
+    struct Raw { uint32_t d, m, qh, q[4]; };
+    struct Lane { int blk_off; };
+    __device__ static void init(Lane& ln, int slot) { ln.blk_off = slot * BLOCK_BYTES; }
+    __device__ static int x_index(int slot, int i) { return slot * 32 + i; }
+    __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
+        const uint8_t* p = row + ln.blk_off;                  // 2-byte aligned (Q5_1: 8)
+        r.d = load_u16(p);
+        r.m = FMT == 2 ? load_u16(p + 2) : 0u;
+        r.qh = FMT != 0 ? load_u32_a2(p + QH) : 0u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r.q[i] = load_u32_a2(p + QS + 4 * i);
+    }
+    __device__ static void prep(const float* x, float* xsum) {
+        float a = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) a += x[i];
+        xsum[0] = a;
+    }
+    template <int B>
+    __device__ static void dot(const Raw& r, const Lane&, const float (*x)[NX], const float (*xsum)[1], float* acc) {
+        const float d = half_bits_to_float_fast(r.d);
+        float s[B];
+#pragma unroll
+        for (int b = 0; b < B; ++b) s[b] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t l4 = r.q[i] & 0x0F0F0F0Fu, h4 = (r.q[i] >> 4) & 0x0F0F0F0Fu;
+            if (FMT != 0) {
+                l4 |= ((((r.qh >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+                h4 |= ((((r.qh >> (16 + 4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+            }
+            const float cl[4] = {ubyte0_to_float(l4), ubyte1_to_float(l4), ubyte2_to_float(l4), ubyte3_to_float(l4)};
+            const float ch[4] = {ubyte0_to_float(h4), ubyte1_to_float(h4), ubyte2_to_float(h4), ubyte3_to_float(h4)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    s[b] = fmaf(x[b][i * 4 + j], cl[j], s[b]);
+                    s[b] = fmaf(x[b][16 + i * 4 + j], ch[j], s[b]);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            if (FMT == 0) acc[b] = d * (s[b] - 8.f * xsum[b][0]);
+            else if (FMT == 1) acc[b] = d * (s[b] - 16.f * xsum[b][0]);
+            else acc[b] = d * s[b] + half_bits_to_float_fast(r.m) * xsum[b][0];
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------- Q5_K
+// The Q4_K slot (one 16-byte nibble chunk = 16 + 16 elements of sub-blocks 2g and 2g + 1) plus the matching 16 bytes
+// of the fifth-bit plane: bit 2g of byte l belongs to element l of sub-block 2g, bit 2g + 1 to sub-block 2g + 1.
+// Block: d, dmin, 12 scale bytes, 32 bytes qh at 16, 128 bytes of nibbles at 48 (176 bytes);
+// semantics of ScalarQ5_KMatmulKernel.kt (per sub-block codeSum * (d * sc) - inputSum * (dmin * m)).
+struct Q5KSlot {
+    static constexpr int BLOCK_BYTES = Q5K_BYTES, SLOTS_PER_BLOCK = 8, SLOT_ELEMS = 32, NX = 32;
+    struct Raw { uint4 hdr, qs, qh; };
+    struct Lane { int blk_off, qs_off, qh_off, sh, bit; uint32_t hi_mask; };
+    __device__ static void init(Lane& ln, int slot) {
+        const int blk = slot >> 3, c = slot & 7;
+        ln.blk_off = blk * BLOCK_BYTES;
+        ln.qs_off = ln.blk_off + 48 + c * 16;
+        ln.qh_off = ln.blk_off + 16 + (c & 1) * 16;
+        ln.sh = ((c >> 1) & 1) * 16;
+        ln.bit = 2 * (c >> 1);
+        ln.hi_mask = (c >> 1) >= 2 ? 0xFFFFFFFFu : 0u;
+    }
+    __device__ static int x_index(int slot, int i) { return Q4KSlot::x_index(slot, i); }
+    __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
+        r.hdr = *reinterpret_cast<const uint4*>(row + ln.blk_off);
+        r.qs = *reinterpret_cast<const uint4*>(row + ln.qs_off);
+        r.qh = *reinterpret_cast<const uint4*>(row + ln.qh_off);
+    }
+    __device__ static void prep(const float* x, float* xsum) { Q4KSlot::prep(x, xsum); }
+    template <int B>
+    __device__ static void dot(const Raw& r, const Lane& ln, const float (*x)[NX], const float (*xsum)[2], float* acc) {
+        Q4KSlot::Raw r4{r.hdr, r.qs};
+        Q4KSlot::Lane l4{0, 0, ln.sh, ln.hi_mask};
+        const Q4KSlot::Scales s = Q4KSlot::scales(r4, l4);      // dhi carries the 1/16 of a high nibble kept in place
+        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+        const uint32_t h[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+        float lo[B], hi[B];
+#pragma unroll
+        for (int b = 0; b < B; ++b) lo[b] = hi[b] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t hb = h[i] >> ln.bit;
+            const uint32_t l5 = (q[i] & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4);
+            const uint32_t h5 = ((q[i] >> 4) & 0x0F0F0F0Fu) | (((hb >> 1) & 0x01010101u) << 4);
+            const float cl[4] = {ubyte0_to_float(l5), ubyte1_to_float(l5), ubyte2_to_float(l5), ubyte3_to_float(l5)};
+            const float ch[4] = {ubyte0_to_float(h5), ubyte1_to_float(h5), ubyte2_to_float(h5), ubyte3_to_float(h5)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    lo[b] = fmaf(x[b][i * 4 + j], cl[j], lo[b]);
+                    hi[b] = fmaf(x[b][16 + i * 4 + j], ch[j], hi[b]);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b)
+            acc[b] = s.dlo * lo[b] + 16.f * s.dhi * hi[b] - (s.mlo * xsum[b][0] + s.mhi * xsum[b][1]);
+    }
+};
+
 template <class F> struct XSumCount { static constexpr int N = 1; };
 template <> struct XSumCount<Q4KSlot> { static constexpr int N = 2; };
 template <> struct XSumCount<Q6KSlot> { static constexpr int N = 4; };
+template <> struct XSumCount<Q5KSlot> { static constexpr int N = 2; };
 
 // F: slot policy, B: activation rows per launch (1, 2 or 4; unused ones are zero), R: weight rows in flight.
 template <class F, int B, int R>
@@ -352,7 +472,7 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (!is_packed(enc)) return set_error("gemv: unsupported encoding %d", enc);
     if (k <= 0 || k % block_elems(enc) != 0)
         return set_error("gemv: inputDim must be a positive multiple of %d; got %d", block_elems(enc), k);
-    const int waves_per_cu = g_gemv_waves_per_cu > 0 ? g_gemv_waves_per_cu : (enc == ENC_Q8_0 ? 4 : 8);
+    const int waves_per_cu = g_gemv_waves_per_cu > 0 ? g_gemv_waves_per_cu : (block_elems(enc) == 32 ? 4 : 8);
     for (int b0 = 0; b0 < m;) {
         const int left = m - b0;
         const float* xb = x + (int64_t)b0 * k;
@@ -368,6 +488,10 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
         const int nb = left < 4 ? left : 4;
         if (enc == ENC_Q4_K) rc = launch_format<Q4KSlot>(w, xb, yb, k, n, nb, waves_per_cu);
         else if (enc == ENC_Q6_K) rc = launch_format<Q6KSlot>(w, xb, yb, k, n, nb, waves_per_cu);
+        else if (enc == ENC_Q5_K) rc = launch_format<Q5KSlot>(w, xb, yb, k, n, nb, waves_per_cu);
+        else if (enc == ENC_Q4_0) rc = launch_format<Q45Slot<0>>(w, xb, yb, k, n, nb, waves_per_cu);
+        else if (enc == ENC_Q5_0) rc = launch_format<Q45Slot<1>>(w, xb, yb, k, n, nb, waves_per_cu);
+        else if (enc == ENC_Q5_1) rc = launch_format<Q45Slot<2>>(w, xb, yb, k, n, nb, waves_per_cu);
         else rc = launch_format<Q80Slot>(w, xb, yb, k, n, nb, waves_per_cu);
         if (rc != 0) return rc;
         b0 += nb;

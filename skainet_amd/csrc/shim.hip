@@ -616,6 +616,10 @@ static void packed_matmul_host(int enc, int order, const float* input, int32_t i
 SKH_PACKED_ENTRY(q4k, ENC_Q4_K)
 SKH_PACKED_ENTRY(q6k, ENC_Q6_K)
 SKH_PACKED_ENTRY(q8_0, ENC_Q8_0)
+SKH_PACKED_ENTRY(q4_0, ENC_Q4_0)
+SKH_PACKED_ENTRY(q5_0, ENC_Q5_0)
+SKH_PACKED_ENTRY(q5_1, ENC_Q5_1)
+SKH_PACKED_ENTRY(q5k, ENC_Q5_K)
 
 void skainet_hip_fp32_matmul(const float* a, int32_t a_offset, int32_t a_stride, const float* b, int32_t b_offset,
                              int32_t b_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k) {

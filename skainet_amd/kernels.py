@@ -30,7 +30,8 @@ from . import _lib
 from ._lib import HipError, check
 
 # TensorEncoding.name -> (C ABI id, block elements, bytes per block)
-ENCODINGS = {"Q8_0": (8, 32, 34), "Q4_K": (12, 256, 144), "Q6_K": (14, 256, 210)}
+ENCODINGS = {"Q8_0": (8, 32, 34), "Q4_K": (12, 256, 144), "Q6_K": (14, 256, 210),
+             "Q4_0": (2, 32, 18), "Q5_0": (6, 32, 22), "Q5_1": (7, 32, 24), "Q5_K": (13, 256, 176)}
 ORDER_ROW_MAJOR, ORDER_INPUT_BLOCK_MAJOR = 0, 1
 
 PRIORITY_SCALAR, PRIORITY_PANAMA, PRIORITY_NATIVE = 0, 50, 100   # KernelProvider.kt:15-17
@@ -357,12 +358,13 @@ def _raise_if_failed(before: bytes, what: str) -> None:
 
 
 class HipPackedMatmulKernel:
-    """Q4KMatmulKernel / Q6KMatmulKernel / Q8_0MatmulKernel: one activation row times an input-block-major weight."""
+    """Q4KMatmulKernel / Q6KMatmulKernel / Q8_0MatmulKernel (and the Q4_0 / Q5_0 / Q5_1 / Q5_K ones): one activation row
+    times an input-block-major weight."""
 
     def __init__(self, encoding: str):
         self.encoding = encoding
         self._id, self.block_size, self.bytes_per_block = ENCODINGS[encoding]
-        short = {"Q4_K": "q4k", "Q6_K": "q6k", "Q8_0": "q8_0"}[encoding]
+        short = {"Q4_K": "q4k", "Q6_K": "q6k", "Q8_0": "q8_0", "Q4_0": "q4_0", "Q5_0": "q5_0", "Q5_1": "q5_1", "Q5_K": "q5k"}[encoding]
         self._fn_name, self._fn_rm_name = f"skainet_hip_{short}_matmul", f"skainet_hip_{short}_matmul_rm"
 
     def _run(self, fn_name, input, input_offset, weight, weight_byte_offset, input_dim, output_dim, output, output_offset):
@@ -515,6 +517,10 @@ class HipKernelProvider:
     def matmul_q4k(self): return HipPackedMatmulKernel("Q4_K") if is_available() else None
     def matmul_q6k(self): return HipPackedMatmulKernel("Q6_K") if is_available() else None
     def matmul_q8_0(self): return HipPackedMatmulKernel("Q8_0") if is_available() else None
+    def matmul_q4_0(self): return HipPackedMatmulKernel("Q4_0") if is_available() else None
+    def matmul_q5_0(self): return HipPackedMatmulKernel("Q5_0") if is_available() else None
+    def matmul_q5_1(self): return HipPackedMatmulKernel("Q5_1") if is_available() else None
+    def matmul_q5k(self): return HipPackedMatmulKernel("Q5_K") if is_available() else None
     def softmax_fp32(self): return HipFp32SoftmaxKernel() if is_available() else None
     def norm_fp32(self): return HipFp32NormKernel() if is_available() else None
     def attention_fp32(self): return HipFp32AttentionKernel() if is_available() else None
@@ -524,4 +530,4 @@ class HipKernelProvider:
         if op_name != "matmul" or len(dtype_keys) != 2 or not is_available():
             return False
         inp, weight = dtype_keys
-        return inp == "Float32" and weight in ("Float32", "Q4_K", "Q6_K", "Q8_0")
+        return inp == "Float32" and weight in ("Float32", "Q4_K", "Q6_K", "Q8_0", "Q4_0", "Q5_0", "Q5_1", "Q5_K")

@@ -4,7 +4,8 @@ import numpy as np
 from oracle import golden as G
 
 ENCS = ["Q8_0", "Q4_K", "Q6_K"]
-SHORT = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k"}
+MORE_ENCS = ["Q4_0", "Q5_0", "Q5_1", "Q5_K"]          # formats without a quantizer here: tested on seeded valid blocks
+SHORT = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k", "Q4_0": "q4_0", "Q5_0": "q5_0", "Q5_1": "q5_1", "Q5_K": "q5k"}
 
 
 def dev(torch, a):

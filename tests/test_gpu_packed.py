@@ -12,7 +12,7 @@ import pytest
 
 from oracle import golden as G
 from oracle import lib as L
-from gpu_util import ENCS, dev, gaussian_weight, normalized_err, random_valid_blocks
+from gpu_util import ENCS, MORE_ENCS, dev, gaussian_weight, normalized_err, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -198,3 +198,79 @@ def test_spi_kernels_on_host_arrays(hip_backend, torch_cuda, enc):
     vk.run(a, wrm, n, o)
     assert len(vk._cache) == 1
     assert normalized_err(o, L.gemv(enc, a, wrm, n)) <= GEMV_TOL
+
+
+# ---- the remaining packed formats of the provider SPI (Q4_0, Q5_0, Q5_1, Q5_K): same bars, seeded valid blocks ----
+@pytest.mark.parametrize("enc", MORE_ENCS)
+def test_more_formats_decode_reproduces_the_reference_golden_digest_and_is_bit_exact(hip_backend, torch_cuda, enc):
+    bs = G.PACKED[enc][0]
+    blocks = G.weight_blocks(enc, 4, 3, 0x5EED0001)
+    got = gpu_dequant(hip_backend, torch_cuda, enc, G.row_major(blocks), 4, 3 * bs)
+    assert G.digest(got) == GOLDENS[f"decode/{enc}"]
+    for rows, cols, seed in ((7, 2 * bs, 1), (129, 5 * bs, 2), (1024, 4096, 3)):
+        packed = random_valid_blocks(enc, rows * cols // bs, 500 + seed, subnormal_every=7)
+        got = gpu_dequant(hip_backend, torch_cuda, enc, packed, rows, cols)
+        assert np.array_equal(got.view(np.uint32), L.dequant(enc, packed).view(np.uint32))
+    # packed embedding lookup: a gather of rows decodes to those rows
+    rows, cols = 50, 3 * bs
+    packed = random_valid_blocks(enc, rows * cols // bs, 510)
+    w = hip_backend.DeviceWeight.upload(enc, packed, rows, cols)
+    ids = np.array([49, 0, 7, 7, 31], np.int32)
+    out = torch_cuda.empty((len(ids), cols), dtype=torch_cuda.float32, device="cuda")
+    w.dequantize_rows(dev(torch_cuda, ids), len(ids), out)
+    want = L.dequant(enc, packed).reshape(rows, cols)[ids]
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("enc", MORE_ENCS)
+def test_more_formats_gemv_on_the_reference_golden_inputs(hip_backend, torch_cuda, enc):
+    bs = G.PACKED[enc][0]
+    blocks = G.weight_blocks(enc, 4, 3, 0x5EED0002)
+    x = G.floats(3 * 3 * bs, 0x5EED0002 + 100).reshape(3, 3 * bs)
+    want = L.gemv(enc, x, G.row_major(blocks), 4)
+    assert G.digest(want) == GOLDENS[f"scalar-matmul/{enc}"]
+    got_rm = gpu_matmul(hip_backend, torch_cuda, enc, G.row_major(blocks), 4, 3 * bs, x)
+    got_bm = gpu_matmul(hip_backend, torch_cuda, enc, G.block_major(blocks), 4, 3 * bs, x, order=1)
+    assert normalized_err(got_rm, want) <= GEMV_TOL
+    assert np.array_equal(got_rm, got_bm)
+
+
+@pytest.mark.parametrize("enc", MORE_ENCS)
+@pytest.mark.parametrize("n,k,m", [(1, 256, 1), (3, 512, 2), (65, 2048, 4), (130, 2304, 5), (1000, 4096, 1), (257, 11008, 1),
+                                   (40, 16640, 3), (300, 1024, 24)])
+def test_more_formats_gemv_ragged_shapes_and_batches(hip_backend, torch_cuda, enc, n, k, m):
+    """All row counts run exact-fp32 products here (24 rows: the product entry falls back from the tile kernel, which has
+    no decoder for these formats, to the row kernels), so the one-row bound holds throughout."""
+    bs = G.PACKED[enc][0]
+    packed = random_valid_blocks(enc, n * k // bs, 600 + n)
+    x = np.random.default_rng(n + k).standard_normal((m, k)).astype(np.float32)
+    x[0, :64] = 0.0
+    got = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x, kind=1 if m > 8 else 0)
+    assert not np.isnan(got).any()
+    assert normalized_err(got, L.gemv(enc, x, packed, n)) <= GEMV_TOL
+
+
+@pytest.mark.parametrize("enc", MORE_ENCS)
+def test_more_formats_spi_kernels_on_host_arrays(hip_backend, torch_cuda, enc):
+    provider = hip_backend.HipKernelProvider()
+    assert provider.supports("matmul", ["Float32", enc])
+    kernel = {"Q4_0": provider.matmul_q4_0, "Q5_0": provider.matmul_q5_0, "Q5_1": provider.matmul_q5_1,
+              "Q5_K": provider.matmul_q5k}[enc]()
+    bs, nb = G.PACKED[enc][0], G.PACKED[enc][1]
+    n, nblocks = 70, 4
+    k = nblocks * bs
+    blocks = G.weight_blocks(enc, n, nblocks, 0x5EED0020)
+    x = G.floats(k, 0x5EED0021)
+    want = L.gemv(enc, x, G.row_major(blocks), n)
+    pad_x, pad_w, pad_y = 5, 2 * nb, 3
+    xin = np.concatenate([np.full(pad_x, 9, np.float32), x])
+    wbm = np.concatenate([np.full(pad_w, 0xAB, np.uint8), G.block_major(blocks)])
+    out = np.full(pad_y + n + 2, 7, np.float32)
+    kernel.matmul(xin, pad_x, wbm, pad_w, k, n, out, pad_y)
+    assert (out[:pad_y] == 7).all() and (out[pad_y + n:] == 7).all()
+    assert normalized_err(out[pad_y:pad_y + n], want) <= GEMV_TOL
+    out2 = np.zeros(n, np.float32)
+    kernel.matmul_row_major(x, 0, G.row_major(blocks), 0, k, n, out2, 0)
+    assert np.array_equal(out2, out[pad_y:pad_y + n])
+    with pytest.raises(ValueError):
+        kernel.matmul(x, 0, wbm, 0, k - 1, n, out, 0)
