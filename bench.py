@@ -37,6 +37,11 @@ WORKLOADS = {
     "q4k_gemv_11008x4096_b8": ("Q4_K", 11008, 4096, 8),
     "q8_0_gemv_4096x4096_b1": ("Q8_0", 4096, 4096, 1),
     "q6k_gemv_32000x4096_b1": ("Q6_K", 32000, 4096, 1),
+    # the remaining packed formats of the provider SPI, at the headline shape
+    "q4_0_gemv_11008x4096_b1": ("Q4_0", 11008, 4096, 1),
+    "q5_0_gemv_11008x4096_b1": ("Q5_0", 11008, 4096, 1),
+    "q5_1_gemv_11008x4096_b1": ("Q5_1", 11008, 4096, 1),
+    "q5k_gemv_11008x4096_b1": ("Q5_K", 11008, 4096, 1),
     # prefill: batch > 8 goes to the MFMA dequant-GEMM and is reported in TFLOP/s against the bf16 MFMA peak
     "q4k_gemm_512x4096x4096": ("Q4_K", 4096, 4096, 512),
     "q6k_gemm_512x32000x4096": ("Q6_K", 32000, 4096, 512),
@@ -65,17 +70,21 @@ def cpu_baseline(enc, n, k, m, packed, x, budget_s=12.0):
     m_full = m
     m = min(m, 16)
     from oracle import lib as L
-    short = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k"}[enc]
+    short = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k", "Q4_0": "q4_0", "Q5_0": "q5_0", "Q5_1": "q5_1", "Q5_K": "q5k"}[enc]
     ref = L.ref()
-    if ref is not None:
-        fn, kind, cores = getattr(ref, f"skainet_{short}_matmul_rm"), "reference", 4
-    else:
-        fn, kind, cores = getattr(L.oracle(fast=True), f"orc_native_{short}_matmul_rm"), "port", 1
+    native = enc in ("Q8_0", "Q4_K", "Q6_K")       # the formats the reference's native C library covers
+    if native and ref is not None:
+        fn, kind, cores, extra_args = getattr(ref, f"skainet_{short}_matmul_rm"), "reference", 4, ()
+    elif native:
+        fn, kind, cores, extra_args = getattr(L.oracle(fast=True), f"orc_native_{short}_matmul_rm"), "port", 1, ()
+    else:                                          # the scalar kernel the reference runs for these (restated), row-major
+        fn, kind, cores, extra_args = getattr(L.oracle(fast=True), f"orc_{short}_matmul"), "port", 1, (1,)
+        short = f"scalar_{short}"
     y = np.empty((m, n), np.float32)
 
     def call():
         for r in range(m):
-            fn(L.fp(x), r * k, L.u8(packed), 0, k, n, L.fp(y), r * n)
+            fn(L.fp(x), r * k, L.u8(packed), 0, k, n, L.fp(y), r * n, *extra_args)
 
     t0 = time.perf_counter()
     call()

@@ -146,7 +146,7 @@ def quant() -> C.CDLL:
         if not os.path.exists(QUANT_LIB_PATH):
             raise HipError(f"{QUANT_LIB_PATH} is missing: build it with `python -m skainet_amd.build`")
         lib = C.CDLL(QUANT_LIB_PATH)
-        for n in ("q8_0", "q4k", "q6k"):
+        for n in ("q8_0", "q4k", "q6k", "q4_0", "q5_0", "q5_1", "q5k"):
             fn = getattr(lib, f"skainet_quantize_{n}")
             fn.restype, fn.argtypes = None, [_vp, _i64, _vp]
         _quant = lib

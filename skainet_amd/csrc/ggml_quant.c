@@ -13,6 +13,10 @@
  * against the decoded scales). Their parity with ggml is unpinned; the tests pin them through the
  * bit-exact decoder instead (valid blocks, round trip within one code step, idempotence).
  *
+ * Q4_0 follows the reference's quantizer (.../lang/tensor/data/Q4_0Quantizer.kt:28-66 and its own fp16 rounding, :91-118);
+ * Q5_0 / Q5_1 / Q5_K follow ggml's quantize_row_q5_0_ref / q5_1_ref / q5_K_ref (the reference has none): parity with ggml
+ * unpinned, pinned through the decoder like the other K-quants.
+ *
  * Threads: OpenMP over super-blocks; output is independent of the thread count.
  */
 #include <math.h>
@@ -277,6 +281,160 @@ QAPI void skainet_quantize_q6k(const float* xin, int64_t n, uint8_t* out) {
                 qh[l] = (uint8_t)((L[j + l] >> 4) | ((L[j + l + 32] >> 4) << 2) | ((L[j + l + 64] >> 4) << 4) | ((L[j + l + 96] >> 4) << 6));
             }
             ql += 64; qh += 32;
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- Q4_0, Q5_0, Q5_1 (32-element blocks) */
+
+/* fp32 -> fp16 as Q4_0Quantizer.floatToHalf does it: round on the first dropped bit (no tie rule), truncating subnormals */
+static uint16_t q4_0_half(float value) {
+    const uint32_t bits = f32_bits(value);
+    const uint32_t sign = (bits >> 16) & 0x8000u;
+    const int exp = (int)((bits >> 23) & 0xFF) - 127 + 15;
+    const uint32_t mant = bits & 0x7FFFFFu;
+    if (exp >= 0x1F) return (uint16_t)(sign | 0x7C00u);
+    if (exp <= 0) {
+        if (exp < -10) return (uint16_t)sign;
+        return (uint16_t)(sign | ((mant | 0x800000u) >> (1 - exp + 13)));
+    }
+    return (uint16_t)((sign | ((uint32_t)exp << 10) | (mant >> 13)) + ((mant >> 12) & 1u));
+}
+
+QAPI void skainet_quantize_q4_0(const float* x, int64_t n, uint8_t* out) {
+    const int64_t nb = n / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < nb; ++b) {
+        const float* v = x + b * 32;
+        uint8_t* y = out + b * 18;
+        float amax = 0.f, max = 0.f;
+        for (int i = 0; i < 32; ++i) { const float a = fabsf(v[i]); if (a > amax) { amax = a; max = v[i]; } }
+        const float d = max / -8.f;
+        const float id = d != 0.f ? 1.f / d : 0.f;
+        const uint16_t h = q4_0_half(d);
+        y[0] = (uint8_t)(h & 0xFF); y[1] = (uint8_t)(h >> 8);
+        for (int j = 0; j < 16; ++j) {
+            int lo = (int)(v[j] * id + 8.5f), hi = (int)(v[16 + j] * id + 8.5f);
+            lo = lo < 0 ? 0 : (lo > 15 ? 15 : lo);
+            hi = hi < 0 ? 0 : (hi > 15 ? 15 : hi);
+            y[2 + j] = (uint8_t)((hi << 4) | lo);
+        }
+    }
+}
+
+QAPI void skainet_quantize_q5_0(const float* x, int64_t n, uint8_t* out) {
+    const int64_t nb = n / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < nb; ++b) {
+        const float* v = x + b * 32;
+        uint8_t* y = out + b * 22;
+        float amax = 0.f, max = 0.f;
+        for (int i = 0; i < 32; ++i) { const float a = fabsf(v[i]); if (a > amax) { amax = a; max = v[i]; } }
+        const float d = max / -16.f;
+        const float id = d != 0.f ? 1.f / d : 0.f;
+        const uint16_t h = f2h(d);
+        y[0] = (uint8_t)(h & 0xFF); y[1] = (uint8_t)(h >> 8);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; ++j) {
+            int q0 = (int)(int8_t)(v[j] * id + 16.5f), q1 = (int)(int8_t)(v[16 + j] * id + 16.5f);
+            q0 = q0 > 31 ? 31 : (q0 < 0 ? 0 : q0);
+            q1 = q1 > 31 ? 31 : (q1 < 0 ? 0 : q1);
+            y[6 + j] = (uint8_t)((q0 & 0x0F) | ((q1 & 0x0F) << 4));
+            qh |= (uint32_t)((q0 & 0x10) >> 4) << j;
+            qh |= (uint32_t)((q1 & 0x10) >> 4) << (j + 16);
+        }
+        memcpy(y + 2, &qh, 4);
+    }
+}
+
+QAPI void skainet_quantize_q5_1(const float* x, int64_t n, uint8_t* out) {
+    const int64_t nb = n / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < nb; ++b) {
+        const float* v = x + b * 32;
+        uint8_t* y = out + b * 24;
+        float mn = v[0], mx = v[0];
+        for (int i = 1; i < 32; ++i) { if (v[i] < mn) mn = v[i]; if (v[i] > mx) mx = v[i]; }
+        const float d = (mx - mn) / 31.f;
+        const float id = d != 0.f ? 1.f / d : 0.f;
+        const uint16_t hd = f2h(d), hm = f2h(mn);
+        y[0] = (uint8_t)(hd & 0xFF); y[1] = (uint8_t)(hd >> 8);
+        y[2] = (uint8_t)(hm & 0xFF); y[3] = (uint8_t)(hm >> 8);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; ++j) {
+            int q0 = (int)((v[j] - mn) * id + 0.5f), q1 = (int)((v[16 + j] - mn) * id + 0.5f);
+            q0 = q0 > 31 ? 31 : (q0 < 0 ? 0 : q0);
+            q1 = q1 > 31 ? 31 : (q1 < 0 ? 0 : q1);
+            y[8 + j] = (uint8_t)((q0 & 0x0F) | ((q1 & 0x0F) << 4));
+            qh |= (uint32_t)((q0 & 0x10) >> 4) << j;
+            qh |= (uint32_t)((q1 & 0x10) >> 4) << (j + 16);
+        }
+        memcpy(y + 4, &qh, 4);
+    }
+}
+
+/* ---------------------------------------------------------------- Q5_K: the Q4_K search with 32 levels */
+QAPI void skainet_quantize_q5k(const float* xin, int64_t n, uint8_t* out) {
+    const int64_t nb = n / 256;
+#pragma omp parallel for schedule(static)
+    for (int64_t ib = 0; ib < nb; ++ib) {
+        const float* x = xin + ib * 256;
+        uint8_t* y = out + ib * 176;
+        uint8_t L[256], Laux[32];
+        float weights[32], mins[8], scales[8];
+        float max_scale = 0, max_min = 0;
+        for (int j = 0; j < 8; ++j) {
+            float sum_x2 = 0;
+            for (int l = 0; l < 32; ++l) sum_x2 += x[32 * j + l] * x[32 * j + l];
+            const float av = sqrtf(sum_x2 / 32);
+            for (int l = 0; l < 32; ++l) weights[l] = av + fabsf(x[32 * j + l]);
+            scales[j] = make_qkx2(32, 31, x + 32 * j, weights, L + 32 * j, &mins[j], Laux, -0.5f, 0.1f, 15);
+            if (scales[j] > max_scale) max_scale = scales[j];
+            if (mins[j] > max_min) max_min = mins[j];
+        }
+        const float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
+        const float inv_min = max_min > 0 ? 63.f / max_min : 0.f;
+        uint8_t* sc = y + 4;
+        memset(sc, 0, 12);
+        for (int j = 0; j < 8; ++j) {
+            int ls = nearest_int(inv_scale * scales[j]);
+            int lm = nearest_int(inv_min * mins[j]);
+            ls = ls > 63 ? 63 : (ls < 0 ? 0 : ls);
+            lm = lm > 63 ? 63 : (lm < 0 ? 0 : lm);
+            if (j < 4) { sc[j] = (uint8_t)ls; sc[j + 4] = (uint8_t)lm; }
+            else {
+                sc[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                sc[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                sc[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        const uint16_t hd = f2h(max_scale / 63.f), hm = f2h(max_min / 63.f);
+        y[0] = (uint8_t)(hd & 0xFF); y[1] = (uint8_t)(hd >> 8);
+        y[2] = (uint8_t)(hm & 0xFF); y[3] = (uint8_t)(hm >> 8);
+        const float fd = h2f(hd), fm = h2f(hm);
+        for (int j = 0; j < 8; ++j) {
+            int s, m;
+            scale_min_k4(j, sc, &s, &m);
+            const float d = fd * s;
+            if (d == 0.f) continue;
+            const float dm = fm * m;
+            for (int ii = 0; ii < 32; ++ii) {
+                int l = nearest_int((x[32 * j + ii] + dm) / d);
+                l = l < 0 ? 0 : (l > 31 ? 31 : l);
+                L[32 * j + ii] = (uint8_t)l;
+            }
+        }
+        uint8_t *qh = y + 16, *ql = y + 48;
+        memset(qh, 0, 32);
+        uint8_t m1 = 1, m2 = 2;
+        for (int g = 0; g < 256; g += 64) {
+            for (int j = 0; j < 32; ++j) {
+                int l1 = L[g + j], l2 = L[g + j + 32];
+                if (l1 > 15) { l1 -= 16; qh[j] |= m1; }
+                if (l2 > 15) { l2 -= 16; qh[j] |= m2; }
+                ql[j] = (uint8_t)(l1 | (l2 << 4));
+            }
+            m1 <<= 2; m2 <<= 2; ql += 32;
         }
     }
 }

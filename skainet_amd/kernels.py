@@ -84,15 +84,17 @@ def quantize(encoding: str, values: np.ndarray) -> np.ndarray:
 
     Q8_0 follows Q8_0Quantizer.quantizeToBytes
     (/root/reference/skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/data/Q8_0Quantizer.kt:28-53);
-    Q4_K / Q6_K follow the ggml reference quantizers (the reference has none for them).
+    Q4_0 follows Q4_0Quantizer.quantizeToBytes (same directory, Q4_0Quantizer.kt:28-66);
+    Q4_K / Q6_K / Q5_K / Q5_0 / Q5_1 follow the ggml reference quantizers (the reference has none for them).
     """
     _, bs, nb = ENCODINGS[encoding]
     v = np.ascontiguousarray(values, dtype=np.float32)
     if v.size % bs != 0 or (v.ndim > 0 and v.shape[-1] % bs != 0):
         raise ValueError(f"{encoding} quantization requires a last dimension that is a multiple of {bs}; got {v.shape}")
     out = np.empty(v.size // bs * nb, dtype=np.uint8)
-    fn = getattr(_lib.quant(), {"Q8_0": "skainet_quantize_q8_0", "Q4_K": "skainet_quantize_q4k",
-                                "Q6_K": "skainet_quantize_q6k"}[encoding])
+    fn = getattr(_lib.quant(), {"Q8_0": "skainet_quantize_q8_0", "Q4_K": "skainet_quantize_q4k", "Q6_K": "skainet_quantize_q6k",
+                                "Q4_0": "skainet_quantize_q4_0", "Q5_0": "skainet_quantize_q5_0",
+                                "Q5_1": "skainet_quantize_q5_1", "Q5_K": "skainet_quantize_q5k"}[encoding])
     fn(v.ctypes.data, v.size, out.ctypes.data)
     return out
 

@@ -32,7 +32,8 @@ def test_library_exports_every_declared_symbol():
 
 def test_quantizer_library_exports():
     lib = ctypes.CDLL(_lib.QUANT_LIB_PATH)
-    for n in ("skainet_quantize_q8_0", "skainet_quantize_q4k", "skainet_quantize_q6k"):
+    for n in ("skainet_quantize_q8_0", "skainet_quantize_q4k", "skainet_quantize_q6k", "skainet_quantize_q4_0",
+              "skainet_quantize_q5_0", "skainet_quantize_q5_1", "skainet_quantize_q5k"):
         assert hasattr(lib, n)
 
 

@@ -1,8 +1,9 @@
 """Host-side GGUF quantizers (skainet_amd/csrc/ggml_quant.c).
 
 Q8_0 has a reference implementation (Q8_0Quantizer.kt) and is checked byte-for-byte against the oracle's
-restatement of it. Q4_K / Q6_K have none in the reference (parity unpinned): they are pinned through the bit-exact
-decoder by invariants -- valid super-blocks, round trip within one code step, determinism, idempotence.
+restatement of it; Q4_0 has one too (Q4_0Quantizer.kt) and is held to the known answers of the reference's own
+Q4_0QuantizerTest.kt. Q4_K / Q6_K / Q5_K / Q5_0 / Q5_1 have none in the reference (parity unpinned): they are pinned
+through the bit-exact decoder by invariants -- valid blocks, round trip within one code step, determinism, idempotence.
 """
 import numpy as np
 import pytest
@@ -93,3 +94,45 @@ def test_to_kernel_order_matches_the_oracle_relayout():
         want = np.empty_like(q)
         L.oracle().orc_relayout(L.u8(q), L.u8(want), 6, 768 // bs, nb, 0)
         assert np.array_equal(kernels.to_kernel_order(enc, q, 6, 768 // bs), want)
+
+
+def test_q4_0_known_answers_of_the_reference_quantizer_test():
+    """Q4_0QuantizerTest.kt: 18 bytes per block; round trip within one step (|max| / 8) per block on
+    (rng - 0.5) * 4 values; the dominant negative element recovered within 0.05; an all-zero block stays zero."""
+    assert kernels.quantize("Q4_0", (0.1 * np.arange(64)).astype(np.float32)).size == 2 * 18
+    with pytest.raises(ValueError):
+        kernels.quantize("Q4_0", np.zeros(31, np.float32))
+    v = ((np.random.default_rng(7).random(32 * 8, dtype=np.float32) - 0.5) * 4).astype(np.float32)
+    back = L.dequant("Q4_0", kernels.quantize("Q4_0", v))
+    step = np.abs(v.reshape(-1, 32)).max(1, keepdims=True) / 8
+    assert (np.abs(back.reshape(-1, 32) - v.reshape(-1, 32)) <= step + 1e-4).all()
+    one = np.zeros(32, np.float32); one[5] = -3.7; one[9] = 1.2
+    assert abs(L.dequant("Q4_0", kernels.quantize("Q4_0", one))[5] + 3.7) <= 0.05
+    assert not L.dequant("Q4_0", kernels.quantize("Q4_0", np.zeros(32, np.float32))).any()
+    # the algorithm itself, restated: d = max / -8 (sign of the largest magnitude), code = trunc(x / d + 8.5) in 0..15
+    blk = v[:32]
+    mx = blk[np.argmax(np.abs(blk))]
+    d = np.float32(mx) / np.float32(-8)
+    codes = np.clip((blk * (np.float32(1) / d) + np.float32(8.5)).astype(np.int32), 0, 15)
+    q = kernels.quantize("Q4_0", blk)
+    assert np.array_equal(q[2:] & 0x0F, codes[:16]) and np.array_equal(q[2:] >> 4, codes[16:])
+    assert abs(float(q[:2].view(np.float16)[0]) - float(d)) <= abs(float(d)) * 2 ** -10
+
+
+@pytest.mark.parametrize("enc,levels,rel_rms", [("Q4_0", 16, 0.12), ("Q5_0", 32, 0.06), ("Q5_1", 32, 0.05), ("Q5_K", 32, 0.045)])
+def test_q4_0_q5_blocks_round_trip_within_one_step_and_are_deterministic(enc, levels, rel_rms):
+    w = weights(8, 1024, 5)
+    w[0, :256] = 0.0
+    q = kernels.quantize(enc, w)
+    assert q.size == w.size // kernels.ENCODINGS[enc][1] * kernels.ENCODINGS[enc][2]
+    back = L.dequant(enc, q).reshape(w.shape)
+    assert np.isfinite(back).all() and not back[0, :256].any()
+    blk = 32
+    amax = np.abs(w.reshape(-1, blk)).max(1, keepdims=True)
+    rng_ = w.reshape(-1, blk).max(1, keepdims=True) - w.reshape(-1, blk).min(1, keepdims=True)
+    step = {"Q4_0": amax / 8, "Q5_0": amax / 16, "Q5_1": rng_ / 31, "Q5_K": rng_ / 31 * 1.2}[enc]
+    assert (np.abs(back.reshape(-1, blk) - w.reshape(-1, blk)) <= step * 1.02 + 1e-6).all()
+    assert np.sqrt(((back - w) ** 2).mean()) / w.std() < rel_rms
+    assert np.array_equal(q, kernels.quantize(enc, w))
+    once = L.dequant(enc, kernels.quantize(enc, back))
+    assert np.sqrt(((once - back.ravel()) ** 2).mean()) / w.std() < rel_rms
