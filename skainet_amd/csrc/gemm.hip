@@ -158,10 +158,76 @@ __device__ __forceinline__ void decode_dword(const RawQ80& r, const DecQ80& c, f
     for (int j = 0; j < 4; ++j) w4[j] = (float)(int8_t)(q >> (8 * j)) * c.d;
 }
 
+// Q4_0 / Q5_0 / Q5_1 (FMT 0 / 1 / 2): a thread's 32 weights are one block -- fp16 d [fp16 m] [32 fifth bits], then 16 bytes
+// whose low nibbles are elements 0..15 and high nibbles elements 16..31. Blocks are 2-byte aligned (Q5_1: 8).
+template <int FMT> struct RawQ45 { uint32_t d, m, qh, q[4]; };
+template <int FMT>
+__device__ __forceinline__ void load_raw(RawQ45<FMT>& r, const uint8_t* row, int e) {
+    constexpr int BYTES = FMT == 0 ? Q40_BYTES : (FMT == 1 ? Q50_BYTES : Q51_BYTES);
+    constexpr int QH = FMT == 2 ? 4 : 2, QS = FMT == 0 ? 2 : QH + 4;
+    const uint8_t* blk = row + (e >> 5) * BYTES;
+    r.d = load_u16(blk);
+    r.m = FMT == 2 ? load_u16(blk + 2) : 0u;
+    r.qh = FMT != 0 ? load_u32_a2(blk + QH) : 0u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.q[i] = load_u32_a2(blk + QS + 4 * i);
+}
+struct DecQ45 { float d, add; };
+template <int FMT>
+__device__ __forceinline__ void decode_prepare(const RawQ45<FMT>& r, int, DecQ45& c) {
+    c.d = half_bits_to_float_fast(r.d);
+    // w = d * code + add:  Q4_0 d * (code - 8),  Q5_0 d * (code5 - 16),  Q5_1 d * code5 + m
+    c.add = FMT == 0 ? -8.f * c.d : (FMT == 1 ? -16.f * c.d : half_bits_to_float_fast(r.m));
+}
+template <int I, int FMT>
+__device__ __forceinline__ void decode_dword(const RawQ45<FMT>& r, const DecQ45& c, float* w4) {
+    // parts 0..3: low nibbles of code dword I (elements 4I ..), parts 4..7: high nibbles of dword I - 4 (elements 16 + ..)
+    uint32_t v = (r.q[I & 3] >> (I < 4 ? 0 : 4)) & 0x0F0F0F0Fu;
+    if (FMT != 0) v |= ((((r.qh >> (4 * I)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;   // fifth bits 4I .. 4I + 3
+    w4[0] = fmaf(ubyte0_to_float(v), c.d, c.add);
+    w4[1] = fmaf(ubyte1_to_float(v), c.d, c.add);
+    w4[2] = fmaf(ubyte2_to_float(v), c.d, c.add);
+    w4[3] = fmaf(ubyte3_to_float(v), c.d, c.add);
+}
+
+// Q5_K: the Q4_K sub-block plus bit sb of the 32-byte fifth-bit plane at byte 16 (nibbles at byte 48).
+struct RawQ5K { uint4 hdr, q0, q1, h0, h1; };
+__device__ __forceinline__ void load_raw(RawQ5K& r, const uint8_t* row, int e) {
+    const uint8_t* blk = row + (e >> 8) * Q5K_BYTES;
+    const int g = (e & 255) >> 6;
+    r.hdr = *reinterpret_cast<const uint4*>(blk);
+    r.h0 = *reinterpret_cast<const uint4*>(blk + 16);
+    r.h1 = *reinterpret_cast<const uint4*>(blk + 32);
+    r.q0 = *reinterpret_cast<const uint4*>(blk + 48 + g * 32);
+    r.q1 = *reinterpret_cast<const uint4*>(blk + 64 + g * 32);
+}
+struct DecQ5K { float scale, offset; int shift, bit; };
+__device__ __forceinline__ void decode_prepare(const RawQ5K& r, int e, DecQ5K& c) {
+    const RawQ4K r4{r.hdr, r.q0, r.q1};
+    DecQ4K c4;
+    decode_prepare(r4, e, c4);                       // same d / dmin / 6-bit scale and min packing
+    c.scale = c4.scale; c.offset = c4.offset; c.shift = c4.shift;
+    c.bit = (e & 255) >> 5;
+}
+template <int I>
+__device__ __forceinline__ void decode_dword(const RawQ5K& r, const DecQ5K& c, float* w4) {
+    const uint32_t q = I == 0 ? r.q0.x : I == 1 ? r.q0.y : I == 2 ? r.q0.z : I == 3 ? r.q0.w
+                     : I == 4 ? r.q1.x : I == 5 ? r.q1.y : I == 6 ? r.q1.z : r.q1.w;
+    const uint32_t h = I == 0 ? r.h0.x : I == 1 ? r.h0.y : I == 2 ? r.h0.z : I == 3 ? r.h0.w
+                     : I == 4 ? r.h1.x : I == 5 ? r.h1.y : I == 6 ? r.h1.z : r.h1.w;
+    const uint32_t v = ((q >> c.shift) & 0x0F0F0F0Fu) | (((h >> c.bit) & 0x01010101u) << 4);
+    w4[0] = fmaf(ubyte0_to_float(v), c.scale, -c.offset);
+    w4[1] = fmaf(ubyte1_to_float(v), c.scale, -c.offset);
+    w4[2] = fmaf(ubyte2_to_float(v), c.scale, -c.offset);
+    w4[3] = fmaf(ubyte3_to_float(v), c.scale, -c.offset);
+}
+
 template <class Raw> struct DecOf;
 template <> struct DecOf<RawQ4K> { typedef DecQ4K type; };
 template <> struct DecOf<RawQ6K> { typedef DecQ6K type; };
 template <> struct DecOf<RawQ80> { typedef DecQ80 type; };
+template <int FMT> struct DecOf<RawQ45<FMT>> { typedef DecQ45 type; };
+template <> struct DecOf<RawQ5K> { typedef DecQ5K type; };
 
 typedef __bf16 gemm_bf16x4 __attribute__((ext_vector_type(4)));
 // part I (0..7) of a thread's 32 weights -> 4 bf16 values
@@ -373,9 +439,7 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     // shapes the tile loader cannot take (a Q8_0 row that is not a whole number of 256-element groups: the K loop
     // runs pairs of 64-element steps over whole groups; unaligned operands) go through the row kernels: same result
     // to fp32 rounding, the weight streamed once per 4 rows
-    // (so do the formats the tile loader has no decoder for: Q4_0, Q5_0, Q5_1, Q5_K)
-    if ((enc != ENC_Q4_K && enc != ENC_Q6_K && enc != ENC_Q8_0) || k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) ||
-        (reinterpret_cast<uintptr_t>(x) & 15))
+    if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15))
         return launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
     const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;
@@ -416,6 +480,10 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     int rc;
     if (enc == ENC_Q4_K) rc = launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     else if (enc == ENC_Q6_K) rc = launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_K) rc = launch_gemm_enc<RawQ5K, QK_ELEMS, Q5K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q4_0) rc = launch_gemm_enc<RawQ45<0>, Q80_ELEMS, Q40_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_0) rc = launch_gemm_enc<RawQ45<1>, Q80_ELEMS, Q50_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_1) rc = launch_gemm_enc<RawQ45<2>, Q80_ELEMS, Q51_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     if (rc != 0 || ksplit == 1) return rc;
     const int64_t total = (int64_t)m * n;

@@ -31,7 +31,7 @@ GGML_TYPES = {
     26: ("I32", 1, 4), 27: ("I64", 1, 8), 28: ("F64", 1, 8), 30: ("BF16", 1, 2),
 }
 TYPE_ID = {v[0]: k for k, v in GGML_TYPES.items()}
-DEVICE_ENCODINGS = ("Q8_0", "Q4_K", "Q6_K")      # what the kernels consume packed
+DEVICE_ENCODINGS = ("Q8_0", "Q4_K", "Q6_K", "Q4_0", "Q5_0", "Q5_1", "Q5_K")      # what the kernels consume packed
 
 # metadata value types (Constants.kt:142-156)
 _SCALARS = {0: "<B", 1: "<b", 2: "<H", 3: "<h", 4: "<I", 5: "<i", 6: "<f", 7: "<?", 10: "<Q", 11: "<q", 12: "<d"}

@@ -382,3 +382,33 @@ def test_gguf_round_trip_gives_the_same_model(small_model, tmp_path):
     w.layers[1].w_down.matmul(x, 1, y2)
     kx.sync()
     assert torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("linear,head", [("Q5_K", "Q5_0"), ("Q4_0", "Q5_1")])
+def test_decoder_over_the_other_packed_formats(hip_backend, linear, head, tmp_path):
+    """The same stack with Q5_K / Q4_0 linears and Q5_0 / Q5_1 heads (composed launches: only Q4_K has the fused decode
+    kernels; the 8-token prompt runs exact-fp32 row kernels): prefill and greedy decode against the float64 checker,
+    and the model survives a GGUF round trip."""
+    import dataclasses
+    from skainet_amd.decoder import LlamaDecoder, LlamaWeights
+    cfg = dataclasses.replace(small_config(), linear_encoding=linear, head_encoding=head)
+    w = LlamaWeights(cfg, seed=13, sigma=0.05, keep_host=True)
+    prompt = np.random.default_rng(3).integers(0, cfg.vocab, 8)
+    dec = LlamaDecoder(w, max_prefill=32)
+    tok = dec.prefill(prompt)
+    chk = CheckDecoder(cfg, w.host)
+    h_ref, logits_ref = chk.forward(prompt)
+    assert max_norm_err(dec.hidden_rows(len(prompt)), h_ref) < 1e-3
+    assert max_norm_err(dec.last_logits(), logits_ref) < 1e-3
+    assert tok == int(np.argmax(dec.last_logits()))
+    for i in range(4):
+        _, logits_ref = chk.forward([tok])
+        tok = int(dec.decode(1, use_graph=i > 0)[0])
+        assert max_norm_err(dec.last_logits(), logits_ref) < 1e-3, f"step {i}"
+        assert tok == int(np.argmax(dec.last_logits()))
+    path = str(tmp_path / "m.gguf")
+    w.to_gguf(path)
+    w2 = LlamaWeights.from_gguf(path, ctx_max=cfg.ctx_max, keep_host=True)
+    assert w2.cfg.linear_encoding == linear and w2.cfg.head_encoding == head
+    for name, a in w.host.items():
+        assert np.array_equal(np.asarray(a), np.asarray(w2.host[name])), name

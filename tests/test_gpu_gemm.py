@@ -9,7 +9,9 @@ import pytest
 
 from oracle import golden as G
 from oracle import lib as L
-from gpu_util import ENCS, dev, gaussian_weight, normalized_err, random_valid_blocks
+from gpu_util import ENCS, MORE_ENCS, dev, gaussian_weight, normalized_err, random_valid_blocks
+
+ALL_ENCS = ENCS + MORE_ENCS
 
 pytestmark = pytest.mark.gpu
 GEMM_TOL = 2e-2       # max |got - ref| / ||ref||_inf against the exact-fp32 oracle
@@ -47,7 +49,7 @@ def gpu_gemm(kernels, torch, enc, packed, n, k, x, kind=1):
     return y.cpu().numpy()
 
 
-@pytest.mark.parametrize("enc", ENCS)
+@pytest.mark.parametrize("enc", ALL_ENCS)
 @pytest.mark.parametrize("m,n,k", [(9, 5, 256), (33, 130, 512), (256, 128, 1024), (300, 257, 768), (64, 1000, 2304), (1, 64, 256)])
 def test_gemm_ragged_tiles(hip_backend, torch_cuda, enc, m, n, k):
     packed = gaussian_weight(hip_backend, enc, n, k, 200 + n)
@@ -62,7 +64,7 @@ def test_gemm_ragged_tiles(hip_backend, torch_cuda, enc, m, n, k):
     check(auto, want)
 
 
-@pytest.mark.parametrize("enc", ENCS)
+@pytest.mark.parametrize("enc", ALL_ENCS)
 def test_gemm_on_random_valid_blocks_and_forced_k_splits(hip_backend, torch_cuda, enc):
     bs = G.PACKED[enc][0]
     m, n, k = 40, 200, 2048

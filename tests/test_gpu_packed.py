@@ -239,13 +239,12 @@ def test_more_formats_gemv_on_the_reference_golden_inputs(hip_backend, torch_cud
 @pytest.mark.parametrize("n,k,m", [(1, 256, 1), (3, 512, 2), (65, 2048, 4), (130, 2304, 5), (1000, 4096, 1), (257, 11008, 1),
                                    (40, 16640, 3), (300, 1024, 24)])
 def test_more_formats_gemv_ragged_shapes_and_batches(hip_backend, torch_cuda, enc, n, k, m):
-    """All row counts run exact-fp32 products here (24 rows: the product entry falls back from the tile kernel, which has
-    no decoder for these formats, to the row kernels), so the one-row bound holds throughout."""
+    """Exact-fp32 products through the row kernels at every row count (kind 0 forces them; 24 rows = six passes)."""
     bs = G.PACKED[enc][0]
     packed = random_valid_blocks(enc, n * k // bs, 600 + n)
     x = np.random.default_rng(n + k).standard_normal((m, k)).astype(np.float32)
     x[0, :64] = 0.0
-    got = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x, kind=1 if m > 8 else 0)
+    got = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x, kind=0)
     assert not np.isnan(got).any()
     assert normalized_err(got, L.gemv(enc, x, packed, n)) <= GEMV_TOL
 
