@@ -46,6 +46,8 @@ WORKLOADS = {
     "q4k_gemm_512x4096x4096": ("Q4_K", 4096, 4096, 512),
     "q6k_gemm_512x32000x4096": ("Q6_K", 32000, 4096, 512),
     "q4k_gemm_512x14336x4096": ("Q4_K", 14336, 4096, 512),
+    "q5k_gemm_512x4096x4096": ("Q5_K", 4096, 4096, 512),
+    "q4_0_gemm_512x4096x4096": ("Q4_0", 4096, 4096, 512),
 }
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 ATTENTION_PREFILL_USES_MFMA = True    # the prompt-shape attention kernel runs bf16 operands on the matrix cores
