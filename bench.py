@@ -74,12 +74,11 @@ def cpu_baseline(enc, n, k, m, packed, x, budget_s=12.0):
     from oracle import lib as L
     short = {"Q8_0": "q8_0", "Q4_K": "q4k", "Q6_K": "q6k", "Q4_0": "q4_0", "Q5_0": "q5_0", "Q5_1": "q5_1", "Q5_K": "q5k"}[enc]
     ref = L.ref()
-    native = enc in ("Q8_0", "Q4_K", "Q6_K")       # the formats the reference's native C library covers
-    if native and ref is not None:
+    if ref is not None and hasattr(ref, f"skainet_{short}_matmul_rm"):
         fn, kind, cores, extra_args = getattr(ref, f"skainet_{short}_matmul_rm"), "reference", 4, ()
-    elif native:
+    elif enc in ("Q8_0", "Q4_K", "Q6_K"):
         fn, kind, cores, extra_args = getattr(L.oracle(fast=True), f"orc_native_{short}_matmul_rm"), "port", 1, ()
-    else:                                          # the scalar kernel the reference runs for these (restated), row-major
+    else:                                          # the reference's scalar kernel restated, canonical order
         fn, kind, cores, extra_args = getattr(L.oracle(fast=True), f"orc_{short}_matmul"), "port", 1, (1,)
         short = f"scalar_{short}"
     y = np.empty((m, n), np.float32)

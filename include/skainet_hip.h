@@ -170,10 +170,10 @@ SKAINET_HIP_API void skainet_hip_q8_0_matmul(const float* input, int32_t input_o
     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
 SKAINET_HIP_API void skainet_hip_q8_0_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
-/* The remaining packed formats of the provider SPI (API/KernelProvider.kt:74-104): Q4_0MatmulKernel.matmul
- * (API/Q4_0MatmulKernel.kt:40), Q5_0MatmulKernel.matmul (API/Q5_0MatmulKernel.kt:37), Q5_1MatmulKernel.matmul
- * (API/Q5_1MatmulKernel.kt:47), Q5KMatmulKernel.matmul (API/Q5KMatmulKernel.kt:53). The reference has no native C
- * twin for these; the signatures follow the ones above. Plain name: input-block-major weight, `_rm`: canonical order. */
+/* The remaining packed formats of the provider SPI (API/KernelProvider.kt:74-104): NAT:353 skainet_q4_0_matmul / NAT:197
+ * skainet_q4_0_matmul_rm (Q4_0MatmulKernel.matmul, API/Q4_0MatmulKernel.kt:40), NAT:381 / NAT:215 (Q5_0MatmulKernel.matmul,
+ * API/Q5_0MatmulKernel.kt:37), NAT:409 / NAT:233 (Q5_1MatmulKernel.matmul, API/Q5_1MatmulKernel.kt:47), NAT:105 / NAT:251
+ * (Q5KMatmulKernel.matmul, API/Q5KMatmulKernel.kt:53). Plain name: input-block-major weight, `_rm`: canonical order. */
 SKAINET_HIP_API void skainet_hip_q4_0_matmul(const float* input, int32_t input_offset, const uint8_t* weight,
     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
 SKAINET_HIP_API void skainet_hip_q4_0_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
@@ -190,6 +190,15 @@ SKAINET_HIP_API void skainet_hip_q5k_matmul(const float* input, int32_t input_of
     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
 SKAINET_HIP_API void skainet_hip_q5k_matmul_rm(const float* input, int32_t input_offset, const uint8_t* weight,
     int32_t weight_byte_offset, int32_t input_dim, int32_t output_dim, float* output, int32_t output_offset);
+
+/* NAT:290 skainet_bf16_matmul / NAT:307 skainet_fp16_matmul (Bf16MatmulKernel.matmul / Fp16MatmulKernel.matmul,
+ * API/NarrowFloatMatmulKernel.kt:44-49): C(m,n) = A(m,k) B(k,n), A and C fp32 with float strides, B two bytes per element
+ * (bf16 = the high half of an fp32; fp16 = IEEE binary16, little-endian) with BYTE offset and row stride; full overwrite,
+ * k == 0 zeroes C. */
+SKAINET_HIP_API void skainet_hip_bf16_matmul(const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b,
+    int32_t b_byte_offset, int32_t b_byte_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k);
+SKAINET_HIP_API void skainet_hip_fp16_matmul(const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b,
+    int32_t b_byte_offset, int32_t b_byte_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k);
 
 /* NAT:271 skainet_fp32_matmul (Fp32MatmulKernel.matmul, API/Fp32MatmulKernel.kt:25-50): C(m,n) = A(m,k) B(k,n),
  * strides in floats, full overwrite; k == 0 zeroes C. */

@@ -32,6 +32,7 @@ def i32(a):
 
 
 _GEMV_ARGS = [_f32p, C.c_int32, _u8p, C.c_int32, C.c_int32, C.c_int32, _f32p, C.c_int32]
+_NARROW_ARGS = [_f32p, C.c_int32, C.c_int32, _u8p, C.c_int32, C.c_int32, _f32p, C.c_int32, C.c_int32] + [C.c_int32] * 3
 _SDPA_ARGS = [_f32p, _f32p, _f32p, _f32p] + [C.c_int32] * 6 + [C.c_float] + [C.c_int32] * 3 + \
              [_i32p, _f32p] + [C.c_int32] * 4
 
@@ -63,6 +64,10 @@ def oracle(fast: bool = False) -> C.CDLL:
         f = getattr(lib, f"orc_native_{n}_matmul_rm")
         f.argtypes = _GEMV_ARGS
         f.restype = None
+    for n in ("bf16", "fp16"):
+        f = getattr(lib, f"orc_{n}_matmul")
+        f.argtypes = _NARROW_ARGS
+        f.restype = None
     lib.orc_relayout.argtypes = [_u8p, _u8p, C.c_int64, C.c_int64, C.c_int32, C.c_int32]
     lib.orc_relayout.restype = None
     lib.orc_q8_0_quantize.argtypes = [_f32p, C.c_int64, _u8p]
@@ -89,10 +94,16 @@ def ref():
     lib = None
     if os.path.exists(path):
         lib = C.CDLL(path)
-        for n in ("q8_0", "q4k", "q6k"):
+        for n in ("q8_0", "q4k", "q6k", "q4_0", "q5_0", "q5_1", "q5k"):
             for suffix in ("", "_rm"):
-                f = getattr(lib, f"skainet_{n}_matmul{suffix}")
-                f.argtypes = _GEMV_ARGS
+                f = getattr(lib, f"skainet_{n}_matmul{suffix}", None)   # an older build of _ref has only the first three
+                if f is not None:
+                    f.argtypes = _GEMV_ARGS
+                    f.restype = None
+        for n in ("bf16", "fp16"):
+            f = getattr(lib, f"skainet_{n}_matmul", None)
+            if f is not None:
+                f.argtypes = _NARROW_ARGS
                 f.restype = None
         lib.skainet_f32_sdpa.argtypes = _SDPA_ARGS
         lib.skainet_f32_sdpa.restype = None
@@ -155,4 +166,15 @@ def sdpa(q, k, v, scale, causal=False, window=0, right_context=0, lengths=None, 
     fn = oracle().orc_f32_sdpa if lib is None else lib.skainet_f32_sdpa
     fn(fp(q), fp(k), fp(v), fp(out), b, h, hkv, sq, skv, d, float(scale), int(causal), window,
        right_context, i32(lengths), fp(mask), *md)
+    return out
+
+
+def narrow_matmul(kind: str, a: np.ndarray, b_bytes: np.ndarray, m: int, n: int, k: int, lib=None) -> np.ndarray:
+    """C(m, n) = A(m, k) B(k, n) with B as contiguous bf16 / fp16 bytes (`kind` "bf16" / "fp16"); `lib` picks the checker
+    (default: the oracle; pass ref() for the reference's C library)."""
+    a = np.ascontiguousarray(a, np.float32)
+    b_bytes = np.ascontiguousarray(b_bytes, np.uint8)
+    out = np.empty((m, n), np.float32)
+    fn = getattr(oracle(), f"orc_{kind}_matmul") if lib is None else getattr(lib, f"skainet_{kind}_matmul")
+    fn(fp(a), 0, k, u8(b_bytes), 0, 2 * n, fp(out), 0, n, m, n, k)
     return out

@@ -21,6 +21,7 @@
  *   [Q5KD]   Q5_KTensorData.kt:126-142 (decode), :190-219 (scale/min index), :221-236 (code)
  *   [Q40M]   .../exec/kernel/ScalarQ4_0MatmulKernel.kt:29-63, [Q50M] ScalarQ5_0MatmulKernel.kt, [Q51M] ScalarQ5_1MatmulKernel.kt,
  *   [Q5KM]   ScalarQ5_KMatmulKernel.kt (all: one `override fun matmul`)
+ *   [NARROW] .../exec/kernel/ScalarBf16MatmulKernel.kt:8-46 and ScalarFp16MatmulKernel.kt (same loop, Fp16Codec.decode)
  *   [Q80Q]   skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/data/Q8_0Quantizer.kt:28-53
  *   [FP16E]  skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/types/NarrowFloatCodec.kt:87-130
  *   [SDPA]   skainet-backends/skainet-backend-native-cpu/native/src/f32_fused.c:304-396 and
@@ -39,6 +40,8 @@
  *   orc_dequant_{q4_0,q5_0,q5_1,q5k} and orc_{q4_0,q5_0,q5_1,q5k}_matmul
  *                              reference golden digests decode/, transpose/, scalar-matmul/, dispatch-bridge/ of
  *                              Q4_0, Q5_0, Q5_1, Q5_K, pinned
+ *   orc_bf16_matmul, orc_fp16_matmul  exact on integer-valued operands (every partial sum representable), the reference
+ *                              C library's skainet_bf16_matmul / skainet_fp16_matmul (oracle/_ref and recorded vectors), float64, pinned
  *   orc_q8_0_quantize          known answers of the reference's Q8_0QuantizerTest + numpy fp16 RNE, pinned
  *   orc_f32_sdpa, rms_norm,    the reference C library compiled from its own sources (oracle/_ref),
  *   softmax, fp32 matmuls      fp64 closed forms and mask-rule invariants, pinned
@@ -702,4 +705,32 @@ ORC_API void orc_native_q8_0_matmul_rm(const float* input, int32_t input_offset,
         }
         output[output_offset + o] = acc;
     }
+}
+
+/* ---------------------------------------------------------------- fp32 x bf16 / fp16 dense matmul [NARROW]
+ * C(m, n) = A(m, k) B(k, n): A and C fp32 with float strides, B two bytes per element with a byte row stride;
+ * sum in fp32 over ascending p; k == 0 zeroes the block. */
+static void narrow_matmul(const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b, int32_t b_byte_offset,
+                          int32_t b_byte_stride, float* out, int32_t out_offset, int32_t out_stride, int32_t m, int32_t n,
+                          int32_t k, int is_fp16) {
+    if (m <= 0 || n <= 0) return;
+    for (int32_t i = 0; i < m; ++i) {
+        for (int32_t j = 0; j < n; ++j) {
+            float sum = 0.0f;
+            for (int32_t p = 0; p < k; ++p) {
+                const uint32_t h = le16(b + b_byte_offset + (int64_t)p * b_byte_stride + 2 * j);
+                const float bf = is_fp16 ? orc_half_to_float(h) : bits_f32(h << 16);
+                sum += a[a_offset + (int64_t)i * a_stride + p] * bf;
+            }
+            out[out_offset + (int64_t)i * out_stride + j] = sum;
+        }
+    }
+}
+ORC_API void orc_bf16_matmul(const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b, int32_t b_byte_offset,
+                             int32_t b_byte_stride, float* out, int32_t out_offset, int32_t out_stride, int32_t m, int32_t n, int32_t k) {
+    narrow_matmul(a, a_offset, a_stride, b, b_byte_offset, b_byte_stride, out, out_offset, out_stride, m, n, k, 0);
+}
+ORC_API void orc_fp16_matmul(const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b, int32_t b_byte_offset,
+                             int32_t b_byte_stride, float* out, int32_t out_offset, int32_t out_stride, int32_t m, int32_t n, int32_t k) {
+    narrow_matmul(a, a_offset, a_stride, b, b_byte_offset, b_byte_stride, out, out_offset, out_stride, m, n, k, 1);
 }

@@ -64,6 +64,8 @@ SIGNATURES = {
     "skainet_hip_q5k_matmul_rm": (None, _GEMV),
     "skainet_hip_fp32_matmul": (None, _SGEMM),
     "skainet_hip_fp32_matmul_wt": (None, _SGEMM_WT),
+    "skainet_hip_bf16_matmul": (None, _SGEMM),
+    "skainet_hip_fp16_matmul": (None, _SGEMM),
     "skainet_hip_f32_rms_norm": (None, [_vp, _vp, _vp, _i32, _i32, _f32]),
     "skainet_hip_f32_layer_norm": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _f32]),
     "skainet_hip_f32_softmax_rows": (None, [_vp, _vp, _i32, _i32, _i32]),

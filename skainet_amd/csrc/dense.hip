@@ -6,16 +6,21 @@
 //                   /root/reference/skainet-backends/skainet-backend-native-cpu/native/include/skainet_kernels.h:262-276
 //   fp32_matmul_wt  out[i,o] = sum_p in[i,p] * w[o,p]
 //                   /root/reference/skainet-backends/skainet-backend-native-cpu/native/include/skainet_kernels.h:495-515
+//   bf16 / fp16 matmul  C(m,n) = A(m,k) B(k,n) with B two bytes per element, byte row stride (bf16: the high half of
+//                   an fp32; fp16: IEEE binary16), same tile kernel with the decode in the tile load
+//                   /root/reference/skainet-backends/skainet-backend-native-cpu/native/include/skainet_kernels.h:278-312
 #include "common.h"
 
 namespace skh {
 
 constexpr int DT = 64, DK = 16;
 
-// BT == false: B(p, j) = b[p * b_stride + j];  BT == true: B(p, j) = b[j * b_stride + p] (x . W^T).
-template <bool BT>
+// BK 0: B(p, j) = b[p * b_stride + j];  BK 1: B(p, j) = b[j * b_stride + p] (x . W^T);
+// BK 2 / 3: B(p, j) = bf16 / fp16 at byte p * b_stride + 2 j of b (b_stride in bytes, any alignment: read bytewise).
+template <int BK>
 __global__ __launch_bounds__(256) void sgemm_kernel(const float* __restrict__ a, int64_t a_stride, const float* __restrict__ b,
                                                     int64_t b_stride, float* __restrict__ c, int64_t c_stride, int m, int n, int k) {
+    constexpr bool BT = BK == 1;
     __shared__ float as[DK][DT + 1];
     __shared__ float bs[DK][DT + 1];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
@@ -29,9 +34,18 @@ __global__ __launch_bounds__(256) void sgemm_kernel(const float* __restrict__ a,
             if (BT) {
                 const int bj = t / DK, bp = t % DK;
                 bs[bp][bj] = (j0 + bj < n && p0 + bp < k) ? b[(int64_t)(j0 + bj) * b_stride + p0 + bp] : 0.f;
-            } else {
+            } else if (BK == 0) {
                 const int bp = t / DT, bj = t % DT;
                 bs[bp][bj] = (j0 + bj < n && p0 + bp < k) ? b[(int64_t)(p0 + bp) * b_stride + j0 + bj] : 0.f;
+            } else {
+                const int bp = t / DT, bj = t % DT;
+                float v = 0.f;
+                if (j0 + bj < n && p0 + bp < k) {
+                    const uint8_t* e = reinterpret_cast<const uint8_t*>(b) + (int64_t)(p0 + bp) * b_stride + 2 * (j0 + bj);
+                    const uint32_t h = (uint32_t)e[0] | ((uint32_t)e[1] << 8);
+                    v = BK == 2 ? __uint_as_float(h << 16) : half_bits_to_float(h);
+                }
+                bs[bp][bj] = v;
             }
         }
         __syncthreads();
@@ -61,8 +75,21 @@ int launch_fp32_matmul(const float* a, int64_t a_stride, const float* b, int64_t
     if (m <= 0 || n <= 0) return 0;
     if (k < 0) k = 0;
     const dim3 grid((n + DT - 1) / DT, (m + DT - 1) / DT);
-    if (b_transposed) sgemm_kernel<true><<<grid, dim3(256), 0, current_stream()>>>(a, a_stride, b, b_stride, c, c_stride, m, n, k);
-    else sgemm_kernel<false><<<grid, dim3(256), 0, current_stream()>>>(a, a_stride, b, b_stride, c, c_stride, m, n, k);
+    if (b_transposed) sgemm_kernel<1><<<grid, dim3(256), 0, current_stream()>>>(a, a_stride, b, b_stride, c, c_stride, m, n, k);
+    else sgemm_kernel<0><<<grid, dim3(256), 0, current_stream()>>>(a, a_stride, b, b_stride, c, c_stride, m, n, k);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
+// C(m, n) = A(m, k) B(k, n), B bf16 (fp16 != 0: IEEE binary16) bytes with a byte row stride.
+int launch_narrow_matmul(const float* a, int64_t a_stride, const uint8_t* b, int64_t b_byte_stride, float* c, int64_t c_stride,
+                         int m, int n, int k, int fp16) {
+    if (m <= 0 || n <= 0) return 0;
+    if (k < 0) k = 0;
+    const dim3 grid((n + DT - 1) / DT, (m + DT - 1) / DT);
+    const float* bf = reinterpret_cast<const float*>(b);
+    if (fp16) sgemm_kernel<3><<<grid, dim3(256), 0, current_stream()>>>(a, a_stride, bf, b_byte_stride, c, c_stride, m, n, k);
+    else sgemm_kernel<2><<<grid, dim3(256), 0, current_stream()>>>(a, a_stride, bf, b_byte_stride, c, c_stride, m, n, k);
     SKH_CHECK(hipGetLastError());
     return 0;
 }

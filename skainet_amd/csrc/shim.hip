@@ -38,6 +38,8 @@ int launch_rope_qkv(const float* qkv, float* q_out, float* k_cache, float* v_cac
                     int head_dim, int kv_capacity, int pos_start, const int32_t* pos_dev, float theta);
 int launch_i32_store_at(int32_t* dst, const int32_t* index, int32_t offset, const int32_t* src);
 int launch_rope_table(const int32_t* pos, float theta, int head_dim, float* table);
+int launch_narrow_matmul(const float* a, int64_t a_stride, const uint8_t* b, int64_t b_byte_stride, float* c, int64_t c_stride,
+                         int m, int n, int k, int fp16);
 int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log);
 int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim);
 int launch_i32_increment(int32_t* v, int32_t delta);
@@ -638,6 +640,32 @@ void skainet_hip_fp32_matmul(const float* a, int32_t a_offset, int32_t a_stride,
     if (check_hip(hipMemcpy2DAsync(c + c_offset, sizeof(float) * (size_t)c_stride, cd, sizeof(float) * (size_t)n,
                                    sizeof(float) * (size_t)n, (size_t)m, hipMemcpyDeviceToHost, t_stream), "hipMemcpy2D d2h") != 0) return;
     check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+
+static void narrow_matmul_host(int fp16, const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b, int32_t b_byte_offset,
+                               int32_t b_byte_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k) {
+    t_error[0] = 0;
+    if (m <= 0 || n <= 0) return;
+    if (ensure_device() != 0) return;
+    if (k < 0) { set_error("narrow matmul: k must be non-negative; got %d", k); return; }
+    const size_t a_span = k > 0 ? (size_t)(m - 1) * a_stride + k : 0, b_span = k > 0 ? (size_t)(k - 1) * b_byte_stride + 2 * (size_t)n : 0;
+    float* ad = static_cast<float*>(stage_in(0, a + a_offset, sizeof(float) * a_span));
+    uint8_t* bd = static_cast<uint8_t*>(stage_in(1, b + b_byte_offset, b_span));
+    float* cd = static_cast<float*>(scratch_get(t_stage[2], sizeof(float) * (size_t)m * n));
+    if ((k > 0 && (!ad || !bd)) || !cd) return;
+    if (launch_narrow_matmul(ad, a_stride, bd, b_byte_stride, cd, n, m, n, k, fp16) != 0) return;
+    if (c_stride == n) { stage_out(c + c_offset, cd, sizeof(float) * (size_t)m * n); return; }
+    if (check_hip(hipMemcpy2DAsync(c + c_offset, sizeof(float) * (size_t)c_stride, cd, sizeof(float) * (size_t)n,
+                                   sizeof(float) * (size_t)n, (size_t)m, hipMemcpyDeviceToHost, t_stream), "hipMemcpy2D d2h") != 0) return;
+    check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+}
+void skainet_hip_bf16_matmul(const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b, int32_t b_byte_offset,
+                             int32_t b_byte_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k) {
+    narrow_matmul_host(0, a, a_offset, a_stride, b, b_byte_offset, b_byte_stride, c, c_offset, c_stride, m, n, k);
+}
+void skainet_hip_fp16_matmul(const float* a, int32_t a_offset, int32_t a_stride, const uint8_t* b, int32_t b_byte_offset,
+                             int32_t b_byte_stride, float* c, int32_t c_offset, int32_t c_stride, int32_t m, int32_t n, int32_t k) {
+    narrow_matmul_host(1, a, a_offset, a_stride, b, b_byte_offset, b_byte_stride, c, c_offset, c_stride, m, n, k);
 }
 
 void skainet_hip_fp32_matmul_wt(const float* in, int32_t in_offset, const float* w, int32_t w_offset, float* out,

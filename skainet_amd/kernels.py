@@ -403,6 +403,30 @@ class HipFp32MatmulKernel:
         _raise_if_failed(before, "fp32_matmul")
 
 
+class HipNarrowFloatMatmulKernel:
+    """Bf16MatmulKernel / Fp16MatmulKernel (skainet-backend-api kernel/NarrowFloatMatmulKernel.kt:25-49,
+    ScalarBf16MatmulKernel.kt:19-46): C(m, n) = A(m, k) B(k, n) with B two bytes per element (little-endian bf16 or IEEE
+    binary16), byte offset and byte row stride for B, float strides for A and C, fp32 sums, k == 0 zeroes the block."""
+
+    def __init__(self, codec: str):
+        if codec not in ("BFloat16", "Float16"):
+            raise ValueError(f"codec must be BFloat16 or Float16, got {codec!r}")
+        self.codec = codec
+
+    def matmul(self, a, a_offset, a_stride, b, b_byte_offset, b_byte_stride, out, out_offset, out_stride, m, n, k):
+        if m < 0 or n < 0 or k < 0:
+            raise ValueError(f"{self.codec} matmul: m, n, k must be non-negative; got m={m} n={n} k={k}")
+        _require_available()
+        lib = _lib.hip()
+        if not (isinstance(b, np.ndarray) and b.dtype == np.uint8 and b.flags.c_contiguous):
+            raise TypeError("b must be a C-contiguous uint8 numpy array")
+        fn = lib.skainet_hip_bf16_matmul if self.codec == "BFloat16" else lib.skainet_hip_fp16_matmul
+        before = lib.skainet_hip_last_error()
+        fn(_f32(a, "a").ctypes.data, a_offset, a_stride, b.ctypes.data, b_byte_offset, b_byte_stride,
+           _f32(out, "out").ctypes.data, out_offset, out_stride, m, n, k)
+        _raise_if_failed(before, f"{self.codec} matmul")
+
+
 class HipFp32MatmulWtKernel:
     def matmul_wt(self, input, input_offset, weight, weight_offset, out, out_offset, m, n, k):
         _require_available()
@@ -516,6 +540,8 @@ class HipKernelProvider:
 
     def matmul_fp32(self): return HipFp32MatmulKernel() if is_available() else None
     def matmul_fp32_wt(self): return HipFp32MatmulWtKernel() if is_available() else None
+    def matmul_bf16(self): return HipNarrowFloatMatmulKernel("BFloat16") if is_available() else None
+    def matmul_fp16(self): return HipNarrowFloatMatmulKernel("Float16") if is_available() else None
     def matmul_q4k(self): return HipPackedMatmulKernel("Q4_K") if is_available() else None
     def matmul_q6k(self): return HipPackedMatmulKernel("Q6_K") if is_available() else None
     def matmul_q8_0(self): return HipPackedMatmulKernel("Q8_0") if is_available() else None
@@ -532,4 +558,4 @@ class HipKernelProvider:
         if op_name != "matmul" or len(dtype_keys) != 2 or not is_available():
             return False
         inp, weight = dtype_keys
-        return inp == "Float32" and weight in ("Float32", "Q4_K", "Q6_K", "Q8_0", "Q4_0", "Q5_0", "Q5_1", "Q5_K")
+        return inp == "Float32" and weight in ("Float32", "BFloat16", "Float16", "Q4_K", "Q6_K", "Q8_0", "Q4_0", "Q5_0", "Q5_1", "Q5_K")

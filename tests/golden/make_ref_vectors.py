@@ -2,7 +2,8 @@
 oracle/Makefile from the sources under /root/reference) on closed-form / seeded inputs.
 
 Run here (the reference is not present on a GPU box):  python tests/golden/make_ref_vectors.py
-The vectors pin the oracle's attention and int8-activation port where the reference library is absent.
+The vectors pin the oracle's attention, its int8-activation port, its exact kernels for Q4_0 / Q5_0 / Q5_1 / Q5_K and its
+bf16 / fp16 dense matmul where the reference library is absent.
 """
 import os
 import sys
@@ -15,7 +16,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 from oracle import golden as G  # noqa: E402
 from oracle import lib as L  # noqa: E402
-from test_oracle_golden import SDPA_GRID, sdpa_inputs  # noqa: E402
+from test_oracle_golden import SDPA_GRID, narrow_inputs, sdpa_inputs  # noqa: E402
 
 
 def main():
@@ -34,6 +35,18 @@ def main():
         y = np.empty(n, np.float32)
         getattr(ref, f"skainet_{short}_matmul_rm")(L.fp(x), 0, L.u8(w), 0, nblocks * bs, n, L.fp(y), 0)
         out[f"native_rm/{enc}"] = y
+    # exact fp32 kernels of the reference library (no int8 activations on these formats)
+    for enc in ("Q4_0", "Q5_0", "Q5_1", "Q5_K"):
+        bs = G.PACKED[enc][0]
+        n, nblocks = 6, 3
+        w = G.row_major(G.weight_blocks(enc, n, nblocks, 0x5EED0010))
+        x = G.floats(nblocks * bs, 0x5EED0011)
+        y = np.empty(n, np.float32)
+        getattr(ref, f"skainet_{L._SHORT[enc]}_matmul_rm")(L.fp(x), 0, L.u8(w), 0, nblocks * bs, n, L.fp(y), 0)
+        out[f"native_rm/{enc}"] = y
+    for kind in ("bf16", "fp16"):
+        a, b, m, n, k = narrow_inputs(kind)
+        out[f"narrow/{kind}"] = L.narrow_matmul(kind, a, b, m, n, k, lib=ref)
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")

@@ -295,3 +295,43 @@ def test_dense_matmuls(hip_backend, torch_cuda):
     o = np.zeros((70, 33), np.float32)
     prov.matmul_fp32_wt().matmul_wt(a, 0, w, 0, o, 0, 70, 33, 130)
     close(o, a.astype(np.float64) @ w.T, rel=1e-5, abs_=1e-4)
+
+
+@pytest.mark.parametrize("kind,codec", [("bf16", "BFloat16"), ("fp16", "Float16")])
+def test_narrow_float_matmuls(hip_backend, torch_cuda, kind, codec):
+    """Bf16MatmulKernel / Fp16MatmulKernel through the host entry: the oracle on the recorded inputs (with the formats'
+    specials), then a ragged larger product with offsets, an odd byte offset and a padded byte row stride for B."""
+    from test_oracle_golden import narrow_inputs, narrow_values
+    prov = hip_backend.HipKernelProvider()
+    kern = prov.matmul_bf16() if kind == "bf16" else prov.matmul_fp16()
+    assert kern.codec == codec and prov.supports("matmul", ["Float32", codec])
+    a, b, m, n, k = narrow_inputs(kind)
+    c = np.full((m, n), np.nan, np.float32)
+    kern.matmul(a, 0, k, b, 0, 2 * n, c, 0, n, m, n, k)
+    want = L.narrow_matmul(kind, a, b, m, n, k)
+    close(c, want.astype(np.float64), rel=1e-5, abs_=1e-6)
+    recorded = np.load(os.path.join(HERE, "golden", "ref_vectors.npz"))[f"narrow/{kind}"]
+    close(c, recorded.astype(np.float64), rel=1e-5, abs_=1e-6)
+    # 70 x 83 x 150 out of wider buffers; B starts at an odd byte and its rows are 2 * 90 + 6 bytes apart
+    rng = np.random.default_rng(12)
+    m, n, k = 70, 83, 150
+    a = rng.standard_normal((m + 2, k + 9)).astype(np.float32)
+    bv = rng.standard_normal((k, n)).astype(np.float32)
+    bits = (bv.view(np.uint32) >> 16).astype("<u2") if kind == "bf16" else bv.astype("<f2").view("<u2")
+    stride = 2 * 90 + 6
+    raw = np.full(3 + k * stride, 0xA5, np.uint8)
+    rows = np.lib.stride_tricks.as_strided(raw[3:], (k, 2 * n), (stride, 1))
+    rows[:] = np.ascontiguousarray(bits).view(np.uint8).reshape(k, 2 * n)
+    c = np.full((m + 1, n + 5), 3.0, np.float32)
+    kern.matmul(a, 2 * (k + 9) + 4, k + 9, raw, 3, stride, c, (n + 5) + 2, n + 5, m, n, k)
+    want = a[2:, 4:4 + k].astype(np.float64) @ narrow_values(kind, np.ascontiguousarray(bits).view(np.uint8).reshape(-1), k, n).astype(np.float64)
+    close(c[1:, 2:2 + n], want, rel=1e-5, abs_=1e-5)
+    assert (c[0] == 3).all() and (c[:, :2] == 3).all() and (c[:, 2 + n:] == 3).all()
+    ref = np.full_like(c, 3.0)
+    getattr(L.oracle(), f"orc_{kind}_matmul")(L.fp(a), 2 * (k + 9) + 4, k + 9, L.u8(raw), 3, stride, L.fp(ref), (n + 5) + 2, n + 5, m, n, k)
+    close(c, ref.astype(np.float64), rel=1e-5, abs_=1e-5)
+    z = np.full((4, 6), 9.0, np.float32)
+    kern.matmul(a, 0, k + 9, raw, 0, stride, z, 0, 6, 4, 6, 0)              # k == 0 zeroes C
+    assert not z.any()
+    with pytest.raises(ValueError):
+        kern.matmul(a, 0, k + 9, raw, 0, stride, z, 0, 6, 4, 6, -1)

@@ -263,6 +263,81 @@ def test_native_port_is_bit_identical_to_the_reference_library(enc):
     assert np.sqrt(((y - exact) ** 2).mean()) / np.sqrt((exact ** 2).mean()) < 0.03
 
 
+@pytest.mark.parametrize("enc", ["Q4_0", "Q5_0", "Q5_1", "Q5_K"])
+def test_exact_kernels_of_the_other_formats_against_the_reference_library(enc):
+    """The reference's C kernels for these formats multiply in fp32 (no int8 activations); they and the oracle's
+    restatement of the Kotlin scalar kernels differ by summation order only."""
+    bs = G.PACKED[enc][0]
+    n, nblocks = 6, 3
+    blocks = G.weight_blocks(enc, n, nblocks, 0x5EED0010)
+    w = G.row_major(blocks)
+    x = G.floats(nblocks * bs, 0x5EED0011)
+    recorded = np.load(os.path.join(HERE, "golden", "ref_vectors.npz"))[f"native_rm/{enc}"]
+    got = L.gemv(enc, x, w, n)
+    scale = np.abs(recorded).max()
+    assert np.abs(got - recorded).max() <= 1e-5 * scale
+    ref = L.ref()
+    if ref is not None and getattr(ref, f"skainet_{L._SHORT[enc]}_matmul_rm", None) is not None:
+        yr, yb = np.empty(n, np.float32), np.empty(n, np.float32)
+        getattr(ref, f"skainet_{L._SHORT[enc]}_matmul_rm")(L.fp(x), 0, L.u8(w), 0, nblocks * bs, n, L.fp(yr), 0)
+        assert np.array_equal(yr.view(np.uint32), recorded.view(np.uint32))
+        getattr(ref, f"skainet_{L._SHORT[enc]}_matmul")(L.fp(x), 0, L.u8(G.block_major(blocks)), 0, nblocks * bs, n, L.fp(yb), 0)
+        np.testing.assert_allclose(yb, yr, rtol=1e-6, atol=1e-6 * scale)
+
+
+def narrow_inputs(kind):
+    """A (5 x 37, fp32) and B (37 x 11) as bf16 / fp16 bytes: seeded, with the specials of the format in B's first row
+    (zero, negative zero, the smallest subnormal, the largest finite value)."""
+    m, n, k = 5, 11, 37
+    a = G.floats(m * k, 0x5EED0020).reshape(m, k)
+    b = G.floats(k * n, 0x5EED0021).reshape(k, n) * 3
+    if kind == "bf16":
+        bits = (b.view(np.uint32) >> 16).astype("<u2")
+        bits[0, :4] = [0x0000, 0x8000, 0x0001, 0x7F7F]
+    else:
+        bits = b.astype("<f2").view("<u2").copy()
+        bits[0, :4] = [0x0000, 0x8000, 0x0001, 0x7BFF]
+    return a, np.ascontiguousarray(bits).view(np.uint8).reshape(-1), m, n, k
+
+
+def narrow_values(kind, b_bytes, k, n):
+    bits = b_bytes.view("<u2").reshape(k, n)
+    return (bits.astype(np.uint32) << 16).view(np.float32) if kind == "bf16" else bits.view("<f2").astype(np.float32)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp16"])
+def test_narrow_float_matmul(kind):
+    """ScalarBf16MatmulKernel.kt:19-46 (and the fp16 twin): numpy's own decode of the 16-bit values, float64 sums; the
+    reference C library's result (recorded, and live when built); byte offset / strides; k == 0 zeroes the block;
+    integer-valued operands give exact sums whatever the order."""
+    a, b, m, n, k = narrow_inputs(kind)
+    got = L.narrow_matmul(kind, a, b, m, n, k)
+    bv = narrow_values(kind, b, k, n)
+    want = a.astype(np.float64) @ bv.astype(np.float64)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+    recorded = np.load(os.path.join(HERE, "golden", "ref_vectors.npz"))[f"narrow/{kind}"]
+    np.testing.assert_allclose(got, recorded, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+    if L.ref() is not None and getattr(L.ref(), f"skainet_{kind}_matmul", None) is not None:
+        assert np.array_equal(L.narrow_matmul(kind, a, b, m, n, k, lib=L.ref()).view(np.uint32), recorded.view(np.uint32))
+    # offsets and strides: a sub-block of A (rows 1.., columns 2..), of B (rows 2.., columns 3..) into a wider C
+    fn = getattr(L.oracle(), f"orc_{kind}_matmul")
+    c = np.full((m, 16), 7.0, np.float32)
+    mm, nn, kk = m - 1, n - 3, k - 2
+    fn(L.fp(a), 1 * k + 2, k, L.u8(b), 2 * n * 2 + 3 * 2, 2 * n, L.fp(c), 16 + 1, 16, mm, nn, kk)
+    sub = a[1:, 2:].astype(np.float64) @ bv[2:, 3:].astype(np.float64)
+    np.testing.assert_allclose(c[1:, 1:1 + nn], sub, rtol=1e-5, atol=1e-5 * np.abs(sub).max())
+    assert (c[0] == 7.0).all() and (c[:, 0] == 7.0).all() and (c[:, 1 + nn:] == 7.0).all()
+    fn(L.fp(a), 0, k, L.u8(b), 0, 2 * n, L.fp(c), 0, 16, m, n, 0)
+    assert (c[:, :n] == 0.0).all() and (c[:, n:] == 7.0).all()
+    # small integers: every product and partial sum is representable, so the result is exact
+    rng = np.random.default_rng(3)
+    ai = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    bi = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    bb = (bi.view(np.uint32) >> 16).astype("<u2") if kind == "bf16" else bi.astype("<f2").view("<u2")
+    exact = L.narrow_matmul(kind, ai, np.ascontiguousarray(bb).view(np.uint8).reshape(-1), m, n, k)
+    assert np.array_equal(exact, ai @ bi)
+
+
 def test_recorded_reference_sdpa_vectors():
     """Vectors written by tests/golden/make_ref_vectors.py from the reference C library pin the oracle's attention."""
     z = np.load(os.path.join(HERE, "golden", "ref_vectors.npz"))
