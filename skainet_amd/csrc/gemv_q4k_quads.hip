@@ -1,21 +1,27 @@
-// Q4_K dequant-GEMV for 3 to 8 activation rows on the fp32 matrix instruction, canonical row-major GGUF weight.
+// Q4_K dequant-GEMV for 3 to 8 activation rows on the matrix cores, canonical row-major GGUF weight.
 //
-//   y[b, o] = sum_j x[b, j] * dequant(W[o, j])     exact fp32 products and sums, like the one-row kernel
+//   y[b, o] = sum_j x[b, j] * dequant(W[o, j])
 //
 // Same products as the reference's exact-fp32 kernel, other summation order
 //   /root/reference/skainet-backends/skainet-backend-cpu/src/commonMain/kotlin/sk/ainet/exec/kernel/ScalarQ4_KMatmulKernel.kt:40-78
 //
 // With one activation row a weight costs a conversion and an FMA per lane; with eight rows it would cost eight FMAs
-// and the kernel would be bound by the vector ALU, not by HBM. v_mfma_f32_4x4x1_16b_f32 multiplies, in each of its 16
-// independent blocks of four lanes, the four A values of the block with its four B values: a lane's converted weight
-// meets four activation rows in one instruction, at the full fp32 matrix rate and with fp32 operands.
-//   * Lane l = 4 * blk + j. As B operand it supplies the weight of output row j of the wave's current row quad; as A
-//     operand the activation of batch row j; both at the K position of block blk. The four result registers of lane
-//     4 * blk + j are batch rows 0..3 against output row j.
+// and the kernel would be bound by the vector ALU, not by HBM. Here the products run on v_mfma_f32_4x4x4_16b_bf16:
+//   * a 4-bit code q is the bf16 value 128 + q after one mask-and-merge (0x4300 | q: bf16 has ulp 1 on [128, 256)), two
+//     codes per instruction; the 128 is taken out again by starting each accumulator at -128 * sum(x);
+//   * an activation is split into two bf16 values, hi = bf16(x) and lo = bf16(x - hi) (16 to 17 significant bits
+//     together, every product exact in fp32); hi and lo run through the same accumulator.
+//   (The fp16 form of the same instruction would take the codes as they lie in the code dword, as fp16 subnormals, and
+//   22 bits of activation; measured on this device it adds its four products and the accumulator in a truncating
+//   adder of about 19 bits below the largest addend, which leaves a one-sided error of 2.5e-5 of the largest output:
+//   more than this kernel's whole error with bf16 operands.)
+//   * Lane l = 4 * blk + j. As B operand it supplies four weights of output row j of the wave's current row quad; as A
+//     operand four activations (hi or lo part) of batch row j of a batch quad; both at the K position of block blk.
+//     The four result registers of lane 4 * blk + j are the quad's batch rows against output row j.
 //   * Block blk owns one 32-byte nibble group (64 weights: sub-blocks 2g and 2g + 1) of every super-block quartet, so
-//     a wave covers 1024 consecutive K elements ("pass") and a lane keeps its 64 activations per batch quad in
-//     registers for all the row quads of the workgroup. Per row quad a lane loads its row's block header and its 32
-//     bytes of codes: across the wave, four spans of 576 contiguous bytes.
+//     a wave covers 1024 consecutive K elements ("pass") and a lane keeps its 64 activations per batch row in registers
+//     (hi and lo: 64 packed dwords) for all the row quads of the workgroup. Per row quad a lane loads its row's block header and
+//     its 32 bytes of codes: across the wave, four spans of 576 contiguous bytes.
 //   * The four waves of a workgroup take the passes round-robin (K = 4096: one pass each) and all walk the same row
 //     quads; per-lane sums are folded across the 16 blocks with a multi-value butterfly and across the waves in LDS.
 #include "gemv_q4k.h"
@@ -23,7 +29,7 @@
 namespace skh {
 
 typedef float f32x4_q __attribute__((ext_vector_type(4)));
-constexpr int QD_SLICE = 68;   // 64 activations + 4 floats of padding: 16-byte aligned, bank-conflict free
+constexpr int QD_SLICE = 36;   // dwords per slice: 64 bf16 activations + 4 dwords of padding (16-byte aligned rows that spread over the banks)
 
 
 // Fold 16 per-lane values across the 16 four-lane blocks of a wave (lane bits 2..5), leaving bits 0..1 apart: on
@@ -47,14 +53,16 @@ __device__ __forceinline__ int block_fold_index(int lane) {
     return ((lane & 4) ? 8 : 0) + ((lane & 8) ? 4 : 0) + ((lane & 16) ? 2 : 0) + ((lane & 32) ? 1 : 0);
 }
 
-// NB: batch quads (batch <= 4 * NB). Q: row quads a workgroup owns. R: row quads whose loads are in flight per wave.
-// OCC: workgroups per CU the register budget is cut for (two batch quads keep 128 activations per lane: one per CU).
-template <int NB, int Q, int R, int OCC>
+typedef short bf16x4_q __attribute__((ext_vector_type(4)));   // four bf16 bit patterns: one matrix operand of a lane
+
+// NM: batch quads (batch <= 4 * NM). Q: row quads a workgroup owns. R: row quads whose loads are in flight per wave.
+// OCC: workgroups per CU the register and LDS budgets are cut for.
+template <int NM, int Q, int R, int OCC>
 __global__ __launch_bounds__(256, OCC) void q4k_gemv_quads_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                              float* __restrict__ y, int k, int n, int batch) {
-    constexpr int NVAL = Q * 4 * NB, NG = (NVAL + 15) / 16;
-    extern __shared__ __attribute__((aligned(16))) float xlds[];   // [4 NB batch rows][64 slices][QD_SLICE]; then the wave partials
-    float (*part)[NG][64] = reinterpret_cast<float (*)[NG][64]>(xlds + 4 * NB * 64 * QD_SLICE);
+    constexpr int NBATCH = 4 * NM, NVAL = Q * NBATCH, NG = (NVAL + 15) / 16;
+    // [NM batch quads][hi, lo][4 batch rows][64 slices][QD_SLICE dwords]; reused for the wave partials at the end
+    extern __shared__ __attribute__((aligned(16))) uint32_t xlds[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int blk = lane >> 2, j = lane & 3;
     // Every workgroup computes exactly Q row quads: rows past N are clamped to the last row and never stored. With no
@@ -68,33 +76,34 @@ __global__ __launch_bounds__(256, OCC) void q4k_gemv_quads_kernel(const uint8_t*
     const int sh = (g & 1) * 16;
     const uint32_t hi_mask = g >= 2 ? 0xFFFFFFFFu : 0u;
     const int q_off = 16 + g * 32;
+    // kept out of the optimiser's sight so that (v & mask) | bias stays one three-operand instruction
+    uint32_t code_mask = 0x000F000Fu, code_bias = 0x43004300u;
+    asm volatile("" : "+v"(code_bias), "+s"(code_mask));
 
-    float acc[Q][4 * NB];
+    float acc[Q][NBATCH];
 #pragma unroll
     for (int q = 0; q < Q; ++q)
 #pragma unroll
-        for (int e = 0; e < 4 * NB; ++e) acc[q][e] = 0.f;
+        for (int e = 0; e < NBATCH; ++e) acc[q][e] = 0.f;
 
     // K is taken in rounds of four passes (4096 elements), one pass per wave. A round's activations are fetched once per
-    // workgroup with coalesced 16-byte loads and parked in LDS as 64-float slices (one per batch row and K group,
-    // padded to 68 floats so the lanes' 16-byte reads spread over the banks); a lane then reads its own slices.
+    // workgroup with coalesced 16-byte loads, split into bf16 hi / lo and parked in LDS as slices of 64 activations per
+    // batch row and part (32 dwords in operand order, padded to QD_SLICE); a lane then reads its own slices.
     const int nrounds = (npass + 3) >> 2;
     for (int round = 0; round < nrounds; ++round) {
         const int pass = round * 4 + wave;
         const int sb = pass * 4 + (blk >> 2);
-        const bool inside = sb < bpr;
         const int sb_c = min(sb, bpr - 1);                 // blocks past K re-read a valid super-block against zero activations
         // this lane's weight row of quad q: r0 + 4 q + j, clamped (rows past N are computed and never stored)
         auto row_ptr = [&](int q) { return w + (int64_t)min(r0 + 4 * q + j, n - 1) * row_bytes + (int64_t)sb_c * Q4K_BYTES; };
 
         // The round's activations are requested first and the first quads' weights right behind them: loads return in
         // issue order, and the (L2-resident) activations must not queue behind the weight stream.
-        // float4 number f (of 1024) of batch row b goes to slice f / 16 of that row, position f % 16.
         Q4KRow raw[R];
         {
-            float4 xv[4 * NB][4];
+            float4 xv[NBATCH][4];
 #pragma unroll
-            for (int b = 0; b < 4 * NB; ++b)
+            for (int b = 0; b < NBATCH; ++b)
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int e = min(round * 4096 + (threadIdx.x + 256 * u) * 4, k - 4);
@@ -110,120 +119,129 @@ __global__ __launch_bounds__(256, OCC) void q4k_gemv_quads_kernel(const uint8_t*
             }
             __builtin_amdgcn_sched_barrier(0);
             __syncthreads();                               // the previous round's slices have been read
+            // float4 number f (of 1024) of batch row b: slice f / 16; inside the slice, sub-block (f % 16) / 8 and code
+            // dword f % 8, whose four activations e0..e3 go out as the dword pair (e0, e2), (e1, e3) -- the order in
+            // which one mask pulls two codes out of a code dword. Rows past the batch and elements past K become
+            // zeros through a mask on the packed values (no branch, no product with what was loaded).
+            typedef float f32x2_q __attribute__((ext_vector_type(2)));
+            typedef __bf16 bf16x2_q __attribute__((ext_vector_type(2)));
 #pragma unroll
-            for (int b = 0; b < 4 * NB; ++b)
+            for (int b = 0; b < NBATCH; ++b)
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int f = threadIdx.x + 256 * u;
-                    float4 v4 = xv[b][u];
-                    if (round * 4096 + f * 4 >= k || b >= batch) v4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                    *reinterpret_cast<float4*>(&xlds[(b * 64 + (f >> 4)) * QD_SLICE + (f & 15) * 4]) = v4;
+                    const float4 v4 = xv[b][u];
+                    const uint32_t live = (round * 4096 + f * 4 < k && b < batch) ? 0xFFFFFFFFu : 0u;
+                    const f32x2_q pr[2] = {f32x2_q{v4.x, v4.z}, f32x2_q{v4.y, v4.w}};
+                    uint32_t hi[2], lo[2];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        hi[t] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pr[t], bf16x2_q)) & live;
+                        const f32x2_q rest = {pr[t].x - __uint_as_float(hi[t] << 16), pr[t].y - __uint_as_float(hi[t] & 0xFFFF0000u)};
+                        lo[t] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2_q)) & live;
+                    }
+                    const int pos = ((f >> 3) & 1) * 16 + (f & 7) * 2;
+                    uint32_t* dst = &xlds[(((b >> 2) * 8 + (b & 3)) * 64 + (f >> 4)) * QD_SLICE + pos];
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(hi[0], hi[1]);
+                    *reinterpret_cast<uint2*>(dst + 4 * 64 * QD_SLICE) = make_uint2(lo[0], lo[1]);
                 }
             __syncthreads();
         }
 
-        // the 64 activations of this lane's K group, for batch rows j and (NB = 2) 4 + j
-        float xs[NB][64], xlo[NB][4], xhi[NB][4];
+        // this lane's operand registers: batch row j of every batch quad at this lane's K group, hi then lo part;
+        // [0..7] go with the low nibbles of code dwords 0..7, [8..15] with the high nibbles
+        bf16x4_q xs[NM][2][16];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            const float* src = &xlds[((nb * 4 + j) * 64 + wave * 16 + blk) * QD_SLICE];
+        for (int nm = 0; nm < NM; ++nm)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float4 v4 = *reinterpret_cast<const float4*>(src + 4 * i);
-                xs[nb][4 * i] = v4.x; xs[nb][4 * i + 1] = v4.y; xs[nb][4 * i + 2] = v4.z; xs[nb][4 * i + 3] = v4.w;
+            for (int part = 0; part < 2; ++part) {
+                const uint32_t* src = &xlds[(((nm * 2 + part) * 4 + j) * 64 + wave * 16 + blk) * QD_SLICE];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint4 v4 = *reinterpret_cast<const uint4*>(src + 4 * i);
+                    xs[nm][part][2 * i] = __builtin_bit_cast(bf16x4_q, make_uint2(v4.x, v4.y));
+                    xs[nm][part][2 * i + 1] = __builtin_bit_cast(bf16x4_q, make_uint2(v4.z, v4.w));
+                }
             }
-            float s0 = 0.f, s1 = 0.f;
+        // 128 * (sum of the batch row's activations, hi + lo) per sub-block, by the same instruction against a constant
+        // operand: negated, the start value of every accumulator; divided by 128, the sum the block minimum multiplies
+        f32x4_q tl[NM], th[NM];
+        float xlo[NBATCH], xhi[NBATCH];
+        {
+            const bf16x4_q ones = __builtin_bit_cast(bf16x4_q, make_uint2(code_bias, code_bias));
 #pragma unroll
-            for (int i = 0; i < 32; ++i) { s0 += xs[nb][i]; s1 += xs[nb][32 + i]; }
-            // the sub-block sums of all four batch rows of the block (a lane holds its own row's)
+            for (int nm = 0; nm < NM; ++nm) {
+                tl[nm] = f32x4_q{0.f, 0.f, 0.f, 0.f}; th[nm] = f32x4_q{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                xlo[nb][e] = __shfl(s0, (lane & ~3) + e, 64);
-                xhi[nb][e] = __shfl(s1, (lane & ~3) + e, 64);
+                for (int i = 0; i < 8; ++i)
+#pragma unroll
+                    for (int part = 0; part < 2; ++part) {
+                        tl[nm] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(xs[nm][part][i], ones, tl[nm], 0, 0, 0);
+                        th[nm] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(xs[nm][part][8 + i], ones, th[nm], 0, 0, 0);
+                    }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    xlo[4 * nm + e] = tl[nm][e] * 0.0078125f;
+                    xhi[4 * nm + e] = th[nm][e] * 0.0078125f;
+                }
+                tl[nm] = -tl[nm]; th[nm] = -th[nm];
             }
         }
-        (void)inside;
 
 #pragma unroll
         for (int q = 0; q < Q; ++q) {
-            {
-                const Q4KRow& r = raw[q % R];
-                float dlo, dhi, mlo, mhi;
-                q4k_lane_scales(r.hdr, sh, hi_mask, dlo, dhi, mlo, mhi);
-                dhi *= 0.0625f;                            // high nibbles enter as 16 * code
-                const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-                // NCH independent accumulation chains per sub-block and batch quad
-                constexpr int NCH = 2;
-                f32x4_q dlc[NB][NCH], dhc[NB][NCH];
+            const Q4KRow& r = raw[q % R];
+            float dlo, dhi, mlo, mhi;
+            q4k_lane_scales(r.hdr, sh, hi_mask, dlo, dhi, mlo, mhi);
+            const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+            // a batch row's hi and lo parts run through the same accumulator: their sum costs nothing
+            f32x4_q dl[NM], dh[NM];
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
+            for (int nm = 0; nm < NM; ++nm) { dl[nm] = tl[nm]; dh[nm] = th[nm]; }
 #pragma unroll
-                    for (int c = 0; c < NCH; ++c) { dlc[nb][c] = f32x4_q{0.f, 0.f, 0.f, 0.f}; dhc[nb][c] = f32x4_q{0.f, 0.f, 0.f, 0.f}; }
-                // The conversions are plain C so the compiler sees the vector-ALU write of every matrix-instruction
-                // operand (an operand written by the instruction just before needs wait states, which the compiler
-                // cannot insert for inline assembly: the matrix instruction then reads the register's old value).
-                // The empty asm emits nothing: it hides the nibble masks from the optimiser, which otherwise turns
-                // each byte conversion into a bit-field extract plus a conversion instead of one v_cvt_f32_ubyteN.
-                // Program order is pinned so that the conversions of code dword i + 1 sit between the matrix
-                // instructions of dword i: each operand is written a dword ahead of its use.
-                float cl[2][4], ch[2][4];
-                auto convert = [&](int set, int t, uint32_t l4, uint32_t h4) __attribute__((always_inline)) {
-                    cl[set][t] = t == 0 ? (float)(l4 & 0xFFu) : t == 1 ? (float)((l4 >> 8) & 0xFFu) : t == 2 ? (float)((l4 >> 16) & 0xFFu) : (float)(l4 >> 24);
-                    ch[set][t] = t == 0 ? (float)(h4 & 0xFFu) : t == 1 ? (float)((h4 >> 8) & 0xFFu) : t == 2 ? (float)((h4 >> 16) & 0xFFu) : (float)(h4 >> 24);
-                };
-                uint32_t l4 = qw[0] & 0x0F0F0F0Fu, h4 = qw[0] & 0xF0F0F0F0u;
-                asm volatile("" : "+v"(l4), "+v"(h4));
+            for (int i = 0; i < 8; ++i) {
+                // codes of bytes (0, 2) and (1, 3) of the dword as bf16 pairs 128 + q: low nibbles, then high nibbles
+                const uint32_t v = qw[i];
+                const bf16x4_q wl = __builtin_bit_cast(bf16x4_q, make_uint2((v & code_mask) | code_bias, ((v >> 8) & code_mask) | code_bias));
+                const bf16x4_q wh = __builtin_bit_cast(bf16x4_q, make_uint2(((v >> 4) & code_mask) | code_bias, ((v >> 12) & code_mask) | code_bias));
 #pragma unroll
-                for (int t = 0; t < 4; ++t) convert(0, t, l4, h4);
+                for (int part = 0; part < 2; ++part)
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if (i < 7) {
-                        l4 = qw[i + 1] & 0x0F0F0F0Fu; h4 = qw[i + 1] & 0xF0F0F0F0u;
-                        asm volatile("" : "+v"(l4), "+v"(h4));
+                    for (int nm = 0; nm < NM; ++nm) {
+                        dl[nm] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(xs[nm][part][i], wl, dl[nm], 0, 0, 0);
+                        dh[nm] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(xs[nm][part][8 + i], wh, dh[nm], 0, 0, 0);
                     }
-                    __builtin_amdgcn_sched_barrier(0);
+            }
+            const float nmlo = -mlo, nmhi = -mhi;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
+            for (int nm = 0; nm < NM; ++nm)
 #pragma unroll
-                        for (int nb = 0; nb < NB; ++nb) {
-                            dlc[nb][t % NCH] = __builtin_amdgcn_mfma_f32_4x4x1f32(xs[nb][i * 4 + t], cl[i & 1][t], dlc[nb][t % NCH], 0, 0, 0);
-                            dhc[nb][t % NCH] = __builtin_amdgcn_mfma_f32_4x4x1f32(xs[nb][32 + i * 4 + t], ch[i & 1][t], dhc[nb][t % NCH], 0, 0, 0);
-                        }
-                        if (i < 7) convert((i + 1) & 1, t, l4, h4);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    float a = acc[q][4 * nm + e];
+                    a = fmaf(nmlo, xlo[4 * nm + e], a);
+                    a = fmaf(nmhi, xhi[4 * nm + e], a);
+                    a = fmaf(dlo, dl[nm][e], a);
+                    acc[q][4 * nm + e] = fmaf(dhi, dh[nm][e], a);
                 }
-                f32x4_q dl[NB], dh[NB];
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    dl[nb] = dlc[nb][0]; dh[nb] = dhc[nb][0];
-#pragma unroll
-                    for (int c = 1; c < NCH; ++c) { dl[nb] += dlc[nb][c]; dh[nb] += dhc[nb][c]; }
-                }
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        acc[q][nb * 4 + e] += dlo * dl[nb][e] + dhi * dh[nb][e] - (mlo * xlo[nb][e] + mhi * xhi[nb][e]);
-                if (q + R < Q) {                           // compile-time: refill with the quad R ahead
-                    const uint8_t* p = row_ptr(q + R);
-                    raw[q % R].hdr = *reinterpret_cast<const uint4*>(p);
-                    raw[q % R].q0 = *reinterpret_cast<const uint4*>(p + q_off);
-                    raw[q % R].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
-                }
+            if (q + R < Q) {                           // compile-time: refill with the quad R ahead
+                const uint8_t* p = row_ptr(q + R);
+                raw[q % R].hdr = *reinterpret_cast<const uint4*>(p);
+                raw[q % R].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                raw[q % R].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
             }
         }
     }
 
-    // value v = q * 4 NB + (batch row) of a lane, in groups of 16: fold across the blocks, park per wave, total the waves
-    const int fidx = block_fold_index(lane);
+    // value v = q * NBATCH + (batch row) of a lane, in groups of 16: fold across the blocks, park per wave, total the waves
+    __syncthreads();                                       // every wave is done with the activation slices
+    float (*part)[NG][64] = reinterpret_cast<float (*)[NG][64]>(xlds);
 #pragma unroll
     for (int grp = 0; grp < NG; ++grp) {
         float v[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int vi = grp * 16 + i;
-            v[i] = vi < NVAL ? acc[vi / (4 * NB)][vi % (4 * NB)] : 0.f;
+            v[i] = vi < NVAL ? acc[vi / NBATCH][vi % NBATCH] : 0.f;
         }
         block_fold16(v, lane);
         part[wave][grp][lane] = v[0];
@@ -232,24 +250,24 @@ __global__ __launch_bounds__(256, OCC) void q4k_gemv_quads_kernel(const uint8_t*
     for (int t = threadIdx.x; t < NG * 64; t += 256) {
         const int grp = t >> 6, ln = t & 63;
         const int vi = grp * 16 + block_fold_index(ln);
-        const int q = vi / (4 * NB), brow = vi % (4 * NB), row = r0 + 4 * q + (ln & 3);
+        const int q = vi / NBATCH, brow = vi % NBATCH, row = r0 + 4 * q + (ln & 3);
         if (vi < NVAL && brow < batch && row < r0 + nrows)
             y[(int64_t)brow * n + row] = part[0][grp][ln] + part[1][grp][ln] + part[2][grp][ln] + part[3][grp][ln];
     }
-    (void)fidx;
 }
 
-template <int NB, int Q, int R, int OCC>
+template <int NM, int Q, int R, int OCC>
 static int launch_quads(hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int batch) {
-    constexpr size_t smem = (size_t)(4 * NB * 64 * QD_SLICE + 4 * ((Q * 4 * NB + 15) / 16) * 64) * sizeof(float);
+    constexpr size_t smem = (size_t)(8 * NM * 64 * QD_SLICE) * sizeof(uint32_t);
+    static_assert(4 * ((Q * 4 * NM + 15) / 16) * 64 <= 8 * NM * 64 * QD_SLICE, "wave partials must fit in the slices");
     static bool attr_set = false;
     if (!attr_set) {
-        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&q4k_gemv_quads_kernel<NB, Q, R, OCC>),
+        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&q4k_gemv_quads_kernel<NM, Q, R, OCC>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     const int grid = (n + 4 * Q - 1) / (4 * Q);
-    q4k_gemv_quads_kernel<NB, Q, R, OCC><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, batch);
+    q4k_gemv_quads_kernel<NM, Q, R, OCC><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, batch);
     SKH_CHECK(hipGetLastError());
     return 1;
 }
@@ -259,8 +277,8 @@ int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int
     if (batch < 3 || batch > 8) return 0;
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 255)) return 0;
     hipStream_t s = current_stream();
-    // one round of workgroups over the chip where N allows: two per CU owning up to 6 row quads (one batch quad), one
-    // per CU owning up to 12 (two batch quads); the quad count is a template parameter
+    // one round of workgroups over the chip where N allows: two per CU owning up to 6 row quads (one batch quad: 74 KB
+    // of activation slices), one per CU owning up to 12 (two batch quads); the quad count is a template parameter
     const int occ = batch <= 4 ? 2 : 1;
     const int q = (n + 4 * occ * num_cus() - 1) / (4 * occ * num_cus());
     if (batch <= 4) {
@@ -275,9 +293,9 @@ int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int
     }
     if (q <= 2) return launch_quads<2, 2, 2, 1>(s, w, x, y, k, n, batch);
     if (q <= 4) return launch_quads<2, 4, 4, 1>(s, w, x, y, k, n, batch);
-    if (q <= 6) return launch_quads<2, 6, 4, 1>(s, w, x, y, k, n, batch);
-    if (q <= 8) return launch_quads<2, 8, 4, 1>(s, w, x, y, k, n, batch);
-    return launch_quads<2, 12, 4, 1>(s, w, x, y, k, n, batch);
+    if (q <= 6) return launch_quads<2, 6, 6, 1>(s, w, x, y, k, n, batch);
+    if (q <= 8) return launch_quads<2, 8, 6, 1>(s, w, x, y, k, n, batch);
+    return launch_quads<2, 12, 6, 1>(s, w, x, y, k, n, batch);
 }
 
 }  // namespace skh

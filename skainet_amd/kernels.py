@@ -554,8 +554,17 @@ class HipKernelProvider:
     def attention_fp32(self): return HipFp32AttentionKernel() if is_available() else None
 
     def supports(self, op_name: str, dtype_keys) -> bool:
-        """KernelProvider.supports (KernelProvider.kt:161-190): matmul over (input, weight) dtype keys."""
-        if op_name != "matmul" or len(dtype_keys) != 2 or not is_available():
+        """KernelProvider.supports (KernelProvider.kt:161-190): true iff the accessor for the combination returns a kernel.
+        One key ["Float32"]: "softmax", "layer_norm", "rms_norm", "sdpa"; two keys [input, weight]: "matmul" over the
+        weight names below, "matmul_wt" over Float32 x Float32."""
+        if not is_available():
             return False
-        inp, weight = dtype_keys
-        return inp == "Float32" and weight in ("Float32", "BFloat16", "Float16", "Q4_K", "Q6_K", "Q8_0", "Q4_0", "Q5_0", "Q5_1", "Q5_K")
+        keys = list(dtype_keys)
+        if len(keys) == 1:
+            return keys[0] == "Float32" and op_name in ("softmax", "layer_norm", "rms_norm", "sdpa")
+        if len(keys) != 2 or keys[0] != "Float32":
+            return False
+        if op_name == "matmul_wt":
+            return keys[1] == "Float32"
+        return op_name == "matmul" and keys[1] in ("Float32", "BFloat16", "Float16", "Q4_K", "Q6_K", "Q8_0", "Q4_0", "Q5_0",
+                                                   "Q5_1", "Q5_K")

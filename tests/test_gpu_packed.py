@@ -135,9 +135,11 @@ def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cud
 
 @pytest.mark.parametrize("n,k,m", [(5, 256, 3), (25, 1280, 8), (77, 2304, 7), (1000, 11008, 4), (11008, 4096, 6), (4096, 14336, 8),
                                    (130, 4096, 9), (64, 1024, 11)])
-def test_q4k_three_to_eight_rows_on_the_fp32_matrix_instruction(hip_backend, torch_cuda, n, k, m):
-    """3 to 8 activation rows take the 4x4x1 fp32 MFMA kernel (9 and 11 rows: 8 + the rest): exact fp32 products, so
-    the one-row bound holds; every batch row must also equal that row run alone to fp32 rounding."""
+def test_q4k_three_to_eight_rows_on_the_matrix_instruction(hip_backend, torch_cuda, n, k, m):
+    """3 to 8 activation rows take the 4x4x4 bf16 MFMA kernel (9 and 11 rows: 8 + the rest). Codes are exact in bf16 and
+    an activation enters as bf16 hi + bf16 lo (16 to 17 significant bits, exact products, fp32 sums): the one-row bound
+    holds with room, and every batch row equals that row run alone (exact fp32) to the split's precision -- 2^-17 per
+    term, seen through this metric's floor of 1 % of the largest output."""
     for packed in (gaussian_weight(hip_backend, "Q4_K", n, k, 81), random_valid_blocks("Q4_K", n * k // 256, 82)):
         x = np.random.default_rng(83 + m).standard_normal((m, k)).astype(np.float32)
         x[1, :64] = 0.0
@@ -146,7 +148,7 @@ def test_q4k_three_to_eight_rows_on_the_fp32_matrix_instruction(hip_backend, tor
         assert got.shape == (m, n) and not np.isnan(got).any()
         assert normalized_err(got, L.gemv("Q4_K", x, packed, n)) <= GEMV_TOL
         alone = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x[m - 1:m])
-        assert normalized_err(got[m - 1], alone[0]) <= 1e-4
+        assert normalized_err(got[m - 1], alone[0]) <= 3e-4
 
 
 def test_gemv_is_linear_and_deterministic_at_full_size(hip_backend, torch_cuda):
@@ -162,7 +164,7 @@ def test_gemv_is_linear_and_deterministic_at_full_size(hip_backend, torch_cuda):
     assert np.array_equal(y1, gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x1))
     # a batch row equals the same row run alone
     yb = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, np.concatenate([x1, x2, x1, x2]))
-    assert normalized_err(yb[1], y2[0]) <= 1e-4   # another kernel (4 rows per pass) sums in another order
+    assert normalized_err(yb[1], y2[0]) <= 5e-4   # another kernel: activations as bf16 hi + lo, another summation order
 
 
 @pytest.mark.parametrize("enc", ENCS)

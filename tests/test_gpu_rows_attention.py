@@ -275,6 +275,12 @@ def test_argmax_split_and_single_kernels(hip_backend, torch_cuda, rows, cols):
 
 def test_dense_matmuls(hip_backend, torch_cuda):
     prov = hip_backend.HipKernelProvider()
+    # capability answers of KernelProvider.supports (KernelProvider.kt:161-190)
+    for op in ("softmax", "layer_norm", "rms_norm", "sdpa"):
+        assert prov.supports(op, ["Float32"]) and not prov.supports(op, ["Float16"])
+    assert prov.supports("matmul_wt", ["Float32", "Float32"]) and not prov.supports("matmul_wt", ["Float32", "Q4_K"])
+    assert not prov.supports("matmul", ["Float16", "Float32"]) and not prov.supports("matmul", ["Float32", "Q3_K"])
+    assert not prov.supports("gather", ["Float32"]) and not prov.supports("matmul", ["Float32"])
     rng = np.random.default_rng(9)
     a = rng.standard_normal((70, 130)).astype(np.float32)
     b = rng.standard_normal((130, 90)).astype(np.float32)
