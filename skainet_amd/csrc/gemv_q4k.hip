@@ -249,8 +249,8 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
     }
 }
 
-static int g_q4k_rows_waves_per_cu = 8;
-void set_q4k_rows_waves_per_cu(int v) { if (v > 0) g_q4k_rows_waves_per_cu = v; }
+static int g_q4k_rows_waves_per_cu = 0;   // 0: chosen from K (below)
+void set_q4k_rows_waves_per_cu(int v) { if (v >= 0) g_q4k_rows_waves_per_cu = v; }
 int q4k_rows_waves_per_cu() { return g_q4k_rows_waves_per_cu; }
 
 template <int B, int R, int NR>
@@ -290,7 +290,13 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     // one round of workgroups over the chip: a wave's rows, taken in equal chunks of at most Q4K_RMAX (the chunk size
     // is a template parameter, so the share is rounded up to a whole number of chunks)
     // (more waves per CU when that keeps a wave's share in one chunk: a second chunk stages the activations again)
-    int waves_per_cu = g_q4k_rows_waves_per_cu;
+    // Measured (2 to 16 waves per CU): a lone product with K of one pass (<= 4096) is fastest at one workgroup per CU
+    // -- a wave stages the activations once for up to 12 rows (11008 x 4096: 7.9 us against 8.2 at 8 waves). With
+    // several passes the staging and its barriers repeat per pass and a second workgroup per CU hides them (4096 x
+    // 14336: 11.7 us at 8 waves against 12.2 at 4), and inside the decoder's chain of fused launches 8 waves measured
+    // 0.6 % faster per token than 4 although each launch alone prefers 4.
+    const bool lone = !gain && epilogue == EPI_NONE;
+    int waves_per_cu = g_q4k_rows_waves_per_cu > 0 ? g_q4k_rows_waves_per_cu : (lone && k <= 4096 ? 4 : 8);
     while (waves_per_cu < 32 && (n + num_cus() * waves_per_cu - 1) / (num_cus() * waves_per_cu) > Q4K_RMAX) waves_per_cu += 4;
     const int total_waves = num_cus() * waves_per_cu;
     const int share = (n + total_waves - 1) / total_waves;
