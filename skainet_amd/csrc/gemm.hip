@@ -36,22 +36,73 @@ constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16); 
 
 void* kernel_workspace(size_t bytes);   // shim.hip
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);   // gemv.hip
+int launch_add(const float* a, const float* b, float* out, int64_t n);                        // rows.hip
+int launch_swiglu_pairs(const float* gate_up, float* out, int64_t n);                         // rows.hip
 
-// The pass in front of the GEMM: activations fp32 -> bf16 (nearest even). Thread i handles float4 number i.
+// The pass in front of the GEMM: activations fp32 -> bf16 (nearest even). A thread handles PREPASS_UNROLL float4s a
+// whole workgroup stride apart, all loaded before the first is stored (clamped index, guarded store).
+constexpr int PREPASS_UNROLL = 4;
 __global__ __launch_bounds__(256) void gemm_prepass_kernel(const float* __restrict__ in, __bf16* __restrict__ out, int64_t n4) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n4) {
-        const float4 v = reinterpret_cast<const float4*>(in)[i];
-        typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-        bf16x4 o = {(__bf16)v.x, (__bf16)v.y, (__bf16)v.z, (__bf16)v.w};
-        reinterpret_cast<bf16x4*>(out)[i] = o;
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    const int64_t i0 = (int64_t)blockIdx.x * (256 * PREPASS_UNROLL) + threadIdx.x;
+    float4 v[PREPASS_UNROLL];
+#pragma unroll
+    for (int u = 0; u < PREPASS_UNROLL; ++u) v[u] = reinterpret_cast<const float4*>(in)[min(i0 + 256 * u, n4 - 1)];
+#pragma unroll
+    for (int u = 0; u < PREPASS_UNROLL; ++u) {
+        const int64_t i = i0 + 256 * u;
+        if (i < n4) reinterpret_cast<bf16x4*>(out)[i] = bf16x4{(__bf16)v[u].x, (__bf16)v[u].y, (__bf16)v[u].z, (__bf16)v[u].w};
     }
 }
+
+// The same pass with an RMSNorm folded in: out = bf16(x / sqrt(mean(x^2) + eps) * gain), one workgroup per activation row,
+// the row held in registers between the sum of squares and the scaling (k a multiple of 4, at most 256 * 4 * V floats).
+template <int V>
+__global__ __launch_bounds__(256) void gemm_prepass_rmsnorm_kernel(const float* __restrict__ in, const float* __restrict__ gain,
+                                                                   __bf16* __restrict__ out, int k, float eps) {
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    __shared__ float red[4];
+    const float4* x = reinterpret_cast<const float4*>(in + (int64_t)blockIdx.x * k);
+    const float4* g4 = reinterpret_cast<const float4*>(gain);
+    bf16x4* o = reinterpret_cast<bf16x4*>(out + (int64_t)blockIdx.x * k);
+    const int k4 = k >> 2;
+    float4 xr[V], gr[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        xr[j] = i < k4 ? x[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        gr[j] = i < k4 ? g4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j) { s = fmaf(xr[j].x, xr[j].x, s); s = fmaf(xr[j].y, xr[j].y, s); s = fmaf(xr[j].z, xr[j].z, s); s = fmaf(xr[j].w, xr[j].w, s); }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    const float scale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) * (1.0f / (float)k) + eps);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < k4) o[i] = bf16x4{(__bf16)(xr[j].x * scale * gr[j].x), (__bf16)(xr[j].y * scale * gr[j].y),
+                                  (__bf16)(xr[j].z * scale * gr[j].z), (__bf16)(xr[j].w * scale * gr[j].w)};
+    }
+}
+
+// What happens to a product on its way out, applied by the launch that sums K splits (a GEMM that is not split writes
+// the plain product and the row kernels finish it: an epilogue in the tile kernel's own stores measured slower --
+// +20 us on 512 x 28672 x 4096 for SwiGLU against 17 us for the separate pass, and it cost the kernels without an
+// epilogue 5 % through the register allocation of their main loop):
+//   GEMM_EPI_NONE      c[row, col] = p
+//   GEMM_EPI_RESIDUAL  c[row, col] = residual[row, col] + p          (residual may be c)
+//   GEMM_EPI_SWIGLU    c[row, col / 2] = silu(p[row, col]) * p[row, col + 1] for even col (c has n / 2 columns)
+enum { GEMM_EPI_NONE = 0, GEMM_EPI_RESIDUAL = 1, GEMM_EPI_SWIGLU = 2 };
+__device__ __forceinline__ float silu_f(float g) { return g * (1.0f / (1.0f + expf(-g))); }
 
 // Split K: C = sum over the splits, in split order, of the partial products parked `stride` floats apart (stride a
 // multiple of 4, the buffer 16-byte aligned). Thread i owns elements 4i .. 4i + 3.
 __global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float* __restrict__ part, int64_t stride, int splits,
-                                                              float* __restrict__ c, int64_t total, int c_aligned) {
+                                                              float* c, int64_t total, int c_aligned, const float* residual,
+                                                              int epilogue) {
     const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= total) return;
     float4 acc = *reinterpret_cast<const float4*>(part + i);
@@ -59,8 +110,18 @@ __global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float* __res
         const float4 v = *reinterpret_cast<const float4*>(part + z * stride + i);
         acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
     }
-    if (c_aligned && i + 4 <= total) { *reinterpret_cast<float4*>(c + i) = acc; return; }
-    const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+    float v[4] = {acc.x, acc.y, acc.z, acc.w};
+    if (epilogue == GEMM_EPI_SWIGLU) {
+        // n is even and elements 4i .. 4i + 3 start at an even column: two (gate, up) pairs, outputs 2i and 2i + 1
+        if (i + 1 < total) c[i >> 1] = silu_f(v[0]) * v[1];
+        if (i + 3 < total) c[(i >> 1) + 1] = silu_f(v[2]) * v[3];
+        return;
+    }
+    if (epilogue == GEMM_EPI_RESIDUAL) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) if (i + j < total) v[j] += residual[i + j];
+    }
+    if (c_aligned && i + 4 <= total) { *reinterpret_cast<float4*>(c + i) = make_float4(v[0], v[1], v[2], v[3]); return; }
     for (int j = 0; j < 4 && i + j < total; ++j) c[i + j] = v[j];
 }
 
@@ -431,7 +492,13 @@ static int launch_gemm_enc(const __bf16* a, const uint8_t* w, float* c, int m, i
 static int g_gemm_ksplit = 0;   // 0 = choose from the tile count
 void set_gemm_ksplit(int v) { g_gemm_ksplit = v; }
 
-int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y) {
+// y = epilogue(prologue(x) . W^T): gain != null normalises every activation row first (RMSNorm, folded into the pass that
+// rounds the activations to bf16); epilogue is one of GEMM_EPI_* (residual [m, n] may be y; SwiGLU: y is [m, n / 2]).
+// `tmp` ([m, n] floats, needed when an epilogue is asked for) takes the plain product when K is not split.
+// Returns 1, having launched nothing, when the shape is outside the tile kernel's range and a prologue or epilogue was
+// asked for (the caller composes the same arithmetic from separate launches).
+int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y, const float* gain, float eps,
+                      const float* residual, int epilogue, float* tmp) {
     if (m <= 0 || n <= 0) return 0;
     if (!is_packed(enc)) return set_error("gemm: unsupported encoding %d", enc);
     if (k <= 0 || k % block_elems(enc) != 0)
@@ -439,8 +506,11 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     // shapes the tile loader cannot take (a Q8_0 row that is not a whole number of 256-element groups: the K loop
     // runs pairs of 64-element steps over whole groups; unaligned operands) go through the row kernels: same result
     // to fp32 rounding, the weight streamed once per 4 rows
-    if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15))
-        return launch_gemv(enc, w, x, m, k, n, y);
+    const bool fused = gain != nullptr || epilogue != GEMM_EPI_NONE;
+    if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) ||
+        (gain && ((reinterpret_cast<uintptr_t>(gain) & 15) || k > 256 * 4 * 16)) || (epilogue == GEMM_EPI_SWIGLU && (n & 1)) ||
+        (epilogue != GEMM_EPI_NONE && !tmp))
+        return fused ? 1 : launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
     const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;
     const int tiles = tiles_m * tiles_n;
@@ -473,10 +543,12 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     __bf16* a = reinterpret_cast<__bf16*>(ws);
     float* part = reinterpret_cast<float*>(ws + a_bytes);
     const int64_t n4 = (int64_t)m * k / 4;                      // k is a multiple of 64
-    gemm_prepass_kernel<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s>>>(x, a, n4);
+    if (!gain) gemm_prepass_kernel<<<dim3((unsigned)((n4 + 256 * PREPASS_UNROLL - 1) / (256 * PREPASS_UNROLL))), dim3(256), 0, s>>>(x, a, n4);
+    else if (k <= 256 * 4 * 4) gemm_prepass_rmsnorm_kernel<4><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
+    else gemm_prepass_rmsnorm_kernel<16><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
     SKH_CHECK(hipGetLastError());
     const dim3 grid(tiles_n, tiles_m, ksplit);
-    float* c = ksplit > 1 ? part : y;
+    float* c = ksplit > 1 ? part : (epilogue != GEMM_EPI_NONE ? tmp : y);
     int rc;
     if (enc == ENC_Q4_K) rc = launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     else if (enc == ENC_Q6_K) rc = launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
@@ -485,12 +557,21 @@ int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     else if (enc == ENC_Q5_0) rc = launch_gemm_enc<RawQ45<1>, Q80_ELEMS, Q50_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     else if (enc == ENC_Q5_1) rc = launch_gemm_enc<RawQ45<2>, Q80_ELEMS, Q51_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    if (rc != 0 || ksplit == 1) return rc;
+    if (rc != 0) return rc;
+    if (ksplit == 1) {
+        if (epilogue == GEMM_EPI_RESIDUAL) return launch_add(residual, tmp, y, (int64_t)m * n);
+        if (epilogue == GEMM_EPI_SWIGLU) return launch_swiglu_pairs(tmp, y, (int64_t)m * (n / 2));
+        return 0;
+    }
     const int64_t total = (int64_t)m * n;
     gemm_splitk_sum_kernel<<<dim3((unsigned)((total / 4 + 256) / 256)), dim3(256), 0, s>>>(
-        part, split_stride, ksplit, y, total, (reinterpret_cast<uintptr_t>(y) & 15) == 0);
+        part, split_stride, ksplit, y, total, (reinterpret_cast<uintptr_t>(y) & 15) == 0, residual, epilogue);
     SKH_CHECK(hipGetLastError());
     return 0;
+}
+
+int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y) {
+    return launch_gemm_fused(enc, w, x, m, k, n, y, nullptr, 0.f, nullptr, GEMM_EPI_NONE, nullptr);
 }
 
 }  // namespace skh

@@ -22,6 +22,8 @@ namespace skh {
 int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr);
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
 int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
+int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y, const float* gain, float eps,
+                      const float* residual, int epilogue, float* tmp);
 int set_tuning(const char* key, int value);
 int launch_rms_norm(const float* in, const float* gamma, float* out, int rows, int cols, float eps);
 int launch_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int rows, int cols, float eps);
@@ -291,7 +293,8 @@ int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int3
 //   gain != NULL: x is RMS-normalised first (x / sqrt(mean(x^2) + eps) * gain, per activation row);
 //   epilogue 0: out [m, rows] = product; 1: out = residual + product (residual [m, rows], may be `out`);
 //   2: out [m, rows / 2], out[j] = silu(p[2j]) * p[2j + 1] (the weight's rows alternate gate row, up row).
-// Decode shapes of Q4_K weights run as ONE kernel; everything else runs the same arithmetic as separate launches.
+// Decode shapes of Q4_K weights run as ONE kernel, prompt shapes (m > 8) as the tile GEMM with the norm in its bf16 pass and
+// the epilogue in the launch that sums its K splits; everything else runs the same arithmetic as separate launches.
 int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out, const float* gain,
                                      float eps, const float* residual, int32_t epilogue) {
     if (ensure_device() != 0) return -1;
@@ -304,6 +307,14 @@ int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x
     if (w->encoding == ENC_Q4_K && m <= 2) {
         const int r = launch_q4k_gemv_rows_fused(w->data, x, out, w->cols, w->rows, m, gain, eps, residual, epilogue, nullptr);
         if (r != 0) return r < 0 ? -1 : 0;
+    }
+    if (m > 8 && is_packed(w->encoding)) {
+        // prompt shapes: the norm rides in the pass that rounds the activations to bf16, the epilogue in the launch that
+        // sums K splits (no split: a row kernel over the plain product, parked in tmp)
+        float* tmp = epilogue != 0 ? static_cast<float*>(scratch_get(t_fuse[1], sizeof(float) * (size_t)m * w->rows)) : nullptr;
+        if (epilogue != 0 && !tmp) return -1;
+        const int r = launch_gemm_fused(w->encoding, w->data, x, m, w->cols, w->rows, out, gain, eps, residual, epilogue, tmp);
+        if (r <= 0) return r;
     }
     const float* xin = x;
     if (gain) {

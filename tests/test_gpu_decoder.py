@@ -136,7 +136,9 @@ def test_rope_qkv_equals_three_scatters(hip_backend, torch_cuda):
 
 @pytest.mark.parametrize("enc,n,k,m", [("Q4_K", 1536, 1024, 1), ("Q4_K", 1030, 512, 2), ("Q4_K", 24, 4096 + 256, 1),
                                         ("Q4_K", 640, 512, 5), ("Q6_K", 512, 512, 1), ("Q4_K", 768, 1024, 24),
-                                        ("Q4_K", 1030, 14336, 1), ("Q4_K", 26, 16640, 1), ("Q4_K", 4096, 12288, 1)])
+                                        ("Q4_K", 1030, 14336, 1), ("Q4_K", 26, 16640, 1), ("Q4_K", 4096, 12288, 1),
+                                        ("Q4_K", 300, 512, 40), ("Q6_K", 258, 1024, 33), ("Q8_0", 130, 2048, 64),
+                                        ("Q4_K", 64, 5120, 300), ("Q8_0", 66, 96, 12)])
 def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
     """Every prologue / epilogue combination against float64 arithmetic on the oracle-decoded weight; the decode
     shapes of Q4_K run the one-kernel route (also with K of several passes), the other cases the composed route of the
@@ -165,6 +167,20 @@ def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
                            residual=out if epi == kx.EPI_RESIDUAL else None, epilogue=epi)   # residual aliases the output
             kx.sync()
             assert max_norm_err(out.cpu().numpy(), want) < tol, (use_gain, epi)
+    if m > 8 and k % 256 == 0:
+        # the same through forced K splits: the epilogue then runs in the launch that sums the splits
+        try:
+            for ks in (2, 3):
+                kx.set_tuning("gemm_ksplit", ks)
+                for epi in (kx.EPI_RESIDUAL, kx.EPI_SWIGLU):
+                    p = xn @ wd.T
+                    want = p + res if epi == kx.EPI_RESIDUAL else p[:, 0::2] / (1 + np.exp(-p[:, 0::2])) * p[:, 1::2]
+                    out = dev(torch, res.copy()) if epi == kx.EPI_RESIDUAL else torch.full((m, want.shape[1]), 9.0, device="cuda")
+                    w.matmul_fused(d_x, m, out, gain=d_gain, eps=eps, residual=out if epi == kx.EPI_RESIDUAL else None, epilogue=epi)
+                    kx.sync()
+                    assert max_norm_err(out.cpu().numpy(), want) < tol, (ks, epi)
+        finally:
+            kx.set_tuning("gemm_ksplit", 0)
     from skainet_amd._lib import HipError
     with pytest.raises(HipError):
         w.matmul_fused(d_x, m, out, epilogue=kx.EPI_RESIDUAL)          # residual epilogue without a residual
