@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-graph] [--skip-cpu]
 
 A "step" is one pass of the hot path over one batch of synthetic input: one y = W.x product with the packed
-weight already resident in HBM. Workload (BASELINE.json configs[1]): W 11008x4096 ~ N(0, 0.02^2) quantised to GGUF
+weight already resident in HBM. Default workload (the configuration the metric is quoted on): W 11008x4096 ~ N(0, 0.02^2) quantised to GGUF
 Q4_K (25 362 432 B), x ~ N(0, 1) fp32[4096], batch 1. Consecutive steps read DIFFERENT copies of the weight
 (enough copies to exceed twice the 256 MB memory-side cache), so the reported rate is an HBM rate, not a cache rate;
 the cache-warm figure (one copy) is reported next to it under "extra".
