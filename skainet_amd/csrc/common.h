@@ -71,6 +71,12 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
     return __uint_as_float(bits);
 }
 
+// RoPE rotation of an adjacent pair by (cos, sin), with the roundings spelled out so that every kernel that rotates
+// (prompt scatter, decode epilogue) produces the same bits whatever the compiler contracts elsewhere.
+__device__ __forceinline__ float2 rope_rotate(float x0, float x1, float cs, float sn) {
+    return make_float2(__fmaf_rn(x0, cs, -__fmul_rn(x1, sn)), __fmaf_rn(x0, sn, __fmul_rn(x1, cs)));
+}
+
 // Hardware fp16 -> fp32 (v_cvt_f32_f16): one instruction; used where the result feeds tolerance-checked sums.
 __device__ __forceinline__ float half_bits_to_float_fast(uint32_t h) {
     const uint16_t b = (uint16_t)h;

@@ -86,7 +86,7 @@ __device__ __forceinline__ void q4k_rows_epilogue(float val, int lane, int row, 
                 float sn, cs;
                 if (rope.table) { const float2 t = rope.table[dd >> 1]; cs = t.x; sn = t.y; }
                 else sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
-                out2 = make_float2(val * cs - odd * sn, val * sn + odd * cs);
+                out2 = rope_rotate(val, odd, cs, sn);
             }
             float* dst;
             if (slot < rope.heads) dst = y + (int64_t)slot * rope.head_dim;

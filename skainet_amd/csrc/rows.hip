@@ -266,8 +266,7 @@ __global__ __launch_bounds__(256) void rope_scatter_kernel(const float* __restri
         const float freq = powf(theta, -2.0f * (float)i / (float)head_dim);
         float sn, cs;
         sincosf((float)(p0 + t) * freq, &sn, &cs);
-        y.x = x.x * cs - x.y * sn;
-        y.y = x.x * sn + x.y * cs;
+        y = rope_rotate(x.x, x.y, cs, sn);
     }
     const int row = (out_row_is_pos ? p0 : 0) + t;
     *reinterpret_cast<float2*>(out + h * out_head_stride + (int64_t)row * head_dim + 2 * i) = y;
@@ -276,32 +275,42 @@ __global__ __launch_bounds__(256) void rope_scatter_kernel(const float* __restri
 // The three scatters of a decoder block in one launch: token rows of [q | k | v] (heads, kv_heads, kv_heads heads of
 // head_dim) -> rotated queries [heads, tokens, head_dim], rotated keys and raw values into cache rows p0 + t of
 // [kv_heads, kv_capacity, head_dim] caches. p0 = *pos_dev when given, else pos_start.
+// A thread owns one (token, pair) and walks ROPE_SLOTS_PER_BLOCK head slots with it: the angle's sine and cosine are
+// worked out once per thread instead of once per element (same expressions as before, so the same bits).
+constexpr int ROPE_SLOTS_PER_BLOCK = 8;
 __global__ __launch_bounds__(256) void rope_qkv_kernel(const float* __restrict__ qkv, float* __restrict__ q_out,
                                                        float* __restrict__ k_cache, float* __restrict__ v_cache, int tokens,
                                                        int heads, int kv_heads, int head_dim, int kv_capacity, int pos_start,
                                                        const int32_t* __restrict__ pos_dev, float theta) {
     const int half = head_dim >> 1;
     const int slots = heads + 2 * kv_heads;
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (token, head slot, pair)
-    if (idx >= (int64_t)tokens * slots * half) return;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (token, pair)
+    if (idx >= (int64_t)tokens * half) return;
     const int i = (int)(idx % half);
-    const int hs = (int)((idx / half) % slots);
-    const int t = (int)(idx / ((int64_t)half * slots));
+    const int t = (int)(idx / half);
     const int p0 = pos_dev ? pos_dev[0] : pos_start;
-    const float2 x = *reinterpret_cast<const float2*>(qkv + ((int64_t)t * slots + hs) * head_dim + 2 * i);
-    float2 y = x;
-    if (hs < heads + kv_heads) {
-        const float freq = powf(theta, -2.0f * (float)i / (float)head_dim);
-        float sn, cs;
-        sincosf((float)(p0 + t) * freq, &sn, &cs);
-        y.x = x.x * cs - x.y * sn;
-        y.y = x.x * sn + x.y * cs;
+    const float freq = powf(theta, -2.0f * (float)i / (float)head_dim);
+    float sn, cs;
+    sincosf((float)(p0 + t) * freq, &sn, &cs);
+    const int hs0 = blockIdx.y * ROPE_SLOTS_PER_BLOCK;
+    float2 x[ROPE_SLOTS_PER_BLOCK];
+#pragma unroll
+    for (int u = 0; u < ROPE_SLOTS_PER_BLOCK; ++u)
+        x[u] = *reinterpret_cast<const float2*>(qkv + ((int64_t)t * slots + min(hs0 + u, slots - 1)) * head_dim + 2 * i);
+#pragma unroll
+    for (int u = 0; u < ROPE_SLOTS_PER_BLOCK; ++u) {
+        const int hs = hs0 + u;
+        if (hs >= slots) break;
+        float2 y = x[u];
+        if (hs < heads + kv_heads) {
+            y = rope_rotate(x[u].x, x[u].y, cs, sn);
+        }
+        float* dst;
+        if (hs < heads) dst = q_out + ((int64_t)hs * tokens + t) * head_dim;
+        else if (hs < heads + kv_heads) dst = k_cache + ((int64_t)(hs - heads) * kv_capacity + p0 + t) * head_dim;
+        else dst = v_cache + ((int64_t)(hs - heads - kv_heads) * kv_capacity + p0 + t) * head_dim;
+        *reinterpret_cast<float2*>(dst + 2 * i) = y;
     }
-    float* dst;
-    if (hs < heads) dst = q_out + ((int64_t)hs * tokens + t) * head_dim;
-    else if (hs < heads + kv_heads) dst = k_cache + ((int64_t)(hs - heads) * kv_capacity + p0 + t) * head_dim;
-    else dst = v_cache + ((int64_t)(hs - heads - kv_heads) * kv_capacity + p0 + t) * head_dim;
-    *reinterpret_cast<float2*>(dst + 2 * i) = y;
 }
 
 // [heads, tokens, head_dim] -> [tokens, heads * head_dim]: attention output back to the token-major rows a projection takes.
@@ -372,8 +381,9 @@ int launch_rope_qkv(const float* qkv, float* q_out, float* k_cache, float* v_cac
     if (head_dim & 1) return set_error("rope: head_dim must be even; got %d", head_dim);
     if (!pos_dev && (pos_start < 0 || pos_start + tokens > kv_capacity))
         return set_error("rope_qkv: positions [%d, %d) do not fit a cache of %d rows", pos_start, pos_start + tokens, kv_capacity);
-    const int64_t n = (int64_t)tokens * (heads + 2 * kv_heads) * (head_dim / 2);
-    rope_qkv_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, current_stream()>>>(
+    const int64_t n = (int64_t)tokens * (head_dim / 2);
+    const int slot_blocks = (heads + 2 * kv_heads + ROPE_SLOTS_PER_BLOCK - 1) / ROPE_SLOTS_PER_BLOCK;
+    rope_qkv_kernel<<<dim3((unsigned)((n + 255) / 256), slot_blocks), dim3(256), 0, current_stream()>>>(
         qkv, q_out, k_cache, v_cache, tokens, heads, kv_heads, head_dim, kv_capacity, pos_start, pos_dev, theta);
     SKH_CHECK(hipGetLastError());
     return 0;
