@@ -24,6 +24,26 @@ def test_header_and_binding_table_agree():
     assert sorted(_lib.SIGNATURES) == names
 
 
+@pytest.mark.parametrize("compiler,lang", [("gcc", "c"), ("g++", "c++")])
+def test_header_is_plain_c_and_cpp(compiler, lang, tmp_path):
+    """The boundary is a C ABI: the header compiles on its own as C and as C++ (no torch or HIP types in it), and a
+    program written against it links with nothing but the shared library."""
+    import shutil
+    import subprocess
+    if shutil.which(compiler) is None:
+        pytest.skip(f"{compiler} not installed")
+    src = tmp_path / ("use." + ("c" if lang == "c" else "cpp"))
+    src.write_text('#include "skainet_hip.h"\n#include <stdio.h>\n'
+                   'int main(void) { printf("%d\\n", (int)skainet_hip_available()); return 0; }\n')
+    exe = tmp_path / "use"
+    pkg = os.path.dirname(_lib.HIP_LIB_PATH)
+    r = subprocess.run([compiler, "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                        "-L", pkg, "-lskainet_hip", f"-Wl,-rpath,{pkg}"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0 and run.stdout.strip() in ("0", "1"), (run.stdout, run.stderr)
+
+
 def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.HIP_LIB_PATH)
     missing = [n for n in declared_symbols() if not hasattr(lib, n)]
