@@ -24,15 +24,20 @@ namespace skh {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int G_WTN = 2;                                      // 32-column MFMA tiles per wave along N (rows: always 4)
+// The tile comes in two widths, WTN = 2 or 4 32-column MFMA tiles per wave along N (rows: always 4): 256 x 128 and
+// 256 x 256. Per K step a CU's LDS moves 144 KB for the narrow tile (1152 cycles at 128 B/clk against the 1024 cycles of
+// its MFMAs; measured in isolation, 32 MFMAs take 505 ns, with the 24 fragment reads 688 ns, with the 12 tile stores
+// 820 ns: a wave that issues an LDS instruction is held while the LDS moves its 1 KB) and 192 KB for the wide tile with
+// twice the MFMAs, so the wide tile is the one that can keep the matrix cores busy; it needs 32 tiles per CU round
+// fewer to fill the chip, so it serves the wide weights (N >= 128 rows per CU) and the narrow one the rest.
 constexpr int G_WAVES_M = 2, G_WAVES_N = 2;
-constexpr int GM = 128 * G_WAVES_M, GN = 32 * G_WTN * G_WAVES_N, GK = 64;
+constexpr int GM = 128 * G_WAVES_M, GK = 64;
 constexpr int G_THREADS = G_WAVES_M * G_WAVES_N * 64;
 constexpr int G_A_LOADS = GM * (GK / 8) / G_THREADS;          // 16-byte chunks of the activation tile per thread
-constexpr int G_W_TASKS = GN * 2 / G_THREADS;                 // 32-weight decode tasks per thread and step
 constexpr int GSTRIDE = GK + 8;                               // bf16 elements per LDS row (144 bytes)
-constexpr int G_A_ELEMS = GM * GSTRIDE, G_W_ELEMS = GN * GSTRIDE;
-constexpr size_t G_SMEM = 2 * (size_t)(G_A_ELEMS + G_W_ELEMS) * sizeof(__bf16);   // two stages
+constexpr int G_A_ELEMS = GM * GSTRIDE;
+constexpr int gemm_gn(int wtn) { return 32 * wtn * G_WAVES_N; }
+constexpr size_t gemm_smem(int wtn) { return 2 * (size_t)(G_A_ELEMS + gemm_gn(wtn) * GSTRIDE) * sizeof(__bf16); }   // two stages
 
 void* kernel_workspace(size_t bytes);   // shim.hip
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);   // gemv.hip
@@ -290,34 +295,50 @@ template <> struct DecOf<RawQ80> { typedef DecQ80 type; };
 template <int FMT> struct DecOf<RawQ45<FMT>> { typedef DecQ45 type; };
 template <> struct DecOf<RawQ5K> { typedef DecQ5K type; };
 
-typedef __bf16 gemm_bf16x4 __attribute__((ext_vector_type(4)));
-// part I (0..7) of a thread's 32 weights -> 4 bf16 values
-template <int I, class Raw, class Dec>
-__device__ __forceinline__ gemm_bf16x4 decode_part(const Raw& r, const Dec& c) {
+typedef __bf16 gemm_bf16x2 __attribute__((ext_vector_type(2)));
+// Half H (0 / 1) of part I (0..7) of a thread's 32 weights -> weights 4 I + 2 H and 4 I + 2 H + 1 as one packed bf16
+// pair. The part's whole 4-weight expression is written out and the unused half is dropped by the compiler, so a
+// half is about seven vector instructions: what fits between two MFMAs without holding the matrix core up.
+template <int I, int H, class Raw, class Dec>
+__device__ __forceinline__ uint32_t decode_half(const Raw& r, const Dec& c) {
     float w4[4];
     decode_dword<I>(r, c, w4);
-    return gemm_bf16x4{(__bf16)w4[0], (__bf16)w4[1], (__bf16)w4[2], (__bf16)w4[3]};
+    return __builtin_bit_cast(uint32_t, gemm_bf16x2{(__bf16)w4[2 * H], (__bf16)w4[2 * H + 1]});
 }
-
-// part I of a thread's 32 weights with I a (constant-folded) loop variable
+// half-part h (0..15) with h a (constant-folded) loop variable
 template <class Raw, class Dec>
-__device__ __forceinline__ gemm_bf16x4 decode_part_at(int i, const Raw& r, const Dec& c) {
-    switch (i) {
-        case 0: return decode_part<0>(r, c);
-        case 1: return decode_part<1>(r, c);
-        case 2: return decode_part<2>(r, c);
-        case 3: return decode_part<3>(r, c);
-        case 4: return decode_part<4>(r, c);
-        case 5: return decode_part<5>(r, c);
-        case 6: return decode_part<6>(r, c);
-        default: return decode_part<7>(r, c);
+__device__ __forceinline__ uint32_t decode_half_at(int h, const Raw& r, const Dec& c) {
+    switch (h) {
+        case 0: return decode_half<0, 0>(r, c);
+        case 1: return decode_half<0, 1>(r, c);
+        case 2: return decode_half<1, 0>(r, c);
+        case 3: return decode_half<1, 1>(r, c);
+        case 4: return decode_half<2, 0>(r, c);
+        case 5: return decode_half<2, 1>(r, c);
+        case 6: return decode_half<3, 0>(r, c);
+        case 7: return decode_half<3, 1>(r, c);
+        case 8: return decode_half<4, 0>(r, c);
+        case 9: return decode_half<4, 1>(r, c);
+        case 10: return decode_half<5, 0>(r, c);
+        case 11: return decode_half<5, 1>(r, c);
+        case 12: return decode_half<6, 0>(r, c);
+        case 13: return decode_half<6, 1>(r, c);
+        case 14: return decode_half<7, 0>(r, c);
+        default: return decode_half<7, 1>(r, c);
     }
 }
 
-template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES>
+template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES, int WTN>
 __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
                                                            float* __restrict__ c, int m, int n, int k, int k_chunk,
                                                            int64_t split_stride) {
+    constexpr int G_WTN = WTN, GN = gemm_gn(WTN);
+    constexpr int G_W_TASKS = GN * 2 / G_THREADS;             // 32-weight decode tasks per thread and step
+    constexpr int G_W_ELEMS = GN * GSTRIDE;
+    // Register slots of the activation ring. Narrow tile: two (requested two steps ahead, like the weights). Wide tile:
+    // one -- the second slot's 32 registers are what the 256 accumulators leave no room for: a step parks the slot in
+    // LDS at its end and requests the step after next into it right away, a full step ahead of its own parking.
+    constexpr int A_SLOTS = WTN == 2 ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) __bf16 smem[];
     // stage `buf` (0 / 1): activation tile, then weight tile
     auto a_tile = [&](int buf) { return smem + buf * (G_A_ELEMS + G_W_ELEMS); };
@@ -343,27 +364,32 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     // to be used. Loads are unconditional (clamped rows, never stored) so a step's loads are in flight together.
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     typedef typename DecOf<Raw>::type Dec;
-    u32x4 aring[2][G_A_LOADS];
+    u32x4 aring[A_SLOTS][G_A_LOADS];
     Raw wring[2][G_W_TASKS];
     auto step_k = [&](int step) { return k_begin + min(step, nsteps - 1) * GK; };   // loads past the end re-read the last step
-    auto load_step = [&](int slot, int step) __attribute__((always_inline)) {
-        const int k0 = step_k(step);
+    auto load_a_chunk = [&](int slot, int step, int j) __attribute__((always_inline)) {
+        const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
+        aring[slot][j] = *reinterpret_cast<const u32x4*>(a + (int64_t)min(m0 + row, m - 1) * k + step_k(step) + 8 * kp);
+    };
+    auto load_a = [&](int slot, int step) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < G_A_LOADS; ++j) {
-            const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
-            aring[slot][j] = *reinterpret_cast<const u32x4*>(a + (int64_t)min(m0 + row, m - 1) * k + k0 + 8 * kp);
-        }
+        for (int j = 0; j < G_A_LOADS; ++j) load_a_chunk(slot, step, j);
+    };
+    auto load_w_task = [&](int slot, int step, int t) __attribute__((always_inline)) {
+        load_raw(wring[slot][t], wrow_ptr[t], step_k(step) + 32 * wsub);
+    };
+    auto load_w = [&](int slot, int step) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < G_W_TASKS; ++t) load_raw(wring[slot][t], wrow_ptr[t], k0 + 32 * wsub);
+        for (int t = 0; t < G_W_TASKS; ++t) load_w_task(slot, step, t);
     };
     auto park_a = [&](int slot, int stage, int j) __attribute__((always_inline)) {      // chunk j of a step's activation tile -> LDS stage
         const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
         *reinterpret_cast<u32x4*>(a_tile(stage) + row * GSTRIDE + 8 * kp) = aring[slot][j];
     };
-    gemm_bf16x4 wp[G_W_TASKS][8];
+    uint32_t wp[G_W_TASKS][16];                                                         // packed bf16 pairs: weights 2 h, 2 h + 1
     auto park_w = [&](int stage, int t, int i) __attribute__((always_inline)) {         // weights 8 i .. 8 i + 7 of task t's 32
         __bf16* dst = w_tile(stage) + (wrow + (G_THREADS / 2) * t) * GSTRIDE + 32 * wsub;
-        *reinterpret_cast<bf16x8*>(dst + 8 * i) = __builtin_shufflevector(wp[t][2 * i], wp[t][2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+        *reinterpret_cast<u32x4*>(dst + 8 * i) = u32x4{wp[t][4 * i], wp[t][4 * i + 1], wp[t][4 * i + 2], wp[t][4 * i + 3]};
     };
 
     f32x16 acc[4][G_WTN];
@@ -376,16 +402,29 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
 
     const int fr = lane & 31, fk = (lane >> 5) * 8;   // fragment row inside a 32-row tile, first k of this lane's 8
 
-    // One K step of a wave: its MFMAs on LDS stage `stage`, with everything that prepares the NEXT step placed between
-    // them in program order -- the fragment reads of the next 16-wide slice, the decode of the next step's weights in
-    // 4-weight parts, the LDS stores into the other stage. A wave issues in order and an MFMA occupies the matrix core
-    // for 32 cycles: what sits between two MFMAs runs for free, what sits after the last one is paid for.
-    // sched_barrier(0) pins the order. The decode parts are spread over the first MFMAs, the LDS stores take one slot
-    // each behind the last N_STORES MFMAs (every weight chunk after its parts, the activation chunks as late as possible).
-    auto step_body = [&](int stage, int slot_next, int step_next) __attribute__((always_inline)) {
-        constexpr int N_MFMA = 4 * G_WTN * (GK / 16), N_PARTS = 8 * G_W_TASKS, N_STORES = G_A_LOADS + 4 * G_W_TASKS;
-        constexpr int PSTRIDE = (N_MFMA - N_STORES) / N_PARTS;      // a decode part after every PSTRIDE-th MFMA
-        static_assert(PSTRIDE >= 1, "more work items than slots between the MFMAs");
+    // One K step of a wave: its MFMAs on LDS stage `stage`, with everything that prepares the steps after it placed
+    // between them in program order. A wave issues in order and an MFMA occupies the matrix core for 32 cycles: about
+    // seven vector instructions between two MFMAs run for free, what sits in front of the first MFMA or behind the last
+    // one is paid for in full -- so nothing but the first fragment reads precedes the first MFMA. sched_barrier(0)
+    // pins the order:
+    //   behind MFMA t (t < tasks)            the global loads of weight task t for step `load_step` (ring slot `load_slot`)
+    //   behind MFMA tasks + t                the scale / offset header of task t of the next step's weights
+    //   behind the following MFMAs           the next step's weights, decoded in two-weight items of about seven
+    //                                        instructions, evenly spread (a four-weight item behind every third MFMA
+    //                                        held the matrix core up each time)
+    //                                        (refilling the registers right behind their last use instead, for a load
+    //                                        lead of well over a step, changed nothing: the waits are not a lead problem)
+    //   behind the slice's first MFMA        the fragment reads of the next 16-wide slice
+    //   behind the last N_STORES MFMAs       one LDS store each into the other stage: every weight chunk after its
+    //                                        items, the activation chunks as late as possible, each followed by the
+    //                                        global load that refills its ring register
+    auto step_body = [&](int stage, int slot_next, int step_next, int load_slot, int load_step) __attribute__((always_inline)) {
+        const int a_slot_next = A_SLOTS == 2 ? slot_next : 0;
+        const int a_load_slot = A_SLOTS == 2 ? load_slot : 0, a_load_step = A_SLOTS == 2 ? load_step : step_next + 1;
+        constexpr int N_MFMA = 4 * G_WTN * (GK / 16), N_HALVES = 16 * G_W_TASKS, N_STORES = G_A_LOADS + 4 * G_W_TASKS;
+        constexpr int FIRST_ITEM = 2 * G_W_TASKS;                  // MFMAs whose slots hold the loads and the headers
+        constexpr int N_GAPS = N_MFMA - N_STORES - FIRST_ITEM;      // MFMAs with a decode slot behind them
+        static_assert(N_GAPS >= N_HALVES, "more decode items than slots between the MFMAs");
         const __bf16* at = a_tile(stage) + (128 * wm + fr) * GSTRIDE + fk;
         const __bf16* wt = w_tile(stage) + (32 * G_WTN * wn + fr) * GSTRIDE + fk;
         bf16x8 af[2][4], bf[2][G_WTN];
@@ -397,8 +436,6 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
         };
         Dec dc[G_W_TASKS];
         frags(0, 0);
-#pragma unroll
-        for (int t = 0; t < G_W_TASKS; ++t) decode_prepare(wring[slot_next][t], step_k(step_next) + 32 * wsub, dc[t]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma clang loop unroll(full)
         for (int q = 0; q < N_MFMA; ++q) {
@@ -409,20 +446,32 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
                 frags(set ^ 1, 16 * (kk + 1));
                 __builtin_amdgcn_sched_barrier(0);
             }
-
-            if (q < N_PARTS * PSTRIDE && q % PSTRIDE == PSTRIDE - 1) {
-                const int item = q / PSTRIDE;
-                wp[item / 8][item % 8] = decode_part_at(item % 8, wring[slot_next][item / 8], dc[item / 8]);
+            if (q < G_W_TASKS) {
+                load_w_task(load_slot, load_step, q);
                 __builtin_amdgcn_sched_barrier(0);
-            }
-            if (q >= N_MFMA - N_STORES) {
+            } else if (q < FIRST_ITEM) {
+                const int t = q - G_W_TASKS;
+                decode_prepare(wring[slot_next][t], step_k(step_next) + 32 * wsub, dc[t]);
+                __builtin_amdgcn_sched_barrier(0);
+            } else if (q < FIRST_ITEM + N_GAPS) {
+                // decode item h sits behind MFMA FIRST_ITEM + h * N_GAPS / N_HALVES: evenly spread, at most one per slot
+                const int g = q - FIRST_ITEM;
+                const int h0 = (g * N_HALVES + N_GAPS - 1) / N_GAPS, h1 = ((g + 1) * N_HALVES + N_GAPS - 1) / N_GAPS;
+                if (h0 < h1 && h0 < N_HALVES) {
+                    wp[h0 / 16][h0 % 16] = decode_half_at(h0 % 16, wring[slot_next][h0 / 16], dc[h0 / 16]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
                 // first the weight chunks of all but the last task, then the activation chunks (their loads are the
                 // youngest), then the last task's weight chunks
                 const int sidx = q - (N_MFMA - N_STORES);
                 constexpr int W_FIRST = 4 * (G_W_TASKS - 1);
                 if (sidx < W_FIRST) park_w(stage ^ 1, sidx / 4, sidx % 4);
-                else if (sidx < W_FIRST + G_A_LOADS) park_a(slot_next, stage ^ 1, sidx - W_FIRST);
-                else park_w(stage ^ 1, G_W_TASKS - 1, sidx - W_FIRST - G_A_LOADS);
+                else if (sidx < W_FIRST + G_A_LOADS) {
+                    park_a(a_slot_next, stage ^ 1, sidx - W_FIRST);
+                    if (A_SLOTS == 1) load_a_chunk(0, a_load_step, sidx - W_FIRST);   // the register has just been parked
+                } else park_w(stage ^ 1, G_W_TASKS - 1, sidx - W_FIRST - G_A_LOADS);
+                if (A_SLOTS == 2 && sidx < G_A_LOADS) load_a_chunk(a_load_slot, a_load_step, sidx);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -431,7 +480,8 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     // nsteps is a multiple of 4 (K chunks are whole 256-element groups) and > 0. The loop body is one straight-line
     // block (no branches), which is what lets the compiler's wait-count bookkeeping leave the newest step's loads in
     // flight while the older ones are parked.
-    load_step(0, 0);
+    load_a(0, 0);
+    load_w(0, 0);
 #pragma unroll
     for (int j = 0; j < G_A_LOADS; ++j) park_a(0, 0, j);
 #pragma unroll
@@ -439,26 +489,40 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
         Dec d0;
         decode_prepare(wring[0][t], step_k(0) + 32 * wsub, d0);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) wp[t][i] = decode_part_at(i, wring[0][t], d0);
+        for (int h = 0; h < 16; ++h) wp[t][h] = decode_half_at(h, wring[0][t], d0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) park_w(0, t, i);
     }
-    load_step(1, 1);
+    load_a(A_SLOTS == 2 ? 1 : 0, 1);
+    load_w(1, 1);
     __syncthreads();
     for (int s0 = 0; s0 < nsteps; s0 += 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int step = s0 + u;
-            // ring slot u held this step's bytes (parked one step ago): refill it with the step after next
-            load_step(u, step + 2);
-            // MFMAs of this step on stage u; step + 1 (ring slot u ^ 1) is decoded and parked in stage u ^ 1 meanwhile
-            step_body(u, u ^ 1, step + 1);
+            // MFMAs of this step on stage u; step + 1 (ring slot u ^ 1) is decoded and parked in stage u ^ 1 meanwhile;
+            // ring slot u held this step's bytes (parked one step ago) and is refilled with the step after next (the
+            // wide tile's single activation slot: chunk by chunk behind its parking, with the step after next)
+            step_body(u, u ^ 1, step + 1, u, step + 2);
             __syncthreads();
         }
     }
 
     float* cz = c + (int64_t)blockIdx.z * split_stride;      // split K: this split's partial product
-    // accumulator element e of lane l sits at row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32 of its 32 x 32 tile
+    // accumulator element e of lane l sits at row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32 of its 32 x 32 tile.
+    // A tile that lies inside C stores without guards: a guard is a branch per store, and at the join after a branch
+    // the stores queue one behind the other (the compiler waits for everything in flight there).
+    if (m0 + GM <= m && n0 + GN <= n) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < G_WTN; ++j) {
+                float* dst = cz + (int64_t)(m0 + 128 * wm + 32 * i + 4 * (lane >> 5)) * n + n0 + 32 * G_WTN * wn + 32 * j + (lane & 31);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) dst[(int64_t)(8 * (e >> 2) + (e & 3)) * n] = acc[i][j][e];
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -475,22 +539,30 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
         }
 }
 
-template <class Raw, int BE, int BB>
-static int launch_gemm_enc(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
-                           int64_t split_stride, hipStream_t s) {
+template <class Raw, int BE, int BB, int WTN>
+static int launch_gemm_tile(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
+                            int64_t split_stride, hipStream_t s) {
     static bool attr_set = false;
     if (!attr_set) {
-        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&dequant_gemm_kernel<Raw, BE, BB>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)G_SMEM));
+        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&dequant_gemm_kernel<Raw, BE, BB, WTN>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_smem(WTN)));
         attr_set = true;
     }
-    dequant_gemm_kernel<Raw, BE, BB><<<grid, dim3(G_THREADS), G_SMEM, s>>>(a, w, c, m, n, k, k_chunk, split_stride);
+    dequant_gemm_kernel<Raw, BE, BB, WTN><<<grid, dim3(G_THREADS), gemm_smem(WTN), s>>>(a, w, c, m, n, k, k_chunk, split_stride);
     SKH_CHECK(hipGetLastError());
     return 0;
+}
+template <class Raw, int BE, int BB>
+static int launch_gemm_enc(int wtn, const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
+                           int64_t split_stride, hipStream_t s) {
+    if (wtn == 4) return launch_gemm_tile<Raw, BE, BB, 4>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    return launch_gemm_tile<Raw, BE, BB, 2>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
 }
 
 static int g_gemm_ksplit = 0;   // 0 = choose from the tile count
 void set_gemm_ksplit(int v) { g_gemm_ksplit = v; }
+static int g_gemm_wide = -1;    // -1 = choose from the shape, 0 / 1 = narrow / wide tile
+void set_gemm_wide(int v) { g_gemm_wide = v; }
 
 // y = epilogue(prologue(x) . W^T): gain != null normalises every activation row first (RMSNorm, folded into the pass that
 // rounds the activations to bf16); epilogue is one of GEMM_EPI_* (residual [m, n] may be y; SwiGLU: y is [m, n / 2]).
@@ -512,7 +584,12 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         (epilogue != GEMM_EPI_NONE && !tmp))
         return fused ? 1 : launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
-    const int tiles_m = (m + GM - 1) / GM, tiles_n = (n + GN - 1) / GN;
+    // the wide tile where it alone fills most of the chip in one round
+    const int tiles_m = (m + GM - 1) / GM;
+    const int wide_tiles = tiles_m * ((n + gemm_gn(4) - 1) / gemm_gn(4));
+    const bool wide = g_gemm_wide >= 0 ? g_gemm_wide != 0 : 4 * wide_tiles >= 3 * num_cus();
+    const int wtn = wide ? 4 : 2;
+    const int tiles_n = (n + gemm_gn(wtn) - 1) / gemm_gn(wtn);
     const int tiles = tiles_m * tiles_n;
     // K chunks are whole 256-element groups so every encoding's blocks stay intact
     const int kgroups = (k + 255) / 256;
@@ -527,7 +604,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         for (int ks = 1; ks <= 8 && ks <= kgroups; ++ks) {
             const int rounds = (tiles * ks + cus - 1) / cus;
             const int steps = ((kgroups + ks - 1) / ks) * (256 / GK);
-            double t = rounds * (8.0 + 1.04 * steps);
+            double t = rounds * (8.0 + (wide ? 2.0 : 1.04) * steps);
             if (ks > 1) t += 2.3 + (double)(ks + 1) * m * n * 4.0 / 8.0e6;
             if (ks == 1 || t < best) { best = t; ksplit = ks; }
         }
@@ -550,13 +627,13 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     const dim3 grid(tiles_n, tiles_m, ksplit);
     float* c = ksplit > 1 ? part : (epilogue != GEMM_EPI_NONE ? tmp : y);
     int rc;
-    if (enc == ENC_Q4_K) rc = launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q6_K) rc = launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q5_K) rc = launch_gemm_enc<RawQ5K, QK_ELEMS, Q5K_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q4_0) rc = launch_gemm_enc<RawQ45<0>, Q80_ELEMS, Q40_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q5_0) rc = launch_gemm_enc<RawQ45<1>, Q80_ELEMS, Q50_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q5_1) rc = launch_gemm_enc<RawQ45<2>, Q80_ELEMS, Q51_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    if (enc == ENC_Q4_K) rc = launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q6_K) rc = launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_K) rc = launch_gemm_enc<RawQ5K, QK_ELEMS, Q5K_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q4_0) rc = launch_gemm_enc<RawQ45<0>, Q80_ELEMS, Q40_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_0) rc = launch_gemm_enc<RawQ45<1>, Q80_ELEMS, Q50_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_1) rc = launch_gemm_enc<RawQ45<2>, Q80_ELEMS, Q51_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     if (rc != 0) return rc;
     if (ksplit == 1) {
         if (epilogue == GEMM_EPI_RESIDUAL) return launch_add(residual, tmp, y, (int64_t)m * n);

@@ -451,6 +451,7 @@ static int launch_format(const uint8_t* w, const float* x, float* y, int k, int 
 static int g_gemv_waves_per_cu = 0;   // 0: per encoding (measured best: Q8_0 4, Q4_K / Q6_K 8)
 static int g_q4k_rows_enable = 1;
 void set_q4k_rows_waves_per_cu(int v);
+void set_gemm_wide(int v);
 void set_gemm_ksplit(int v);
 void set_sdpa_prefill_mfma(int v);
 int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch);   // gemv_q4k.hip
@@ -460,6 +461,7 @@ int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int
 int set_tuning(const char* key, int value) {
     if (!strcmp(key, "gemv_waves_per_cu")) { if (value >= 0) g_gemv_waves_per_cu = value; return 0; }
     if (!strcmp(key, "q4k_rows_waves_per_cu")) { set_q4k_rows_waves_per_cu(value); return 0; }
+    if (!strcmp(key, "gemm_wide")) { set_gemm_wide(value); return 0; }
     if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }
     if (!strcmp(key, "gemm_ksplit")) { set_gemm_ksplit(value); return 0; }
     if (!strcmp(key, "sdpa_prefill_mfma")) { set_sdpa_prefill_mfma(value); return 0; }

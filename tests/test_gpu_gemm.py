@@ -62,6 +62,15 @@ def test_gemm_ragged_tiles(hip_backend, torch_cuda, enc, m, n, k):
     # the automatic choice (m > 8 -> GEMM, else GEMV) gives the same product
     auto = gpu_gemm(hip_backend, torch_cuda, enc, packed, n, k, x, kind=None)
     check(auto, want)
+    # and so does the wide (256 x 256) tile, which the launcher would only pick for weights of many rows
+    try:
+        hip_backend.set_tuning("gemm_wide", 1)
+        wide = gpu_gemm(hip_backend, torch_cuda, enc, packed, n, k, x)
+        assert not np.isnan(wide).any()
+        check(wide, want)
+        check_exact(torch_cuda, enc, wide, x, packed, n)
+    finally:
+        hip_backend.set_tuning("gemm_wide", -1)
 
 
 @pytest.mark.parametrize("enc", ALL_ENCS)
@@ -72,13 +81,16 @@ def test_gemm_on_random_valid_blocks_and_forced_k_splits(hip_backend, torch_cuda
     x = np.random.default_rng(5).standard_normal((m, k)).astype(np.float32)
     want = L.gemv(enc, x, packed, n)
     try:
-        for ks in (1, 2, 3, 8):
-            hip_backend.set_tuning("gemm_ksplit", ks)
-            got = gpu_gemm(hip_backend, torch_cuda, enc, packed, n, k, x)
-            check(got, want)
-            check_exact(torch_cuda, enc, got, x, packed, n)
+        for wide in (0, 1):
+            hip_backend.set_tuning("gemm_wide", wide)
+            for ks in (1, 2, 3, 8):
+                hip_backend.set_tuning("gemm_ksplit", ks)
+                got = gpu_gemm(hip_backend, torch_cuda, enc, packed, n, k, x)
+                check(got, want)
+                check_exact(torch_cuda, enc, got, x, packed, n)
     finally:
         hip_backend.set_tuning("gemm_ksplit", 0)
+        hip_backend.set_tuning("gemm_wide", -1)
 
 
 @pytest.mark.parametrize("k", [96, 192, 320, 448])
