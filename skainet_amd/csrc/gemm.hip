@@ -174,8 +174,14 @@ __device__ __forceinline__ void load_raw(RawQ6K& r, const uint8_t* row, int e) {
     const int half = (e & 255) >> 7, kq = (e & 127) >> 5;   // quarter kq of the half: output offset 32 * kq
     const uint8_t* ql = blk + half * 64 + (kq & 1) * 32;
     const uint8_t* qh = blk + 128 + half * 32;
+    // two 16-byte loads per 32-byte run (2-byte aligned): 6 loads per task instead of 18, so that two steps of weights in
+    // flight stay far below the 63 loads a wave's memory counter can track
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { r.ql[i] = load_u32_a2(ql + 4 * i); r.qh[i] = load_u32_a2(qh + 4 * i); }
+    for (int h = 0; h < 2; ++h) {
+        const u32x4_vec l4 = load_u32x4_a2(ql + 16 * h), h4 = load_u32x4_a2(qh + 16 * h);
+        r.ql[4 * h] = l4.x; r.ql[4 * h + 1] = l4.y; r.ql[4 * h + 2] = l4.z; r.ql[4 * h + 3] = l4.w;
+        r.qh[4 * h] = h4.x; r.qh[4 * h + 1] = h4.y; r.qh[4 * h + 2] = h4.z; r.qh[4 * h + 3] = h4.w;
+    }
     // the two int8 scales of this quarter: sc[half * 8 + 2 * kq] (elements 0..15) and [.. + 1] (elements 16..31)
     r.sc = load_u16(blk + 192 + half * 8 + 2 * kq);
     r.d = load_u16(blk + 208);
