@@ -130,7 +130,16 @@ __global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float* __res
     for (int j = 0; j < 4 && i + j < total; ++j) c[i + j] = v[j];
 }
 
+// byte N of a dword as float, N a compile-time index
+template <int N>
+__device__ __forceinline__ float gemm_byte_to_float(uint32_t v) {
+    return N == 0 ? ubyte0_to_float(v) : N == 1 ? ubyte1_to_float(v) : N == 2 ? ubyte2_to_float(v) : ubyte3_to_float(v);
+}
+
 // ---- raw bytes a thread needs to decode 32 consecutive weights of one row, per encoding ----
+// Per encoding: load_raw (global loads of a thread's 32 weights), decode_prepare (scales of the 32), and the decode of
+// part I (0..7, four weights) in two stages the main loop places separately: decode_codes<I> gathers the part's four
+// codes into the bytes of one dword, decode_pair<I, H> turns bytes 2 H and 2 H + 1 of it into two fp32 weights.
 struct RawQ4K { uint4 hdr, q0, q1; };
 struct RawQ6K { uint32_t ql[8], qh[8]; uint32_t sc, d; };
 struct RawQ80 { u32x4_vec lo, hi; uint32_t edge, odd; };   // aligned 32-byte body, the 2 bytes outside it, start parity
@@ -152,21 +161,25 @@ __device__ __forceinline__ void decode_prepare(const RawQ4K& r, int e, DecQ4K& c
     // ggml get_scale_min_k4 on the 12 scale bytes s[0..11] (hdr.y = s[0..3], hdr.z = s[4..7], hdr.w = s[8..11])
     const int sh = (sb & 3) * 8;
     const uint32_t sa = (r.hdr.y >> sh) & 0xFFu, sbm = (r.hdr.z >> sh) & 0xFFu, st = (r.hdr.w >> sh) & 0xFFu;
-    const uint32_t sc = sb < 4 ? (sa & 63u) : ((st & 0xFu) | ((sa >> 6) << 4));
-    const uint32_t mn = sb < 4 ? (sbm & 63u) : ((st >> 4) | ((sbm >> 6) << 4));
+    // both packings are evaluated and one is picked with a mask: a select written as a conditional becomes a branch
+    // here, and a branch inside the K loop makes every wait behind it cover all the loads in flight
+    const uint32_t hi = (uint32_t)-(int)(sb >> 2);            // sb >= 4: all ones
+    const uint32_t sc = ((sa & 63u) & ~hi) | (((st & 0xFu) | ((sa >> 6) << 4)) & hi);
+    const uint32_t mn = ((sbm & 63u) & ~hi) | (((st >> 4) | ((sbm >> 6) << 4)) & hi);
     c.scale = d * (float)sc;
     c.offset = dmin * (float)mn;
     c.shift = (sb & 1) * 4;
 }
 template <int I>
-__device__ __forceinline__ void decode_dword(const RawQ4K& r, const DecQ4K& c, float* w4) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ4K& r, const DecQ4K& c) {
     const uint32_t q = I == 0 ? r.q0.x : I == 1 ? r.q0.y : I == 2 ? r.q0.z : I == 3 ? r.q0.w
                      : I == 4 ? r.q1.x : I == 5 ? r.q1.y : I == 6 ? r.q1.z : r.q1.w;
-    const uint32_t v = (q >> c.shift) & 0x0F0F0F0Fu;
-    w4[0] = fmaf(ubyte0_to_float(v), c.scale, -c.offset);
-    w4[1] = fmaf(ubyte1_to_float(v), c.scale, -c.offset);
-    w4[2] = fmaf(ubyte2_to_float(v), c.scale, -c.offset);
-    w4[3] = fmaf(ubyte3_to_float(v), c.scale, -c.offset);
+    return (q >> c.shift) & 0x0F0F0F0Fu;
+}
+template <int I, int H>
+__device__ __forceinline__ void decode_pair(uint32_t v, const DecQ4K& c, float& w0, float& w1) {
+    w0 = fmaf(gemm_byte_to_float<2 * H>(v), c.scale, -c.offset);
+    w1 = fmaf(gemm_byte_to_float<2 * H + 1>(v), c.scale, -c.offset);
 }
 
 __device__ __forceinline__ void load_raw(RawQ6K& r, const uint8_t* row, int e) {
@@ -186,25 +199,29 @@ __device__ __forceinline__ void load_raw(RawQ6K& r, const uint8_t* row, int e) {
     r.sc = load_u16(blk + 192 + half * 8 + 2 * kq);
     r.d = load_u16(blk + 208);
 }
-struct DecQ6K { float s0, s1; int nib, hs; };
+struct DecQ6K { float s0, s1, n0, n1; int nib, hs; };   // n = -32 s
 __device__ __forceinline__ void decode_prepare(const RawQ6K& r, int e, DecQ6K& c) {
     const int kq = (e & 127) >> 5;
     const float d = half_bits_to_float_fast(r.d);
     c.s0 = d * (float)(int8_t)(r.sc & 0xFF);
     c.s1 = d * (float)(int8_t)(r.sc >> 8);
+    c.n0 = -32.f * c.s0;
+    c.n1 = -32.f * c.s1;
     c.nib = (kq >> 1) * 4;
     c.hs = 2 * kq;
 }
 template <int I>
-__device__ __forceinline__ void decode_dword(const RawQ6K& r, const DecQ6K& c, float* w4) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ6K& r, const DecQ6K& c) {
     const uint32_t lo = (r.ql[I] >> c.nib) & 0x0F0F0F0Fu;
     const uint32_t hi = ((r.qh[I] >> c.hs) & 0x03030303u) << 4;
-    const uint32_t q = lo | hi;                              // four 6-bit codes, one per byte
-    const float sc = I < 4 ? c.s0 : c.s1;
-    w4[0] = sc * (ubyte0_to_float(q) - 32.f);
-    w4[1] = sc * (ubyte1_to_float(q) - 32.f);
-    w4[2] = sc * (ubyte2_to_float(q) - 32.f);
-    w4[3] = sc * (ubyte3_to_float(q) - 32.f);
+    return lo | hi;                                          // four 6-bit codes, one per byte
+}
+template <int I, int H>
+__device__ __forceinline__ void decode_pair(uint32_t v, const DecQ6K& c, float& w0, float& w1) {
+    // sc * (q - 32) as one FMA: q - 32 is exact and so is 32 * sc, so the single rounding gives the same bits
+    const float sc = I < 4 ? c.s0 : c.s1, off = I < 4 ? c.n0 : c.n1;
+    w0 = fmaf(gemm_byte_to_float<2 * H>(v), sc, off);
+    w1 = fmaf(gemm_byte_to_float<2 * H + 1>(v), sc, off);
 }
 
 __device__ __forceinline__ void load_raw(RawQ80& r, const uint8_t* row, int e) {
@@ -223,11 +240,14 @@ __device__ __forceinline__ void decode_prepare(const RawQ80& r, int, DecQ80& c) 
     c.drop = r.odd ? 0u : 2u;                        // bytes in front of the codes in the loaded dwords
 }
 template <int I>
-__device__ __forceinline__ void decode_dword(const RawQ80& r, const DecQ80& c, float* w4) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ80& r, const DecQ80& c) {
     const uint32_t v[9] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w, r.edge};
-    const uint32_t q = __builtin_amdgcn_alignbyte(v[I + 1], v[I], c.drop);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) w4[j] = (float)(int8_t)(q >> (8 * j)) * c.d;
+    return __builtin_amdgcn_alignbyte(v[I + 1], v[I], c.drop);
+}
+template <int I, int H>
+__device__ __forceinline__ void decode_pair(uint32_t q, const DecQ80& c, float& w0, float& w1) {
+    w0 = (float)(int8_t)(q >> (16 * H)) * c.d;
+    w1 = (float)(int8_t)(q >> (16 * H + 8)) * c.d;
 }
 
 // Q4_0 / Q5_0 / Q5_1 (FMT 0 / 1 / 2): a thread's 32 weights are one block -- fp16 d [fp16 m] [32 fifth bits], then 16 bytes
@@ -252,14 +272,16 @@ __device__ __forceinline__ void decode_prepare(const RawQ45<FMT>& r, int, DecQ45
     c.add = FMT == 0 ? -8.f * c.d : (FMT == 1 ? -16.f * c.d : half_bits_to_float_fast(r.m));
 }
 template <int I, int FMT>
-__device__ __forceinline__ void decode_dword(const RawQ45<FMT>& r, const DecQ45& c, float* w4) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ45<FMT>& r, const DecQ45&) {
     // parts 0..3: low nibbles of code dword I (elements 4I ..), parts 4..7: high nibbles of dword I - 4 (elements 16 + ..)
     uint32_t v = (r.q[I & 3] >> (I < 4 ? 0 : 4)) & 0x0F0F0F0Fu;
     if (FMT != 0) v |= ((((r.qh >> (4 * I)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;   // fifth bits 4I .. 4I + 3
-    w4[0] = fmaf(ubyte0_to_float(v), c.d, c.add);
-    w4[1] = fmaf(ubyte1_to_float(v), c.d, c.add);
-    w4[2] = fmaf(ubyte2_to_float(v), c.d, c.add);
-    w4[3] = fmaf(ubyte3_to_float(v), c.d, c.add);
+    return v;
+}
+template <int I, int H>
+__device__ __forceinline__ void decode_pair(uint32_t v, const DecQ45& c, float& w0, float& w1) {
+    w0 = fmaf(gemm_byte_to_float<2 * H>(v), c.d, c.add);
+    w1 = fmaf(gemm_byte_to_float<2 * H + 1>(v), c.d, c.add);
 }
 
 // Q5_K: the Q4_K sub-block plus bit sb of the 32-byte fifth-bit plane at byte 16 (nibbles at byte 48).
@@ -282,16 +304,17 @@ __device__ __forceinline__ void decode_prepare(const RawQ5K& r, int e, DecQ5K& c
     c.bit = (e & 255) >> 5;
 }
 template <int I>
-__device__ __forceinline__ void decode_dword(const RawQ5K& r, const DecQ5K& c, float* w4) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ5K& r, const DecQ5K& c) {
     const uint32_t q = I == 0 ? r.q0.x : I == 1 ? r.q0.y : I == 2 ? r.q0.z : I == 3 ? r.q0.w
                      : I == 4 ? r.q1.x : I == 5 ? r.q1.y : I == 6 ? r.q1.z : r.q1.w;
     const uint32_t h = I == 0 ? r.h0.x : I == 1 ? r.h0.y : I == 2 ? r.h0.z : I == 3 ? r.h0.w
                      : I == 4 ? r.h1.x : I == 5 ? r.h1.y : I == 6 ? r.h1.z : r.h1.w;
-    const uint32_t v = ((q >> c.shift) & 0x0F0F0F0Fu) | (((h >> c.bit) & 0x01010101u) << 4);
-    w4[0] = fmaf(ubyte0_to_float(v), c.scale, -c.offset);
-    w4[1] = fmaf(ubyte1_to_float(v), c.scale, -c.offset);
-    w4[2] = fmaf(ubyte2_to_float(v), c.scale, -c.offset);
-    w4[3] = fmaf(ubyte3_to_float(v), c.scale, -c.offset);
+    return ((q >> c.shift) & 0x0F0F0F0Fu) | (((h >> c.bit) & 0x01010101u) << 4);
+}
+template <int I, int H>
+__device__ __forceinline__ void decode_pair(uint32_t v, const DecQ5K& c, float& w0, float& w1) {
+    w0 = fmaf(gemm_byte_to_float<2 * H>(v), c.scale, -c.offset);
+    w1 = fmaf(gemm_byte_to_float<2 * H + 1>(v), c.scale, -c.offset);
 }
 
 template <class Raw> struct DecOf;
@@ -302,35 +325,37 @@ template <int FMT> struct DecOf<RawQ45<FMT>> { typedef DecQ45 type; };
 template <> struct DecOf<RawQ5K> { typedef DecQ5K type; };
 
 typedef __bf16 gemm_bf16x2 __attribute__((ext_vector_type(2)));
-// Half H (0 / 1) of part I (0..7) of a thread's 32 weights -> weights 4 I + 2 H and 4 I + 2 H + 1 as one packed bf16
-// pair. The part's whole 4-weight expression is written out and the unused half is dropped by the compiler, so a
-// half is about seven vector instructions: what fits between two MFMAs without holding the matrix core up.
+// Decode item h (0..15) of a thread's 32 weights: half H = h % 2 of part I = h / 2 -> weights 2 h and 2 h + 1 as one
+// packed bf16 pair. The first item of a part gathers its codes into `codes`, the second reuses them: about seven
+// vector instructions for the first, five for the second -- what fits between two MFMAs without holding the matrix
+// core up.
 template <int I, int H, class Raw, class Dec>
-__device__ __forceinline__ uint32_t decode_half(const Raw& r, const Dec& c) {
-    float w4[4];
-    decode_dword<I>(r, c, w4);
-    return __builtin_bit_cast(uint32_t, gemm_bf16x2{(__bf16)w4[2 * H], (__bf16)w4[2 * H + 1]});
+__device__ __forceinline__ uint32_t decode_item(const Raw& r, const Dec& c, uint32_t& codes) {
+    if (H == 0) codes = decode_codes<I>(r, c);
+    float w0, w1;
+    decode_pair<I, H>(codes, c, w0, w1);
+    return __builtin_bit_cast(uint32_t, gemm_bf16x2{(__bf16)w0, (__bf16)w1});
 }
-// half-part h (0..15) with h a (constant-folded) loop variable
+// item h with h a (constant-folded) loop variable
 template <class Raw, class Dec>
-__device__ __forceinline__ uint32_t decode_half_at(int h, const Raw& r, const Dec& c) {
+__device__ __forceinline__ uint32_t decode_item_at(int h, const Raw& r, const Dec& c, uint32_t& codes) {
     switch (h) {
-        case 0: return decode_half<0, 0>(r, c);
-        case 1: return decode_half<0, 1>(r, c);
-        case 2: return decode_half<1, 0>(r, c);
-        case 3: return decode_half<1, 1>(r, c);
-        case 4: return decode_half<2, 0>(r, c);
-        case 5: return decode_half<2, 1>(r, c);
-        case 6: return decode_half<3, 0>(r, c);
-        case 7: return decode_half<3, 1>(r, c);
-        case 8: return decode_half<4, 0>(r, c);
-        case 9: return decode_half<4, 1>(r, c);
-        case 10: return decode_half<5, 0>(r, c);
-        case 11: return decode_half<5, 1>(r, c);
-        case 12: return decode_half<6, 0>(r, c);
-        case 13: return decode_half<6, 1>(r, c);
-        case 14: return decode_half<7, 0>(r, c);
-        default: return decode_half<7, 1>(r, c);
+        case 0: return decode_item<0, 0>(r, c, codes);
+        case 1: return decode_item<0, 1>(r, c, codes);
+        case 2: return decode_item<1, 0>(r, c, codes);
+        case 3: return decode_item<1, 1>(r, c, codes);
+        case 4: return decode_item<2, 0>(r, c, codes);
+        case 5: return decode_item<2, 1>(r, c, codes);
+        case 6: return decode_item<3, 0>(r, c, codes);
+        case 7: return decode_item<3, 1>(r, c, codes);
+        case 8: return decode_item<4, 0>(r, c, codes);
+        case 9: return decode_item<4, 1>(r, c, codes);
+        case 10: return decode_item<5, 0>(r, c, codes);
+        case 11: return decode_item<5, 1>(r, c, codes);
+        case 12: return decode_item<6, 0>(r, c, codes);
+        case 13: return decode_item<6, 1>(r, c, codes);
+        case 14: return decode_item<7, 0>(r, c, codes);
+        default: return decode_item<7, 1>(r, c, codes);
     }
 }
 
@@ -441,6 +466,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
             for (int j = 0; j < G_WTN; ++j) bf[set][j] = *reinterpret_cast<const bf16x8*>(wt + 32 * j * GSTRIDE + kk);
         };
         Dec dc[G_W_TASKS];
+        uint32_t codes[G_W_TASKS];                                  // the codes of the part a task's items are working on
         frags(0, 0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma clang loop unroll(full)
@@ -464,7 +490,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
                 const int g = q - FIRST_ITEM;
                 const int h0 = (g * N_HALVES + N_GAPS - 1) / N_GAPS, h1 = ((g + 1) * N_HALVES + N_GAPS - 1) / N_GAPS;
                 if (h0 < h1 && h0 < N_HALVES) {
-                    wp[h0 / 16][h0 % 16] = decode_half_at(h0 % 16, wring[slot_next][h0 / 16], dc[h0 / 16]);
+                    wp[h0 / 16][h0 % 16] = decode_item_at(h0 % 16, wring[slot_next][h0 / 16], dc[h0 / 16], codes[h0 / 16]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
@@ -494,8 +520,9 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     for (int t = 0; t < G_W_TASKS; ++t) {
         Dec d0;
         decode_prepare(wring[0][t], step_k(0) + 32 * wsub, d0);
+        uint32_t codes0 = 0;
 #pragma unroll
-        for (int h = 0; h < 16; ++h) wp[t][h] = decode_half_at(h, wring[0][t], d0);
+        for (int h = 0; h < 16; ++h) wp[t][h] = decode_item_at(h, wring[0][t], d0, codes0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) park_w(0, t, i);
     }
