@@ -174,37 +174,43 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
 }
 
 // Merge the per-split (unnormalised output, max, sum) triples of one query row. 4 * D threads: thread (j, d) folds
-// splits j, j + 4, ... of output element d (independent loads, all in flight together), LDS folds the four.
+// splits j, j + 4, ... of output element d (independent loads, all in flight together), LDS folds the four. The
+// softmax weights of the splits -- exp(max_s - max) / sum -- are worked out once, by the first wave: one split per
+// lane, maximum and sum by wave reductions (splits <= 64), parked in LDS for everyone.
 template <int D>
 __global__ __launch_bounds__(4 * D) void sdpa_decode_combine_kernel(const float* __restrict__ part, float* __restrict__ out, int splits) {
-    __shared__ float sm[SDPA_DECODE_MAX_SPLITS], sl[SDPA_DECODE_MAX_SPLITS];
+    __shared__ float sw[SDPA_DECODE_MAX_SPLITS];
     __shared__ float so[4][D];
     const float* src = part + (int64_t)blockIdx.x * splits * (D + 2);
     const int d = threadIdx.x % D, j = threadIdx.x / D;
-    if ((int)threadIdx.x < splits) { sm[threadIdx.x] = src[threadIdx.x * (D + 2) + D]; sl[threadIdx.x] = src[threadIdx.x * (D + 2) + D + 1]; }
     float pv[SDPA_DECODE_MAX_SPLITS / 4];
 #pragma unroll
     for (int i = 0; i < SDPA_DECODE_MAX_SPLITS / 4; ++i) {
         const int sp = j + 4 * i;
-        pv[i] = sp < splits ? src[sp * (D + 2) + d] : 0.f;
+        pv[i] = src[min(sp, splits - 1) * (D + 2) + d];         // clamped: a split past the end gets weight zero below
+    }
+    if (threadIdx.x < 64) {
+        const int sp = threadIdx.x;
+        const bool live = sp < splits;
+        const float m = live ? src[sp * (D + 2) + D] : -INFINITY;
+        const float l = live ? src[sp * (D + 2) + D + 1] : 0.f;
+        float mm = m;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mm = fmaxf(mm, __shfl_xor(mm, off, 64));
+        const float w = exp_diff(m, mm);
+        const float ls = wave_sum(l * w);
+        if (sp < SDPA_DECODE_MAX_SPLITS) sw[sp] = ls > 0.f ? w / ls : 0.f;
     }
     __syncthreads();
-    float mm = -INFINITY;
-    for (int sp = 0; sp < splits; ++sp) mm = fmaxf(mm, sm[sp]);
     float o = 0.f;
 #pragma unroll
     for (int i = 0; i < SDPA_DECODE_MAX_SPLITS / 4; ++i) {
         const int sp = j + 4 * i;
-        if (sp < splits) o = fmaf(pv[i], exp_diff(sm[sp], mm), o);
+        o = fmaf(pv[i], sp < splits ? sw[sp] : 0.f, o);
     }
     so[j][d] = o;
     __syncthreads();
-    if (j == 0) {
-        float ls = 0.f;
-        for (int sp = 0; sp < splits; ++sp) ls = fmaf(sl[sp], exp_diff(sm[sp], mm), ls);
-        const float t = so[0][d] + so[1][d] + so[2][d] + so[3][d];
-        out[(int64_t)blockIdx.x * D + d] = ls > 0.f ? t / ls : 0.f;
-    }
+    if (j == 0) out[(int64_t)blockIdx.x * D + d] = so[0][d] + so[1][d] + so[2][d] + so[3][d];
 }
 
 float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
