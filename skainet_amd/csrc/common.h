@@ -109,6 +109,10 @@ __device__ __forceinline__ uint32_t load_u16(const uint8_t* p) { return *reinter
 typedef uint32_t u32x4_vec __attribute__((ext_vector_type(4)));
 struct __attribute__((packed, aligned(4))) u32x4_a4 { u32x4_vec v; };
 __device__ __forceinline__ u32x4_vec load_u32x4_a4(const uint8_t* p) { return reinterpret_cast<const u32x4_a4*>(p)->v; }
+// 8 bytes from a 2-byte aligned address as one load.
+typedef uint32_t u32x2_vec __attribute__((ext_vector_type(2)));
+struct __attribute__((packed, aligned(2))) u32x2_a2 { u32x2_vec v; };
+__device__ __forceinline__ u32x2_vec load_u32x2_a2(const uint8_t* p) { return reinterpret_cast<const u32x2_a2*>(p)->v; }
 // The same from a 2-byte aligned address (Q6_K code runs): still one global_load_dwordx4, which this device serves.
 struct __attribute__((packed, aligned(2))) u32x4_a2 { u32x4_vec v; };
 __device__ __forceinline__ u32x4_vec load_u32x4_a2(const uint8_t* p) { return reinterpret_cast<const u32x4_a2*>(p)->v; }

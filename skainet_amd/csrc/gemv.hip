@@ -106,61 +106,77 @@ struct Q4KSlot {
 
 // ---------------------------------------------------------------------------------------------- Q6_K
 struct Q6KSlot {
-    static constexpr int BLOCK_BYTES = Q6K_BYTES, SLOTS_PER_BLOCK = 16, SLOT_ELEMS = 16, NX = 16;
-    struct Raw { uint32_t qla, qlb, qh, sc0, sc1, d; };
+    // A slot is 32 weights: 8 consecutive positions l of one half of a super-block, in all four quarters (elements
+    // half * 128 + 32 k + l). Their codes sit in three 8-byte runs (two of low / high nibbles, one of the two-bit
+    // planes), read with one 8-byte load each; the half's eight scale bytes are a fourth.
+    static constexpr int BLOCK_BYTES = Q6K_BYTES, SLOTS_PER_BLOCK = 8, SLOT_ELEMS = 32, NX = 32;
+    struct Raw { u32x2_vec qla, qlb, qh, sc; uint32_t d; };
     struct Lane { int blk_off, ql_off, qh_off, sc_off, sc_shift; };
     __device__ static void init(Lane& ln, int slot) {
-        const int blk = slot >> 4, t = slot & 15, half = t >> 3, l0 = (t & 7) * 4;
+        const int blk = slot >> 3, t = slot & 7, half = t >> 2, l0 = (t & 3) * 8;
         ln.blk_off = blk * BLOCK_BYTES;
         ln.ql_off = ln.blk_off + half * 64 + l0;
         ln.qh_off = ln.blk_off + 128 + half * 32 + l0;
         ln.sc_off = ln.blk_off + 192 + half * 8;
         ln.sc_shift = (l0 >> 4) * 8;
     }
-    // Register i = 4 * k + j pairs with element half*128 + 32*k + l0 + j.
+    // Register i = 8 * k + j pairs with element half*128 + 32*k + l0 + j.
     __device__ static int x_index(int slot, int i) {
-        const int blk = slot >> 4, t = slot & 15, half = t >> 3, l0 = (t & 7) * 4;
-        return blk * 256 + half * 128 + (i >> 2) * 32 + l0 + (i & 3);
+        const int blk = slot >> 3, t = slot & 7, half = t >> 2, l0 = (t & 3) * 8;
+        return blk * 256 + half * 128 + (i >> 3) * 32 + l0 + (i & 7);
     }
     __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
-        r.qla = load_u32_a2(row + ln.ql_off);
-        r.qlb = load_u32_a2(row + ln.ql_off + 32);
-        r.qh = load_u32_a2(row + ln.qh_off);
-        r.sc0 = load_u32_a2(row + ln.sc_off);
-        r.sc1 = load_u32_a2(row + ln.sc_off + 4);
+        r.qla = load_u32x2_a2(row + ln.ql_off);
+        r.qlb = load_u32x2_a2(row + ln.ql_off + 32);
+        r.qh = load_u32x2_a2(row + ln.qh_off);
+        r.sc = load_u32x2_a2(row + ln.sc_off);
         r.d = load_u16(row + ln.blk_off + 208);
     }
     __device__ static void prep(const float* x, float* xsum) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) xsum[k] = 32.f * (x[4 * k] + x[4 * k + 1] + x[4 * k + 2] + x[4 * k + 3]);
+        for (int k = 0; k < 4; ++k) {
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s += x[8 * k + j];
+            xsum[k] = 32.f * s;
+        }
     }
     template <int B>
     __device__ static void dot(const Raw& r, const Lane& ln, const float (*x)[NX], const float (*xsum)[4], float* acc) {
         const float d = half_bits_to_float_fast(r.d);
         // signed scales of the four quarters: bytes is, is+2, is+4, is+6 of the half's 8 scale bytes
-        const uint32_t s0 = r.sc0 >> ln.sc_shift, s1 = r.sc1 >> ln.sc_shift;
+        const uint32_t s0 = r.sc.x >> ln.sc_shift, s1 = r.sc.y >> ln.sc_shift;
         const float sc[4] = {d * (float)(int8_t)(s0), d * (float)(int8_t)(s0 >> 16),
                              d * (float)(int8_t)(s1), d * (float)(int8_t)(s1 >> 16)};
-        const uint32_t c[4] = {
-            (r.qla & 0x0F0F0F0Fu) | ((r.qh << 4) & 0x30303030u),
-            (r.qlb & 0x0F0F0F0Fu) | ((r.qh << 2) & 0x30303030u),
-            ((r.qla >> 4) & 0x0F0F0F0Fu) | (r.qh & 0x30303030u),
-            ((r.qlb >> 4) & 0x0F0F0F0Fu) | ((r.qh >> 2) & 0x30303030u)};
+        const uint32_t qla[2] = {r.qla.x, r.qla.y}, qlb[2] = {r.qlb.x, r.qlb.y}, qh[2] = {r.qh.x, r.qh.y};
+        float s[4][B];
 #pragma unroll
-        for (int b = 0; b < B; ++b) acc[b] = 0.f;
+        for (int k = 0; k < 4; ++k)
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            float s[B];
+            for (int b = 0; b < B; ++b) s[k][b] = -xsum[b][k];       // the -32 bias of every code, taken out of the loop
 #pragma unroll
-            for (int b = 0; b < B; ++b) s[b] = -xsum[b][k];   // the -32 bias of every code, taken out of the loop
-            const float cf[4] = {ubyte0_to_float(c[k]), ubyte1_to_float(c[k]), ubyte2_to_float(c[k]), ubyte3_to_float(c[k])};
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t c[4] = {
+                (qla[h] & 0x0F0F0F0Fu) | ((qh[h] << 4) & 0x30303030u),
+                (qlb[h] & 0x0F0F0F0Fu) | ((qh[h] << 2) & 0x30303030u),
+                ((qla[h] >> 4) & 0x0F0F0F0Fu) | (qh[h] & 0x30303030u),
+                ((qlb[h] >> 4) & 0x0F0F0F0Fu) | ((qh[h] >> 2) & 0x30303030u)};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int k = 0; k < 4; ++k) {
+                const float cf[4] = {ubyte0_to_float(c[k]), ubyte1_to_float(c[k]), ubyte2_to_float(c[k]), ubyte3_to_float(c[k])};
 #pragma unroll
-                for (int b = 0; b < B; ++b) s[b] = fmaf(x[b][4 * k + j], cf[j], s[b]);
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int b = 0; b < B; ++b) s[k][b] = fmaf(x[b][8 * k + 4 * h + j], cf[j], s[k][b]);
+                }
             }
+        }
 #pragma unroll
-            for (int b = 0; b < B; ++b) acc[b] = fmaf(sc[k], s[b], acc[b]);
+        for (int b = 0; b < B; ++b) {
+            float a = 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) a = fmaf(sc[k], s[k][b], a);
+            acc[b] = a;
         }
     }
 };
