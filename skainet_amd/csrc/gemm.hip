@@ -261,8 +261,8 @@ __device__ __forceinline__ void load_raw(RawQ45<FMT>& r, const uint8_t* row, int
     r.d = load_u16(blk);
     r.m = FMT == 2 ? load_u16(blk + 2) : 0u;
     r.qh = FMT != 0 ? load_u32_a2(blk + QH) : 0u;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) r.q[i] = load_u32_a2(blk + QS + 4 * i);
+    const u32x4_vec q4 = load_u32x4_a2(blk + QS);           // the 16 code bytes as one load (2-byte aligned)
+    r.q[0] = q4.x; r.q[1] = q4.y; r.q[2] = q4.z; r.q[3] = q4.w;
 }
 struct DecQ45 { float d, add; };
 template <int FMT>

@@ -250,8 +250,8 @@ struct Q45Slot {
         r.d = load_u16(p);
         r.m = FMT == 2 ? load_u16(p + 2) : 0u;
         r.qh = FMT != 0 ? load_u32_a2(p + QH) : 0u;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) r.q[i] = load_u32_a2(p + QS + 4 * i);
+        const u32x4_vec q4 = load_u32x4_a2(p + QS);          // the 16 code bytes as one load (2-byte aligned)
+        r.q[0] = q4.x; r.q[1] = q4.y; r.q[2] = q4.z; r.q[3] = q4.w;
     }
     __device__ static void prep(const float* x, float* xsum) {
         float a = 0.f;
