@@ -130,6 +130,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // register read, which this target expands into a compare/select chain per element).
 template <int NV>
 __device__ __forceinline__ void wave_fold(float* v, int lane) {
+    static_assert(NV >= 1 && NV <= 64 && (NV & (NV - 1)) == 0, "every halving must pair all values: NV is a power of two");
     int mask = 1;
 #pragma unroll
     for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) {
