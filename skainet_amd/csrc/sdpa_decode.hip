@@ -35,7 +35,30 @@ struct SdpaDecodeParams {
     float* part;          // [batch * heads][splits][D + 2]
 };
 
-__device__ __forceinline__ float exp_diff(float m_old, float m_new) { return m_old == -INFINITY ? 0.f : expf(m_old - m_new); }
+// Scores are kept in units of ln 2 (the query is scaled by scale * log2(e) once), so every exponential of the softmax is
+// one v_exp_f32 of a difference: no range reduction, no multiply. For the differences that carry weight (|x| < 30) the
+// rounding of the scaled score moves the result by under 3e-6 relative.
+constexpr float SDPA_LOG2E = 1.44269504088896340736f;
+__device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+// 2^(m_old - m_new), 0 for an empty state; the exponential is evaluated unconditionally (a select, not a branch)
+__device__ __forceinline__ float exp_diff(float m_old, float m_new) {
+    const float e = exp2_raw(m_old - m_new);
+    return m_old == -INFINITY ? 0.f : e;
+}
+
+// Sum over the 16 lanes of a DPP row (lanes 16 r .. 16 r + 15), result in every lane: four rotate-and-add steps inside
+// the vector ALU instead of four round trips through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_row_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_row_move<0x128>(v);   // row_ror:8
+    v += dpp_row_move<0x124>(v);   // row_ror:4
+    v += dpp_row_move<0x122>(v);   // row_ror:2
+    v += dpp_row_move<0x121>(v);   // row_ror:1
+    return v;
+}
 
 template <int GS, int DPL>
 __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
@@ -44,7 +67,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
     __shared__ float wacc[4][GS][D];
     __shared__ float wm[4][GS], wl[4][GS];
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform, and said so: the key loop's exits stay scalar branches
     const int sub = lane & 15, kg = lane >> 4;
     const int split = blockIdx.x, b = blockIdx.z;
     const int per_kv = p.heads / p.kv_heads;
@@ -66,6 +90,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
     const int lo = first + split * chunk;
     const int hi = min(end, lo + chunk);
 
+    const float qscale = p.scale * SDPA_LOG2E;
     float qr[GS][DPL];
 #pragma unroll
     for (int g = 0; g < GS; ++g) {
@@ -73,7 +98,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
 #pragma unroll
         for (int d = 0; d < DPL; d += 4) {
             const float4 t = *reinterpret_cast<const float4*>(qp + d);
-            qr[g][d] = t.x * p.scale; qr[g][d + 1] = t.y * p.scale; qr[g][d + 2] = t.z * p.scale; qr[g][d + 3] = t.w * p.scale;
+            qr[g][d] = t.x * qscale; qr[g][d + 1] = t.y * qscale; qr[g][d + 2] = t.z * qscale; qr[g][d + 3] = t.w * qscale;
         }
     }
     float m[GS], l[GS], acc[GS][DPL];
@@ -86,14 +111,13 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
 
     const float* kb = p.k + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * DPL;
     const float* vb = p.v + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * DPL;
-    for (int k0 = lo + wave * 4; k0 < hi; k0 += 16 * U) {       // wave-uniform trip count
-        float kr[U][DPL], vr[U][DPL];
-        bool valid[U];
+    // The K / V rows of a pass (U groups of 4 keys per wave) are requested one pass ahead of their use, into the other of
+    // two register sets: a split of 64 keys is two passes per wave, and both are in flight from the start.
+    constexpr int STEP = 16 * U;
+    auto request = [&](float (&kr)[U][DPL], float (&vr)[U][DPL], int k0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int key = k0 + 16 * u + kg;
-            valid[u] = key < hi;
-            const int64_t off = (int64_t)min(key, hi - 1) * D;   // a lane past the range re-reads the last row
+            const int64_t off = (int64_t)min(k0 + 16 * u + kg, hi - 1) * D;   // a lane past the range re-reads the last row
 #pragma unroll
             for (int d = 0; d < DPL; d += 4) {
                 const float4 a = *reinterpret_cast<const float4*>(kb + off + d);
@@ -102,6 +126,15 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
                 vr[u][d] = c.x; vr[u][d + 1] = c.y; vr[u][d + 2] = c.z; vr[u][d + 3] = c.w;
             }
         }
+    };
+    auto consume = [&](const float (&kr)[U][DPL], const float (&vr)[U][DPL], int k0) {
+        bool valid[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) valid[u] = k0 + 16 * u + kg < hi;
+        // Branch-free from here to the end of the body: the U x GS score chains (dot product, row reduction, exponentials)
+        // are independent and the compiler interleaves them; behind a per-key branch each ran on its own, one
+        // dependent instruction at a time -- with one wave per SIMD that chain, not the memory, set the pace.
+        float sc[U][GS];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -109,22 +142,50 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
                 float s = 0.f;
 #pragma unroll
                 for (int d = 0; d < DPL; ++d) s = fmaf(qr[g][d], kr[u][d], s);
-                s += __shfl_xor(s, 1, 64);
-                s += __shfl_xor(s, 2, 64);
-                s += __shfl_xor(s, 4, 64);
-                s += __shfl_xor(s, 8, 64);
+                s = row16_sum(s);
                 if (uniform) s = SDPA_DECODE_MASKED;
-                if (valid[u]) {
-                    const float m_new = fmaxf(m[g], s);
-                    const float alpha = exp_diff(m[g], m_new);
-                    const float pr = expf(s - m_new);
-                    l[g] = l[g] * alpha + pr;
-#pragma unroll
-                    for (int d = 0; d < DPL; ++d) acc[g][d] = fmaf(pr, vr[u][d], acc[g][d] * alpha);
-                    m[g] = m_new;
-                }
+                sc[u][g] = valid[u] ? s : -INFINITY;
             }
         }
+#pragma unroll
+        for (int g = 0; g < GS; ++g) {
+            // both key groups enter the running state in one update: one rescale of the accumulator per pass
+            float m_new = m[g];
+#pragma unroll
+            for (int u = 0; u < U; ++u) m_new = fmaxf(m_new, sc[u][g]);
+            const float alpha = exp_diff(m[g], m_new);
+            float pr[U], psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float e = exp2_raw(sc[u][g] - m_new);        // NaN for (-inf) - (-inf): discarded by the select
+                pr[u] = valid[u] ? e : 0.f;
+                psum += pr[u];
+            }
+            l[g] = fmaf(l[g], alpha, psum);
+#pragma unroll
+            for (int d = 0; d < DPL; ++d) {
+                float a = acc[g][d] * alpha;
+#pragma unroll
+                for (int u = 0; u < U; ++u) a = fmaf(pr[u], vr[u][d], a);
+                acc[g][d] = a;
+            }
+            m[g] = m_new;
+        }
+    };
+    // Passes are taken in pairs so that the loop has one exit and one back edge (with an exit between the two halves
+    // the compiler's wait-count pass sees a path on which the second set is still in flight at the loop head and makes
+    // every request wait for it). The second half of the last pair may lie past the range: none of its keys is valid
+    // and it leaves the running state as it is.
+    float ka[U][DPL], va[U][DPL], kb2[U][DPL], vb2[U][DPL];
+    const int k_first = lo + wave * 4;
+    if (k_first < hi) request(ka, va, k_first);                 // wave-uniform
+    for (int k0 = k_first; k0 < hi; k0 += 2 * STEP) {
+        request(kb2, vb2, k0 + STEP);                           // past the range: clamped re-reads of the last row
+        __builtin_amdgcn_sched_barrier(0);                      // requests are issued where they are written, ahead of the arithmetic
+        consume(ka, va, k0);
+        request(ka, va, k0 + 2 * STEP);
+        __builtin_amdgcn_sched_barrier(0);
+        consume(kb2, vb2, k0 + STEP);
     }
 
     // merge the four lane groups of the wave (lanes 16 and 32 apart hold the same dims of other keys)
