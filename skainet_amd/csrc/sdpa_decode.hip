@@ -12,8 +12,8 @@
 //   * 16 lanes hold one key row (D / 16 consecutive floats each), a wave covers 4 adjacent keys per load
 //     instruction (one contiguous span of 4 rows), the 4 waves interleave groups of 4 keys;
 //   * every 16-lane group keeps its own online-softmax state (running max, sum, output slice) for its keys, so
-//     the key loop has no cross-lane traffic beyond the 4-step dot-product reduction; states are merged across
-//     lane groups by shuffles, across waves through LDS;
+//     the key loop has no cross-lane traffic beyond the 4-step dot-product reduction (DPP rotates inside a row of 16
+//     lanes); the 16 states of a workgroup are merged once, through LDS;
 //   * splits > 1: each workgroup writes an unnormalised partial (output, max, sum) and a second, small kernel
 //     merges them. (Merging in the last-arriving workgroup instead needs an agent-scope release / acquire per
 //     workgroup, which on this multi-die part writes back and invalidates whole L2s: measured slower.)
@@ -52,6 +52,13 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_row_move(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_row_move<0x128>(v));
+    v = fmaxf(v, dpp_row_move<0x124>(v));
+    v = fmaxf(v, dpp_row_move<0x122>(v));
+    v = fmaxf(v, dpp_row_move<0x121>(v));
+    return v;
+}
 __device__ __forceinline__ float row16_sum(float v) {
     v += dpp_row_move<0x128>(v);   // row_ror:8
     v += dpp_row_move<0x124>(v);   // row_ror:4
@@ -64,8 +71,9 @@ template <int GS, int DPL>
 __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
     constexpr int D = 16 * DPL;
     constexpr int U = 2;                       // groups of 4 keys a wave has in flight
-    __shared__ float wacc[4][GS][D];
-    __shared__ float wm[4][GS], wl[4][GS];
+    __shared__ __attribute__((aligned(16))) float wacc[16][GS][D];
+    __shared__ __attribute__((aligned(16))) float cw[GS][16];
+    __shared__ float wm[GS][16], wl[GS][16], wmm[GS], wls[GS];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform, and said so: the key loop's exits stay scalar branches
@@ -188,48 +196,60 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
         consume(kb2, vb2, k0 + STEP);
     }
 
-    // merge the four lane groups of the wave (lanes 16 and 32 apart hold the same dims of other keys)
+    // Merge the 16 running states of the workgroup (4 lane groups x 4 waves) through LDS: every lane parks its slice,
+    // one 16-lane row per head works out the 16 weights 2^(m_s - max) and the weighted sum of the l_s, then each thread
+    // sums its output elements over the states. (Merging lane groups by shuffles first cost 80 crossbar round trips and
+    // 16 exponentials per lane.) An element's position inside a state is permuted so that the 16 lanes of a row store
+    // 256 contiguous bytes: float4 number j of lane `sub` sits at j * 64 + sub * 4.
+    const int state = wave * 4 + kg;
 #pragma unroll
-    for (int step = 16; step <= 32; step <<= 1) {
+    for (int g = 0; g < GS; ++g) {
 #pragma unroll
-        for (int g = 0; g < GS; ++g) {
-            const float mo = __shfl_xor(m[g], step, 64), lo_ = __shfl_xor(l[g], step, 64);
-            const float mm = fmaxf(m[g], mo);
-            const float a = exp_diff(m[g], mm), c = exp_diff(mo, mm);
-            l[g] = l[g] * a + lo_ * c;
-#pragma unroll
-            for (int d = 0; d < DPL; ++d) acc[g][d] = acc[g][d] * a + __shfl_xor(acc[g][d], step, 64) * c;
-            m[g] = mm;
-        }
+        for (int j = 0; j < DPL / 4; ++j)
+            *reinterpret_cast<float4*>(&wacc[state][g][j * 64 + sub * 4]) =
+                make_float4(acc[g][4 * j], acc[g][4 * j + 1], acc[g][4 * j + 2], acc[g][4 * j + 3]);
+        if (sub == 0) { wm[g][state] = m[g]; wl[g][state] = l[g]; }
     }
-    if (kg == 0) {
-#pragma unroll
-        for (int g = 0; g < GS; ++g) {
-#pragma unroll
-            for (int d = 0; d < DPL; ++d) wacc[wave][g][sub * DPL + d] = acc[g][d];
-            if (sub == 0) { wm[wave][g] = m[g]; wl[wave][g] = l[g]; }
-        }
+    __syncthreads();
+    if (threadIdx.x < 16 * GS) {
+        const int g = threadIdx.x >> 4, st = threadIdx.x & 15;
+        const float ms = wm[g][st];
+        const float mm = row16_max(ms);
+        const float c = exp_diff(ms, mm);
+        const float ls = row16_sum(c * wl[g][st]);
+        cw[g][st] = c;
+        if (st == 0) { wmm[g] = mm; wls[g] = ls; }
     }
     __syncthreads();
 
-    // merge the four waves; element (g, d) by thread
-    for (int t = threadIdx.x; t < GS * D; t += 256) {
-        const int g = t / D, d = t % D;
-        const float mm = fmaxf(fmaxf(wm[0][g], wm[1][g]), fmaxf(wm[2][g], wm[3][g]));
-        float o = 0.f, ls = 0.f;
+    constexpr int EPT = GS * D >= 256 ? GS * D / 256 : 1;       // output elements per thread, adjacent inside one head
+    if (threadIdx.x * EPT < GS * D) {
+        const int g = threadIdx.x * EPT / D, i0 = threadIdx.x * EPT % D;
+        float c[16], o[EPT];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float c = exp_diff(wm[w][g], mm);
-            o = fmaf(wacc[w][g][d], c, o);
-            ls = fmaf(wl[w][g], c, ls);
+        for (int q4 = 0; q4 < 4; ++q4) {
+            const float4 t = *reinterpret_cast<const float4*>(&cw[g][4 * q4]);
+            c[4 * q4] = t.x; c[4 * q4 + 1] = t.y; c[4 * q4 + 2] = t.z; c[4 * q4 + 3] = t.w;
         }
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) o[e] = 0.f;
+#pragma unroll
+        for (int st = 0; st < 16; ++st)
+#pragma unroll
+            for (int e = 0; e < EPT; ++e) o[e] = fmaf(wacc[st][g][i0 + e], c[st], o[e]);
+        const float mm = wmm[g], ls = wls[g];
         const int64_t row = (int64_t)b * p.heads + h0 + g;
-        if (p.splits == 1) {
-            p.out[row * D + d] = ls > 0.f ? o / ls : 0.f;
-        } else {
-            float* dst = p.part + (row * p.splits + split) * (D + 2);
-            dst[d] = o;
-            if (d == 0) { dst[D] = mm; dst[D + 1] = ls; }
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+            const int i = i0 + e;
+            const int d = ((i & 63) >> 2) * DPL + (i >> 6) * 4 + (i & 3);
+            if (p.splits == 1) {
+                p.out[row * D + d] = ls > 0.f ? o[e] / ls : 0.f;
+            } else {
+                float* dst = p.part + (row * p.splits + split) * (D + 2);
+                dst[d] = o[e];
+                if (d == 0) { dst[D] = mm; dst[D + 1] = ls; }
+            }
         }
     }
 }
