@@ -249,9 +249,109 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
     }
 }
 
+// Long rows, few of them (the down projection: 4096 rows of 14336): with the shape above a wave would own two rows and
+// walk K in several passes, each with its staging barriers, and every workgroup would stage all of x for eight rows.
+// Here the four waves of a workgroup own the same NR rows and a quarter of K each: a wave stages only its own quarter,
+// through its own LDS region, so the pass loop has no workgroup barrier and (for K <= 16384) a single pass per wave
+// with all NR rows streaming behind one staging; the four partial sums per row meet in LDS at the end.
+template <int R, int NR>
+__global__ __launch_bounds__(256, 2) void q4k_gemv_ksplit_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                              float* y, int k, int n, const float* residual, int epilogue) {
+    constexpr int NV = 16, SLICE = 68;
+    static_assert(NR >= 1 && NR <= Q4K_RMAX && R <= NR, "rows per workgroup");
+    __shared__ __attribute__((aligned(16))) float xlds[4][64 * SLICE];
+    __shared__ float part[4][NV];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r0 = blockIdx.x * NR;
+    const int nrows = min(n - r0, NR);
+    const int bpr = k >> 8;
+    const int bpw = (bpr + 3) >> 2;                              // super-blocks of a row per wave
+    const int wb0 = wave * bpw, wb1 = min(bpr, wb0 + bpw);
+    const int64_t row_bytes = (int64_t)bpr * Q4K_BYTES;
+    const int g = lane & 3;
+    const int sh = (g & 1) * 16;
+    const uint32_t hi_mask = g >= 2 ? 0xFFFFFFFFu : 0u;
+    const int q_off = 16 + g * 32;
+    float* xw = &xlds[wave][0];
+
+    float acc[16][1];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i][0] = 0.f;
+
+    for (int blk0 = wb0; blk0 < wb1; blk0 += 16) {
+        const int blk_c = min(blk0 + (lane >> 2), wb1 - 1);     // lanes past the quarter re-read a valid block against zero activations
+        auto row_ptr = [&](int i) { return w + (int64_t)min(r0 + i, n - 1) * row_bytes + (int64_t)blk_c * Q4K_BYTES; };
+        // the pass's activations first (coalesced: float4 number f = lane + 64 j), the first R rows right behind them
+        float4 xv[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) xv[j] = *reinterpret_cast<const float4*>(x + min(blk0 * 256 + (lane + 64 * j) * 4, k - 4));
+        __builtin_amdgcn_sched_barrier(0);
+        Q4KRow raw[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const uint8_t* p = row_ptr(i);
+            raw[i].hdr = *reinterpret_cast<const uint4*>(p);
+            raw[i].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+            raw[i].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // through the wave's own LDS region into one 64-float slice per lane; a wave's LDS accesses complete in order,
+        // so the region needs no barrier
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int f = lane + 64 * j;
+            const float inside = blk0 * 256 + f * 4 < wb1 * 256 ? 1.0f : 0.0f;
+            float4 v4 = xv[j];
+            v4.x *= inside; v4.y *= inside; v4.z *= inside; v4.w *= inside;
+            *reinterpret_cast<float4*>(&xw[(f >> 4) * SLICE + (f & 15) * 4]) = v4;
+        }
+        float xs[1][64], xsum[1][2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float4 v4 = *reinterpret_cast<const float4*>(&xw[lane * SLICE + i * 4]);
+            xs[0][4 * i] = v4.x; xs[0][4 * i + 1] = v4.y; xs[0][4 * i + 2] = v4.z; xs[0][4 * i + 3] = v4.w;
+        }
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) { s0 += xs[0][i]; s1 += xs[0][32 + i]; }
+        xsum[0][0] = s0; xsum[0][1] = s1;
+
+#pragma unroll
+        for (int c = 0; c < NR; ++c) {
+            q4k_row_dot<1>(raw[c % R], sh, hi_mask, xs, xsum, acc[c]);
+            if (c + R < NR) {                                   // compile-time: refill with the row R ahead
+                const uint8_t* p = row_ptr(c + R);
+                raw[c % R].hdr = *reinterpret_cast<const uint4*>(p);
+                raw[c % R].q0 = *reinterpret_cast<const uint4*>(p + q_off);
+                raw[c % R].q1 = *reinterpret_cast<const uint4*>(p + q_off + 16);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    float v[NV];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = acc[i][0];
+    wave_fold<NV>(v, lane);
+    if (lane < NV) part[wave][lane] = v[0];
+    __syncthreads();
+    if (wave == 0 && lane < NV) {
+        const int row = wave_fold_index<NV>(lane);
+        if (row < nrows) {
+            float val = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+            const int64_t o = r0 + row;
+            if (epilogue == EPI_RESIDUAL) val += residual[o];
+            y[o] = val;
+        }
+    }
+}
+
 static int g_q4k_rows_waves_per_cu = 0;   // 0: chosen from K (below)
 void set_q4k_rows_waves_per_cu(int v) { if (v >= 0) g_q4k_rows_waves_per_cu = v; }
 int q4k_rows_waves_per_cu() { return g_q4k_rows_waves_per_cu; }
+static int g_q4k_ksplit_enable = 1;      // 0: long rows take the plain row shape too
+void set_q4k_ksplit_enable(int v) { g_q4k_ksplit_enable = v; }
 
 template <int B, int R, int NR>
 static void launch_rows(bool pro, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int nchunks,
@@ -285,6 +385,22 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     }
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 3)) return 0;
     if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return 0;
+    if (g_q4k_ksplit_enable && batch == 1 && !gain && epilogue <= EPI_RESIDUAL && k >= 8192) {
+        // long rows: K over the four waves of a workgroup when the plain shape would leave a wave three rows or fewer
+        const int nr = (n + 2 * num_cus() - 1) / (2 * num_cus());
+        if (nr >= 4 && nr <= Q4K_RMAX && (n + num_cus() * 8 - 1) / (num_cus() * 8) <= 3) {
+            const int grid = (n + nr - 1) / nr;
+            hipStream_t s = current_stream();
+#define SKH_KS_CASE(N) case N: q4k_gemv_ksplit_kernel<(6 < N ? 6 : N), N><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, residual, epilogue); break;
+            switch (nr) {
+                SKH_KS_CASE(4) SKH_KS_CASE(5) SKH_KS_CASE(6) SKH_KS_CASE(7) SKH_KS_CASE(8) SKH_KS_CASE(9)
+                SKH_KS_CASE(10) SKH_KS_CASE(11) SKH_KS_CASE(12)
+            }
+#undef SKH_KS_CASE
+            SKH_CHECK(hipGetLastError());
+            return 1;
+        }
+    }
     const bool pairs = epilogue >= EPI_SWIGLU;                   // a (gate, up) or rotation pair never straddles two waves
     if (pairs && (n & 1)) return 0;
     // one round of workgroups over the chip: a wave's rows, taken in equal chunks of at most Q4K_RMAX (the chunk size

@@ -296,6 +296,9 @@ __global__ __launch_bounds__(4 * D) void sdpa_decode_combine_kernel(const float*
 
 float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
 
+static int g_sdpa_decode_split_keys = 64;   // least keys per split (a multiple of 16)
+void set_sdpa_decode_split_keys(int v) { if (v >= 16) g_sdpa_decode_split_keys = (v + 15) & ~15; }
+
 template <int GS, int DPL>
 static int launch_decode_variant(const SdpaDecodeParams& p, int subs) {
     constexpr int D = 16 * DPL;
@@ -327,7 +330,7 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
     // keys: 32 keys per split 4 % slower per token, 128 keys 1 % slower)
     const int64_t groups = (int64_t)batch * kv_heads * subs;
     int splits = (int)((2 * (int64_t)num_cus() + groups - 1) / groups);
-    splits = min(splits, min(SDPA_DECODE_MAX_SPLITS, (seq_kv + 63) / 64));
+    splits = min(splits, min(SDPA_DECODE_MAX_SPLITS, (seq_kv + g_sdpa_decode_split_keys - 1) / g_sdpa_decode_split_keys));
     if (splits < 1) splits = 1;
     p.splits = splits;
     if (splits > 1) {

@@ -136,7 +136,7 @@ def test_rope_qkv_equals_three_scatters(hip_backend, torch_cuda):
 
 @pytest.mark.parametrize("enc,n,k,m", [("Q4_K", 1536, 1024, 1), ("Q4_K", 1030, 512, 2), ("Q4_K", 24, 4096 + 256, 1),
                                         ("Q4_K", 640, 512, 5), ("Q6_K", 512, 512, 1), ("Q4_K", 768, 1024, 24),
-                                        ("Q4_K", 1030, 14336, 1), ("Q4_K", 26, 16640, 1), ("Q4_K", 4096, 12288, 1),
+                                        ("Q4_K", 1030, 14336, 1), ("Q4_K", 26, 16640, 1), ("Q4_K", 4096, 12288, 1), ("Q4_K", 2050, 8448, 1),
                                         ("Q4_K", 300, 512, 40), ("Q6_K", 258, 1024, 33), ("Q8_0", 130, 2048, 64),
                                         ("Q4_K", 64, 5120, 300), ("Q8_0", 66, 96, 12)])
 def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
