@@ -71,20 +71,42 @@ __device__ __forceinline__ void q4k_row_dot(const Q4KRow& r, int sh, uint32_t hi
 // Epilogue of a chunk: after the fold lane l < 16 B holds the total of row `row` (of the chunk that starts at output
 // row r0) for activation row b. Plain store, `+ residual`, SwiGLU over adjacent (gate, up) rows, or RoPE + scatter of
 // one token's [q | k | v] rows.
+//
+// What the epilogue reads besides the sum -- the residual element, the token position, the (cos, sin) pair -- is
+// requested by q4k_epilogue_prefetch at the start of the chunk, ahead of the weight stream: read where it is used it would
+// be one more memory round trip at the very end of the kernel.
+struct Q4KEpiloguePrefetch { float residual; int pos; float2 cs; };
+template <int B>
+__device__ __forceinline__ Q4KEpiloguePrefetch q4k_epilogue_prefetch(int lane, int r0, int nrows, int n, const float* x,
+                                                                       const float* residual, int epilogue,
+                                                                       const RopeQkvEpilogue& rope) {
+    constexpr int NV = 16 * B;
+    const int idx = wave_fold_index<NV>(lane), row = idx / B, b = idx % B;
+    const bool live = lane < NV && row < nrows;
+    // lanes (and epilogues) without such an operand read the first activations instead: no branch around a load
+    const float* rp = (epilogue == EPI_RESIDUAL && live) ? residual + ((int64_t)b * n + r0 + row) : x;
+    const bool rot = epilogue == EPI_ROPE_QKV && live;
+    const int32_t* pp = rot ? rope.pos_dev : reinterpret_cast<const int32_t*>(x);
+    const int dd = (r0 + row) % max(rope.head_dim, 1);
+    const float2* tp = (rot && rope.table) ? rope.table + (dd >> 1) : reinterpret_cast<const float2*>(x);
+    Q4KEpiloguePrefetch pre;
+    pre.residual = *rp; pre.pos = *pp; pre.cs = *tp;
+    return pre;
+}
 template <int B>
 __device__ __forceinline__ void q4k_rows_epilogue(float val, int lane, int row, int b, int r0, int nrows, int n, float* y,
-                                                  const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+                                                  int epilogue, const RopeQkvEpilogue& rope, const Q4KEpiloguePrefetch& pre) {
     constexpr int NV = 16 * B;
     if (epilogue == EPI_ROPE_QKV) {
         // rows 2i and 2i + 1 of a head are one rotation pair; like the SwiGLU pairs they sit NV / (2B) lanes apart
         const float odd = __shfl_xor(val, NV / (2 * B), 64);
         if (lane < NV && !(row & 1) && row < nrows) {
             const int o = r0 + row, slot = o / rope.head_dim, dd = o % rope.head_dim;
-            const int p0 = rope.pos_dev[0];
+            const int p0 = pre.pos;
             float2 out2 = make_float2(val, odd);
             if (slot < rope.heads + rope.kv_heads) {
                 float sn, cs;
-                if (rope.table) { const float2 t = rope.table[dd >> 1]; cs = t.x; sn = t.y; }
+                if (rope.table) { cs = pre.cs.x; sn = pre.cs.y; }
                 else sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
                 out2 = rope_rotate(val, odd, cs, sn);
             }
@@ -100,7 +122,7 @@ __device__ __forceinline__ void q4k_rows_epilogue(float val, int lane, int row, 
         if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
     } else if (lane < NV && row < nrows) {
         const int64_t o = (int64_t)b * n + r0 + row;
-        if (epilogue == EPI_RESIDUAL) val += residual[o];
+        if (epilogue == EPI_RESIDUAL) val += pre.residual;
         y[o] = val;
     }
 }
@@ -141,6 +163,7 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
         const int r0 = wave_r0 + c0 * NR;
         const int nrows = max(0, min(n - r0, NR));               // rows of this chunk that exist (the rest are clamped copies)
         const float first = c0 == 0 ? 1.0f : 0.0f;               // the squares are summed during the first chunk only
+        const Q4KEpiloguePrefetch pre = q4k_epilogue_prefetch<B>(lane, r0, nrows, n, x, residual, epilogue, rope);
 
         float acc[16][B];
 #pragma unroll
@@ -245,7 +268,7 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
         const int idx = wave_fold_index<NV>(lane);
         const int row = idx / B, b = idx % B;
         float val = v[0] * (B == 1 ? xscale[0] : (b == 0 ? xscale[0] : xscale[B - 1]));
-        q4k_rows_epilogue<B>(val, lane, row, b, r0, nrows, n, y, residual, epilogue, rope);
+        q4k_rows_epilogue<B>(val, lane, row, b, r0, nrows, n, y, epilogue, rope, pre);
     }
 }
 
@@ -274,6 +297,10 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_ksplit_kernel(const uint8_t* 
     const uint32_t hi_mask = g >= 2 ? 0xFFFFFFFFu : 0u;
     const int q_off = 16 + g * 32;
     float* xw = &xlds[wave][0];
+
+    // the residual element a lane will add at the end, requested ahead of the weight stream (a valid address either way)
+    const int e_row = wave_fold_index<NV>(lane);
+    const float res_pre = *((epilogue == EPI_RESIDUAL && lane < NV && e_row < nrows) ? residual + r0 + e_row : x);
 
     float acc[16][1];
 #pragma unroll
@@ -337,12 +364,10 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_ksplit_kernel(const uint8_t* 
     if (lane < NV) part[wave][lane] = v[0];
     __syncthreads();
     if (wave == 0 && lane < NV) {
-        const int row = wave_fold_index<NV>(lane);
-        if (row < nrows) {
+        if (e_row < nrows) {
             float val = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
-            const int64_t o = r0 + row;
-            if (epilogue == EPI_RESIDUAL) val += residual[o];
-            y[o] = val;
+            if (epilogue == EPI_RESIDUAL) val += res_pre;
+            y[r0 + e_row] = val;
         }
     }
 }
