@@ -117,6 +117,27 @@ __device__ __forceinline__ u32x2_vec load_u32x2_a2(const uint8_t* p) { return re
 struct __attribute__((packed, aligned(2))) u32x4_a2 { u32x4_vec v; };
 __device__ __forceinline__ u32x4_vec load_u32x4_a2(const uint8_t* p) { return reinterpret_cast<const u32x4_a2*>(p)->v; }
 
+// Sum over the 16 lanes of a DPP row (lanes 16 r .. 16 r + 15), result in every lane: four rotate-and-add steps inside
+// the vector ALU instead of four round trips through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_row_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_row_move<0x128>(v));
+    v = fmaxf(v, dpp_row_move<0x124>(v));
+    v = fmaxf(v, dpp_row_move<0x122>(v));
+    v = fmaxf(v, dpp_row_move<0x121>(v));
+    return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_row_move<0x128>(v);   // row_ror:8
+    v += dpp_row_move<0x124>(v);   // row_ror:4
+    v += dpp_row_move<0x122>(v);   // row_ror:2
+    v += dpp_row_move<0x121>(v);   // row_ror:1
+    return v;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);

@@ -144,6 +144,7 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
     constexpr int SLICE = 68;    // 64 activations + 4 floats of padding: 16-byte aligned and bank-conflict free
     static_assert(NR >= 1 && NR <= Q4K_RMAX, "rows per chunk");
     __shared__ __attribute__((aligned(16))) float xlds[B][64 * SLICE];
+    __shared__ __attribute__((aligned(16))) float ssq_rows[B][16];   // squares of x summed per 16-lane row (RMSNorm prologue)
     const int lane = threadIdx.x & 63;
     // readfirstlane: the wave index is uniform across a wave, and saying so keeps the row addresses scalar
     const int gw = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
@@ -215,7 +216,30 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
                     *reinterpret_cast<float4*>(&xlds[b][(f >> 4) * SLICE + (f & 15) * 4]) = v4;
                 }
             }
+            // RMSNorm prologue: once the last pass of the first chunk is staged every thread has its share of the squares.
+            // Row sums go to LDS in front of the barrier the staging needs anyway, the total is read behind it -- all in
+            // the shadow of the weight loads that are still on their way.
+            const bool ssq_done = PRO && c0 == 0 && blk0 + 16 >= bpr;   // uniform
+            if (ssq_done) {
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    const float t = row16_sum(ssq[b]);
+                    if ((lane & 15) == 0) ssq_rows[b][threadIdx.x >> 4] = t;
+                }
+            }
             __syncthreads();
+            if (ssq_done) {
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    float t = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 16; i += 4) {
+                        const float4 r4 = *reinterpret_cast<const float4*>(&ssq_rows[b][i]);
+                        t += (r4.x + r4.y) + (r4.z + r4.w);
+                    }
+                    xscale[b] = 1.0f / sqrtf(t * (1.0f / (float)k) + eps);
+                }
+            }
 
             float xs[B][64], xsum[B][2];
 #pragma unroll
@@ -242,21 +266,6 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_rows_kernel(const uint8_t* __
                 }
                 __builtin_amdgcn_sched_barrier(0);              // a refill is issued where it is written, not later
             }
-        }
-
-        if (PRO && c0 == 0) {
-            // every workgroup has seen all of x: total the squares over its four waves
-            __syncthreads();                                    // the last pass's slices have been read
-            float* red = &xlds[0][0];
-#pragma unroll
-            for (int b = 0; b < B; ++b) {
-                const float t = wave_sum(ssq[b]);
-                if (lane == 0) red[(threadIdx.x >> 6) * B + b] = t;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int b = 0; b < B; ++b)
-                xscale[b] = 1.0f / sqrtf((red[b] + red[B + b] + red[2 * B + b] + red[3 * B + b]) * (1.0f / (float)k) + eps);
         }
 
         float v[NV];

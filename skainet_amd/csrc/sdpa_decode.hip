@@ -46,27 +46,6 @@ __device__ __forceinline__ float exp_diff(float m_old, float m_new) {
     return m_old == -INFINITY ? 0.f : e;
 }
 
-// Sum over the 16 lanes of a DPP row (lanes 16 r .. 16 r + 15), result in every lane: four rotate-and-add steps inside
-// the vector ALU instead of four round trips through the LDS crossbar.
-template <int CTRL>
-__device__ __forceinline__ float dpp_row_move(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float row16_max(float v) {
-    v = fmaxf(v, dpp_row_move<0x128>(v));
-    v = fmaxf(v, dpp_row_move<0x124>(v));
-    v = fmaxf(v, dpp_row_move<0x122>(v));
-    v = fmaxf(v, dpp_row_move<0x121>(v));
-    return v;
-}
-__device__ __forceinline__ float row16_sum(float v) {
-    v += dpp_row_move<0x128>(v);   // row_ror:8
-    v += dpp_row_move<0x124>(v);   // row_ror:4
-    v += dpp_row_move<0x122>(v);   // row_ror:2
-    v += dpp_row_move<0x121>(v);   // row_ror:1
-    return v;
-}
-
 template <int GS, int DPL>
 __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
     constexpr int D = 16 * DPL;
