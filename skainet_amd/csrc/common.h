@@ -138,43 +138,64 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
+// Wave-wide sum, result in every lane: the 16 lanes of a row inside the vector ALU, the four rows by two shuffles.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    v = row16_sum(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
     return v;
 }
-// Fold NV (a power of two, <= 64) per-lane values across the 64 lanes of a wave with a multi-value butterfly:
-// each of the first log2(NV) steps halves the number of live values (a lane keeps the half selected by one bit of
-// its lane id and hands the other half to its partner), the remaining steps are plain xor-shuffle adds. On return
-// v[0] of lane l holds the wave-wide total of value wave_fold_index<NV>(l). The selects are written as bit-field
-// inserts on the raw bits so they stay one instruction each (a ?: on array elements is turned into an indexed
-// register read, which this target expands into a compare/select chain per element).
+
+// The value of the lane that differs from this one in lane-id bit BIT and shares every higher bit: the partner of one
+// butterfly step. Inside a row of 16 lanes these are DPP moves (row_mirror = lane ^ 15, row_half_mirror = lane ^ 7,
+// quad permutes = lane ^ 2, lane ^ 1: bits below BIT may flip as well, which a step that has not used them yet does not
+// mind); across rows a shuffle through the LDS crossbar.
+template <int BIT>
+__device__ __forceinline__ float fold_partner(float v) {
+    if constexpr (BIT == 5) return __shfl_xor(v, 32, 64);
+    else if constexpr (BIT == 4) return __shfl_xor(v, 16, 64);
+    else if constexpr (BIT == 3) return dpp_row_move<0x140>(v);   // row_mirror
+    else if constexpr (BIT == 2) return dpp_row_move<0x141>(v);   // row_half_mirror
+    else if constexpr (BIT == 1) return dpp_row_move<0x4E>(v);    // quad_perm:[2,3,0,1]
+    else return dpp_row_move<0xB1>(v);                            // quad_perm:[1,0,3,2]
+}
+// One halving step of wave_fold on lane bit BIT: HALF values stay (the lower or the upper half, by the lane's bit), the
+// other HALF go to the partner. The selects are written as bit-field inserts on the raw bits so they stay one
+// instruction each (a ?: on array elements is turned into an indexed register read, which this target expands into a
+// compare/select chain per element).
+template <int BIT, int HALF>
+__device__ __forceinline__ void fold_halve(float* v, int lane) {
+    const uint32_t up = ((lane >> BIT) & 1) ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int i = 0; i < HALF; ++i) {
+        const uint32_t a = __float_as_uint(v[i]), b = __float_as_uint(v[i + HALF]);
+        const float send = __uint_as_float((a & up) | (b & ~up));
+        const float keep = __uint_as_float((b & up) | (a & ~up));
+        v[i] = keep + fold_partner<BIT>(send);
+    }
+}
+template <int BIT, int NV>
+__device__ __forceinline__ void fold_steps(float* v, int lane) {
+    if constexpr ((1 << BIT) < NV) fold_halve<BIT, (1 << BIT)>(v, lane);   // 2 << BIT values are live at this step
+    if constexpr (BIT > 0) fold_steps<BIT - 1, NV>(v, lane);
+}
+// Fold NV (a power of two, <= 64) per-lane values across the 64 lanes of a wave with a multi-value butterfly: the
+// log2(NV) low bits of the lane id, taken from the highest down, each halve the number of live values (a lane keeps
+// the half its bit selects and hands the other half to its partner); the remaining, higher bits are plain adds of
+// v[0] (rotations inside a row, which keep the low bits, then the two cross-row shuffles). On return v[0] of lane l
+// holds the wave-wide total of value wave_fold_index<NV>(l) = l mod NV.
 template <int NV>
 __device__ __forceinline__ void wave_fold(float* v, int lane) {
-    static_assert(NV >= 1 && NV <= 64 && (NV & (NV - 1)) == 0, "every halving must pair all values: NV is a power of two");
-    int mask = 1;
-#pragma unroll
-    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) {
-        const int half = nv >> 1;
-        const uint32_t up = (lane & mask) ? 0xFFFFFFFFu : 0u;
-#pragma unroll
-        for (int i = 0; i < half; ++i) {
-            const uint32_t a = __float_as_uint(v[i]), b = __float_as_uint(v[i + half]);
-            const float send = __uint_as_float((a & up) | (b & ~up));
-            const float keep = __uint_as_float((b & up) | (a & ~up));
-            v[i] = keep + __shfl_xor(send, mask, 64);
-        }
-    }
-#pragma unroll
-    for (int m = NV; m < 64; m <<= 1) v[0] += __shfl_xor(v[0], m, 64);
+    static_assert(NV >= 2 && NV <= 64 && (NV & (NV - 1)) == 0, "every halving must pair all values: NV is a power of two");
+    fold_steps<5, NV>(v, lane);
+    if constexpr (NV <= 8) v[0] += dpp_row_move<0x128>(v[0]);     // row_ror:8
+    if constexpr (NV <= 4) v[0] += dpp_row_move<0x124>(v[0]);     // row_ror:4
+    if constexpr (NV <= 2) v[0] += dpp_row_move<0x122>(v[0]);     // row_ror:2
+    if constexpr (NV <= 16) v[0] += __shfl_xor(v[0], 16, 64);
+    if constexpr (NV <= 32) v[0] += __shfl_xor(v[0], 32, 64);
 }
 template <int NV>
-__device__ __forceinline__ int wave_fold_index(int lane) {
-    int idx = 0, mask = 1;
-#pragma unroll
-    for (int nv = NV; nv > 1; nv >>= 1, mask <<= 1) idx += (lane & mask) ? (nv >> 1) : 0;
-    return idx;
-}
+__device__ __forceinline__ int wave_fold_index(int lane) { return lane & (NV - 1); }
 
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

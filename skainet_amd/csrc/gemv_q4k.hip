@@ -98,8 +98,8 @@ __device__ __forceinline__ void q4k_rows_epilogue(float val, int lane, int row, 
                                                   int epilogue, const RopeQkvEpilogue& rope, const Q4KEpiloguePrefetch& pre) {
     constexpr int NV = 16 * B;
     if (epilogue == EPI_ROPE_QKV) {
-        // rows 2i and 2i + 1 of a head are one rotation pair; like the SwiGLU pairs they sit NV / (2B) lanes apart
-        const float odd = __shfl_xor(val, NV / (2 * B), 64);
+        // rows 2i and 2i + 1 of a head are one rotation pair; like the SwiGLU pairs they sit B lanes apart (lane = row * B + b)
+        const float odd = __shfl_xor(val, B, 64);
         if (lane < NV && !(row & 1) && row < nrows) {
             const int o = r0 + row, slot = o / rope.head_dim, dd = o % rope.head_dim;
             const int p0 = pre.pos;
@@ -117,8 +117,8 @@ __device__ __forceinline__ void q4k_rows_epilogue(float val, int lane, int row, 
             *reinterpret_cast<float2*>(dst + dd) = out2;
         }
     } else if (epilogue == EPI_SWIGLU) {
-        // rows 2j (gate) and 2j + 1 (up) of this wave sit NV / (2B) lanes apart after the fold
-        const float up = __shfl_xor(val, NV / (2 * B), 64);
+        // rows 2j (gate) and 2j + 1 (up) of this wave sit B lanes apart after the fold (lane = row * B + b)
+        const float up = __shfl_xor(val, B, 64);
         if (lane < NV && !(row & 1) && row < nrows) y[(int64_t)b * (n >> 1) + ((r0 + row) >> 1)] = val * (1.0f / (1.0f + expf(-val))) * up;
     } else if (lane < NV && row < nrows) {
         const int64_t o = (int64_t)b * n + r0 + row;
