@@ -56,7 +56,7 @@ ATTENTION_PREFILL_USES_MFMA = True    # the prompt-shape attention kernel runs b
 # measured report null.
 MEASURED_TRAFFIC_BYTES = {"q4k_gemv_11008x4096_b1": 25776538, "q4k_gemv_11008x4096_b8": 27202560, "q4k_gemv_11008x4096_b4": 26220954,
                           "q8_0_gemv_4096x4096_b1": 18091400, "q4k_gemm_512x4096x4096": 76910600,
-                          "sdpa_decode_4096_b1": 34923300, "sdpa_decode_4096_b8": 270405900, "sdpa_prefill_2048": 131414600}
+                          "sdpa_decode_4096_b1": 34856300, "sdpa_decode_4096_b8": 270339900, "sdpa_prefill_2048": 131414600}
 
 
 def algorithmic_bytes(enc, n, k, m):
