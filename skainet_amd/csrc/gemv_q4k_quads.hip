@@ -34,20 +34,35 @@ constexpr int QD_SLICE = 36;   // dwords per slice: 64 bf16 activations + 4 dwor
 
 // Fold 16 per-lane values across the 16 four-lane blocks of a wave (lane bits 2..5), leaving bits 0..1 apart: on
 // return v[0] of lane l is the total, over the lanes with the same l % 4, of value block_fold_index(l).
-__device__ __forceinline__ void block_fold16(float* v, int lane) {
-    int mask = 4;
-#pragma unroll
-    for (int nv = 16; nv > 1; nv >>= 1, mask <<= 1) {
-        const int half = nv >> 1;
-        const uint32_t up = (lane & mask) ? 0xFFFFFFFFu : 0u;
-#pragma unroll
-        for (int i = 0; i < half; ++i) {
-            const uint32_t a = __float_as_uint(v[i]), b = __float_as_uint(v[i + half]);
-            const float send = __uint_as_float((a & up) | (b & ~up));
-            const float keep = __uint_as_float((b & up) | (a & ~up));
-            v[i] = keep + __shfl_xor(send, mask, 64);
-        }
+// The partners 4 and 8 lanes away are inside the lane's row of 16: DPP moves (lane ^ 8 is a rotation by 8; lane ^ 4 is a
+// shift left by 4 for the lanes of banks 0 and 2 and a shift right by 4 for banks 1 and 3, two moves under bank masks).
+template <int MASK>
+__device__ __forceinline__ float block_fold_partner(float v) {
+    if constexpr (MASK == 4) {
+        const int up = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x104, 0xF, 0x5, false);      // row_shl:4 -> lane + 4
+        return __int_as_float(__builtin_amdgcn_update_dpp(up, __float_as_int(v), 0x114, 0xF, 0xA, false));   // row_shr:4 -> lane - 4
+    } else if constexpr (MASK == 8) {
+        return dpp_row_move<0x128>(v);                                                                    // row_ror:8
+    } else {
+        return __shfl_xor(v, MASK, 64);
     }
+}
+template <int MASK, int HALF>
+__device__ __forceinline__ void block_fold_step(float* v, int lane) {
+    const uint32_t up = (lane & MASK) ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int i = 0; i < HALF; ++i) {
+        const uint32_t a = __float_as_uint(v[i]), b = __float_as_uint(v[i + HALF]);
+        const float send = __uint_as_float((a & up) | (b & ~up));
+        const float keep = __uint_as_float((b & up) | (a & ~up));
+        v[i] = keep + block_fold_partner<MASK>(send);
+    }
+}
+__device__ __forceinline__ void block_fold16(float* v, int lane) {
+    block_fold_step<4, 8>(v, lane);
+    block_fold_step<8, 4>(v, lane);
+    block_fold_step<16, 2>(v, lane);
+    block_fold_step<32, 1>(v, lane);
 }
 __device__ __forceinline__ int block_fold_index(int lane) {
     return ((lane & 4) ? 8 : 0) + ((lane & 8) ? 4 : 0) + ((lane & 16) ? 2 : 0) + ((lane & 32) ? 1 : 0);
