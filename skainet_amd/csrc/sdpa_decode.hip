@@ -309,7 +309,7 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
     SdpaDecodeParams p{q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, scale, window, right_context, lengths, 1,
                        nullptr};
     // enough workgroups to put every CU on the cache, at least 64 keys per split (measured in the decoder at 500 to 650
-    // keys: 32 keys per split 4 % slower per token, 128 keys 1 % slower)
+    // keys: 32 or 48 keys per split 2.5 % slower per token, 96 and 128 keys the same as 64)
     const int64_t groups = (int64_t)batch * kv_heads * subs;
     int splits = (int)((2 * (int64_t)num_cus() + groups - 1) / groups);
     splits = min(splits, min(SDPA_DECODE_MAX_SPLITS, (seq_kv + g_sdpa_decode_split_keys - 1) / g_sdpa_decode_split_keys));
