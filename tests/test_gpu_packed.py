@@ -115,13 +115,14 @@ def test_gemv_at_config_sizes(hip_backend, torch_cuda, enc, n, k, batches):
 
 
 @pytest.mark.parametrize("mode", ["slot-fp32", "rows-fp32"])
-@pytest.mark.parametrize("n,k,m", [(11008, 4096, 1), (11008, 4096, 2), (4096, 14336, 1), (2050, 8448, 1), (1000, 11008, 1), (77, 2304, 2),
-                                   (5, 256, 1)])
+@pytest.mark.parametrize("n,k,m", [(11008, 4096, 1), (11008, 4096, 2), (4096, 14336, 1), (2050, 8448, 1), (1537, 16640, 1), (6144, 8192, 1),
+                                   (1000, 11008, 1), (77, 2304, 2), (5, 256, 1)])
 def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cuda, mode, n, k, m):
     """Both Q4_K decode kernels (the generic slot kernel and the row-streaming kernel) are held to the same bound
     against the exact-fp32 oracle, on quantised Gaussian weights and on random valid blocks with large scales. The
-    long-row shapes (4096 x 14336, 2050 x 8448: 33 super-blocks per row, a ragged last workgroup) take the form of the
-    row kernel that splits K over the waves of a workgroup."""
+    long-row shapes (4096 x 14336; 2050 x 8448: 33 super-blocks per row, a ragged last workgroup; 1537 x 16640: 65
+    super-blocks, two passes per wave, four rows per workgroup; 6144 x 8192: twelve) take the form of the row kernel that
+    splits K over the waves of a workgroup."""
     hip_backend.set_tuning("q4k_rows_enable", 1 if mode == "rows-fp32" else 0)
     try:
         for packed in (gaussian_weight(hip_backend, "Q4_K", n, k, 71), random_valid_blocks("Q4_K", n * k // 256, 72)):
