@@ -359,7 +359,9 @@ template <class F, int B, int R>
 __global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
     const uint8_t* __restrict__ w, const float* __restrict__ x, float* __restrict__ y,
     int k, int n, int batch, int64_t row_bytes, int rows_per_wg) {
-    constexpr int NX = F::NX, NS = XSumCount<F>::N, NV = R * B;
+    constexpr int NX = F::NX, NS = XSumCount<F>::N;
+    constexpr int NV = (R * B <= 2) ? 2 : (R * B <= 4) ? 4 : (R * B <= 8) ? 8 : 16;   // fold width: the next power of two, zero padded
+    static_assert(R * B <= 16, "at most 16 values per fold");
     __shared__ float partial[GEMV_MAX_WAVES][GEMV_MAX_ROWS][B];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
@@ -408,6 +410,8 @@ __global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
         for (int r = 0; r < nrows; r += R) {
             float acc[NV];
 #pragma unroll
+            for (int i = R * B; i < NV; ++i) acc[i] = 0.f;
+#pragma unroll
             for (int i = 0; i < R; ++i) {
                 float a[B];
 #pragma unroll
@@ -421,7 +425,7 @@ __global__ __launch_bounds__(64 * GEMV_MAX_WAVES) void gemv_kernel(
             wave_fold<NV>(acc, lane);
             if (lane < NV) {
                 const int i = my_value / B, b = my_value % B;
-                if (r + i < nrows) {
+                if (i < R && r + i < nrows) {
                     float* dst = &partial[wave][r + i][b];
                     *dst = pass == 0 ? acc[0] : *dst + acc[0];
                 }
@@ -457,9 +461,16 @@ static int launch_one(const uint8_t* w, const float* x, float* y, int k, int n, 
     return 0;
 }
 
+// Weight rows a wave keeps in flight at batch 1, per format (measured over 2 .. 8 on the 11008 x 4096, 32000 x 4096 and
+// 4096 x 4096 shapes: the formats with many loads per row are faster with fewer rows requested at once).
+template <class F> struct RowsInFlight { static constexpr int B1 = 8; };
+template <> struct RowsInFlight<Q80Slot> { static constexpr int B1 = 3; };
+template <> struct RowsInFlight<Q6KSlot> { static constexpr int B1 = 2; };
+template <> struct RowsInFlight<Q5KSlot> { static constexpr int B1 = 3; };
+
 template <class F>
 static int launch_format(const uint8_t* w, const float* x, float* y, int k, int n, int batch, int waves_per_cu) {
-    if (batch == 1) return launch_one<F, 1, 8>(w, x, y, k, n, batch, waves_per_cu);
+    if (batch == 1) return launch_one<F, 1, RowsInFlight<F>::B1>(w, x, y, k, n, batch, waves_per_cu);
     if (batch == 2) return launch_one<F, 2, 4>(w, x, y, k, n, batch, waves_per_cu);
     return launch_one<F, 4, 2>(w, x, y, k, n, batch, waves_per_cu);
 }
