@@ -37,6 +37,8 @@ WORKLOADS = {
     "q4k_gemv_11008x4096_b8": ("Q4_K", 11008, 4096, 8),
     "q8_0_gemv_4096x4096_b1": ("Q8_0", 4096, 4096, 1),
     "q6k_gemv_32000x4096_b1": ("Q6_K", 32000, 4096, 1),
+    # the decoder's down projection: long rows, K split over the waves of a workgroup
+    "q4k_gemv_4096x14336_b1": ("Q4_K", 4096, 14336, 1),
     # the remaining packed formats of the provider SPI, at the headline shape
     "q4_0_gemv_11008x4096_b1": ("Q4_0", 11008, 4096, 1),
     "q5_0_gemv_11008x4096_b1": ("Q5_0", 11008, 4096, 1),
@@ -55,7 +57,7 @@ ATTENTION_PREFILL_USES_MFMA = True    # the prompt-shape attention kernel runs b
 # of the dominant kernel; the runs and their raw readings are in the summaries under profiles/. Workloads not
 # measured report null.
 MEASURED_TRAFFIC_BYTES = {"q4k_gemv_11008x4096_b1": 25776538, "q4k_gemv_11008x4096_b8": 27202560, "q4k_gemv_11008x4096_b4": 26220954,
-                          "q8_0_gemv_4096x4096_b1": 18091400, "q4k_gemm_512x4096x4096": 76910600,
+                          "q8_0_gemv_4096x4096_b1": 18091400, "q4k_gemv_4096x14336_b1": 33662400, "q4k_gemm_512x4096x4096": 76910600,
                           "sdpa_decode_4096_b1": 34856300, "sdpa_decode_4096_b8": 270339900, "sdpa_prefill_2048": 131414600}
 
 
