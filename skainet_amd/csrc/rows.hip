@@ -284,10 +284,10 @@ __global__ __launch_bounds__(256) void rope_qkv_kernel(const float* __restrict__
                                                        const int32_t* __restrict__ pos_dev, float theta) {
     const int half = head_dim >> 1;
     const int slots = heads + 2 * kv_heads;
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (token, pair)
-    if (idx >= (int64_t)tokens * half) return;
-    const int i = (int)(idx % half);
-    const int t = (int)(idx / half);
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (token, pair); the host checks the count fits 31 bits
+    if (idx >= (uint32_t)tokens * (uint32_t)half) return;
+    const int i = (int)(idx % (uint32_t)half);
+    const int t = (int)(idx / (uint32_t)half);
     const int p0 = pos_dev ? pos_dev[0] : pos_start;
     const float freq = powf(theta, -2.0f * (float)i / (float)head_dim);
     float sn, cs;
@@ -382,6 +382,7 @@ int launch_rope_qkv(const float* qkv, float* q_out, float* k_cache, float* v_cac
     if (!pos_dev && (pos_start < 0 || pos_start + tokens > kv_capacity))
         return set_error("rope_qkv: positions [%d, %d) do not fit a cache of %d rows", pos_start, pos_start + tokens, kv_capacity);
     const int64_t n = (int64_t)tokens * (head_dim / 2);
+    if (n >= (int64_t)1 << 31) return set_error("rope_qkv: %d tokens x %d pairs exceed the 31-bit thread index", tokens, head_dim / 2);
     const int slot_blocks = (heads + 2 * kv_heads + ROPE_SLOTS_PER_BLOCK - 1) / ROPE_SLOTS_PER_BLOCK;
     rope_qkv_kernel<<<dim3((unsigned)((n + 255) / 256), slot_blocks), dim3(256), 0, current_stream()>>>(
         qkv, q_out, k_cache, v_cache, tokens, heads, kv_heads, head_dim, kv_capacity, pos_start, pos_dev, theta);
