@@ -69,6 +69,11 @@ SKAINET_HIP_API int32_t skainet_hip_compute_units(void);
 SKAINET_HIP_API int32_t skainet_hip_set_stream(void* stream);
 /* Wait for this thread's stream. */
 SKAINET_HIP_API int32_t skainet_hip_sync(void);
+/* Frees the calling thread's scratch (workspace, staging buffers of the host-pointer entries, counters, timer events)
+ * after waiting for its stream. For worker threads that end before the process does (the reference's schedule workers,
+ * skainet-backend-api/.../kernel/KernelDispatch.kt:28-32, may call in from any thread); no reference counterpart: the CPU
+ * library's per-call malloc / free needs none. Free this thread's recorded graphs first. 0 on success. */
+SKAINET_HIP_API int32_t skainet_hip_thread_release(void);
 
 /* Device buffers: the backing store of a Storage.Device
  * (REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/memory/Storage.kt:230). */

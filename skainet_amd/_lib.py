@@ -27,6 +27,7 @@ SIGNATURES = {
     "skainet_hip_compute_units": (_i32, []),
     "skainet_hip_set_stream": (_i32, [_vp]),
     "skainet_hip_sync": (_i32, []),
+    "skainet_hip_thread_release": (_i32, []),
     "skainet_hip_malloc": (_vp, [_sz]),
     "skainet_hip_free": (_i32, [_vp]),
     "skainet_hip_memcpy_h2d": (_i32, [_vp, _vp, _sz]),

@@ -177,6 +177,30 @@ int32_t skainet_hip_sync(void) {
     if (ensure_device() != 0) return -1;
     return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
 }
+// The calling thread's scratch (kernel workspace, staging of the host-pointer entries, counters, timer events) goes back
+// to the device: for worker threads that end while the process lives on. Recorded graphs of this thread hold the old
+// addresses and must be freed first; the next call on this thread allocates afresh.
+int32_t skainet_hip_thread_release(void) {
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        if (g_state != 1) return 0;   // nothing was ever allocated
+    }
+    if (ensure_device() != 0) return -1;
+    int rc = check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+    auto drop = [&](Scratch& sc) {
+        if (sc.ptr && check_hip(hipFree(sc.ptr), "hipFree(scratch)") != 0) rc = -1;
+        sc.ptr = nullptr; sc.cap = 0;
+    };
+    drop(t_workspace);
+    for (Scratch& sc : t_stage) drop(sc);
+    for (Scratch& sc : t_fuse) drop(sc);
+    if (t_sync && check_hip(hipFree(t_sync), "hipFree(sync scratch)") != 0) rc = -1;
+    t_sync = nullptr;
+    if (t_ev0 && check_hip(hipEventDestroy(t_ev0), "hipEventDestroy") != 0) rc = -1;
+    if (t_ev1 && check_hip(hipEventDestroy(t_ev1), "hipEventDestroy") != 0) rc = -1;
+    t_ev0 = t_ev1 = nullptr;
+    return rc;
+}
 void* skainet_hip_malloc(size_t bytes) {
     if (ensure_device() != 0) return nullptr;
     void* p = nullptr;

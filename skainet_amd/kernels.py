@@ -213,6 +213,12 @@ def sync() -> None:
     check(_lib.hip().skainet_hip_sync(), "sync")
 
 
+def thread_release() -> None:
+    """Give the calling thread's library scratch back to the device (skainet_hip_thread_release): for worker threads
+    that end before the process does. Graphs recorded on this thread must be freed first."""
+    check(_lib.hip().skainet_hip_thread_release(), "thread_release")
+
+
 def rms_norm_dev(x, gamma, out, rows: int, cols: int, eps: float) -> None:
     check(_lib.hip().skainet_hip_f32_rms_norm_dev(_ptr(x), _ptr(gamma), _ptr(out), rows, cols, eps), "rms_norm")
 

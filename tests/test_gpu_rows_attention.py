@@ -341,3 +341,51 @@ def test_narrow_float_matmuls(hip_backend, torch_cuda, kind, codec):
     assert not z.any()
     with pytest.raises(ValueError):
         kern.matmul(a, 0, k + 9, raw, 0, stride, z, 0, 6, 4, 6, -1)
+
+
+def test_thread_release_frees_and_regrows_scratch(hip_backend, torch_cuda):
+    """A worker thread's scratch can be handed back (skainet_hip_thread_release); calls after it allocate afresh and
+    give the same bits, and the memory the thread held is free again."""
+    import threading
+    from oracle import golden as G
+    torch = torch_cuda
+    provider = hip_backend.HipKernelProvider()
+    n, nblocks = 96, 4
+    k = nblocks * 256
+    blocks = G.weight_blocks("Q4_K", n, nblocks, 0x5EED0700)
+    x = G.floats(k, 0x5EED0701)
+    want = L.gemv("Q4_K", x, G.row_major(blocks), n)
+    b, h, hkv, skv, d = 2, 8, 2, 300, 64           # decode shape: split partials live in the thread's workspace
+    q, kk, vv = sdpa_inputs(b, h, hkv, 1, skv, d, 31)
+    results, errors = {}, []
+
+    def worker():
+        try:
+            kernel = provider.matmul_q4k()
+            att = provider.attention_fp32()
+            for tag in ("before", "after"):
+                y = np.zeros(n, np.float32)
+                kernel.matmul_row_major(x, 0, G.row_major(blocks), 0, k, n, y, 0)
+                o = np.zeros(b * h * d, np.float32)
+                att.sdpa(q, kk, vv, o, b, h, hkv, 1, skv, d, 0.125, True, 0, 0)
+                big = np.ones((4096, 4096), np.float32)              # 64 MiB staged on the device by the host-pointer entry
+                provider.norm_fp32().rms_norm(big, 0, np.ones(4096, np.float32), np.empty_like(big), 0, 4096, 4096, 1e-5)
+                results[tag] = (y, o)
+                if tag == "before":
+                    hip_backend.sync()
+                    held = torch.cuda.mem_get_info()[0]
+                    hip_backend.thread_release()
+                    results["freed"] = torch.cuda.mem_get_info()[0] - held
+            hip_backend.thread_release()
+            hip_backend.thread_release()                              # idempotent
+        except Exception as e:                                        # surfaced in the main thread below
+            errors.append(e)
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert not errors, errors
+    assert normalized_err(results["before"][0], want) <= 1e-3
+    assert np.array_equal(results["before"][0], results["after"][0])
+    assert np.array_equal(results["before"][1], results["after"][1])
+    assert results["freed"] >= 64 << 20, results["freed"]
