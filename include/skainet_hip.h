@@ -306,7 +306,8 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
 
 /* Launch-shape knobs for experiments (defaults are the measured best). Keys: "gemv_waves_per_cu",
  * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares, 0 = chosen from the shape),
- * "q4k_rows_enable" (0: Q4_K decode shapes take the generic slot kernel), "q4k_ksplit_enable" (0: long Q4_K rows are not
+ * "q4k_rows_enable" (0: Q4_K decode shapes take the generic slot kernel), "q6k_slot64" (0: Q6_K at batch 1 keeps the
+ * 32-weight slot of the batched kernel), "q4k_ksplit_enable" (0: long Q4_K rows are not
  * split over the waves of a workgroup), "gemm_ksplit" (K splits of the MFMA GEMM,
  * 0 = automatic), "gemm_wide" (1 / 0: force the 256 x 256 / 256 x 128 tile, -1 = chosen from the shape),
  * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_decode_split_keys" (least keys per split of

@@ -19,6 +19,7 @@
 //     order, so results are deterministic.
 //   * Grid: contiguous row ranges, sized so the whole chip gets an even share (rows_per_wg from the host).
 #include "common.h"
+#include <type_traits>
 
 #include <cstring>
 
@@ -168,6 +169,82 @@ struct Q6KSlot {
                 for (int j = 0; j < 4; ++j) {
 #pragma unroll
                     for (int b = 0; b < B; ++b) s[k][b] = fmaf(x[b][8 * k + 4 * h + j], cf[j], s[k][b]);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            float a = 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) a = fmaf(sc[k], s[k][b], a);
+            acc[b] = a;
+        }
+    }
+};
+
+// Q6_K at batch 1: a slot is 64 weights -- 16 consecutive positions l of one half of a super-block in all four quarters
+// (elements half * 128 + 32 k + l) -- so the three code runs are one 16-byte load each (2-byte aligned) instead of two
+// slots of 8-byte loads: half the load instructions per weight. Four lanes per super-block; a 4096-wide row is one wave.
+struct Q6KSlot64 {
+    static constexpr int BLOCK_BYTES = Q6K_BYTES, SLOTS_PER_BLOCK = 4, SLOT_ELEMS = 64, NX = 64;
+    struct Raw { u32x4_vec qla, qlb, qh; u32x2_vec sc; uint32_t d; };
+    struct Lane { int blk_off, ql_off, qh_off, sc_off, sc_shift; };
+    __device__ static void init(Lane& ln, int slot) {
+        const int blk = slot >> 2, t = slot & 3, half = t >> 1, l0 = (t & 1) * 16;
+        ln.blk_off = blk * BLOCK_BYTES;
+        ln.ql_off = ln.blk_off + half * 64 + l0;
+        ln.qh_off = ln.blk_off + 128 + half * 32 + l0;
+        ln.sc_off = ln.blk_off + 192 + half * 8;
+        ln.sc_shift = (l0 >> 4) * 8;
+    }
+    // Register i = 16 * k + j pairs with element half*128 + 32*k + l0 + j.
+    __device__ static int x_index(int slot, int i) {
+        const int blk = slot >> 2, t = slot & 3, half = t >> 1, l0 = (t & 1) * 16;
+        return blk * 256 + half * 128 + (i >> 4) * 32 + l0 + (i & 15);
+    }
+    __device__ static void load(Raw& r, const uint8_t* row, const Lane& ln) {
+        r.qla = load_u32x4_a2(row + ln.ql_off);
+        r.qlb = load_u32x4_a2(row + ln.ql_off + 32);
+        r.qh = load_u32x4_a2(row + ln.qh_off);
+        r.sc = load_u32x2_a2(row + ln.sc_off);
+        r.d = load_u16(row + ln.blk_off + 208);
+    }
+    __device__ static void prep(const float* x, float* xsum) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s += x[16 * k + j];
+            xsum[k] = 32.f * s;
+        }
+    }
+    template <int B>
+    __device__ static void dot(const Raw& r, const Lane& ln, const float (*x)[NX], const float (*xsum)[4], float* acc) {
+        const float d = half_bits_to_float_fast(r.d);
+        const uint32_t s0 = r.sc.x >> ln.sc_shift, s1 = r.sc.y >> ln.sc_shift;
+        const float sc[4] = {d * (float)(int8_t)(s0), d * (float)(int8_t)(s0 >> 16),
+                             d * (float)(int8_t)(s1), d * (float)(int8_t)(s1 >> 16)};
+        const uint32_t qla[4] = {r.qla.x, r.qla.y, r.qla.z, r.qla.w}, qlb[4] = {r.qlb.x, r.qlb.y, r.qlb.z, r.qlb.w},
+                       qh[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+        float s[4][B];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int b = 0; b < B; ++b) s[k][b] = -xsum[b][k];       // the -32 bias of every code, taken out of the loop
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            const uint32_t c[4] = {
+                (qla[h] & 0x0F0F0F0Fu) | ((qh[h] << 4) & 0x30303030u),
+                (qlb[h] & 0x0F0F0F0Fu) | ((qh[h] << 2) & 0x30303030u),
+                ((qla[h] >> 4) & 0x0F0F0F0Fu) | (qh[h] & 0x30303030u),
+                ((qlb[h] >> 4) & 0x0F0F0F0Fu) | ((qh[h] >> 2) & 0x30303030u)};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float cf[4] = {ubyte0_to_float(c[k]), ubyte1_to_float(c[k]), ubyte2_to_float(c[k]), ubyte3_to_float(c[k])};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int b = 0; b < B; ++b) s[k][b] = fmaf(x[b][16 * k + 4 * h + j], cf[j], s[k][b]);
                 }
             }
         }
@@ -352,6 +429,7 @@ struct Q5KSlot {
 template <class F> struct XSumCount { static constexpr int N = 1; };
 template <> struct XSumCount<Q4KSlot> { static constexpr int N = 2; };
 template <> struct XSumCount<Q6KSlot> { static constexpr int N = 4; };
+template <> struct XSumCount<Q6KSlot64> { static constexpr int N = 4; };
 template <> struct XSumCount<Q5KSlot> { static constexpr int N = 2; };
 
 // F: slot policy, B: activation rows per launch (1, 2 or 4; unused ones are zero), R: weight rows in flight.
@@ -468,14 +546,22 @@ template <> struct RowsInFlight<Q80Slot> { static constexpr int B1 = 3; };
 template <> struct RowsInFlight<Q6KSlot> { static constexpr int B1 = 2; };
 template <> struct RowsInFlight<Q5KSlot> { static constexpr int B1 = 3; };
 
+static int g_gemv_waves_per_cu = 0;   // 0: per encoding (measured best: Q8_0 4, Q6_K at batch 1 6, the others 8)
+static int g_q6k_slot64 = 1;   // 0: Q6_K at batch 1 stays on the 32-weight slot
+
 template <class F>
 static int launch_format(const uint8_t* w, const float* x, float* y, int k, int n, int batch, int waves_per_cu) {
-    if (batch == 1) return launch_one<F, 1, RowsInFlight<F>::B1>(w, x, y, k, n, batch, waves_per_cu);
+    if (batch == 1) {
+        // Q6_K: the 64-weight slot, 2 rows in flight, 6 waves per CU unless the caller set a count (measured on 32000 x 4096
+        // over 1 .. 4 rows and 5 .. 16 waves: 23.1 us against 25.5 us for the 32-weight slot at its best, 2 rows and 8 waves)
+        if (std::is_same<F, Q6KSlot>::value && g_q6k_slot64)
+            return launch_one<Q6KSlot64, 1, 2>(w, x, y, k, n, batch, g_gemv_waves_per_cu > 0 ? g_gemv_waves_per_cu : 6);
+        return launch_one<F, 1, RowsInFlight<F>::B1>(w, x, y, k, n, batch, waves_per_cu);
+    }
     if (batch == 2) return launch_one<F, 2, 4>(w, x, y, k, n, batch, waves_per_cu);
     return launch_one<F, 4, 2>(w, x, y, k, n, batch, waves_per_cu);
 }
 
-static int g_gemv_waves_per_cu = 0;   // 0: per encoding (measured best: Q8_0 4, Q4_K / Q6_K 8)
 static int g_q4k_rows_enable = 1;
 void set_q4k_rows_waves_per_cu(int v);
 void set_gemm_wide(int v);
@@ -490,6 +576,7 @@ int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int
 int set_tuning(const char* key, int value) {
     if (!strcmp(key, "gemv_waves_per_cu")) { if (value >= 0) g_gemv_waves_per_cu = value; return 0; }
     if (!strcmp(key, "q4k_rows_waves_per_cu")) { set_q4k_rows_waves_per_cu(value); return 0; }
+    if (!strcmp(key, "q6k_slot64")) { g_q6k_slot64 = value != 0; return 0; }
     if (!strcmp(key, "gemm_wide")) { set_gemm_wide(value); return 0; }
     if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }
     if (!strcmp(key, "gemm_ksplit")) { set_gemm_ksplit(value); return 0; }

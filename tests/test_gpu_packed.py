@@ -137,6 +137,26 @@ def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cud
         hip_backend.set_tuning("q4k_rows_enable", 1)
 
 
+@pytest.mark.parametrize("slot64", [1, 0])
+@pytest.mark.parametrize("n,k", [(8000, 4096), (515, 4096), (70, 768), (33, 256), (257, 14336), (3, 16640)])
+def test_q6k_batch1_slot_variants_agree_with_the_oracle(hip_backend, torch_cuda, slot64, n, k):
+    """Q6_K at batch 1 with the 64-weight slot (16-byte code loads, the default) and with the 32-weight slot of the
+    batched kernel: the same bound against the exact-fp32 oracle, on quantised Gaussian weights and on random valid
+    blocks; rows of one super-block, rows longer than one wave pass, ragged last workgroups."""
+    hip_backend.set_tuning("q6k_slot64", slot64)
+    try:
+        for packed in (gaussian_weight(hip_backend, "Q6_K", n, k, 81), random_valid_blocks("Q6_K", n * k // 256, 82)):
+            x = np.random.default_rng(83).standard_normal((1, k)).astype(np.float32)
+            x[0, :64] = 0.0
+            x[0, 100] = 37.5
+            got = gpu_matmul(hip_backend, torch_cuda, "Q6_K", packed, n, k, x)
+            err = normalized_err(got, L.gemv("Q6_K", x, packed, n))
+            print(f"slot64={slot64} {n}x{k}: {err:.2e}")
+            assert err <= GEMV_TOL
+    finally:
+        hip_backend.set_tuning("q6k_slot64", 1)
+
+
 @pytest.mark.parametrize("n,k,m", [(5, 256, 3), (25, 1280, 8), (77, 2304, 7), (1000, 11008, 4), (11008, 4096, 6), (4096, 14336, 8),
                                    (130, 4096, 9), (64, 1024, 11)])
 def test_q4k_three_to_eight_rows_on_the_matrix_instruction(hip_backend, torch_cuda, n, k, m):
