@@ -57,7 +57,7 @@ ATTENTION_PREFILL_USES_MFMA = True    # the prompt-shape attention kernel runs b
 # of the dominant kernel; the runs and their raw readings are in the summaries under profiles/. Workloads not
 # measured report null.
 MEASURED_TRAFFIC_BYTES = {"q4k_gemv_11008x4096_b1": 25776538, "q4k_gemv_11008x4096_b8": 27202560, "q4k_gemv_11008x4096_b4": 26220954,
-                          "q8_0_gemv_4096x4096_b1": 18091400, "q4k_gemv_4096x14336_b1": 33662400, "q4k_gemm_512x4096x4096": 76910600,
+                          "q8_0_gemv_4096x4096_b1": 18091400, "q6k_gemv_32000x4096_b1": 107947150, "q4k_gemv_4096x14336_b1": 33662400, "q4k_gemm_512x4096x4096": 76910600,
                           "sdpa_decode_4096_b1": 34856300, "sdpa_decode_4096_b8": 270339900, "sdpa_prefill_2048": 131414600}
 
 
