@@ -262,6 +262,13 @@ SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_cache_dev(const float* q, const flo
 SKAINET_HIP_API int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* out, int64_t n);
 SKAINET_HIP_API int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int64_t n);
 SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
+/* skainet_hip_f32_argmax_rows_dev for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it). No counterpart in the reference. Same result (first maximum of each row);
+ * the partial pairs and arrival counters live in a fixed 33 KiB array inside the library's code object instead of scratch
+ * the library allocates, so the call makes no allocation of any kind. At most 64 rows per call (more is refused with
+ * -1 and a message; cols is unbounded). Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (two streams, two threads) race, calls on one stream are safe. */
+SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_noalloc_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
 
 /* Decoder glue the reference keeps in its external transformer repository (no counterpart in /root/reference; the
  * semantics are the standard Llama ones and are checked against closed forms):

@@ -9,6 +9,9 @@
 //   silu_mul      x * (1 / (1 + exp(-x))) * up                 f32_ops.c:222-244 (silu), binary mul
 //   argmax        first index of the row maximum               TensorOps.kt:263-277 (ties -> lowest index)
 #include "common.h"
+#include "../../include/skainet_hip.h"
+
+#include <mutex>
 
 namespace skh {
 
@@ -485,6 +488,49 @@ int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out) {
     SKH_CHECK(hipGetLastError());
     return 0;
 }
+// ---- arg-max for callers that cannot allocate ----
+// The same many-workgroups-per-row kernel, with its pairs and counters in a fixed array that is part of the loaded code
+// object: every GPU the library runs on holds its own copy until the process ends. In host code the array's name is
+// only a handle; the device address comes from hipGetSymbolAddress, once per device, and that address is what the
+// kernels are given.
+static __device__ __align__(256) unsigned char scratch[sizeof(ArgmaxScratch)];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static void* g_noalloc_scratch[NOALLOC_MAX_DEVICES];    // per device, filled on first use
+static std::mutex g_noalloc_mutex;
+
+__global__ void argmax_clear_kernel(ArgmaxScratch* __restrict__ sc, int rows) {
+    if ((int)threadIdx.x < rows) sc->done[threadIdx.x] = 0u;
+}
+
+static ArgmaxScratch* noalloc_scratch() {
+    int dev = -1;
+    if (check_hip(hipGetDevice(&dev), "hipGetDevice") != 0) return nullptr;
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) { set_error("argmax_rows_noalloc: device ordinal %d is beyond the %d this entry keeps scratch for", dev, NOALLOC_MAX_DEVICES); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    if (!g_noalloc_scratch[dev]) {
+        void* ptr = nullptr;
+        if (check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)") != 0) return nullptr;
+        if (!ptr) { set_error("argmax_rows_noalloc: no device address for the scratch array"); return nullptr; }
+        g_noalloc_scratch[dev] = ptr;
+    }
+    return static_cast<ArgmaxScratch*>(g_noalloc_scratch[dev]);
+}
+
+int launch_argmax_rows_noalloc(const float* in, int rows, int cols, int32_t* out) {
+    if (rows <= 0 || cols <= 0) return 0;
+    if (rows > ARGMAX_MAX_ROWS)
+        return set_error("argmax_rows_noalloc: %d rows exceed the %d rows the fixed scratch holds; use skainet_hip_f32_argmax_rows_dev", rows, ARGMAX_MAX_ROWS);
+    ArgmaxScratch* sc = noalloc_scratch();
+    if (!sc) return -1;
+    // the array keeps what the last call left: the arrival counters must start at zero (a fill kernel, not a memset
+    // node, so the pair can be recorded into a graph)
+    argmax_clear_kernel<<<dim3(1), dim3(ARGMAX_MAX_ROWS), 0, current_stream()>>>(sc, rows);
+    SKH_CHECK(hipGetLastError());
+    argmax_split_kernel<<<dim3(ARGMAX_SPLIT, rows), dim3(ROW_THREADS), 0, current_stream()>>>(in, cols, out, sc);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
 int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes) {
     if (rows <= 0 || bpr <= 0) return 0;
     relayout_to_row_major_kernel<<<dim3((unsigned)((int64_t)rows * bpr)), dim3(64), 0, current_stream()>>>(src, dst, rows, bpr, block_bytes);
@@ -493,3 +539,9 @@ int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int
 }
 
 }  // namespace skh
+
+extern "C" int32_t skainet_hip_f32_argmax_rows_noalloc_dev(const float* in, int32_t rows, int32_t cols, int32_t* out) {
+    if (skh::ensure_device() != 0) return -1;
+    if (rows > 0 && cols > 0 && (!in || !out)) return skh::set_error("argmax_rows_noalloc: null pointer");
+    return skh::launch_argmax_rows_noalloc(in, rows, cols, out);
+}

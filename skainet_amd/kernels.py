@@ -258,6 +258,11 @@ def argmax_rows_dev(x, rows: int, cols: int, out) -> None:
     check(_lib.hip().skainet_hip_f32_argmax_rows_dev(_ptr(x), rows, cols, _ptr(out)), "argmax_rows")
 
 
+def argmax_rows_noalloc_dev(x, rows: int, cols: int, out) -> None:
+    """argmax_rows_dev without any device allocation: scratch is a fixed array inside the library, at most 64 rows."""
+    check(_lib.hip().skainet_hip_f32_argmax_rows_noalloc_dev(_ptr(x), rows, cols, _ptr(out)), "argmax_rows_noalloc")
+
+
 def rope_scatter_dev(x, out, tokens, heads, head_dim, pos_start=0, pos_dev=None, theta=10000.0, rotate=True,
                      out_head_stride=None, out_row_is_pos=False, in_row_pitch=None) -> None:
     if out_head_stride is None:
