@@ -317,6 +317,9 @@ def bench_decoder(a):
     toks = [first] + [int(x) for x in dec.decode(max(1, warmup), use_graph=not a.no_graph)]
     kernels.sync()
     pos0 = dec.position()
+    if pos0 + steps > cfg.ctx_max:
+        print(f"bench.py: {steps} decode steps from position {pos0} would pass the context limit {cfg.ctx_max}", file=sys.stderr)
+        sys.exit(2)
     t0 = time.perf_counter()
     with kernels.Timer() as t:               # HIP events on the launch stream around exactly K decode steps
         if a.no_graph:

@@ -109,8 +109,10 @@ SKAINET_HIP_API int64_t skainet_hip_weight_nbytes(const skainet_hip_weight* w);
 /* out[m, rows] = x[m, cols] . W^T, fp32 in and out, device pointers. What a ViewKernel registered for
  * matmul(F32 dense x packed BLOCKED_ROW_MAJOR) runs (API/MatmulKernels.kt:11-40; CPU twin
  * REF/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/FfmRowMajorKernels.kt:52-106).
- * m <= 8 streams the weight once per 4 rows (GEMV kernels, fp32 arithmetic); larger m uses the MFMA
- * dequant-GEMM (bf16 operands, fp32 accumulation). */
+ * m <= 8 streams the weight once per 4 rows (GEMV kernels, fp32 arithmetic, within 1e-3 of the exact fp32 product);
+ * larger m uses the MFMA dequant-GEMM, which rounds activations and decoded weights to bf16 and accumulates in fp32
+ * (within 2e-2 of the largest output): the switch at m = 9 is a switch of precision class as well as of kernel, and
+ * skainet_hip_matmul_kind_dev pins either one. */
 SKAINET_HIP_API int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out);
 /* Same product, forcing one of the two kernels (kind 0 = GEMV path, 1 = MFMA GEMM path). */
 SKAINET_HIP_API int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out, int32_t kind);
@@ -294,20 +296,30 @@ SKAINET_HIP_API int32_t skainet_hip_f32_rope_qkv_dev(const float* qkv, float* q_
 SKAINET_HIP_API int32_t skainet_hip_f32_heads_to_rows_dev(const float* in, float* out, int32_t heads, int32_t tokens, int32_t head_dim);
 SKAINET_HIP_API int32_t skainet_hip_i32_increment_dev(int32_t* value, int32_t delta);
 /* dst[index_dev[0] + offset] = src[0], all on the device: appends a sampled token to a log at the device-side position. */
-/* End of a greedy decode step: *pos += 1, *kv_len += 1, log[*pos] = *token (all device memory, one launch). */
-SKAINET_HIP_API int32_t skainet_hip_decode_advance_dev(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log);
+/* End of a greedy decode step: *pos += 1, *kv_len += 1, log[*pos] = *token (all device memory, one launch). `capacity` is
+ * the cache's row count (the log holds capacity + 1 entries): at *pos == capacity the call changes nothing, so a recorded
+ * step replayed past the end of the cache writes nowhere (the K / V append of that step is skipped the same way) and the
+ * host reads the saturated position. */
+SKAINET_HIP_API int32_t skainet_hip_decode_advance_dev(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log,
+    int32_t capacity);
 SKAINET_HIP_API int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t* index_dev, int32_t offset, const int32_t* src);
 
 /* HIP graphs (no reference counterpart; for launch-bound loops such as a decode step): graph_begin redirects this
  * thread's device entries into a stream capture, graph_end closes it and returns an executable graph (NULL on
  * failure), graph_launch replays it on the calling thread's stream (in order with that thread's eager device
  * entries), graph_sync waits for that stream. Nothing that
- * allocates (a first call that grows the library's scratch) may run between begin and end: run the sequence once
- * eagerly first. Only kernel launches are recorded. */
+ * allocates (a first call that grows the library's scratch) may run between begin and end: such a call fails with a
+ * message instead of freeing memory under the capture, so run the sequence once eagerly first. A graph is tied to the
+ * scratch addresses of its recording: when a later call on the thread makes the library reallocate scratch, the graph
+ * is refused from then on (graph_valid / graph_launch). Only kernel launches are recorded. */
 typedef struct skainet_hip_graph skainet_hip_graph;
 SKAINET_HIP_API int32_t skainet_hip_graph_begin(void);
 SKAINET_HIP_API skainet_hip_graph* skainet_hip_graph_end(void);
 SKAINET_HIP_API int32_t skainet_hip_graph_launch(skainet_hip_graph* graph);
+/* 1 while the graph may still be launched from this thread, 0 once the thread's scratch has been reallocated since the
+ * recording (a later call needed more, or skainet_hip_thread_release ran): graph_launch then returns -1 without
+ * launching anything, and the sequence has to be recorded again. */
+SKAINET_HIP_API int32_t skainet_hip_graph_valid(const skainet_hip_graph* graph);
 SKAINET_HIP_API int32_t skainet_hip_graph_sync(skainet_hip_graph* graph);
 SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
 

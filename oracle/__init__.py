@@ -3,5 +3,4 @@
 `oracle.lib`     ctypes bindings of liboracle.so (this repo's strict-fp32 restatement) and, when it
                  was built, of _ref/libskainet_ref.so (the reference's own C kernels).
 `oracle.golden`  the reference's golden-test input generator and digest, restated.
-`oracle.quant`   numpy generators of valid Q4_K / Q6_K super-blocks from fp32 weights.
 """

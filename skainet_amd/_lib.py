@@ -84,7 +84,7 @@ SIGNATURES = {
     "skainet_hip_f32_argmax_rows_dev": (_i32, [_vp, _i32, _i32, _vp]),
     "skainet_hip_f32_argmax_rows_noalloc_dev": (_i32, [_vp, _i32, _i32, _vp]),
     "skainet_hip_f32_rope_scatter_dev": (_i32, [_vp, _i64, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _i32, _i64, _i32]),
-    "skainet_hip_decode_advance_dev": (_i32, [_vp, _vp, _vp, _vp]),
+    "skainet_hip_decode_advance_dev": (_i32, [_vp, _vp, _vp, _vp, _i32]),
     "skainet_hip_i32_store_at_dev": (_i32, [_vp, _vp, _i32, _vp]),
     "skainet_hip_f32_swiglu_pairs_dev": (_i32, [_vp, _vp, _i64]),
     "skainet_hip_f32_rope_qkv_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _f32]),
@@ -93,6 +93,7 @@ SIGNATURES = {
     "skainet_hip_graph_begin": (_i32, []),
     "skainet_hip_graph_end": (_vp, []),
     "skainet_hip_graph_launch": (_i32, [_vp]),
+    "skainet_hip_graph_valid": (_i32, [_vp]),
     "skainet_hip_graph_sync": (_i32, [_vp]),
     "skainet_hip_graph_free": (None, [_vp]),
     "skainet_hip_set_tuning": (_i32, [C.c_char_p, _i32]),

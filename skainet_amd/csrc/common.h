@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <mutex>
+
 namespace skh {
 
 // GGUF block geometry (elements per block, bytes per block); see
@@ -45,6 +48,20 @@ int num_cus();
     } while (0)
 
 #define SKH_LAUNCH_CHECK(name) SKH_CHECK((hipGetLastError()))
+
+// Raises a kernel's dynamic-LDS limit exactly once per process, whichever thread launches it first (every thread
+// passes through the same once-flag; a failure is remembered and reported to every caller).
+#define SKH_SET_MAX_DYNAMIC_LDS_ONCE(kernel_ptr, bytes)                                                         \
+    do {                                                                                                        \
+        static std::once_flag skh_once;                                                                         \
+        static int skh_once_rc = 0;                                                                             \
+        std::call_once(skh_once, [&] {                                                                          \
+            skh_once_rc = skh::check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_ptr),        \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)), \
+                                         "hipFuncSetAttribute(max dynamic LDS)");                               \
+        });                                                                                                     \
+        if (skh_once_rc != 0) return skh::set_error("kernel attribute could not be set: dynamic LDS of %d bytes refused", (int)(bytes)); \
+    } while (0)
 
 // ---- device helpers ----
 

@@ -17,19 +17,21 @@
 
 namespace skh {
 
-// Output block b reads source block b, or -- for a row gather -- block (b % bpr) of source row row_ids[b / bpr].
-__device__ __forceinline__ int64_t source_block(int64_t b, const int32_t* row_ids, int bpr) {
-    return row_ids ? (int64_t)row_ids[b / bpr] * bpr + (b % bpr) : b;
+// Output block b reads source block b, or -- for a row gather -- block (b % bpr) of source row row_ids[b / bpr]. A row
+// id outside [0, rows) (ids that reach the device unchecked, e.g. a sampled token fed back) is clamped into the weight:
+// the read stays inside the allocation; hosts that hold the ids validate them before the call.
+__device__ __forceinline__ int64_t source_block(int64_t b, const int32_t* row_ids, int bpr, int rows) {
+    return row_ids ? (int64_t)min(max(row_ids[b / bpr], 0), rows - 1) * bpr + (b % bpr) : b;
 }
 
 // One thread per 8 output elements; 4 threads per Q8_0 block.
 __global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                           int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr) {
+                                                           int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr, int rows) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t b = t >> 2;
     if (b >= nblocks) return;
     const int part = (int)(t & 3);
-    const uint8_t* p = w + source_block(b, row_ids, bpr) * Q80_BYTES;
+    const uint8_t* p = w + source_block(b, row_ids, bpr, rows) * Q80_BYTES;
     const float d = half_bits_to_float(load_u16(p));
     const uint8_t* c = p + 2 + part * 8;
     const uint32_t lo = load_u32_a2(c), hi = load_u32_a2(c + 4);
@@ -60,12 +62,12 @@ __device__ __forceinline__ void q4k_scale_min(const uint8_t* s, int j, int& sc, 
 // One thread per 8 output elements; 32 threads per Q4_K block. Thread u: sub-block sb = u / 4,
 // elements [8 * (u % 4), +8) of it, i.e. 8 consecutive bytes of 32-byte group sb / 2, low or high nibble.
 __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr) {
+                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr, int rows) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t b = t >> 5;
     if (b >= nblocks) return;
     const int u = (int)(t & 31), sb = u >> 2, e0 = (u & 3) * 8;
-    const uint8_t* p = w + source_block(b, row_ids, bpr) * Q4K_BYTES;
+    const uint8_t* p = w + source_block(b, row_ids, bpr, rows) * Q4K_BYTES;
     const uint32_t dd = *reinterpret_cast<const uint32_t*>(p);
     const float d = half_bits_to_float(dd & 0xFFFFu), dmin = half_bits_to_float(dd >> 16);
     int sc, mn;
@@ -88,12 +90,12 @@ __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t* __restr
 // One thread per 8 output elements; 32 threads per Q6_K block. Thread u: half = u / 16, quarter k = (u / 4) % 4
 // (output offset 32 * k inside the half), elements l in [8 * (u % 4), +8).
 __global__ __launch_bounds__(256) void dequant_q6k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr) {
+                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr, int rows) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t b = t >> 5;
     if (b >= nblocks) return;
     const int u = (int)(t & 31), half = u >> 4, k = (u >> 2) & 3, l0 = (u & 3) * 8;
-    const uint8_t* p = w + source_block(b, row_ids, bpr) * Q6K_BYTES;
+    const uint8_t* p = w + source_block(b, row_ids, bpr, rows) * Q6K_BYTES;
     const float d = half_bits_to_float(load_u16(p + 208));
     const int8_t sc = (int8_t)p[192 + half * 8 + (l0 >> 4) + 2 * k];
     const float ds = __fmul_rn(d, (float)sc);
@@ -120,14 +122,14 @@ __global__ __launch_bounds__(256) void dequant_q6k_kernel(const uint8_t* __restr
 // 8p .. 8p+7, part p >= 2 the high nibbles of bytes 8(p-2) .. 8(p-2)+7. FMT: 0 = Q4_0, 1 = Q5_0, 2 = Q5_1.
 template <int FMT>
 __global__ __launch_bounds__(256) void dequant_q45_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr) {
+                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr, int rows) {
     constexpr int BYTES = FMT == 0 ? Q40_BYTES : (FMT == 1 ? Q50_BYTES : Q51_BYTES);
     constexpr int QH = FMT == 2 ? 4 : 2, QS = FMT == 0 ? 2 : QH + 4;
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t b = t >> 2;
     if (b >= nblocks) return;
     const int part = (int)(t & 3), byte0 = (part & 1) * 8, shift = (part >> 1) * 4;
-    const uint8_t* p = w + source_block(b, row_ids, bpr) * BYTES;
+    const uint8_t* p = w + source_block(b, row_ids, bpr, rows) * BYTES;
     const float d = half_bits_to_float(load_u16(p));
     float m = 0.f;
     uint32_t qh = 0;
@@ -151,12 +153,12 @@ __global__ __launch_bounds__(256) void dequant_q45_kernel(const uint8_t* __restr
 // Q5_K: the Q4_K layout with a 32-byte plane of fifth bits at byte 16 and the nibbles at byte 48 (176 bytes). Thread
 // u of 32: sub-block sb = u / 4, elements [8 * (u % 4), +8): bytes e0 .. e0+7 of nibble group sb / 2, bit sb of qh[e0 ..].
 __global__ __launch_bounds__(256) void dequant_q5k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr) {
+                                                          int64_t nblocks, const int32_t* __restrict__ row_ids, int bpr, int rows) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t b = t >> 5;
     if (b >= nblocks) return;
     const int u = (int)(t & 31), sb = u >> 2, e0 = (u & 3) * 8;
-    const uint8_t* p = w + source_block(b, row_ids, bpr) * Q5K_BYTES;
+    const uint8_t* p = w + source_block(b, row_ids, bpr, rows) * Q5K_BYTES;
     const uint32_t dd = *reinterpret_cast<const uint32_t*>(p);
     const float d = half_bits_to_float(dd & 0xFFFFu), dmin = half_bits_to_float(dd >> 16);
     int sc, mn;
@@ -181,20 +183,20 @@ __global__ __launch_bounds__(256) void dequant_q5k_kernel(const uint8_t* __restr
 
 // Decodes `nblocks` consecutive output blocks; with `row_ids` (device int32) output row r is source row row_ids[r]
 // of a weight with `bpr` blocks per row.
-int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr) {
+int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr, int rows) {
     if (nblocks <= 0) return 0;
     if (!is_packed(enc)) return set_error("dequantize: unsupported encoding %d", enc);
     hipStream_t s = current_stream();
     const int64_t threads = nblocks * (block_elems(enc) / 8);
     const int64_t grid = (threads + 255) / 256;
     if (grid > 0x7FFFFFFFLL) return set_error("dequantize: %lld blocks exceed one launch", (long long)nblocks);
-    if (enc == ENC_Q8_0) dequant_q8_0_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
-    else if (enc == ENC_Q4_K) dequant_q4k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
-    else if (enc == ENC_Q5_K) dequant_q5k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
-    else if (enc == ENC_Q4_0) dequant_q45_kernel<0><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
-    else if (enc == ENC_Q5_0) dequant_q45_kernel<1><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
-    else if (enc == ENC_Q5_1) dequant_q45_kernel<2><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
-    else dequant_q6k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr);
+    if (enc == ENC_Q8_0) dequant_q8_0_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr, rows);
+    else if (enc == ENC_Q4_K) dequant_q4k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr, rows);
+    else if (enc == ENC_Q5_K) dequant_q5k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr, rows);
+    else if (enc == ENC_Q4_0) dequant_q45_kernel<0><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr, rows);
+    else if (enc == ENC_Q5_0) dequant_q45_kernel<1><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr, rows);
+    else if (enc == ENC_Q5_1) dequant_q45_kernel<2><<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr, rows);
+    else dequant_q6k_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(w, out, nblocks, row_ids, bpr, rows);
     SKH_CHECK(hipGetLastError());
     return 0;
 }

@@ -575,12 +575,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
 template <class Raw, int BE, int BB, int WTN>
 static int launch_gemm_tile(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
                             int64_t split_stride, hipStream_t s) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&dequant_gemm_kernel<Raw, BE, BB, WTN>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_smem(WTN)));
-        attr_set = true;
-    }
+    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&dequant_gemm_kernel<Raw, BE, BB, WTN>), gemm_smem(WTN));
     dequant_gemm_kernel<Raw, BE, BB, WTN><<<grid, dim3(G_THREADS), gemm_smem(WTN), s>>>(a, w, c, m, n, k, k_chunk, split_stride);
     SKH_CHECK(hipGetLastError());
     return 0;
@@ -592,9 +587,9 @@ static int launch_gemm_enc(int wtn, const __bf16* a, const uint8_t* w, float* c,
     return launch_gemm_tile<Raw, BE, BB, 2>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
 }
 
-static int g_gemm_ksplit = 0;   // 0 = choose from the tile count
+static std::atomic<int> g_gemm_ksplit{0};   // 0 = choose from the tile count
 void set_gemm_ksplit(int v) { g_gemm_ksplit = v; }
-static int g_gemm_wide = -1;    // -1 = choose from the shape, 0 / 1 = narrow / wide tile
+static std::atomic<int> g_gemm_wide{-1};    // -1 = choose from the shape, 0 / 1 = narrow / wide tile
 void set_gemm_wide(int v) { g_gemm_wide = v; }
 
 // y = epilogue(prologue(x) . W^T): gain != null normalises every activation row first (RMSNorm, folded into the pass that
@@ -620,7 +615,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     // the wide tile where it alone fills most of the chip in one round
     const int tiles_m = (m + GM - 1) / GM;
     const int wide_tiles = tiles_m * ((n + gemm_gn(4) - 1) / gemm_gn(4));
-    const bool wide = g_gemm_wide >= 0 ? g_gemm_wide != 0 : 4 * wide_tiles >= 3 * num_cus();
+    const bool wide = g_gemm_wide.load() >= 0 ? g_gemm_wide.load() != 0 : 4 * wide_tiles >= 3 * num_cus();
     const int wtn = wide ? 4 : 2;
     const int tiles_n = (n + gemm_gn(wtn) - 1) / gemm_gn(wtn);
     const int tiles = tiles_m * tiles_n;

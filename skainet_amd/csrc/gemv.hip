@@ -546,8 +546,8 @@ template <> struct RowsInFlight<Q80Slot> { static constexpr int B1 = 3; };
 template <> struct RowsInFlight<Q6KSlot> { static constexpr int B1 = 2; };
 template <> struct RowsInFlight<Q5KSlot> { static constexpr int B1 = 3; };
 
-static int g_gemv_waves_per_cu = 0;   // 0: per encoding (measured best: Q8_0 4, Q6_K at batch 1 6, the others 8)
-static int g_q6k_slot64 = 1;   // 0: Q6_K at batch 1 stays on the 32-weight slot
+static std::atomic<int> g_gemv_waves_per_cu{0};   // 0: per encoding (measured best: Q8_0 4, Q6_K at batch 1 6, the others 8)
+static std::atomic<int> g_q6k_slot64{1};   // 0: Q6_K at batch 1 stays on the 32-weight slot
 
 template <class F>
 static int launch_format(const uint8_t* w, const float* x, float* y, int k, int n, int batch, int waves_per_cu) {
@@ -555,14 +555,14 @@ static int launch_format(const uint8_t* w, const float* x, float* y, int k, int 
         // Q6_K: the 64-weight slot, 2 rows in flight, 6 waves per CU unless the caller set a count (measured on 32000 x 4096
         // over 1 .. 4 rows and 5 .. 16 waves: 23.1 us against 25.5 us for the 32-weight slot at its best, 2 rows and 8 waves)
         if (std::is_same<F, Q6KSlot>::value && g_q6k_slot64)
-            return launch_one<Q6KSlot64, 1, 2>(w, x, y, k, n, batch, g_gemv_waves_per_cu > 0 ? g_gemv_waves_per_cu : 6);
+            return launch_one<Q6KSlot64, 1, 2>(w, x, y, k, n, batch, g_gemv_waves_per_cu.load() > 0 ? g_gemv_waves_per_cu.load() : 6);
         return launch_one<F, 1, RowsInFlight<F>::B1>(w, x, y, k, n, batch, waves_per_cu);
     }
     if (batch == 2) return launch_one<F, 2, 4>(w, x, y, k, n, batch, waves_per_cu);
     return launch_one<F, 4, 2>(w, x, y, k, n, batch, waves_per_cu);
 }
 
-static int g_q4k_rows_enable = 1;
+static std::atomic<int> g_q4k_rows_enable{1};
 void set_q4k_rows_waves_per_cu(int v);
 void set_gemm_wide(int v);
 void set_gemm_ksplit(int v);
@@ -592,7 +592,7 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
     if (!is_packed(enc)) return set_error("gemv: unsupported encoding %d", enc);
     if (k <= 0 || k % block_elems(enc) != 0)
         return set_error("gemv: inputDim must be a positive multiple of %d; got %d", block_elems(enc), k);
-    const int waves_per_cu = g_gemv_waves_per_cu > 0 ? g_gemv_waves_per_cu : (block_elems(enc) == 32 ? 4 : 8);
+    const int waves_per_cu = g_gemv_waves_per_cu.load() > 0 ? g_gemv_waves_per_cu.load() : (block_elems(enc) == 32 ? 4 : 8);
     for (int b0 = 0; b0 < m;) {
         const int left = m - b0;
         const float* xb = x + (int64_t)b0 * k;

@@ -110,11 +110,12 @@ __device__ __forceinline__ void q4k_rows_epilogue(float val, int lane, int row, 
                 else sincosf((float)p0 * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
                 out2 = rope_rotate(val, odd, cs, sn);
             }
+            const bool in_cache = p0 >= 0 && p0 < rope.capacity;   // a device-side position past the cache writes no K / V row
             float* dst;
             if (slot < rope.heads) dst = y + (int64_t)slot * rope.head_dim;
             else if (slot < rope.heads + rope.kv_heads) dst = rope.k_cache + ((int64_t)(slot - rope.heads) * rope.capacity + p0) * rope.head_dim;
             else dst = rope.v_cache + ((int64_t)(slot - rope.heads - rope.kv_heads) * rope.capacity + p0) * rope.head_dim;
-            *reinterpret_cast<float2*>(dst + dd) = out2;
+            if (slot < rope.heads || in_cache) *reinterpret_cast<float2*>(dst + dd) = out2;
         }
     } else if (epilogue == EPI_SWIGLU) {
         // rows 2j (gate) and 2j + 1 (up) of this wave sit B lanes apart after the fold (lane = row * B + b)
@@ -381,10 +382,10 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_ksplit_kernel(const uint8_t* 
     }
 }
 
-static int g_q4k_rows_waves_per_cu = 0;   // 0: chosen from K (below)
+static std::atomic<int> g_q4k_rows_waves_per_cu{0};   // 0: chosen from K (below)
 void set_q4k_rows_waves_per_cu(int v) { if (v >= 0) g_q4k_rows_waves_per_cu = v; }
 int q4k_rows_waves_per_cu() { return g_q4k_rows_waves_per_cu; }
-static int g_q4k_ksplit_enable = 1;      // 0: long rows take the plain row shape too
+static std::atomic<int> g_q4k_ksplit_enable{1};      // 0: long rows take the plain row shape too
 void set_q4k_ksplit_enable(int v) { g_q4k_ksplit_enable = v; }
 
 template <int B, int R, int NR>
@@ -446,7 +447,7 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     // 14336: 11.7 us at 8 waves against 12.2 at 4), and inside the decoder's chain of fused launches 8 waves measured
     // 0.6 % faster per token than 4 although each launch alone prefers 4.
     const bool lone = !gain && epilogue == EPI_NONE;
-    int waves_per_cu = g_q4k_rows_waves_per_cu > 0 ? g_q4k_rows_waves_per_cu : (lone && k <= 4096 ? 4 : 8);
+    int waves_per_cu = g_q4k_rows_waves_per_cu.load() > 0 ? g_q4k_rows_waves_per_cu.load() : (lone && k <= 4096 ? 4 : 8);
     while (waves_per_cu < 32 && (n + num_cus() * waves_per_cu - 1) / (num_cus() * waves_per_cu) > Q4K_RMAX) waves_per_cu += 4;
     const int total_waves = num_cus() * waves_per_cu;
     const int share = (n + total_waves - 1) / total_waves;

@@ -275,12 +275,7 @@ template <int NM, int Q, int R, int OCC>
 static int launch_quads(hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int batch) {
     constexpr size_t smem = (size_t)(8 * NM * 64 * QD_SLICE) * sizeof(uint32_t);
     static_assert(4 * ((Q * 4 * NM + 15) / 16) * 64 <= 8 * NM * 64 * QD_SLICE, "wave partials must fit in the slices");
-    static bool attr_set = false;
-    if (!attr_set) {
-        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&q4k_gemv_quads_kernel<NM, Q, R, OCC>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
-    }
+    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_quads_kernel<NM, Q, R, OCC>), smem);
     const int grid = (n + 4 * Q - 1) / (4 * Q);
     q4k_gemv_quads_kernel<NM, Q, R, OCC><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, batch);
     SKH_CHECK(hipGetLastError());

@@ -310,8 +310,11 @@ __global__ __launch_bounds__(256) void rope_qkv_kernel(const float* __restrict__
         }
         float* dst;
         if (hs < heads) dst = q_out + ((int64_t)hs * tokens + t) * head_dim;
-        else if (hs < heads + kv_heads) dst = k_cache + ((int64_t)(hs - heads) * kv_capacity + p0 + t) * head_dim;
-        else dst = v_cache + ((int64_t)(hs - heads - kv_heads) * kv_capacity + p0 + t) * head_dim;
+        else {
+            if (p0 < 0 || p0 + t >= kv_capacity) continue;      // a device-side position past the cache: nothing is written
+            if (hs < heads + kv_heads) dst = k_cache + ((int64_t)(hs - heads) * kv_capacity + p0 + t) * head_dim;
+            else dst = v_cache + ((int64_t)(hs - heads - kv_heads) * kv_capacity + p0 + t) * head_dim;
+        }
         *reinterpret_cast<float2*>(dst + 2 * i) = y;
     }
 }
@@ -353,17 +356,20 @@ int launch_rope_table(const int32_t* pos, float theta, int head_dim, float* tabl
 }
 
 // End of a greedy decode step in one launch: the position and the key count advance by one and the token just
-// sampled is appended to the log at the new position.
-__global__ void decode_advance_kernel(int32_t* pos, int32_t* kv_len, const int32_t* __restrict__ token, int32_t* log) {
+// sampled is appended to the log at the new position. The position saturates at `capacity` (the cache's row count, the
+// log holds capacity + 1 entries): a step replayed past the end writes nothing anywhere and the host sees pos == capacity.
+__global__ void decode_advance_kernel(int32_t* pos, int32_t* kv_len, const int32_t* __restrict__ token, int32_t* log, int32_t capacity) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         const int32_t p = pos[0] + 1;
+        if (p > capacity) return;
         pos[0] = p;
-        kv_len[0] += 1;
+        kv_len[0] = min(kv_len[0] + 1, capacity);
         log[p] = token[0];
     }
 }
-int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log) {
-    decode_advance_kernel<<<dim3(1), dim3(64), 0, current_stream()>>>(pos, kv_len, token, log);
+int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log, int32_t capacity) {
+    if (capacity <= 0) return set_error("decode_advance: capacity must be positive; got %d", capacity);
+    decode_advance_kernel<<<dim3(1), dim3(64), 0, current_stream()>>>(pos, kv_len, token, log, capacity);
     SKH_CHECK(hipGetLastError());
     return 0;
 }

@@ -278,7 +278,7 @@ __global__ __launch_bounds__(4 * D) void sdpa_decode_combine_kernel(const float*
 
 float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
 
-static int g_sdpa_decode_split_keys = 64;   // least keys per split (a multiple of 16)
+static std::atomic<int> g_sdpa_decode_split_keys{64};   // least keys per split (a multiple of 16)
 void set_sdpa_decode_split_keys(int v) { if (v >= 16) g_sdpa_decode_split_keys = (v + 15) & ~15; }
 
 template <int GS, int DPL>

@@ -268,7 +268,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
 
 void* kernel_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
 
-static int g_prefill_mfma = 1;
+static std::atomic<int> g_prefill_mfma{1};
 void set_sdpa_prefill_mfma(int v) { g_prefill_mfma = v; }
 
 template <int D>
@@ -288,12 +288,7 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
     PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, hpw};
     const dim3 grid((seq_q + q_per_wg - 1) / q_per_wg, kv_heads * (per_kv / hpw), batch);
     constexpr size_t smem = sizeof(__bf16) * (2 * PF_KB * (D + 8) + 2 * D * (PF_KB + 8));
-    static bool attr_set = false;
-    if (!attr_set) {
-        SKH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&sdpa_prefill_kernel<D>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_set = true;
-    }
+    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D>), smem);
     sdpa_prefill_kernel<D><<<grid, dim3(256), smem, s>>>(p);
     SKH_CHECK(hipGetLastError());
     return 1;

@@ -19,7 +19,7 @@
 namespace skh {
 
 // kernels (one translation unit each)
-int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr);
+int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const int32_t* row_ids, int bpr, int rows);
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
 int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
 int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y, const float* gain, float eps,
@@ -42,7 +42,7 @@ int launch_i32_store_at(int32_t* dst, const int32_t* index, int32_t offset, cons
 int launch_rope_table(const int32_t* pos, float theta, int head_dim, float* table);
 int launch_narrow_matmul(const float* a, int64_t a_stride, const uint8_t* b, int64_t b_byte_stride, float* c, int64_t c_stride,
                          int m, int n, int k, int fp16);
-int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log);
+int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log, int32_t capacity);
 int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim);
 int launch_i32_increment(int32_t* v, int32_t delta);
 int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink);
@@ -118,10 +118,24 @@ int ensure_device() {
     return 0;
 }
 
+// Recorded graphs hold the scratch addresses of the moment they were recorded. Every time a buffer of this thread is
+// given back to the device (it grew, or the thread released its scratch) the thread's scratch generation moves on;
+// a graph remembers the generation it was recorded under and is refused afterwards (skainet_hip_graph_launch). While a
+// capture is open nothing may grow: the call that would need it fails instead of freeing memory under the capture.
+static thread_local uint64_t t_scratch_generation = 1;
+static thread_local hipStream_t t_capture_stream = nullptr;
 static void* scratch_get(Scratch& s, size_t bytes) {
     if (bytes <= s.cap) return s.ptr;
+    if (t_capture_stream) {
+        set_error("scratch of %zu bytes is needed while a graph capture is open (held: %zu): run the sequence once outside the capture first",
+                  bytes, s.cap);
+        return nullptr;
+    }
     // the old buffer may still be read by queued kernels of this thread's stream
-    if (s.ptr) { (void)hipStreamSynchronize(t_stream); (void)hipFree(s.ptr); s.ptr = nullptr; s.cap = 0; }
+    if (s.ptr) {
+        (void)hipStreamSynchronize(t_stream); (void)hipFree(s.ptr); s.ptr = nullptr; s.cap = 0;
+        ++t_scratch_generation;
+    }
     const size_t cap = (bytes + (1u << 20) - 1) & ~((size_t)(1u << 20) - 1);
     void* p = nullptr;
     if (check_hip(hipMalloc(&p, cap), "hipMalloc(scratch)") != 0) return nullptr;
@@ -167,7 +181,9 @@ int32_t skainet_hip_available(void) {
 int32_t skainet_hip_init(int32_t device) {
     std::lock_guard<std::mutex> lock(g_mutex);
     if (g_state == 1 && device == g_device) return 0;
-    return probe_locked(device);
+    // threads bind to the selected device once and their scratch lives there: a process keeps the device it started on
+    if (g_state == 1) return set_error("init: this process already runs on device %d; device %d refused", g_device, device);
+    return probe_locked(device);          // first probe, or a new attempt after a failed one
 }
 const char* skainet_hip_last_error(void) { return t_error; }
 const char* skainet_hip_device_name(void) { return g_name; }
@@ -191,6 +207,7 @@ int32_t skainet_hip_thread_release(void) {
         if (sc.ptr && check_hip(hipFree(sc.ptr), "hipFree(scratch)") != 0) rc = -1;
         sc.ptr = nullptr; sc.cap = 0;
     };
+    ++t_scratch_generation;                       // graphs recorded on this thread are stale from here on
     drop(t_workspace);
     for (Scratch& sc : t_stage) drop(sc);
     for (Scratch& sc : t_fuse) drop(sc);
@@ -439,14 +456,14 @@ float skainet_hip_read_probe_dev(const void* const* buffers, int32_t nbuffers, i
 int32_t skainet_hip_dequantize_dev(const skainet_hip_weight* w, float* out) {
     if (ensure_device() != 0) return -1;
     if (!w || !out) return set_error("dequantize: null argument");
-    return launch_dequant(w->encoding, w->data, (int64_t)w->rows * (w->cols / block_elems(w->encoding)), out, nullptr, 1);
+    return launch_dequant(w->encoding, w->data, (int64_t)w->rows * (w->cols / block_elems(w->encoding)), out, nullptr, 1, w->rows);
 }
 int32_t skainet_hip_dequantize_rows_dev(const skainet_hip_weight* w, const int32_t* row_ids, int32_t count, float* out) {
     if (ensure_device() != 0) return -1;
     if (!w || !out || !row_ids) return set_error("dequantize_rows: null argument");
     if (count <= 0) return 0;
     const int bpr = w->cols / block_elems(w->encoding);
-    return launch_dequant(w->encoding, w->data, (int64_t)count * bpr, out, row_ids, bpr);
+    return launch_dequant(w->encoding, w->data, (int64_t)count * bpr, out, row_ids, bpr, w->rows);
 }
 
 // ------------------------------------------------------------------------------------------ device entries
@@ -516,10 +533,10 @@ int32_t skainet_hip_f32_rope_table_dev(const int32_t* pos_dev, float theta, int3
     if (!pos_dev || !table) return set_error("rope_table: null argument");
     return launch_rope_table(pos_dev, theta, head_dim, table);
 }
-int32_t skainet_hip_decode_advance_dev(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log) {
+int32_t skainet_hip_decode_advance_dev(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log, int32_t capacity) {
     if (ensure_device() != 0) return -1;
     if (!pos || !kv_len || !token || !log) return set_error("decode_advance: null argument");
-    return launch_decode_advance(pos, kv_len, token, log);
+    return launch_decode_advance(pos, kv_len, token, log, capacity);
 }
 int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t* index_dev, int32_t offset, const int32_t* src) {
     if (ensure_device() != 0) return -1;
@@ -545,9 +562,8 @@ int32_t skainet_hip_i32_increment_dev(int32_t* value, int32_t delta) {
 }
 
 // ---- HIP graphs: record this thread's device entries once, replay them with one launch ----
-struct skainet_hip_graph { hipGraph_t graph; hipGraphExec_t exec; };
+struct skainet_hip_graph { hipGraph_t graph; hipGraphExec_t exec; uint64_t scratch_generation; };
 static thread_local hipStream_t t_capture_prev = nullptr;
-static thread_local hipStream_t t_capture_stream = nullptr;
 
 int32_t skainet_hip_graph_begin(void) {
     if (ensure_device() != 0) return -1;
@@ -577,10 +593,17 @@ skainet_hip_graph* skainet_hip_graph_end(void) {
         return nullptr;
     }
     (void)hipStreamDestroy(cap);   // replays run on the calling thread's stream, in order with its eager work
-    return new skainet_hip_graph{graph, exec};
+    return new skainet_hip_graph{graph, exec, t_scratch_generation};
+}
+int32_t skainet_hip_graph_valid(const skainet_hip_graph* g) {
+    return g && g->scratch_generation == t_scratch_generation ? 1 : 0;
 }
 int32_t skainet_hip_graph_launch(skainet_hip_graph* g) {
     if (!g) return set_error("graph_launch: null graph");
+    if (g->scratch_generation != t_scratch_generation)
+        return set_error("graph_launch: refused, the library's scratch was reallocated after this graph was recorded "
+                         "(generation %llu, now %llu); record it again",
+                         (unsigned long long)g->scratch_generation, (unsigned long long)t_scratch_generation);
     return check_hip(hipGraphLaunch(g->exec, t_stream), "hipGraphLaunch");
 }
 int32_t skainet_hip_graph_sync(skainet_hip_graph* g) {
@@ -618,8 +641,11 @@ static void packed_matmul_host(int enc, int order, const float* input, int32_t i
     if (output_dim <= 0) return;
     if (ensure_device() != 0) return;
     if (input_dim % block_elems(enc) != 0) { set_error("matmul: inputDim must be a multiple of %d; got %d", block_elems(enc), input_dim); return; }
-    if (input_dim <= 0) {   // an empty contraction is a row of zeros (Q8_0 scalar kernel) / a no-op (K-quants): write zeros
-        for (int32_t o = 0; o < output_dim; ++o) output[output_offset + o] = 0.f;
+    if (input_dim <= 0) {
+        // an empty contraction: the reference's K-quant entries return with the output untouched (q4k_matmul.c:326), its
+        // 32-element formats write a row of zeros (q8_0_matmul.c:176)
+        if (block_elems(enc) == Q80_ELEMS)
+            for (int32_t o = 0; o < output_dim; ++o) output[output_offset + o] = 0.f;
         return;
     }
     const int bpr = input_dim / block_elems(enc);

@@ -378,10 +378,14 @@ class LlamaDecoder:
     def prefill(self, token_ids) -> int:
         """Run the prompt through the stack, fill the KV cache, return the greedy next token."""
         c = self.cfg
-        ids = np.ascontiguousarray(token_ids, dtype=np.int32)
-        rows = int(ids.size)
+        ids64 = np.ascontiguousarray(token_ids, dtype=np.int64).reshape(-1)
+        rows = int(ids64.size)
         if rows < 1 or rows > self.max_rows or rows > c.ctx_max:
             raise ValueError(f"prompt of {rows} tokens does not fit (max_prefill {self.max_rows}, ctx {c.ctx_max})")
+        if ids64.min() < 0 or ids64.max() >= c.vocab:       # the gather reads embedding rows by id: checked before any launch
+            bad = ids64[(ids64 < 0) | (ids64 >= c.vocab)][0]
+            raise ValueError(f"token id {int(bad)} is outside the vocabulary [0, {c.vocab})")
+        ids = ids64.astype(np.int32)
         ids_dev = DeviceBuffer(ids.nbytes).upload(ids)
         self.w.tok_embd.dequantize_rows(ids_dev, rows, self.h)
         for li in range(c.layers):
@@ -404,7 +408,7 @@ class LlamaDecoder:
         for li in range(c.layers):
             self._block(li, 1, 0, self.pos, c.ctx_max, self.kv_len)
         self._head(0)
-        kernels.decode_advance_dev(self.pos, self.kv_len, self.token, self.generated)
+        kernels.decode_advance_dev(self.pos, self.kv_len, self.token, self.generated, c.ctx_max)
 
     def decode(self, steps: int, use_graph: bool = True) -> np.ndarray:
         """Greedy-decode `steps` tokens after prefill(); returns them. With use_graph the step is recorded once and replayed."""
@@ -412,6 +416,9 @@ class LlamaDecoder:
         if self.position() + steps > c.ctx_max:
             raise ValueError(f"{steps} more tokens would pass the context limit {c.ctx_max}")
         out = np.empty(steps, np.int32)
+        if use_graph and self._graph is not None and not self._graph.valid():
+            self._graph.close()                       # scratch moved since the recording (e.g. a longer prompt): record again
+            self._graph = None
         if use_graph and self._graph is None:
             self._decode_step()                       # eager once: sizes every scratch buffer
             kernels.sync()
@@ -437,7 +444,10 @@ class LlamaDecoder:
         """Replay the recorded step `steps` times without reading tokens back; returns seconds (host clock around
         launch + sync). Tokens stay on the device (greedy feedback happens there)."""
         import time
-        if self._graph is None:
+        record = self._graph is None or not self._graph.valid()      # recording costs one (eager) step of its own
+        if self.position() + steps + int(record) > self.cfg.ctx_max:
+            raise ValueError(f"{steps} more tokens would pass the context limit {self.cfg.ctx_max}")
+        if record:
             self.decode(1, use_graph=True)
         kernels.sync()
         self._graph.sync()
@@ -446,6 +456,18 @@ class LlamaDecoder:
             self._graph.launch()
         self._graph.sync()
         return time.perf_counter() - t0
+
+    def close(self) -> None:
+        """Free the recorded decode graph (device buffers go with their owners)."""
+        if self._graph is not None:
+            self._graph.close()
+            self._graph = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
     def generated_tokens(self) -> np.ndarray:
         """Every token emitted since the last prefill (the prefill's own next-token first), read from the device log."""

@@ -298,8 +298,9 @@ def rope_table_dev(pos_dev, theta: float, head_dim: int, table) -> None:
     check(_lib.hip().skainet_hip_f32_rope_table_dev(_ptr(pos_dev), theta, head_dim, _ptr(table)), "rope_table")
 
 
-def decode_advance_dev(pos, kv_len, token, log) -> None:
-    check(_lib.hip().skainet_hip_decode_advance_dev(_ptr(pos), _ptr(kv_len), _ptr(token), _ptr(log)), "decode_advance")
+def decode_advance_dev(pos, kv_len, token, log, capacity: int) -> None:
+    """*pos += 1, *kv_len += 1, log[*pos] = *token on the device; nothing changes once *pos == capacity."""
+    check(_lib.hip().skainet_hip_decode_advance_dev(_ptr(pos), _ptr(kv_len), _ptr(token), _ptr(log), capacity), "decode_advance")
 
 
 def i32_store_at_dev(dst, index_dev, offset: int, src) -> None:
@@ -326,6 +327,10 @@ class Graph:
     def launch(self) -> None:
         check(_lib.hip().skainet_hip_graph_launch(self._g), "graph_launch")
 
+    def valid(self) -> bool:
+        """False once the library reallocated this thread's scratch after the recording: launch() would be refused."""
+        return bool(self._g) and bool(_lib.hip().skainet_hip_graph_valid(self._g))
+
     def sync(self) -> None:
         check(_lib.hip().skainet_hip_graph_sync(self._g), "graph_sync")
 
@@ -333,6 +338,12 @@ class Graph:
         if self._g:
             _lib.hip().skainet_hip_graph_free(self._g)
             self._g = 0
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def fp32_matmul_dev(a, a_offset, a_stride, b, b_offset, b_stride, out, out_offset, out_stride, m, n, k) -> None:
@@ -363,7 +374,7 @@ class Timer:
 
 # ---------------------------------------------------------------------------------------------- SPI kernels (host arrays)
 
-def _raise_if_failed(before: bytes, what: str) -> None:
+def _raise_if_failed(what: str) -> None:
     # The void host entries clear the thread's error text on entry; a message afterwards means this call failed.
     now = _lib.hip().skainet_hip_last_error()
     if now:
@@ -391,10 +402,9 @@ class HipPackedMatmulKernel:
         if weight.size < need or input.size < input_offset + input_dim or output.size < output_offset + output_dim:
             raise ValueError("operand shorter than the dimensions require")
         lib = _lib.hip()
-        before = lib.skainet_hip_last_error()
         getattr(lib, fn_name)(input.ctypes.data, input_offset, weight.ctypes.data, weight_byte_offset, input_dim, output_dim,
                               output.ctypes.data, output_offset)
-        _raise_if_failed(before, fn_name)
+        _raise_if_failed(fn_name)
 
     def matmul(self, input, input_offset, weight, weight_byte_offset, input_dim, output_dim, output, output_offset):
         self._run(self._fn_name, input, input_offset, weight, weight_byte_offset, input_dim, output_dim, output, output_offset)
@@ -408,10 +418,9 @@ class HipFp32MatmulKernel:
     def matmul(self, a, a_offset, a_stride, b, b_offset, b_stride, out, out_offset, out_stride, m, n, k):
         _require_available()
         lib = _lib.hip()
-        before = lib.skainet_hip_last_error()
         lib.skainet_hip_fp32_matmul(_f32(a, "a").ctypes.data, a_offset, a_stride, _f32(b, "b").ctypes.data, b_offset, b_stride,
                                     _f32(out, "out").ctypes.data, out_offset, out_stride, m, n, k)
-        _raise_if_failed(before, "fp32_matmul")
+        _raise_if_failed("fp32_matmul")
 
 
 class HipNarrowFloatMatmulKernel:
@@ -432,48 +441,43 @@ class HipNarrowFloatMatmulKernel:
         if not (isinstance(b, np.ndarray) and b.dtype == np.uint8 and b.flags.c_contiguous):
             raise TypeError("b must be a C-contiguous uint8 numpy array")
         fn = lib.skainet_hip_bf16_matmul if self.codec == "BFloat16" else lib.skainet_hip_fp16_matmul
-        before = lib.skainet_hip_last_error()
         fn(_f32(a, "a").ctypes.data, a_offset, a_stride, b.ctypes.data, b_byte_offset, b_byte_stride,
            _f32(out, "out").ctypes.data, out_offset, out_stride, m, n, k)
-        _raise_if_failed(before, f"{self.codec} matmul")
+        _raise_if_failed(f"{self.codec} matmul")
 
 
 class HipFp32MatmulWtKernel:
     def matmul_wt(self, input, input_offset, weight, weight_offset, out, out_offset, m, n, k):
         _require_available()
         lib = _lib.hip()
-        before = lib.skainet_hip_last_error()
         lib.skainet_hip_fp32_matmul_wt(_f32(input, "input").ctypes.data, input_offset, _f32(weight, "weight").ctypes.data,
                                        weight_offset, _f32(out, "out").ctypes.data, out_offset, m, n, k)
-        _raise_if_failed(before, "fp32_matmul_wt")
+        _raise_if_failed("fp32_matmul_wt")
 
 
 class HipFp32SoftmaxKernel:
     def softmax_rows(self, input, input_offset, out, out_offset, rows, cols, log):
         _require_available()
         lib = _lib.hip()
-        before = lib.skainet_hip_last_error()
         lib.skainet_hip_f32_softmax_rows(_f32(input, "input").ctypes.data + 4 * input_offset,
                                          _f32(out, "out").ctypes.data + 4 * out_offset, rows, cols, int(log))
-        _raise_if_failed(before, "softmax_rows")
+        _raise_if_failed("softmax_rows")
 
 
 class HipFp32NormKernel:
     def layer_norm(self, input, input_offset, gamma, beta, out, out_offset, rows, cols, eps):
         _require_available()
         lib = _lib.hip()
-        before = lib.skainet_hip_last_error()
         lib.skainet_hip_f32_layer_norm(_f32(input, "input").ctypes.data + 4 * input_offset, _ptr(gamma), _ptr(beta),
                                        _f32(out, "out").ctypes.data + 4 * out_offset, rows, cols, eps)
-        _raise_if_failed(before, "layer_norm")
+        _raise_if_failed("layer_norm")
 
     def rms_norm(self, input, input_offset, gamma, out, out_offset, rows, cols, eps):
         _require_available()
         lib = _lib.hip()
-        before = lib.skainet_hip_last_error()
         lib.skainet_hip_f32_rms_norm(_f32(input, "input").ctypes.data + 4 * input_offset, _ptr(gamma),
                                      _f32(out, "out").ctypes.data + 4 * out_offset, rows, cols, eps)
-        _raise_if_failed(before, "rms_norm")
+        _raise_if_failed("rms_norm")
 
 
 class HipFp32AttentionKernel:
@@ -489,11 +493,10 @@ class HipFp32AttentionKernel:
             md = [1] * (4 - len(dims)) + dims
         kl = None if key_lengths is None else np.ascontiguousarray(key_lengths, dtype=np.int32)
         lib = _lib.hip()
-        before = lib.skainet_hip_last_error()
         lib.skainet_hip_f32_sdpa(_f32(query, "query").ctypes.data, _f32(key, "key").ctypes.data, _f32(value, "value").ctypes.data,
                                  _f32(out, "out").ctypes.data, batch, heads, kv_heads, seq_q, seq_kv, head_dim, scale,
                                  int(causal), window, right_context, _ptr(kl), _ptr(mask), *md)
-        _raise_if_failed(before, "sdpa")
+        _raise_if_failed("sdpa")
 
 
 class HipRowMajorMatmulKernel:

@@ -97,9 +97,14 @@ def test_heads_to_rows_and_swiglu_and_increment(hip_backend, torch_cuda):
     kx.i32_increment_dev(ctr, 3)
     pos, klen = dev(torch, np.array([6], np.int32)), dev(torch, np.array([7], np.int32))
     tok, log = dev(torch, np.array([99], np.int32)), dev(torch, np.zeros(10, np.int32))
-    kx.decode_advance_dev(pos, klen, tok, log)
+    kx.decode_advance_dev(pos, klen, tok, log, 9)
     kx.sync()
     assert int(pos.cpu()[0]) == 7 and int(klen.cpu()[0]) == 8 and log.cpu().tolist() == [0] * 7 + [99, 0, 0]
+    # the position saturates at the capacity: two more steps fit (8, 9), the third changes nothing
+    for _ in range(3):
+        kx.decode_advance_dev(pos, klen, tok, log, 9)
+    kx.sync()
+    assert int(pos.cpu()[0]) == 9 and int(klen.cpu()[0]) == 9 and log.cpu().tolist() == [0] * 7 + [99, 99, 99]
     assert np.array_equal(out.cpu().numpy().reshape(tokens, heads, hd), a.transpose(1, 0, 2))
     g, u = gu[:, 0::2].astype(np.float64), gu[:, 1::2].astype(np.float64)
     assert max_norm_err(act.cpu().numpy().reshape(rows, ffn), g / (1 + np.exp(-g)) * u) < 1e-6
@@ -284,6 +289,135 @@ def test_graph_replays_match_eager(hip_backend, torch_cuda):
         assert np.array_equal(y.cpu().numpy(), y1)
         assert max_norm_err(acc.cpu().numpy(), y1.astype(np.float64) * (2 + i)) < 1e-6
     g.close()
+
+
+def test_graph_is_refused_once_scratch_moved(hip_backend, torch_cuda):
+    """A recorded graph holds the scratch addresses of its recording. When a later call makes the library reallocate
+    that scratch, launching the graph is refused on the host (nothing runs, a message says why); a call that would grow
+    scratch inside an open capture fails instead of freeing memory under the capture."""
+    import threading
+    torch, kx = torch_cuda, hip_backend
+    from skainet_amd import _lib
+    result = {}
+
+    def worker():                                   # a fresh thread: its scratch starts empty, whatever ran before
+        try:
+            heads, kvh, d = 8, 2, 64
+            q = torch.randn((1, heads, 1, d), device="cuda")
+            out = torch.empty_like(q)
+
+            def attend(skv):                        # single-query attention: split-key partials live in the workspace
+                k = torch.randn((1, kvh, skv, d), device="cuda")
+                v = torch.randn((1, kvh, skv, d), device="cuda")
+                kx.sdpa_dev(q, k, v, out, 1, heads, kvh, 1, skv, d, 0.125, False)
+                return k, v
+
+            keep = attend(512)                      # sizes the workspace (1 MiB granule)
+            kx.sync()
+            # a prompt-shaped product parks 4 MiB of bf16 activations in the same workspace
+            from gpu_util import random_valid_blocks
+            n, kk, m = 1024, 4096, 512
+            wbig = kx.DeviceWeight.upload("Q4_K", random_valid_blocks("Q4_K", n * kk // 256, 5), n, kk)
+            xbig = torch.randn((m, kk), device="cuda")
+            ybig = torch.empty((m, n), device="cuda")
+            # growth inside a capture is refused
+            assert _lib.hip().skainet_hip_graph_begin() == 0
+            rc_inside = _lib.hip().skainet_hip_matmul_dev(wbig._h, xbig.data_ptr(), m, ybig.data_ptr())
+            msg_inside = _lib.last_error()
+            g_aborted = _lib.hip().skainet_hip_graph_end()
+            if g_aborted:
+                _lib.hip().skainet_hip_graph_free(g_aborted)
+            result["inside"] = (rc_inside, msg_inside)
+            # a good recording, then the workspace grows: the graph is stale
+            with kx.Graph() as g:
+                kx.sdpa_dev(q, keep[0], keep[1], out, 1, heads, kvh, 1, 512, d, 0.125, False)
+            g.launch(); g.sync()
+            assert g.valid()
+            wbig.matmul(xbig, m, ybig)
+            kx.sync()
+            result["valid_after"] = g.valid()
+            try:
+                g.launch()
+                result["launch"] = "ran"
+            except kx.HipError as e:
+                result["launch"] = str(e)
+            g.close()
+            kx.thread_release()
+        except Exception as e:                      # surfaces in the main thread's assert
+            result["error"] = repr(e)
+
+    t = threading.Thread(target=worker)
+    t.start(); t.join()
+    assert "error" not in result, result
+    assert result["inside"][0] == -1 and "capture is open" in result["inside"][1], result
+    assert result["valid_after"] is False
+    assert "refused" in result["launch"] and "record it again" in result["launch"], result
+
+
+def test_decoder_rerecords_its_graph_after_a_longer_prompt(small_model):
+    """prefill(short) -> decode(graph) -> prefill(longer: the MFMA path grows the workspace) -> decode: the decoder
+    notices the stale graph and records a new one; tokens equal the eager route's."""
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    rng = np.random.default_rng(21)
+    short, longer = rng.integers(0, cfg.vocab, 3), rng.integers(0, cfg.vocab, 40)
+    dec = LlamaDecoder(w, max_prefill=40)
+    dec.prefill(short)
+    dec.decode(3, use_graph=True)
+    first = dec.prefill(longer)
+    toks = dec.decode(5, use_graph=True)
+    ref = LlamaDecoder(w, max_prefill=40)
+    assert ref.prefill(longer) == first
+    assert np.array_equal(ref.decode(5, use_graph=False), toks)
+    dec.close(); ref.close()
+
+
+def test_decode_stops_at_the_end_of_the_cache(small_model):
+    """Replaying the recorded step past the context limit writes nothing: the position saturates, the cache rows and
+    the token log keep their contents, and the host entry points refuse to go there in the first place."""
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    dec = LlamaDecoder(w, max_prefill=8)
+    dec.prefill(np.arange(5) % cfg.vocab)
+    with pytest.raises(ValueError):
+        dec.decode_timed(cfg.ctx_max)               # 5 + 64 > 64
+    dec.decode(cfg.ctx_max - 5, use_graph=True)     # exactly to the end
+    assert dec.position() == cfg.ctx_max
+    log_before = dec.generated.download(np.int32, cfg.ctx_max + 1)
+    k_before = dec.k_cache.download(np.float32, cfg.layers * dec.kv_layer_floats)
+    for _ in range(3):
+        dec._graph.launch()                         # what a caller that skips the check would do
+    dec._graph.sync()
+    assert dec.position() == cfg.ctx_max
+    assert np.array_equal(dec.generated.download(np.int32, cfg.ctx_max + 1), log_before)
+    assert np.array_equal(dec.k_cache.download(np.float32, cfg.layers * dec.kv_layer_floats), k_before)
+    dec.close()
+
+
+def test_prefill_rejects_token_ids_outside_the_vocabulary(small_model):
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    dec = LlamaDecoder(w, max_prefill=4)
+    for bad in ([0, cfg.vocab, 1], [3, -1], [2 ** 31 + 5]):
+        with pytest.raises(ValueError, match="outside the vocabulary"):
+            dec.prefill(np.array(bad, np.int64))
+    dec.close()
+
+
+def test_row_gather_clamps_ids_on_the_device(hip_backend, torch_cuda):
+    """Ids that never pass through a host (a sampled token fed back) cannot read outside the weight: the gather clamps."""
+    torch, kx = torch_cuda, hip_backend
+    rows, cols = 16, 512
+    packed = kx.quantize("Q4_K", (np.random.default_rng(4).standard_normal((rows, cols)) * 0.05).astype(np.float32))
+    w = kx.DeviceWeight.upload("Q4_K", packed, rows, cols)
+    dense = torch.empty(rows * cols, device="cuda")
+    w.dequantize(dense)
+    ids = dev(torch, np.array([3, -5, rows + 1000, rows - 1], np.int32))
+    out = torch.empty(4 * cols, device="cuda")
+    w.dequantize_rows(ids, 4, out)
+    kx.sync()
+    d, o = dense.cpu().numpy().reshape(rows, cols), out.cpu().numpy().reshape(4, cols)
+    assert np.array_equal(o, d[[3, 0, rows - 1, rows - 1]])
 
 
 @pytest.mark.parametrize("prompt_len,tol", [(6, 1e-3), (24, 2e-2)])
