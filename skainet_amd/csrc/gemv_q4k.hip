@@ -29,6 +29,9 @@
 
 namespace skh {
 
+int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n, const float* gain, float eps,
+                         const float* residual, int epilogue, const RopeQkvEpilogue* rope_in);   // gemv_q4k_mfma.hip
+
 // One row's 64 weights of a lane against its 64 activations. The 4-bit codes are never converted: a dword of codes is
 // masked into pairs of 16-bit fields whose low mantissa bits hold a code (0x000F000F: the low nibbles of bytes 0 and 2;
 // 0x00F000F0: their high nibbles, i.e. 16 * code; the same on the dword shifted right by 8 for bytes 1 and 3). Read as
@@ -420,6 +423,11 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     }
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 3)) return 0;
     if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return 0;
+    if (batch == 1) {
+        // one activation row with K in whole slices of 1024: the matrix-core kernel with consecutive-kilobyte loads
+        const int r = launch_q4k_gemv_mfma(w, x, y, k, n, gain, eps, residual, epilogue, epilogue == EPI_ROPE_QKV ? &rope : nullptr);
+        if (r != 0) return r;
+    }
     if (g_q4k_ksplit_enable && batch == 1 && !gain && epilogue <= EPI_RESIDUAL && k >= 8192) {
         // long rows: K over the four waves of a workgroup when the plain shape would leave a wave three rows or fewer
         const int nr = (n + 2 * num_cus() - 1) / (2 * num_cus());

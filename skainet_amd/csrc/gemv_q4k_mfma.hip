@@ -1,0 +1,370 @@
+// Q4_K dequant-GEMV for one activation row on the integer matrix cores, canonical row-major GGUF weight.
+//
+//   y[o] = sum_j x[j] * dequant(W[o, j]),   W[o, j] = code * (d * sc) - dmin * m  per 32-element sub-block
+//
+// Same products as the reference's exact-fp32 kernel up to a 22-bit fixed-point rounding of the activations
+//   /root/reference/skainet-backends/skainet-backend-cpu/src/commonMain/kotlin/sk/ainet/exec/kernel/ScalarQ4_KMatmulKernel.kt:40-78
+// (per sub-block: codeSum * (d * sc) - inputSum * (dmin * m)); the reference's own native kernel rounds the activations to
+// 8 bits per 256-element block (native/src/q4k_matmul.c:74-92), this one keeps 22 bits per 64-element group: measured
+// 3.6e-5 in the GEMV parity metric against the exact product, bound 1e-3.
+//
+// What bounds a read-once pass over 25 MB on this device is the shape of the loads, not the arithmetic: a wave load whose
+// lanes pick 16-byte pieces out of many cache lines (a lane owning "its" 64 weights of every row) streams at 3.6 TB/s
+// with no arithmetic at all, a wave load of 1 KB of consecutive bytes with the non-temporal hint at 5.0 TB/s. So:
+//   * Loads are plain consecutive kilobytes. The four waves of a workgroup split K in slices of 1024 elements (576
+//     bytes of a row; wave w takes slices w, w + 4, ...); a wave's share of a row quad (4 rows x its slices) is one run of
+//     16-byte pieces fetched with full-wave non-temporal loads that write straight into LDS (global_load_lds_dwordx4: no
+//     registers are held while the data is in flight), W quads ahead of the one being computed. The loads are inline
+//     assembly with explicit wait counts: their issue order is the program order and nothing else waits on them.
+//   * The lane that computes is not the lane that loaded: lane 4 * blk + j reads from LDS the header and the 32 code
+//     bytes of row j of the quad, 64-weight group blk of the slice (16 groups = 1024 elements).
+//   * The dot products run on v_mfma_i32_4x4x4_16b_i8 (16 independent 4x4x4 blocks): as B operand a lane supplies four
+//     codes of its row (a nibble mask turns a code dword into two operands: 3 instructions per 8 weights), as A operand
+//     four bytes of one "plane" of the activations of its group. The activations of a group are 22-bit fixed point
+//     against the group's largest magnitude, split into balanced base-256 digits: planes 0 and 1 are the two low signed
+//     digits, plane 2 the top digit + 64 (the byte as it lies in the float x * inv + 1.5 * 2^23 + 0x8080), plane 3 is all
+//     ones: the four result registers of a lane are its row's dots with the three digits and its code sum, which takes
+//     the + 64 out again. One accumulator per sub-block, scaled by d * sc afterwards; the minima use the exact fp32 sum
+//     of the sub-block's activations.
+//   * Per quad a lane ends with one partial sum (its row, its group): parked in LDS, summed over the 16 groups and the
+//     four waves at the end by 16 lanes per row (one float4 each, a DPP row sum).
+//   * Optional fusions as in the row-streaming kernel: RMSNorm prologue (x * gain quantised, outputs scaled by
+//     1 / sqrt(mean(x^2) + eps)), epilogue residual / SwiGLU over adjacent (gate, up) rows / RoPE of one token's
+//     [q | k | v] rows with the K and V rows written into the cache.
+#include "gemv_q4k.h"
+
+#include <type_traits>
+
+namespace skh {
+
+typedef uint32_t u32x4_m __attribute__((ext_vector_type(4)));
+typedef int i32x4_m __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void mfma_plain_load16(u32x4_m& dst, uint32_t off, const void* base) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+typedef float f32x2_m __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void mfma_plain_load8(f32x2_m& dst, uint32_t off, const void* base) {
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void mfma_plain_load4(float& dst, uint32_t off, const void* base) {
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+// 16 bytes per lane from base + off into LDS at lds_addr + 16 * lane (M0 carries the LDS address)
+__device__ __forceinline__ void mfma_stream_to_lds(uint32_t lds_addr, uint32_t off, const uint8_t* base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(off), "s"(base) : "memory");
+}
+template <int N> __device__ __forceinline__ void mfma_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+template <int N> __device__ __forceinline__ void mfma_wait_loads(u32x4_m& v) { asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory"); }
+__device__ __forceinline__ void mfma_wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+template <int I, int N, typename F> __device__ __forceinline__ void mfma_static_for(F&& f) {
+    if constexpr (I < N) { f(std::integral_constant<int, I>{}); mfma_static_for<I + 1, N>(f); }
+}
+
+// d * sc and dmin * m of the two sub-blocks (2g, 2g + 1) of a lane, ggml get_scale_min_k4 through byte selectors that are
+// constant per lane: g < 2 picks bytes 2h, 2h + 1 of the 6-bit fields; g >= 2 the split 4 + 2 bit form.
+__device__ __forceinline__ void q4k_lane_scales_sel(const uint4& hdr, uint32_t sel, uint32_t m1, uint32_t sh_min, float& dlo,
+                                                    float& dhi, float& mlo, float& mhi) {
+    const float d = half_bits_to_float_fast(hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(hdr.x >> 16);
+    const uint32_t A = __builtin_amdgcn_perm(hdr.w, hdr.y, sel), B = __builtin_amdgcn_perm(hdr.w, hdr.z, sel);
+    const uint32_t sc = (A & m1) | ((A >> 18) & 0x3030u);
+    const uint32_t mn = ((B >> sh_min) & m1) | ((B >> 18) & 0x3030u);
+    dlo = d * ubyte0_to_float(sc); dhi = d * ubyte1_to_float(sc);
+    mlo = dmin * ubyte0_to_float(mn); mhi = dmin * ubyte1_to_float(mn);
+}
+
+constexpr int MFMA_XROW = 20;          // dwords per (group, plane) row of 16 operand dwords, padded against bank conflicts
+constexpr int MFMA_MAX_QUADS = 32;     // row quads per workgroup (bounds the final pass: 8 rounds of 256 threads)
+constexpr int MFMA_XA_BYTES = 16 * 4 * MFMA_XROW * 4 + 16 * 16;   // operand planes of 16 groups + {scale, sums} per group
+
+// One wave's pass: K slices wave, wave + 4, ... (NSW of them), row quads [0, qt) of the workgroup, W quads in flight.
+// Leaves one partial sum per (quad, lane) in `partials` (index: quad * 64 + (lane % 4) * 16 + lane / 4) and, with the
+// RMSNorm prologue, the sum of squares of this wave's activations in *ssq_out.
+template <int NSW, int W, int PRO>
+__device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, const float* __restrict__ x, const float* __restrict__ gain,
+                                              int n, int r0, int qt, uint32_t row_bytes, int wave, int lane, uint8_t* ring,
+                                              uint8_t* xa_stage, float* partials, float* ssq_out) {
+    constexpr int NPQ = 144 * NSW;                 // 16-byte pieces of a quad in this wave's slices
+    constexpr int NLI = (NPQ + 63) / 64;           // wave loads per quad
+    constexpr int NX = NSW * 4 * (1 + PRO);        // activation (and gain) loads
+    static_assert(NX + W * NLI <= 63, "loads in flight must fit the wave's counter");
+    const int blk = lane >> 2, j = lane & 3, g = blk & 3, h = g & 1;
+    const uint32_t sel = g < 2 ? (0x0C0C0000u | ((2 * h + 1) << 8) | (2 * h))
+                               : (((2 * h + 1) << 24) | ((2 * h) << 16) | ((4 + 2 * h + 1) << 8) | (4 + 2 * h));
+    const uint32_t m1 = g < 2 ? 0x3F3Fu : 0x0F0Fu, sh_min = g < 2 ? 0u : 4u;
+
+    // activations (and gains) of this wave's slices first, the first W quads right behind them
+    u32x4_m xq[NSW][4], gq[PRO ? NSW : 1][4];
+#pragma unroll
+    for (int t = 0; t < NSW; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t off = (uint32_t)((wave + 4 * t) * 1024 + (i * 64 + lane) * 4) * 4u;
+            mfma_plain_load16(xq[t][i], off, x);
+            if (PRO) mfma_plain_load16(gq[t][i], off, gain);
+        }
+    uint32_t loff[NLI];
+#pragma unroll
+    for (int u = 0; u < NLI; ++u) {
+        const uint32_t p = min(64u * u + lane, (uint32_t)(NPQ - 1)), t = (p * 1821u) >> 18;       // p / 144 for p < 2^12
+        const uint32_t rem = p - 144u * t, row4 = (rem * 1821u) >> 16, pc = rem - 36u * row4;    // rem / 36
+        loff[u] = __umul24(row4, row_bytes) + (wave + 4u * t) * 576u + pc * 16u;
+    }
+    const uint32_t max_off = (uint32_t)n * row_bytes - 16u;
+    const uint32_t ring_addr = (uint32_t)(size_t)(__attribute__((address_space(3))) uint8_t*)ring;
+    constexpr uint32_t SLOT = NLI * 1024u;          // bytes of a quad in the ring; W + 1 slots
+    auto issue_quad = [&](int q) {                  // q uniform; rows past the weight are clamped (computed, never stored)
+        const uint32_t base = (uint32_t)(r0 + 4 * q) * row_bytes;
+        const uint32_t slot = ring_addr + (uint32_t)(q % (W + 1)) * SLOT;
+#pragma unroll
+        for (int u = 0; u < NLI; ++u) mfma_stream_to_lds(slot + 1024u * u, min(base + loff[u], max_off), w);
+    };
+#pragma unroll
+    for (int q = 0; q < W; ++q) issue_quad(min(q, qt - 1));
+    mfma_wait_loads<W * NLI>(xq[0][0]);
+#pragma unroll
+    for (int t = 0; t < NSW; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { mfma_wait_loads<W * NLI>(xq[t][i]); if (PRO) mfma_wait_loads<W * NLI>(gq[t][i]); }
+
+    // activations of a slice: float4 number f = i * 64 + lane belongs to group f / 16 (the 16 lanes of a DPP row share a
+    // group); planes go through LDS into operand order
+    int xa[NSW][16];
+    float s_grp[NSW], xsl[NSW], xsh[NSW];
+    float ssq = 0.f;
+    uint32_t* xa_lds = reinterpret_cast<uint32_t*>(xa_stage);
+    float4* xs_lds = reinterpret_cast<float4*>(xa_stage + 16 * 4 * MFMA_XROW * 4);
+#pragma unroll
+    for (int t = 0; t < NSW; ++t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float4 v = make_float4(__uint_as_float(xq[t][i].x), __uint_as_float(xq[t][i].y), __uint_as_float(xq[t][i].z), __uint_as_float(xq[t][i].w));
+            if (PRO) {
+                ssq = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ssq))));
+                v.x *= __uint_as_float(gq[t][i].x); v.y *= __uint_as_float(gq[t][i].y);
+                v.z *= __uint_as_float(gq[t][i].z); v.w *= __uint_as_float(gq[t][i].w);
+            }
+            const int G = i * 4 + (lane >> 4), tt = lane & 15;
+            const float amax = row16_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+            const float inv = 2097151.0f * __builtin_amdgcn_rcpf(fmaxf(amax, 1e-30f));
+            float s4 = (v.x + v.y) + (v.z + v.w);                  // summed over the 8 lanes of a half row = a sub-block of 32
+            s4 += dpp_row_move<0xB1>(s4); s4 += dpp_row_move<0x4E>(s4); s4 += dpp_row_move<0x141>(s4);
+            const uint32_t b0 = __float_as_uint(fmaf(v.x, inv, 12615808.0f)), b1 = __float_as_uint(fmaf(v.y, inv, 12615808.0f));
+            const uint32_t b2 = __float_as_uint(fmaf(v.z, inv, 12615808.0f)), b3 = __float_as_uint(fmaf(v.w, inv, 12615808.0f));
+            const uint32_t a = __builtin_amdgcn_perm(b1, b0, 0x05010400u), b = __builtin_amdgcn_perm(b3, b2, 0x05010400u);
+            const uint32_t c = __builtin_amdgcn_perm(b1, b0, 0x07030602u), d = __builtin_amdgcn_perm(b3, b2, 0x07030602u);
+            uint32_t* dst = xa_lds + G * 4 * MFMA_XROW + tt;
+            dst[0] = __builtin_amdgcn_perm(b, a, 0x05040100u) ^ 0x80808080u;
+            dst[MFMA_XROW] = __builtin_amdgcn_perm(b, a, 0x07060302u) ^ 0x80808080u;
+            dst[2 * MFMA_XROW] = __builtin_amdgcn_perm(d, c, 0x05040100u);
+            dst[3 * MFMA_XROW] = 0x01010101u;
+            float* xs = reinterpret_cast<float*>(xs_lds + G);
+            if ((tt & 7) == 0) { xs[0] = amax * (1.0f / 2097151.0f); xs[1 + (tt >> 3)] = s4 * inv; }
+        }
+        const uint4* src = reinterpret_cast<const uint4*>(xa_lds + (blk * 4 + j) * MFMA_XROW);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint4 v4 = src[e];
+            xa[t][4 * e] = (int)v4.x; xa[t][4 * e + 1] = (int)v4.y; xa[t][4 * e + 2] = (int)v4.z; xa[t][4 * e + 3] = (int)v4.w;
+        }
+        const float4 xsv = xs_lds[blk];
+        s_grp[t] = xsv.x; xsl[t] = xsv.y; xsh[t] = xsv.z;
+    }
+    if (PRO) *ssq_out = wave_sum(ssq);
+
+    // lane's read offsets inside a quad slot: header of (row j, super-block blk / 4 of the slice), then its two code pieces
+    const uint32_t rd_hdr = (uint32_t)(j * 36 + (blk >> 2) * 9) * 16u, rd_q = rd_hdr + 16u + (uint32_t)g * 32u;
+    const int widx = j * 16 + blk;
+    auto compute_quad = [&](int q) {
+        const uint8_t* slot = ring + (uint32_t)(q % (W + 1)) * SLOT;
+        float total = 0.f;
+#pragma unroll
+        for (int t = 0; t < NSW; ++t) {
+            const uint4 hdr = *reinterpret_cast<const uint4*>(slot + t * 2304 + rd_hdr);
+            const uint4 q0 = *reinterpret_cast<const uint4*>(slot + t * 2304 + rd_q);
+            const uint4 q1 = *reinterpret_cast<const uint4*>(slot + t * 2304 + rd_q + 16);
+            float dlo, dhi, mlo, mhi;
+            q4k_lane_scales_sel(hdr, sel, m1, sh_min, dlo, dhi, mlo, mhi);
+            const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+            i32x4_m dl = {0, 0, 0, 0}, dh = {0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int wlo = (int)(qw[u] & 0x0F0F0F0Fu), whi = (int)((qw[u] >> 4) & 0x0F0F0F0Fu);
+                dl = __builtin_amdgcn_mfma_i32_4x4x4i8(xa[t][u], wlo, dl, 0, 0, 0);
+                dh = __builtin_amdgcn_mfma_i32_4x4x4i8(xa[t][8 + u], whi, dh, 0, 0, 0);
+            }
+            // digits back together: ((top * 256 + mid) * 256 + low) - 64 * 65536 * (code sum)
+            const int tl = __mul24(dl[3], -4194304) + (((dl[2] << 8) + dl[1]) << 8) + dl[0];
+            const int th = __mul24(dh[3], -4194304) + (((dh[2] << 8) + dh[1]) << 8) + dh[0];
+            total = fmaf(s_grp[t], fmaf(dlo, (float)tl, fmaf(dhi, (float)th, -fmaf(mlo, xsl[t], mhi * xsh[t]))), total);
+        }
+        partials[q * 64 + widx] = total;
+    };
+
+    // quads [0, base): wait for the quad, ask for the one W ahead, compute; the last W quads without new requests
+    const int base = max(qt - W, 0);
+    for (int q = 0; q < base; ++q) {
+        mfma_wait_loads<(W - 1) * NLI>();
+        mfma_wait_lds();                             // the slot about to be refilled has been read
+        issue_quad(q + W);
+        compute_quad(q);
+    }
+    mfma_static_for<0, W>([&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        mfma_wait_loads<(W - 1 - m) * NLI>();
+        if (base + m < qt) compute_quad(base + m);
+    });
+}
+
+// What the epilogue of a row reads besides its sum, requested at the start of the kernel.
+struct MfmaRowPre { float residual; f32x2_m cs; };
+
+template <int W, int PRO>
+__global__ __launch_bounds__(256, 2) void q4k_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x, float* y,
+                                                             int k, int n, int qt, const float* __restrict__ gain, float eps,
+                                                             const float* residual, int epilogue, RopeQkvEpilogue rope) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nsl = k >> 10;                                   // slices of 1024 elements
+    const int nsw = (nsl - wave + 3) >> 2;                     // this wave's share (uniform)
+    const int ns_max = (nsl + 3) >> 2;
+    const int nli_max = (144 * ns_max + 63) / 64;
+    const uint32_t ring_bytes = (uint32_t)(W + 1) * nli_max * 1024u;
+    uint8_t* ring = smem + wave * (ring_bytes + MFMA_XA_BYTES);
+    uint8_t* xa_stage = ring + ring_bytes;
+    float* partials_all = reinterpret_cast<float*>(smem + 4 * (ring_bytes + MFMA_XA_BYTES));   // [4 waves][qt][64]
+    float* ssq_lds = partials_all + 4 * qt * 64;
+    float* partials = partials_all + wave * qt * 64;
+    const int r0 = blockIdx.x * (4 * qt);
+    const uint32_t row_bytes = (uint32_t)(k >> 8) * (uint32_t)Q4K_BYTES;
+
+    // what the final pass will add or rotate with: one output row per 16 threads and round
+    constexpr int ROUNDS = MFMA_MAX_QUADS * 4 * 16 / 256;
+    MfmaRowPre pre[ROUNDS];
+    const int pos = epilogue == EPI_ROPE_QKV ? rope.pos_dev[0] : 0;
+    if (epilogue == EPI_RESIDUAL || (epilogue == EPI_ROPE_QKV && rope.table)) {       // uniform
+#pragma unroll
+        for (int it = 0; it < ROUNDS; ++it) {
+            const int row = min(r0 + it * 16 + (threadIdx.x >> 4), n - 1);
+            pre[it].residual = 0.f; pre[it].cs = f32x2_m{1.f, 0.f};
+            if (it * 16 < 4 * qt) {
+                if (epilogue == EPI_RESIDUAL) mfma_plain_load4(pre[it].residual, (uint32_t)row * 4u, residual);
+                else mfma_plain_load8(pre[it].cs, (uint32_t)((row % rope.head_dim) >> 1) * 8u, rope.table);
+            }
+        }
+        mfma_wait_loads<0>();                 // a handful of cached loads, before the stream starts
+    }
+
+    float ssq = 0.f;
+    switch (nsw) {
+        case 1: q4k_mfma_wave<1, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 2: q4k_mfma_wave<2, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 3: q4k_mfma_wave<3, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 4: q4k_mfma_wave<4, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        default:                                               // K below 4 slices: this wave has none
+            for (int i = lane; i < qt * 64; i += 64) partials[i] = 0.f;
+    }
+    if (PRO && lane == 0) ssq_lds[wave] = ssq;
+    __syncthreads();
+
+    float xscale = 1.0f;
+    if (PRO) xscale = 1.0f / sqrtf(((ssq_lds[0] + ssq_lds[1]) + (ssq_lds[2] + ssq_lds[3])) * (1.0f / (float)k) + eps);
+    const int u = threadIdx.x & 15, pw = u >> 2, pp = u & 3;
+#pragma unroll
+    for (int it = 0; it < ROUNDS; ++it) {
+        if (it * 16 >= 4 * qt) break;                          // uniform
+        const int rl = it * 16 + (threadIdx.x >> 4);           // row of the workgroup
+        const int rlc = min(rl, 4 * qt - 1);
+        const float4 p4 = *reinterpret_cast<const float4*>(partials_all + (pw * qt + (rlc >> 2)) * 64 + (rlc & 3) * 16 + pp * 4);
+        float val = row16_sum((p4.x + p4.y) + (p4.z + p4.w)) * xscale;
+        const int row = r0 + rl;
+        const bool live = u == 0 && rl < 4 * qt && row < n;
+        if (epilogue == EPI_SWIGLU) {
+            const float up = __shfl_xor(val, 16, 64);          // rows 2i (gate) and 2i + 1 (up) sit 16 lanes apart
+            if (live && !(row & 1)) y[row >> 1] = val * (1.0f / (1.0f + expf(-val))) * up;
+        } else if (epilogue == EPI_ROPE_QKV) {
+            const float odd = __shfl_xor(val, 16, 64);
+            if (live && !(row & 1)) {
+                const int slot = row / rope.head_dim, dd = row % rope.head_dim;
+                float2 out2 = make_float2(val, odd);
+                if (slot < rope.heads + rope.kv_heads) {
+                    float sn, cs;
+                    if (rope.table) { cs = pre[it].cs.x; sn = pre[it].cs.y; }
+                    else sincosf((float)pos * powf(rope.theta, -(float)dd / (float)rope.head_dim), &sn, &cs);
+                    out2 = rope_rotate(val, odd, cs, sn);
+                }
+                const bool in_cache = pos >= 0 && pos < rope.capacity;
+                float* dst;
+                if (slot < rope.heads) dst = y + (int64_t)slot * rope.head_dim;
+                else if (slot < rope.heads + rope.kv_heads) dst = rope.k_cache + ((int64_t)(slot - rope.heads) * rope.capacity + pos) * rope.head_dim;
+                else dst = rope.v_cache + ((int64_t)(slot - rope.heads - rope.kv_heads) * rope.capacity + pos) * rope.head_dim;
+                if (slot < rope.heads || in_cache) *reinterpret_cast<float2*>(dst + dd) = out2;
+            }
+        } else if (live) {
+            if (epilogue == EPI_RESIDUAL) val += pre[it].residual;
+            y[row] = val;
+        }
+    }
+}
+
+static std::atomic<int> g_q4k_mfma_enable{1};
+void set_q4k_mfma_enable(int v) { g_q4k_mfma_enable = v; }
+
+// quads in flight per wave: three while a quad is at most 5 KB per wave, two for the long rows (9 KB per quad and wave)
+static int mfma_window(int k) { return (((k >> 10) + 3) >> 2) >= 3 ? 2 : 3; }
+
+static size_t mfma_smem_bytes(int k, int qt, int window) {
+    const int ns_max = ((k >> 10) + 3) >> 2;
+    const int nli_max = (144 * ns_max + 63) / 64;
+    return (size_t)4 * ((size_t)(window + 1) * nli_max * 1024 + MFMA_XA_BYTES) + (size_t)4 * qt * 64 * sizeof(float) + 16;
+}
+
+template <int W>
+static int launch_mfma(bool pro, int grid, size_t smem, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int qt,
+                       const float* gain, float eps, const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+    if (pro) {
+        SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, 1>), 160 * 1024);
+        q4k_gemv_mfma_kernel<W, 1><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
+    } else {
+        SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, 0>), 160 * 1024);
+        q4k_gemv_mfma_kernel<W, 0><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
+    }
+    SKH_CHECK(hipGetLastError());
+    return 1;
+}
+
+// Returns 1 when this kernel took the product, 0 when the shape is outside its range (the caller goes on to the
+// row-streaming kernel), -1 on a launch error. One activation row; K a multiple of 1024 up to 16384; the weight below
+// 4 GiB (32-bit byte offsets); operands 16-byte aligned.
+int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n, const float* gain, float eps,
+                         const float* residual, int epilogue, const RopeQkvEpilogue* rope_in) {
+    if (!g_q4k_mfma_enable) return 0;
+    if (k < 1024 || (k & 1023) || k > 16384 || n < 4) return 0;
+    const uint64_t wbytes = (uint64_t)n * (uint64_t)(k >> 8) * Q4K_BYTES;
+    if (wbytes >= ((uint64_t)1 << 32) || (uint64_t)n * 4 >= ((uint64_t)1 << 32)) return 0;
+    if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return 0;
+    if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return 0;
+    RopeQkvEpilogue rope{};
+    if (epilogue == EPI_ROPE_QKV) {
+        if (!rope_in) return 0;
+        rope = *rope_in;
+        if ((rope.head_dim & 1) || n != (rope.heads + 2 * rope.kv_heads) * rope.head_dim) return 0;
+        if (rope.table && (reinterpret_cast<uintptr_t>(rope.table) & 7)) return 0;
+    }
+    if (epilogue >= EPI_SWIGLU && (n & 1)) return 0;
+    if (epilogue == EPI_RESIDUAL && (!residual || (reinterpret_cast<uintptr_t>(residual) & 3))) return 0;
+    // one round of workgroups over the chip: a workgroup's quads are consecutive rows, the last workgroup may own fewer
+    const int quads = (n + 3) / 4;
+    int qt = (quads + num_cus() - 1) / num_cus();
+    if (qt > MFMA_MAX_QUADS) qt = MFMA_MAX_QUADS;
+    if (qt < 1) qt = 1;
+    const int grid = (quads + qt - 1) / qt;
+    const int window = mfma_window(k);
+    const size_t smem = mfma_smem_bytes(k, qt, window);
+    if (smem > 160 * 1024) return 0;
+    if (window == 2) return launch_mfma<2>(gain != nullptr, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
+    return launch_mfma<3>(gain != nullptr, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
+}
+
+}  // namespace skh

@@ -143,7 +143,8 @@ def test_rope_qkv_equals_three_scatters(hip_backend, torch_cuda):
                                         ("Q4_K", 640, 512, 5), ("Q6_K", 512, 512, 1), ("Q4_K", 768, 1024, 24),
                                         ("Q4_K", 1030, 14336, 1), ("Q4_K", 26, 16640, 1), ("Q4_K", 4096, 12288, 1), ("Q4_K", 2050, 8448, 1),
                                         ("Q4_K", 300, 512, 40), ("Q6_K", 258, 1024, 33), ("Q8_0", 130, 2048, 64),
-                                        ("Q4_K", 64, 5120, 300), ("Q8_0", 66, 96, 12)])
+                                        ("Q4_K", 64, 5120, 300), ("Q8_0", 66, 96, 12), ("Q4_K", 1030, 4096, 1), ("Q4_K", 14000, 2048, 1),
+                                        ("Q4_K", 50, 3072, 1), ("Q4_K", 6, 1024, 1)])
 def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
     """Every prologue / epilogue combination against float64 arithmetic on the oracle-decoded weight; the decode
     shapes of Q4_K run the one-kernel route (also with K of several passes), the other cases the composed route of the
@@ -194,7 +195,7 @@ def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
 
 
 @pytest.mark.parametrize("enc,heads,kvh,hd,k", [("Q4_K", 8, 2, 64, 512), ("Q4_K", 32, 8, 128, 4096), ("Q4_K", 3, 1, 64, 256),
-                                                ("Q6_K", 4, 2, 64, 512)])
+                                                ("Q6_K", 4, 2, 64, 512), ("Q4_K", 5, 1, 64, 1024), ("Q4_K", 8, 4, 128, 2048)])
 def test_matmul_qkv_rope_equals_product_then_rope(hip_backend, torch_cuda, enc, heads, kvh, hd, k):
     """The one-launch decode projection (norm + product + RoPE + cache append) against the separate entries, with and
     without the norm, at a device-side position; rows of the caches other than the position stay untouched."""

@@ -114,16 +114,20 @@ def test_gemv_at_config_sizes(hip_backend, torch_cuda, enc, n, k, batches):
         assert err <= GEMV_TOL
 
 
-@pytest.mark.parametrize("mode", ["slot-fp32", "rows-fp32"])
+@pytest.mark.parametrize("mode", ["slot-fp32", "rows-fp32", "mfma-i8"])
 @pytest.mark.parametrize("n,k,m", [(11008, 4096, 1), (11008, 4096, 2), (4096, 14336, 1), (2050, 8448, 1), (1537, 16640, 1), (6144, 8192, 1),
-                                   (1000, 11008, 1), (77, 2304, 2), (5, 256, 1)])
+                                   (1000, 11008, 1), (77, 2304, 2), (5, 256, 1), (1030, 1024, 1), (7, 2048, 1), (515, 3072, 1),
+                                   (2052, 5120, 1), (300, 16384, 1), (28672, 4096, 1), (36000, 1024, 1), (4096, 12288, 1)])
 def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cuda, mode, n, k, m):
-    """Both Q4_K decode kernels (the generic slot kernel and the row-streaming kernel) are held to the same bound
-    against the exact-fp32 oracle, on quantised Gaussian weights and on random valid blocks with large scales. The
-    long-row shapes (4096 x 14336; 2050 x 8448: 33 super-blocks per row, a ragged last workgroup; 1537 x 16640: 65
-    super-blocks, two passes per wave, four rows per workgroup; 6144 x 8192: twelve) take the form of the row kernel that
-    splits K over the waves of a workgroup."""
-    hip_backend.set_tuning("q4k_rows_enable", 1 if mode == "rows-fp32" else 0)
+    """The Q4_K decode kernels (the generic slot kernel, the fp32 row-streaming kernel and the integer matrix-core
+    kernel that takes one-row products with K in whole slices of 1024) are held to the same bound against the
+    exact-fp32 oracle, on quantised Gaussian weights and on random valid blocks with large scales. The long-row shapes
+    (4096 x 14336; 2050 x 8448: 33 super-blocks per row, a ragged last workgroup; 1537 x 16640: 65 super-blocks, two
+    passes per wave, four rows per workgroup; 6144 x 8192: twelve) take the form of the row kernel that splits K over the
+    waves of a workgroup; K of 1 to 16 slices, row counts that are not a multiple of 4, more quads than one round of
+    workgroups holds (28672 and 36000 rows) exercise the matrix-core kernel's slice and quad bookkeeping."""
+    hip_backend.set_tuning("q4k_rows_enable", 0 if mode == "slot-fp32" else 1)
+    hip_backend.set_tuning("q4k_mfma_enable", 1 if mode == "mfma-i8" else 0)
     try:
         for packed in (gaussian_weight(hip_backend, "Q4_K", n, k, 71), random_valid_blocks("Q4_K", n * k // 256, 72)):
             x = np.random.default_rng(73 + m).standard_normal((m, k)).astype(np.float32)
@@ -135,6 +139,7 @@ def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cud
             assert err <= GEMV_TOL
     finally:
         hip_backend.set_tuning("q4k_rows_enable", 1)
+        hip_backend.set_tuning("q4k_mfma_enable", 1)
 
 
 @pytest.mark.parametrize("slot64", [1, 0])
@@ -171,7 +176,11 @@ def test_q4k_three_to_eight_rows_on_the_matrix_instruction(hip_backend, torch_cu
         got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
         assert got.shape == (m, n) and not np.isnan(got).any()
         assert normalized_err(got, L.gemv("Q4_K", x, packed, n)) <= GEMV_TOL
-        alone = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x[m - 1:m])
+        hip_backend.set_tuning("q4k_mfma_enable", 0)          # "alone" on the exact-fp32 row kernel
+        try:
+            alone = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x[m - 1:m])
+        finally:
+            hip_backend.set_tuning("q4k_mfma_enable", 1)
         assert normalized_err(got[m - 1], alone[0]) <= 3e-4
 
 
