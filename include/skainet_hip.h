@@ -328,7 +328,8 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * "q4k_rows_enable" (0: Q4_K decode shapes take the generic slot kernel), "q6k_slot64" (0: Q6_K at batch 1 keeps the
  * 32-weight slot of the batched kernel), "q4k_ksplit_enable" (0: long Q4_K rows are not
  * split over the waves of a workgroup), "q4k_mfma_enable" (0: one-row Q4_K products stay off the integer matrix-core
- * kernel and run the fp32 row-streaming one), "gemm_ksplit" (K splits of the MFMA GEMM,
+ * kernel and run the fp32 row-streaming one), "q4k_mfma_window" (row quads that kernel keeps in flight per wave: 2 or 3,
+ * 0 = chosen from K), "gemm_ksplit" (K splits of the MFMA GEMM,
  * 0 = automatic), "gemm_wide" (1 / 0: force the 256 x 256 / 256 x 128 tile, -1 = chosen from the shape),
  * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_decode_split_keys" (least keys per split of
  * decode-shape attention, default 64).

@@ -260,8 +260,8 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_mfma_kernel(const uint8_t* __
     switch (nsw) {
         case 1: q4k_mfma_wave<1, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
         case 2: q4k_mfma_wave<2, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 3: q4k_mfma_wave<3, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 4: q4k_mfma_wave<4, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 3: if constexpr (W <= 2) q4k_mfma_wave<3, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 4: if constexpr (W <= 2) q4k_mfma_wave<4, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
         default:                                               // K below 4 slices: this wave has none
             for (int i = lane; i < qt * 64; i += 64) partials[i] = 0.f;
     }
@@ -310,6 +310,8 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_mfma_kernel(const uint8_t* __
 
 static std::atomic<int> g_q4k_mfma_enable{1};
 void set_q4k_mfma_enable(int v) { g_q4k_mfma_enable = v; }
+static std::atomic<int> g_q4k_mfma_window{0};      // 0: chosen from K
+void set_q4k_mfma_window(int v) { if (v == 0 || v == 2 || v == 3) g_q4k_mfma_window = v; }
 
 // quads in flight per wave: three while a quad is at most 5 KB per wave, two for the long rows (9 KB per quad and wave)
 static int mfma_window(int k) { return (((k >> 10) + 3) >> 2) >= 3 ? 2 : 3; }
@@ -360,7 +362,9 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
     if (qt > MFMA_MAX_QUADS) qt = MFMA_MAX_QUADS;
     if (qt < 1) qt = 1;
     const int grid = (quads + qt - 1) / qt;
-    const int window = mfma_window(k);
+    // measured on 11008 x 4096 with two / three / four quads in flight: 7.06 / 6.52 / 6.68 us
+    int window = g_q4k_mfma_window.load() > 0 ? g_q4k_mfma_window.load() : mfma_window(k);
+    if (mfma_window(k) == 2) window = 2;                       // long rows: the wave's load counter holds 63
     const size_t smem = mfma_smem_bytes(k, qt, window);
     if (smem > 160 * 1024) return 0;
     if (window == 2) return launch_mfma<2>(gain != nullptr, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
