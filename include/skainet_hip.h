@@ -65,6 +65,9 @@ SKAINET_HIP_API const char* skainet_hip_last_error(void);
 /* Device name ("" when unavailable) and compute-unit count. */
 SKAINET_HIP_API const char* skainet_hip_device_name(void);
 SKAINET_HIP_API int32_t skainet_hip_compute_units(void);
+/* Name of the kernel family the calling thread's last matmul / attention entry launched as its main kernel ("" before
+ * the first): lets a measurement say which kernel a number belongs to. No reference counterpart. */
+SKAINET_HIP_API const char* skainet_hip_last_kernel(void);
 /* Stream (a hipStream_t, NULL = the null stream) used by this thread's later device entries. */
 SKAINET_HIP_API int32_t skainet_hip_set_stream(void* stream);
 /* Wait for this thread's stream. */
@@ -137,12 +140,14 @@ SKAINET_HIP_API int32_t skainet_hip_matmul_qkv_rope_dev(const skainet_hip_weight
 /* table[2i], table[2i+1] = cos, sin of (*pos_dev) * theta^(-2i/head_dim), i < head_dim/2 (head_dim floats). */
 SKAINET_HIP_API int32_t skainet_hip_f32_rope_table_dev(const int32_t* pos_dev, float theta, int32_t head_dim, float* table);
 /* Measurement aid: `iters` such products back to back on this thread's stream, weight number i % nweights at
- * step i, timed with HIP events; returns the elapsed milliseconds (< 0 on failure). use_graph != 0 captures the
- * launches into a HIP graph first and times one replay, so host launch cost stays off the GPU timeline.
+ * step i, timed with HIP events; returns the elapsed milliseconds of one pass of `iters` steps (< 0 on failure): the pass
+ * is timed `replays` times (1 .. 64) and the median is returned. use_graph != 0 captures the launches into a HIP graph
+ * first and times replays of it, so host launch cost stays off the GPU timeline; about 400 untimed launches come first
+ * whatever `iters` is, so a short pass reads the same time per step as a long one.
  * (The reference times its kernels the same way, in a loop around the call: NativeKernel microbench,
  * REF/skainet-backend-native-cpu/src/jvmTest/kotlin/sk/ainet/exec/kernel/Q4KMatmulMicrobenchTest.kt:53-70.) */
 SKAINET_HIP_API float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, int32_t nweights,
-    const float* x, int32_t m, float* out, int32_t iters, int32_t kind, int32_t use_graph);
+    const float* x, int32_t m, float* out, int32_t iters, int32_t kind, int32_t use_graph, int32_t replays);
 /* Calibration aid with no reference counterpart: `iters` launches of a pure streaming-read kernel (16-byte loads,
  * no arithmetic) over buffers[i % nbuffers], each `bytes` long, timed with HIP events; returns milliseconds.
  * The rate it reaches on rotating copies of a weight is the device's ceiling for a read-once pass of that size. */

@@ -25,6 +25,7 @@ SIGNATURES = {
     "skainet_hip_last_error": (C.c_char_p, []),
     "skainet_hip_device_name": (C.c_char_p, []),
     "skainet_hip_compute_units": (_i32, []),
+    "skainet_hip_last_kernel": (C.c_char_p, []),
     "skainet_hip_set_stream": (_i32, [_vp]),
     "skainet_hip_sync": (_i32, []),
     "skainet_hip_thread_release": (_i32, []),
@@ -45,7 +46,7 @@ SIGNATURES = {
     "skainet_hip_matmul_fused_dev": (_i32, [_vp, _vp, _i32, _vp, _vp, _f32, _vp, _i32]),
     "skainet_hip_matmul_qkv_rope_dev": (_i32, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _vp]),
     "skainet_hip_f32_rope_table_dev": (_i32, [_vp, _f32, _i32, _vp]),
-    "skainet_hip_matmul_repeat_dev": (_f32, [_vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32]),
+    "skainet_hip_matmul_repeat_dev": (_f32, [_vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32, _i32]),
     "skainet_hip_read_probe_dev": (_f32, [_vp, _i32, _i64, _i32, _i32]),
     "skainet_hip_dequantize_dev": (_i32, [_vp, _vp]),
     "skainet_hip_dequantize_rows_dev": (_i32, [_vp, _vp, _i32, _vp]),

@@ -41,6 +41,7 @@ int check_hip(hipError_t e, const char* what);  // 0 on success, else records an
 hipStream_t current_stream();                 // the calling thread's launch stream
 int ensure_device();                          // lazily initialises the device; 0 when usable
 int num_cus();
+void note_kernel(const char* family);    // remembers the kernel family this thread launched last (skainet_hip_last_kernel)
 
 #define SKH_CHECK(expr)                                     \
     do {                                                    \

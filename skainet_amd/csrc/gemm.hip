@@ -576,6 +576,7 @@ template <class Raw, int BE, int BB, int WTN>
 static int launch_gemm_tile(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
                             int64_t split_stride, hipStream_t s) {
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&dequant_gemm_kernel<Raw, BE, BB, WTN>), gemm_smem(WTN));
+    note_kernel("dequant_gemm_kernel");
     dequant_gemm_kernel<Raw, BE, BB, WTN><<<grid, dim3(G_THREADS), gemm_smem(WTN), s>>>(a, w, c, m, n, k, k_chunk, split_stride);
     SKH_CHECK(hipGetLastError());
     return 0;

@@ -534,6 +534,7 @@ static int launch_one(const uint8_t* w, const float* x, float* y, int k, int n, 
     if (rows_per_wg < 1) rows_per_wg = 1;
     if (rows_per_wg > GEMV_MAX_ROWS) rows_per_wg = GEMV_MAX_ROWS;
     const int grid = (n + rows_per_wg - 1) / rows_per_wg;
+    note_kernel("gemv_kernel");
     gemv_kernel<F, B, R><<<dim3(grid), dim3(64 * nwaves), 0, current_stream()>>>(w, x, y, k, n, batch, row_bytes, rows_per_wg);
     SKH_CHECK(hipGetLastError());
     return 0;

@@ -394,6 +394,7 @@ void set_q4k_ksplit_enable(int v) { g_q4k_ksplit_enable = v; }
 template <int B, int R, int NR>
 static void launch_rows(bool pro, int grid, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int nchunks,
                         const float* gain, float eps, const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+    note_kernel("q4k_gemv_rows_kernel");
     if (pro) q4k_gemv_rows_kernel<B, R, NR, 1><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, nchunks, gain, eps, residual, epilogue, rope);
     else q4k_gemv_rows_kernel<B, R, NR, 0><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, nchunks, gain, eps, residual, epilogue, rope);
 }
@@ -434,6 +435,7 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
         if (nr >= 4 && nr <= Q4K_RMAX && (n + num_cus() * 8 - 1) / (num_cus() * 8) <= 3) {
             const int grid = (n + nr - 1) / nr;
             hipStream_t s = current_stream();
+            note_kernel("q4k_gemv_ksplit_kernel");
 #define SKH_KS_CASE(N) case N: q4k_gemv_ksplit_kernel<(6 < N ? 6 : N), N><<<dim3(grid), dim3(256), 0, s>>>(w, x, y, k, n, residual, epilogue); break;
             switch (nr) {
                 SKH_KS_CASE(4) SKH_KS_CASE(5) SKH_KS_CASE(6) SKH_KS_CASE(7) SKH_KS_CASE(8) SKH_KS_CASE(9)

@@ -325,6 +325,7 @@ static size_t mfma_smem_bytes(int k, int qt, int window) {
 template <int W>
 static int launch_mfma(bool pro, int grid, size_t smem, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int qt,
                        const float* gain, float eps, const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+    note_kernel("q4k_gemv_mfma_kernel");
     if (pro) {
         SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, 1>), 160 * 1024);
         q4k_gemv_mfma_kernel<W, 1><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);

@@ -277,6 +277,7 @@ static int launch_quads(hipStream_t s, const uint8_t* w, const float* x, float* 
     static_assert(4 * ((Q * 4 * NM + 15) / 16) * 64 <= 8 * NM * 64 * QD_SLICE, "wave partials must fit in the slices");
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_quads_kernel<NM, Q, R, OCC>), smem);
     const int grid = (n + 4 * Q - 1) / (4 * Q);
+    note_kernel("q4k_gemv_quads_kernel");
     q4k_gemv_quads_kernel<NM, Q, R, OCC><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, batch);
     SKH_CHECK(hipGetLastError());
     return 1;

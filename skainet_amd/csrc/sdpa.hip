@@ -236,6 +236,7 @@ int launch_sdpa(const float* q, const float* k, const float* v, float* out, int 
         if (!p.part) return -1;
     }
     const size_t smem = sizeof(float) * ((size_t)SDPA_TILE * (head_dim + 1) + (size_t)group * head_dim + (size_t)group * SDPA_TILE);
+    note_kernel("sdpa_rows_kernel");
     sdpa_rows_kernel<<<dim3((unsigned)grid, (unsigned)splits), dim3(64 * group), smem, s>>>(p);
     SKH_CHECK(hipGetLastError());
     if (splits > 1) {

@@ -284,6 +284,7 @@ void set_sdpa_decode_split_keys(int v) { if (v >= 16) g_sdpa_decode_split_keys =
 template <int GS, int DPL>
 static int launch_decode_variant(const SdpaDecodeParams& p, int subs) {
     constexpr int D = 16 * DPL;
+    note_kernel("sdpa_decode_kernel");
     sdpa_decode_kernel<GS, DPL><<<dim3(p.splits, p.kv_heads * subs, p.batch), dim3(256), 0, current_stream()>>>(p);
     SKH_CHECK(hipGetLastError());
     if (p.splits > 1) {

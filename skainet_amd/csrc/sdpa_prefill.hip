@@ -289,6 +289,7 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
     const dim3 grid((seq_q + q_per_wg - 1) / q_per_wg, kv_heads * (per_kv / hpw), batch);
     constexpr size_t smem = sizeof(__bf16) * (2 * PF_KB * (D + 8) + 2 * D * (PF_KB + 8));
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D>), smem);
+    note_kernel("sdpa_prefill_kernel");
     sdpa_prefill_kernel<D><<<grid, dim3(256), smem, s>>>(p);
     SKH_CHECK(hipGetLastError());
     return 1;

@@ -81,6 +81,8 @@ int check_hip(hipError_t e, const char* what) {
     (void)hipGetLastError();   // clear the sticky error so later calls report their own
     return set_error("%s failed: %s", what, hipGetErrorString(e));
 }
+static thread_local const char* t_last_kernel = "";
+void note_kernel(const char* family) { t_last_kernel = family; }
 hipStream_t current_stream() { return t_stream; }
 int num_cus() { return g_cus > 0 ? g_cus : 256; }
 
@@ -188,6 +190,7 @@ int32_t skainet_hip_init(int32_t device) {
 const char* skainet_hip_last_error(void) { return t_error; }
 const char* skainet_hip_device_name(void) { return g_name; }
 int32_t skainet_hip_compute_units(void) { return g_cus; }
+const char* skainet_hip_last_kernel(void) { return t_last_kernel; }
 int32_t skainet_hip_set_stream(void* stream) { t_stream = static_cast<hipStream_t>(stream); return 0; }
 int32_t skainet_hip_sync(void) {
     if (ensure_device() != 0) return -1;
@@ -402,36 +405,66 @@ int32_t skainet_hip_matmul_qkv_rope_dev(const skainet_hip_weight* w, const float
 // `iters` products back to back on this thread's stream, weight i % nweights each time (several copies of one
 // weight defeat the memory-side cache), bracketed by HIP events. With use_graph the launches are captured once
 // into a HIP graph (kernel nodes only) and replayed, which removes the host's per-launch cost from the GPU timeline.
+// The pass is timed `replays` times (each replay is exactly `iters` steps) and the median is returned.
 float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, int32_t nweights, const float* x, int32_t m,
-                                    float* out, int32_t iters, int32_t kind, int32_t use_graph) {
+                                    float* out, int32_t iters, int32_t kind, int32_t use_graph, int32_t replays) {
     if (ensure_device() != 0) return -1.f;
     if (!weights || nweights <= 0 || iters <= 0 || m <= 0) { set_error("matmul_repeat: bad arguments"); return -1.f; }
+    if (replays < 1) replays = 1;
+    if (replays > 64) replays = 64;
     hipStream_t prev = t_stream, cap = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     float ms = -1.f;
     bool ok = true;
+    float samples[64];
+    auto median = [&](int count) {
+        for (int i = 1; i < count; ++i) for (int j = i; j > 0 && samples[j] < samples[j - 1]; --j) { const float t = samples[j]; samples[j] = samples[j - 1]; samples[j - 1] = t; }
+        return samples[count / 2];
+    };
     if (use_graph) {
         // capture needs a real (non-null) stream; the graph is then launched on it as well
         ok = check_hip(hipStreamCreateWithFlags(&cap, hipStreamNonBlocking), "hipStreamCreate") == 0;
         if (ok) {
             t_stream = cap;
-            ok = check_hip(hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture") == 0;
-            for (int i = 0; ok && i < iters; ++i) ok = skainet_hip_matmul_kind_dev(weights[i % nweights], x, m, out, kind) == 0;
+            // One graph holds about 400 untimed launches (the upload of the graph, clocks and address translations settle
+            // on those whatever the step count) and behind them `replays` passes of exactly `iters` launches, with an
+            // event-record node between consecutive passes: every timed pass runs in the steady state of one long chain
+            // of launches, so a short pass reads the same time per step as a long one (a graph launch of its own per
+            // pass costs about 9 us of idle device per pass, 7 % of a 20-step pass). A pass's time is the span
+            // between its two events.
+            hipEvent_t ev[65] = {};
+            for (int r = 0; ok && r <= replays; ++r) ok = check_hip(hipEventCreate(&ev[r]), "hipEventCreate") == 0;
+            ok = ok && check_hip(hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture") == 0;
+            int step = 0;
+            for (int i = 0; ok && i < 400; ++i, ++step) ok = skainet_hip_matmul_kind_dev(weights[step % nweights], x, m, out, kind) == 0;
+            bool inner = ok && hipEventRecord(ev[0], cap) == hipSuccess;
+            for (int r = 0; ok && r < replays; ++r) {
+                for (int i = 0; ok && i < iters; ++i, ++step) ok = skainet_hip_matmul_kind_dev(weights[step % nweights], x, m, out, kind) == 0;
+                if (inner && hipEventRecord(ev[r + 1], cap) != hipSuccess) inner = false;
+            }
+            if (!inner) (void)hipGetLastError();
             hipError_t e = hipStreamEndCapture(cap, &graph);
             ok = ok && check_hip(e, "hipStreamEndCapture") == 0;
             ok = ok && check_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate") == 0;
-            // one untimed replay (uploads the graph), then the timed one
-            ok = ok && check_hip(hipGraphLaunch(exec, cap), "hipGraphLaunch") == 0;
+            ok = ok && check_hip(hipGraphLaunch(exec, cap), "hipGraphLaunch") == 0;          // uploads the graph
             ok = ok && check_hip(hipStreamSynchronize(cap), "hipStreamSynchronize") == 0;
             ok = ok && skainet_hip_timer_begin() == 0;
             ok = ok && check_hip(hipGraphLaunch(exec, cap), "hipGraphLaunch") == 0;
-            if (ok) ms = skainet_hip_timer_end_ms();
+            float whole = ok ? skainet_hip_timer_end_ms() : -1.f;
+            ok = ok && whole >= 0.f;
+            for (int r = 0; ok && inner && r < replays; ++r)
+                if (hipEventElapsedTime(&samples[r], ev[r], ev[r + 1]) != hipSuccess || samples[r] <= 0.f) { (void)hipGetLastError(); inner = false; }
+            if (ok) ms = inner ? median(replays) : whole * (float)iters / (float)(400 + replays * iters);   // no event nodes: the whole chain's mean
+            for (int r = 0; r <= replays; ++r) if (ev[r]) (void)hipEventDestroy(ev[r]);
         }
     } else {
-        ok = skainet_hip_timer_begin() == 0;
-        for (int i = 0; ok && i < iters; ++i) ok = skainet_hip_matmul_kind_dev(weights[i % nweights], x, m, out, kind) == 0;
-        if (ok) ms = skainet_hip_timer_end_ms();
+        for (int r = 0; ok && r < replays; ++r) {
+            ok = skainet_hip_timer_begin() == 0;
+            for (int i = 0; ok && i < iters; ++i) ok = skainet_hip_matmul_kind_dev(weights[i % nweights], x, m, out, kind) == 0;
+            if (ok) { samples[r] = skainet_hip_timer_end_ms(); ok = samples[r] >= 0.f; }
+        }
+        if (ok) ms = median(replays);
     }
     if (exec) (void)hipGraphExecDestroy(exec);
     if (graph) (void)hipGraphDestroy(graph);

@@ -184,10 +184,11 @@ class DeviceWeight:
             pass
 
 
-def matmul_repeat(weights, x, m: int, out, iters: int, kind: int = 0, use_graph: bool = True) -> float:
-    """Time `iters` back-to-back products rotating over `weights` (DeviceWeight list); returns milliseconds."""
+def matmul_repeat(weights, x, m: int, out, iters: int, kind: int = 0, use_graph: bool = True, replays: int = 1) -> float:
+    """Time `iters` back-to-back products rotating over `weights` (DeviceWeight list); returns the milliseconds of one
+    pass (the median of `replays` timed passes)."""
     arr = (C.c_void_p * len(weights))(*[w._h for w in weights])
-    ms = _lib.hip().skainet_hip_matmul_repeat_dev(arr, len(weights), _ptr(x), m, _ptr(out), iters, kind, int(use_graph))
+    ms = _lib.hip().skainet_hip_matmul_repeat_dev(arr, len(weights), _ptr(x), m, _ptr(out), iters, kind, int(use_graph), replays)
     if ms < 0:
         raise HipError("matmul_repeat: " + _lib.last_error())
     return ms
@@ -202,6 +203,11 @@ def read_probe(buffers, nbytes: int, iters: int, grid: int = 0) -> float:
     if ms < 0:
         raise HipError("read_probe: " + _lib.last_error())
     return ms
+
+
+def last_kernel() -> str:
+    """Kernel family the calling thread's last matmul / attention entry launched as its main kernel."""
+    return _lib.hip().skainet_hip_last_kernel().decode()
 
 
 def set_tuning(key: str, value: int) -> None:
