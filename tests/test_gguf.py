@@ -1,6 +1,7 @@
 """GGUF reader / writer (host logic, no GPU): the file format of the reference's StreamingGGUFReader -- header, metadata
 value types, tensor infos with aligned relative offsets, block geometry -- checked by round trips through the writer,
 by hand-built byte strings, and by the reader's error behaviour on damaged files."""
+import os
 import struct
 
 import numpy as np
@@ -109,3 +110,39 @@ def test_damaged_files_are_rejected(tmp_path):
     w = gguf.GGUFWriter()
     with pytest.raises(gguf.GGUFError):
         w.add_tensor("bad", "Q4_K", (2, 256), np.zeros(100, np.uint8))   # byte count does not match the shape
+
+
+FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "test_experiment.gguf")
+
+
+def test_reference_fixture_parses_as_the_reference_reader_asserts():
+    """The 512-byte file the reference's own reader tests run on
+    (/root/reference/skainet-io/skainet-io-gguf/src/jvmTest/resources/test_experiment.gguf, kept here as a data fixture),
+    with the assertions of StreamingGGUFReaderTest.kt:39-185: version, tensor count, names, shapes, types, offsets at or
+    behind the data section, positive sizes, every tensor loadable at its full size, two loads of a tensor identical,
+    a load into a larger buffer at an offset leaves the prefix alone."""
+    assert os.path.getsize(FIXTURE) == 512
+    with gguf.GGUFReader(FIXTURE) as r:
+        assert r.version == 3 and r.version > 0
+        assert len(r.tensors) == 3 == len(r.names())
+        assert sorted(r.names()) == ["result", "x", "y"]
+        assert r.fields["general.architecture"] == "llama"
+        assert r.fields["general.name"] == "addition_op" and r.fields["general.description"] == "Simple addition"
+        assert r.data_offset > 0 and r.data_offset % r.alignment == 0
+        expected_offsets = {"x": 320, "y": 384, "result": 448}
+        for t in r.tensors:
+            assert t.shape == (3, 3) and t.type_name == "F32" and t.type_id == 0
+            assert t.offset >= r.data_offset and t.offset == expected_offsets[t.name]
+            assert t.n_bytes == 36 > 0 and t.n_elements == 9
+            data = np.array(r.tensor_bytes(t.name))
+            assert data.size == t.n_bytes
+            assert np.array_equal(data, np.array(r.tensor_bytes(t.name)))          # loading twice gives the same bytes
+            buf = np.zeros(t.n_bytes + 100, np.uint8)
+            buf[10:10 + t.n_bytes] = r.tensor_bytes(t.name)
+            assert not buf[:10].any() and np.array_equal(buf[10:10 + t.n_bytes], data) and not buf[10 + t.n_bytes:].any()
+        # the file is a recorded addition: result = x + y, which pins the element order and the float decoding
+        x, y, res = r.tensor_f32("x"), r.tensor_f32("y"), r.tensor_f32("result")
+        assert x.shape == (3, 3) and np.isfinite(res).all()
+        assert np.allclose(x + y, res, rtol=0, atol=1e-6)
+        with pytest.raises(gguf.GGUFError):
+            r.upload("x")                                                          # dense F32 is not a packed matmul weight
