@@ -172,6 +172,8 @@ DECODER_WORKLOADS = {
     # a quarter-depth stack for quick runs; same per-layer shapes
     "llama3_8b_8layers_decode": ({"layers": 8}, 512, 1),
 }
+# The same stack driven through host arrays only (the unchanged kernel SPI): see measure_decoder_spi.
+SPI_DECODER_WORKLOADS = {"llama3_8b_decode_spi": "llama3_8b_decode", "llama3_8b_8layers_decode_spi": "llama3_8b_8layers_decode"}
 
 
 def cpu_baseline_decode(cfg, host, ctx):
@@ -433,7 +435,83 @@ def measure_decoder(workload, steps, warmup, no_graph, skip_cpu):
     return rec, ok
 
 
+def measure_decoder_spi(workload, steps, warmup):
+    """The decode step of `measure_decoder` with every operand a host array: each linear is one call of the library's
+    host-array product (upload, launch, download, wait), attention and the norms go through the SPI's host kernels, the
+    rest runs in numpy. The prompt is prefilled by the resident decoder and its KV cache handed over, so the timed
+    steps run at the same context. A step = one decoded token, timed on the host clock (every call ends in a wait)."""
+    from dataclasses import replace
+    from skainet_amd import _lib, kernels
+    from skainet_amd.decoder import LLAMA3_8B, LlamaDecoder, LlamaWeights
+    from skainet_amd.spi_decoder import SpiDecoder
+    overrides, prompt_len, distinct = DECODER_WORKLOADS[SPI_DECODER_WORKLOADS[workload]]
+    cfg = replace(LLAMA3_8B, **overrides)
+    w = LlamaWeights(cfg, seed=20251125, distinct_layers=distinct)
+    dec = LlamaDecoder(w, max_prefill=prompt_len)
+    prompt = np.random.default_rng(7).integers(0, cfg.vocab, prompt_len)
+    first = dec.prefill(prompt)
+    spi = SpiDecoder(w)
+    shape = (cfg.layers, cfg.kv_heads, cfg.ctx_max, cfg.head_dim)
+    spi.k_cache[...] = dec.k_cache.download(np.float32, int(np.prod(shape))).reshape(shape)
+    spi.v_cache[...] = dec.v_cache.download(np.float32, int(np.prod(shape))).reshape(shape)
+    spi.pos, spi.token = prompt_len, first
+    # parity of the timed route: same token in, logits within the fp32 bar of the resident decoder's
+    resident_next = int(dec.decode(1, use_graph=False)[0])
+    spi.step(first)
+    ref = dec.last_logits().astype(np.float64)
+    err = float(np.abs(spi.logits[0] - ref).max() / np.abs(ref).max())
+    ok = err < 1e-3 and bool(np.isfinite(spi.logits).all())
+    spi.token = resident_next
+    for _ in range(max(0, warmup - 1)):
+        spi.step(spi.token)
+    spi.matmul_seconds, spi.attention_seconds, spi.matmul_calls, spi.calls = 0.0, 0.0, 0, 0
+    pos0 = spi.pos
+    t0 = time.perf_counter()
+    spi.decode(steps)
+    wall = time.perf_counter() - t0
+    ms_per_tok = wall * 1e3 / steps
+    # the resident decoder at the same context, for the comparison
+    dec.decode(max(1, warmup), use_graph=True)
+    with kernels.Timer() as tm:
+        for _ in range(64):
+            dec._graph.launch()
+    resident_ms = tm.ms / 64
+    linears = 4 * cfg.layers + 1
+    us_call = spi.matmul_seconds / spi.matmul_calls * 1e6
+    alg = w.decode_bytes_per_token(pos0 + steps // 2)
+    gbs = alg / (ms_per_tok * 1e-3) / 1e9
+    rec = {
+        "metric": "decode tok/s", "value": round(1e3 / ms_per_tok, 2), "unit": "tok/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(ms_per_tok, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 (packed Q4_K / Q6_K weights)", "data": "synthetic",
+        "config": {"workload": workload, "layers": cfg.layers, "hidden": cfg.hidden, "heads": cfg.heads,
+                   "kv_heads": cfg.kv_heads, "head_dim": cfg.head_dim, "ffn": cfg.ffn, "vocab": cfg.vocab, "batch": 1,
+                   "prompt_tokens": prompt_len, "decoded_tokens": steps, "context_at_end": pos0 + steps,
+                   "route": "kernel SPI with host arrays: weights resident, activations / KV cache / results on the host; "
+                            "driven from Python over ctypes"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "extra": {"boundary_calls_per_token": spi.calls // steps, "linear_calls_per_token": linears,
+                  "us_per_linear_call": round(us_call, 2),
+                  "ms_per_token_in_linears": round(spi.matmul_seconds * 1e3 / steps, 4),
+                  "ms_per_token_in_attention_calls": round(spi.attention_seconds * 1e3 / steps, 4),
+                  "resident_ms_per_token_same_context": round(resident_ms, 5),
+                  "us_per_linear_resident_upper_bound": round(resident_ms * 1e3 / linears, 2),
+                  "host_overhead_us_per_linear": round(us_call - resident_ms * 1e3 / linears, 2),
+                  "logits_err_vs_resident": err, "device": _lib.hip().skainet_hip_device_name().decode()},
+    }
+    if not ok:
+        rec["extra"]["PARITY_FAILED"] = True
+    spi.close()
+    dec.close()
+    return rec, ok
+
+
 def bench_decoder(a):
+    if a.workload in SPI_DECODER_WORKLOADS:
+        rec, ok = measure_decoder_spi(a.workload, 32 if a.steps == 2000 else a.steps, 4 if a.warmup == 200 else a.warmup)
+        print(json.dumps(rec).replace("NaN", "null"))
+        sys.exit(0 if ok else 1)
     steps = 128 if a.steps == 2000 else a.steps
     warmup = 8 if a.warmup == 200 else a.warmup
     rec, ok = measure_decoder(a.workload, steps, warmup, a.no_graph, a.skip_cpu)
@@ -446,7 +524,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000, help="timed steps (default 2000; 200 for the GEMM workloads)")
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS))
+    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(SPI_DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
     ap.add_argument("--hbm-only", action="store_true", help="skip the cache-warm pass and the read probe, so every launch of the "
@@ -468,7 +546,7 @@ def main():
         key, _, val = kv.partition("=")
         _lib.check(_lib.hip().skainet_hip_set_tuning(key.encode(), int(val)), "set_tuning")
 
-    if a.workload in DECODER_WORKLOADS:
+    if a.workload in DECODER_WORKLOADS or a.workload in SPI_DECODER_WORKLOADS:
         bench_decoder(a)
     if a.workload in ATTENTION_WORKLOADS:
         bench_attention(a)

@@ -117,6 +117,12 @@ SKAINET_HIP_API int64_t skainet_hip_weight_nbytes(const skainet_hip_weight* w);
  * (within 2e-2 of the largest output): the switch at m = 9 is a switch of precision class as well as of kernel, and
  * skainet_hip_matmul_kind_dev pins either one. */
 SKAINET_HIP_API int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out);
+/* The same product for the SPI's own calling convention: `x_host` [m, cols] and `out_host` [m, rows] are ordinary
+ * host arrays (what MatmulKernels.kt:11-40 hands a ViewKernel), the weight is the resident handle. One upload, the
+ * product, one download and one wait per call; the page-locked staging and the device buffers belong to the calling
+ * thread and are reused, so a call allocates nothing after the thread's largest shape has been seen. This is the entry
+ * HipRowMajorMatmulKernel.run binds. */
+SKAINET_HIP_API int32_t skainet_hip_matmul_host(const skainet_hip_weight* w, const float* x_host, int32_t m, float* out_host);
 /* Same product, forcing one of the two kernels (kind 0 = GEMV path, 1 = MFMA GEMM path). */
 SKAINET_HIP_API int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out, int32_t kind);
 /* out = epilogue(W . prologue(x)): a product with the row ops a decoder block puts around it folded in (no reference

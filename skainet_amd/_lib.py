@@ -42,6 +42,7 @@ SIGNATURES = {
     "skainet_hip_weight_data": (_vp, [_vp]),
     "skainet_hip_weight_nbytes": (_i64, [_vp]),
     "skainet_hip_matmul_dev": (_i32, [_vp, _vp, _i32, _vp]),
+    "skainet_hip_matmul_host": (_i32, [_vp, _vp, _i32, _vp]),
     "skainet_hip_matmul_kind_dev": (_i32, [_vp, _vp, _i32, _vp, _i32]),
     "skainet_hip_matmul_fused_dev": (_i32, [_vp, _vp, _i32, _vp, _vp, _f32, _vp, _i32]),
     "skainet_hip_matmul_qkv_rope_dev": (_i32, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _vp]),

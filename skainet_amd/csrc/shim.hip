@@ -62,6 +62,7 @@ struct Scratch { void* ptr = nullptr; size_t cap = 0; };
 static thread_local Scratch t_workspace;          // kernel scratch (attention split-K partials, GEMM staging)
 static thread_local Scratch t_stage[6];           // device staging of the host-pointer entries
 static thread_local Scratch t_fuse[2];            // normalised input / raw product of the unfused route of matmul_fused
+static thread_local Scratch t_pinned[2];          // page-locked host staging of skainet_hip_matmul_host (activations in, product out)
 
 static std::mutex g_mutex;
 static int g_state = 0;        // 0 = not probed, 1 = usable, -1 = unusable
@@ -144,6 +145,16 @@ static void* scratch_get(Scratch& s, size_t bytes) {
     s.ptr = p; s.cap = cap;
     return p;
 }
+// Page-locked host memory, grown on demand (allocated, never registered: existing host memory cannot be pinned here).
+static void* pinned_get(Scratch& s, size_t bytes) {
+    if (bytes <= s.cap) return s.ptr;
+    if (s.ptr) { (void)hipStreamSynchronize(t_stream); (void)hipHostFree(s.ptr); s.ptr = nullptr; s.cap = 0; }
+    const size_t cap = (bytes + (1u << 16) - 1) & ~((size_t)(1u << 16) - 1);
+    void* p = nullptr;
+    if (check_hip(hipHostMalloc(&p, cap, hipHostMallocDefault), "hipHostMalloc(staging)") != 0) return nullptr;
+    s.ptr = p; s.cap = cap;
+    return p;
+}
 // Persistent, zero-initialised device memory for cross-workgroup counters (a kernel that uses one leaves it at zero).
 // One allocation per host thread, made on first use and never moved, so recorded graphs keep a valid address.
 constexpr size_t SYNC_SCRATCH_BYTES = 1u << 20;
@@ -214,6 +225,10 @@ int32_t skainet_hip_thread_release(void) {
     drop(t_workspace);
     for (Scratch& sc : t_stage) drop(sc);
     for (Scratch& sc : t_fuse) drop(sc);
+    for (Scratch& sc : t_pinned) {
+        if (sc.ptr && check_hip(hipHostFree(sc.ptr), "hipHostFree(staging)") != 0) rc = -1;
+        sc.ptr = nullptr; sc.cap = 0;
+    }
     if (t_sync && check_hip(hipFree(t_sync), "hipFree(sync scratch)") != 0) rc = -1;
     t_sync = nullptr;
     if (t_ev0 && check_hip(hipEventDestroy(t_ev0), "hipEventDestroy") != 0) rc = -1;
@@ -332,6 +347,29 @@ int32_t skainet_hip_matmul_kind_dev(const skainet_hip_weight* w, const float* x,
 }
 int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out) {
     return skainet_hip_matmul_kind_dev(w, x, m, out, m <= 8 ? 0 : 1);
+}
+// The view-kernel route of the SPI on a resident weight: activations and result live in host memory, the weight stays
+// on the device. One call = copy the rows into page-locked staging, one asynchronous upload, the product, one
+// asynchronous download, one wait; every buffer belongs to the calling thread and is reused, so a call allocates
+// nothing once the thread has seen its largest shape.
+int32_t skainet_hip_matmul_host(const skainet_hip_weight* w, const float* x_host, int32_t m, float* out_host) {
+    if (ensure_device() != 0) return -1;
+    if (!w) return set_error("matmul_host: null weight handle");
+    if (m <= 0) return 0;
+    if (!x_host || !out_host) return set_error("matmul_host: null activation or output pointer");
+    const size_t in_bytes = sizeof(float) * (size_t)m * w->cols, out_bytes = sizeof(float) * (size_t)m * w->rows;
+    void* pin_in = pinned_get(t_pinned[0], in_bytes);
+    void* pin_out = pinned_get(t_pinned[1], out_bytes);
+    float* xd = static_cast<float*>(scratch_get(t_stage[1], in_bytes));
+    float* yd = static_cast<float*>(scratch_get(t_stage[2], out_bytes));
+    if (!pin_in || !pin_out || !xd || !yd) return -1;
+    memcpy(pin_in, x_host, in_bytes);
+    if (check_hip(hipMemcpyAsync(xd, pin_in, in_bytes, hipMemcpyHostToDevice, t_stream), "hipMemcpy h2d") != 0) return -1;
+    if (skainet_hip_matmul_dev(w, xd, m, yd) != 0) return -1;
+    if (check_hip(hipMemcpyAsync(pin_out, yd, out_bytes, hipMemcpyDeviceToHost, t_stream), "hipMemcpy d2h") != 0) return -1;
+    if (check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize") != 0) return -1;
+    memcpy(out_host, pin_out, out_bytes);
+    return 0;
 }
 // out = epilogue(W . prologue(x)), the products of a decoder block with their neighbouring row ops folded in:
 //   gain != NULL: x is RMS-normalised first (x / sqrt(mean(x^2) + eps) * gain, per activation row);

@@ -154,6 +154,14 @@ class DeviceWeight:
         else:
             check(_lib.hip().skainet_hip_matmul_kind_dev(self._h, _ptr(x), m, _ptr(out), kind), "matmul")
 
+    def matmul_host(self, a: np.ndarray, out: np.ndarray) -> None:
+        """out[m, rows] = a[m, cols] . W^T with host arrays on both sides (skainet_hip_matmul_host): one upload, one
+        launch chain, one download, one wait, all on buffers the calling thread re-uses."""
+        a, out = _f32(a, "a"), _f32(out, "out")
+        if a.ndim != 2 or a.shape[1] != self.cols or out.shape != (a.shape[0], self.rows):
+            raise ValueError(f"matmul_host: a {a.shape} x W [{self.rows}, {self.cols}] -> out {out.shape} do not fit")
+        check(_lib.hip().skainet_hip_matmul_host(self._h, a.ctypes.data, a.shape[0], out.ctypes.data), "matmul_host")
+
     def matmul_fused(self, x, m: int, out, gain=None, eps: float = 0.0, residual=None, epilogue: int = 0) -> None:
         """out = epilogue(W . rmsnorm(x) if gain is given else W . x); epilogue EPI_NONE / EPI_RESIDUAL / EPI_SWIGLU."""
         check(_lib.hip().skainet_hip_matmul_fused_dev(self._h, _ptr(x), m, _ptr(out), _ptr(gain), eps, _ptr(residual), epilogue),
@@ -532,21 +540,11 @@ class HipRowMajorMatmulKernel:
             return w
 
     def run(self, a: np.ndarray, w: np.ndarray, n: int, out: np.ndarray) -> None:
+        """One call of the library's host-array entry: the activation rows go up, the product comes down, the weight
+        stays where it is. Nothing is allocated per call."""
         _require_available()
         rows, k = a.shape
-        dw = self._resident(w, n, k)
-        lib = _lib.hip()
-        nbytes_a, nbytes_o = a.size * 4, rows * n * 4
-        da, do = lib.skainet_hip_malloc(nbytes_a), lib.skainet_hip_malloc(nbytes_o)
-        try:
-            if not da or not do:
-                raise HipError("malloc: " + _lib.last_error())
-            check(lib.skainet_hip_memcpy_h2d(da, _f32(a, "a").ctypes.data, nbytes_a), "h2d")
-            dw.matmul(da, rows, do)
-            check(lib.skainet_hip_memcpy_d2h(_f32(out, "out").ctypes.data, do, nbytes_o), "d2h")
-        finally:
-            lib.skainet_hip_free(da)
-            lib.skainet_hip_free(do)
+        self._resident(w, n, k).matmul_host(a, out)
 
 
 class HipKernelProvider:

@@ -563,3 +563,59 @@ def test_decoder_over_the_other_packed_formats(hip_backend, linear, head, tmp_pa
     assert w2.cfg.linear_encoding == linear and w2.cfg.head_encoding == head
     for name, a in w.host.items():
         assert np.array_equal(np.asarray(a), np.asarray(w2.host[name])), name
+
+
+# ---- the host-array route of the kernel SPI -------------------------------------------------------------------------
+@pytest.mark.parametrize("enc,n,k", [("Q4_K", 1536, 1024), ("Q4_K", 260, 512), ("Q6_K", 130, 768), ("Q8_0", 96, 64)])
+def test_host_array_product_equals_the_device_entry(hip_backend, torch_cuda, enc, n, k):
+    """skainet_hip_matmul_host against skainet_hip_matmul_dev on the same handle, bit for bit: a large call, a smaller
+    one on the re-used staging, then a batch that crosses into the GEMM path; padding around the host output stays."""
+    from oracle import golden as G
+    torch = torch_cuda
+    blocks = G.weight_blocks(enc, n, k // G.PACKED[enc][0], 0xC0FFEE)
+    w = hip_backend.DeviceWeight.upload(enc, G.row_major(blocks), n, k)
+    for m in (5, 1, 12):
+        a = G.floats(m * k, 0x1234 + m).reshape(m, k)
+        padded = np.full(m * n + 8, 7, np.float32)
+        out = padded[4:4 + m * n].reshape(m, n)
+        w.matmul_host(a, out)
+        want = torch.empty(m, n, device="cuda:0", dtype=torch.float32)
+        w.matmul(dev(torch, a), m, want)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.view(np.uint32), want.cpu().numpy().view(np.uint32)), f"m={m}"
+        assert (padded[:4] == 7).all() and (padded[-4:] == 7).all()
+    with pytest.raises(ValueError):
+        w.matmul_host(np.zeros((2, k + 1), np.float32), np.zeros((2, n), np.float32))
+    with pytest.raises(TypeError):
+        w.matmul_host(np.zeros((2, k), np.float64), np.zeros((2, n), np.float32))
+    w.matmul_host(np.zeros((0, k), np.float32), np.zeros((0, n), np.float32))      # nothing to do is not an error
+    w.close()
+
+
+def test_spi_route_decoder_follows_the_resident_decoder(small_model):
+    """The decoder written against host arrays only (every linear through the host-array entry, attention and norms
+    through the SPI's host kernels, the rest in numpy) produces the resident decoder's logits within the fp32 bar on a
+    shared token history, and the checker's."""
+    from skainet_amd.decoder import LlamaDecoder
+    from skainet_amd.spi_decoder import SpiDecoder
+    cfg, w = small_model
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 6)
+    dec = LlamaDecoder(w, max_prefill=8)
+    spi = SpiDecoder(w)
+    chk = CheckDecoder(cfg, w.host)
+    tok = dec.prefill(prompt)
+    spi.prefill(prompt)
+    _, logits_ref = chk.forward(prompt)
+    for i in range(8):
+        assert max_norm_err(spi.logits[0], logits_ref) < 1e-3, f"step {i}"
+        assert max_norm_err(spi.logits[0], dec.last_logits()) < 1e-3, f"step {i}"
+        assert spi.pos == dec.position()
+        nxt = int(dec.decode(1, use_graph=False)[0])
+        spi.step(tok)                      # teacher-forced on the resident decoder's token
+        _, logits_ref = chk.forward([tok])
+        tok = nxt
+    per_token = 4 * cfg.layers + 1
+    assert spi.matmul_calls == per_token * (len(prompt) + 8)
+    with pytest.raises(ValueError):
+        spi.step(cfg.vocab)
+    spi.close()
