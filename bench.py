@@ -45,6 +45,11 @@ WORKLOADS = {
     "q6k_gemv_32000x4096_b1": ("Q6_K", 32000, 4096, 1),
     # the decoder's down projection: long rows, K split over the waves of a workgroup
     "q4k_gemv_4096x14336_b1": ("Q4_K", 4096, 14336, 1),
+    # the other products of a Llama-3-8B decode step: fused gate/up, fused q/k/v, attention output, the Q6_K head
+    "q4k_gemv_28672x4096_b1": ("Q4_K", 28672, 4096, 1),
+    "q4k_gemv_6144x4096_b1": ("Q4_K", 6144, 4096, 1),
+    "q4k_gemv_4096x4096_b1": ("Q4_K", 4096, 4096, 1),
+    "q6k_gemv_128256x4096_b1": ("Q6_K", 128256, 4096, 1),
     # the remaining packed formats of the provider SPI, at the headline shape
     "q4_0_gemv_11008x4096_b1": ("Q4_0", 11008, 4096, 1),
     "q5_0_gemv_11008x4096_b1": ("Q5_0", 11008, 4096, 1),
@@ -218,6 +223,7 @@ def cpu_baseline_decode(cfg, host, ctx):
 ATTENTION_WORKLOADS = {
     # name -> (batch, seq_q, seq_kv); 32 query heads, 8 KV heads, head_dim 128, fp32, scale 1/sqrt(128), causal
     "sdpa_prefill_2048": (1, 2048, 2048),
+    "sdpa_decode_576_b1": (1, 1, 576),
     "sdpa_decode_4096_b1": (1, 1, 4096),
     "sdpa_decode_4096_b8": (8, 1, 4096),
 }
@@ -375,12 +381,7 @@ def measure_decoder(workload, steps, warmup, no_graph, skip_cpu):
 
     def timed_steps(count):
         with kernels.Timer() as tm:          # HIP events on the launch stream around exactly `count` decode steps
-            if no_graph:
-                for _ in range(count):
-                    dec._decode_step()
-            else:
-                for _ in range(count):
-                    dec._graph.launch()
+            dec.run_steps(count, use_graph=not no_graph)
         return tm.ms
 
     t0 = time.perf_counter()
@@ -473,8 +474,7 @@ def measure_decoder_spi(workload, steps, warmup):
     # the resident decoder at the same context, for the comparison
     dec.decode(max(1, warmup), use_graph=True)
     with kernels.Timer() as tm:
-        for _ in range(64):
-            dec._graph.launch()
+        dec.run_steps(64)
     resident_ms = tm.ms / 64
     linears = 4 * cfg.layers + 1
     us_call = spi.matmul_seconds / spi.matmul_calls * 1e6

@@ -265,6 +265,18 @@ SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_dev(const float* q, const float* k,
 SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_cache_dev(const float* q, const float* k_cache, const float* v_cache, float* out,
     int32_t batch, int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t kv_capacity, int32_t head_dim,
     float scale, int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths);
+/* One decode token's attention over the KV cache and the output projection behind it:
+ *   out[rows of wo] = (residual ? residual : 0) + Wo . sdpa(q [heads, head_dim], cache [kv_heads, kv_capacity, head_dim]),
+ * causal over seq_kv keys (or lengths[0] of them when `lengths` is given: a device-side key count, so a recorded graph
+ * follows the cache as it grows), `window` as in skainet_hip_f32_sdpa_dev. No reference counterpart as one call: the
+ * parts are f32_fused.c:290-396 (attention), the packed product and a binary add. For a Q4_K projection of at most 4096
+ * inputs and up to "attn_merge_splits" x "attn_merge_max_keys" keys (6 x 176) the attention kernel leaves its key splits unmerged and the projection
+ * merges them while it loads its activations (two launches instead of four); other shapes run attention into
+ * `attn_tmp` [heads * head_dim] and the fused product. `residual` may alias `out`. */
+SKAINET_HIP_API int32_t skainet_hip_attn_out_proj_dev(const skainet_hip_weight* wo, const float* q, const float* k_cache,
+                                                      const float* v_cache, int32_t heads, int32_t kv_heads, int32_t head_dim,
+                                                      int32_t seq_kv, int32_t kv_capacity, float scale, int32_t window,
+                                                      const int32_t* lengths, const float* residual, float* out, float* attn_tmp);
 
 /* Decoder glue with the reference ops' semantics (device pointers):
  *   silu_mul: out[i] = gate[i] * (1 / (1 + exp(-gate[i]))) * up[i]   (NAT:532-539 unary op 2 then binary mul,
@@ -343,7 +355,9 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * 0 = chosen from K), "gemm_ksplit" (K splits of the MFMA GEMM,
  * 0 = automatic), "gemm_wide" (1 / 0: force the 256 x 256 / 256 x 128 tile, -1 = chosen from the shape),
  * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_decode_split_keys" (least keys per split of
- * decode-shape attention, default 64).
+ * decode-shape attention, default 64), "attn_merge_enable" (0: skainet_hip_attn_out_proj_dev always merges the key
+ * splits in a launch of its own), "attn_merge_max_keys" (most keys per split for which that entry leaves the merge to
+ * the projection, default 176), "attn_merge_splits" (most key splits it then uses, 1 to 8, default 6).
  * 0 when the key is known. No reference counterpart. */
 SKAINET_HIP_API int32_t skainet_hip_set_tuning(const char* key, int32_t value);
 

@@ -572,6 +572,9 @@ void set_sdpa_decode_split_keys(int v);
 void set_q4k_ksplit_enable(int v);
 void set_q4k_mfma_enable(int v);
 void set_q4k_mfma_window(int v);
+void set_attn_merge_enable(int v);
+void set_attn_merge_max_keys(int v);
+void set_attn_merge_splits(int v);
 int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch);   // gemv_q4k.hip
 int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int n, int batch);  // gemv_q4k_quads.hip
 
@@ -588,6 +591,9 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q4k_mfma_enable")) { set_q4k_mfma_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_window")) { set_q4k_mfma_window(value); return 0; }
     if (!strcmp(key, "sdpa_decode_split_keys")) { set_sdpa_decode_split_keys(value); return 0; }
+    if (!strcmp(key, "attn_merge_enable")) { set_attn_merge_enable(value); return 0; }
+    if (!strcmp(key, "attn_merge_max_keys")) { set_attn_merge_max_keys(value); return 0; }
+    if (!strcmp(key, "attn_merge_splits")) { set_attn_merge_splits(value); return 0; }
     return -1;
 }
 

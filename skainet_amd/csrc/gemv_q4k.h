@@ -22,6 +22,13 @@ struct RopeQkvEpilogue {
     int heads, kv_heads, head_dim, capacity;
 };
 
+// Activations handed over as the unmerged per-split results of a one-query attention: the consumer forms
+//   x[h * head_dim + d] = sum_s c[h][s] * part[(h * splits + s) * head_dim + d],
+//   c[h][s] = 2^(m[h][s] - max_s m) / sum_s 2^(m[h][s] - max_s m) * l[h][s]   (0 where that sum is 0),
+// (m, l) = ml[(h * splits + s) * 2 ..]: the running maximum in units of ln 2 and the sum of a split's softmax weights.
+constexpr int ATTN_MERGE_MAX_SPLITS = 8;
+struct AttnMergePrologue { const float* part; const float* ml; int splits; int head_dim; };
+
 // d * sc and dmin * m of the two sub-blocks (2g, 2g + 1) a lane owns. ggml get_scale_min_k4: both packings are
 // evaluated and picked with a lane-constant mask (g < 2: bytes j and j + 4; g >= 2: the split 4 + 2 bit form).
 __device__ __forceinline__ void q4k_lane_scales(const uint4& hdr, int sh, uint32_t hi_mask, float& dlo, float& dhi,

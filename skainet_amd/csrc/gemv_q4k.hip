@@ -30,7 +30,8 @@
 namespace skh {
 
 int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n, const float* gain, float eps,
-                         const float* residual, int epilogue, const RopeQkvEpilogue* rope_in);   // gemv_q4k_mfma.hip
+                         const float* residual, int epilogue, const RopeQkvEpilogue* rope_in,
+                         const AttnMergePrologue* merge);   // gemv_q4k_mfma.hip
 
 // One row's 64 weights of a lane against its 64 activations. The 4-bit codes are never converted: a dword of codes is
 // masked into pairs of 16-bit fields whose low mantissa bits hold a code (0x000F000F: the low nibbles of bytes 0 and 2;
@@ -426,7 +427,7 @@ int launch_q4k_gemv_rows_fused(const uint8_t* w, const float* x, float* y, int k
     if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return 0;
     if (batch == 1) {
         // one activation row with K in whole slices of 1024: the matrix-core kernel with consecutive-kilobyte loads
-        const int r = launch_q4k_gemv_mfma(w, x, y, k, n, gain, eps, residual, epilogue, epilogue == EPI_ROPE_QKV ? &rope : nullptr);
+        const int r = launch_q4k_gemv_mfma(w, x, y, k, n, gain, eps, residual, epilogue, epilogue == EPI_ROPE_QKV ? &rope : nullptr, nullptr);
         if (r != 0) return r;
     }
     if (g_q4k_ksplit_enable && batch == 1 && !gain && epilogue <= EPI_RESIDUAL && k >= 8192) {

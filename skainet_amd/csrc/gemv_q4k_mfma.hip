@@ -39,11 +39,11 @@ namespace skh {
 
 typedef uint32_t u32x4_m __attribute__((ext_vector_type(4)));
 typedef int i32x4_m __attribute__((ext_vector_type(4)));
+typedef float f32x2_m __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ void mfma_plain_load16(u32x4_m& dst, uint32_t off, const void* base) {
     asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
 }
-typedef float f32x2_m __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void mfma_plain_load8(f32x2_m& dst, uint32_t off, const void* base) {
     asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
 }
@@ -55,7 +55,7 @@ __device__ __forceinline__ void mfma_stream_to_lds(uint32_t lds_addr, uint32_t o
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(off), "s"(base) : "memory");
 }
 template <int N> __device__ __forceinline__ void mfma_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-template <int N> __device__ __forceinline__ void mfma_wait_loads(u32x4_m& v) { asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory"); }
+template <int N, typename T> __device__ __forceinline__ void mfma_wait_loads(T& v) { asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory"); }
 __device__ __forceinline__ void mfma_wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 template <int I, int N, typename F> __device__ __forceinline__ void mfma_static_for(F&& f) {
@@ -76,34 +76,61 @@ __device__ __forceinline__ void q4k_lane_scales_sel(const uint4& hdr, uint32_t s
 
 constexpr int MFMA_XROW = 20;          // dwords per (group, plane) row of 16 operand dwords, padded against bank conflicts
 constexpr int MFMA_MAX_QUADS = 32;     // row quads per workgroup (bounds the final pass: 8 rounds of 256 threads)
-constexpr int MFMA_XA_BYTES = 16 * 4 * MFMA_XROW * 4 + 16 * 16;   // operand planes of 16 groups + {scale, sums} per group
+constexpr int MFMA_XA_BYTES = 16 * 4 * MFMA_XROW * 4 + 16 * 16 + 16 * ATTN_MERGE_MAX_SPLITS * 4;
+// operand planes of 16 groups + {scale, sums} per group + the merge coefficients of up to 16 heads of a slice
+constexpr int MFMA_XC_OFFSET = 16 * 4 * MFMA_XROW * 4 + 16 * 16;
 
 // One wave's pass: K slices wave, wave + 4, ... (NSW of them), row quads [0, qt) of the workgroup, W quads in flight.
 // Leaves one partial sum per (quad, lane) in `partials` (index: quad * 64 + (lane % 4) * 16 + lane / 4) and, with the
 // RMSNorm prologue, the sum of squares of this wave's activations in *ssq_out.
+// PRO: 0 plain activations, 1 RMSNorm prologue (x * gain, sum of squares), 2 activations = merge of attention partials.
 template <int NSW, int W, int PRO>
 __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, const float* __restrict__ x, const float* __restrict__ gain,
-                                              int n, int r0, int qt, uint32_t row_bytes, int wave, int lane, uint8_t* ring,
-                                              uint8_t* xa_stage, float* partials, float* ssq_out) {
+                                              const AttnMergePrologue& am, int n, int r0, int qt, uint32_t row_bytes, int wave,
+                                              int lane, uint8_t* ring, uint8_t* xa_stage, float* partials, float* ssq_out) {
     constexpr int NPQ = 144 * NSW;                 // 16-byte pieces of a quad in this wave's slices
     constexpr int NLI = (NPQ + 63) / 64;           // wave loads per quad
-    constexpr int NX = NSW * 4 * (1 + PRO);        // activation (and gain) loads
+    constexpr int NX = PRO == 2 ? 2 + 4 * ATTN_MERGE_MAX_SPLITS : NSW * 4 * (1 + PRO);        // activation (and gain) loads
     static_assert(NX + W * NLI <= 63, "loads in flight must fit the wave's counter");
+    static_assert(PRO != 2 || NSW == 1, "the attention-merge prologue serves one slice per wave");
     const int blk = lane >> 2, j = lane & 3, g = blk & 3, h = g & 1;
     const uint32_t sel = g < 2 ? (0x0C0C0000u | ((2 * h + 1) << 8) | (2 * h))
                                : (((2 * h + 1) << 24) | ((2 * h) << 16) | ((4 + 2 * h + 1) << 8) | (4 + 2 * h));
     const uint32_t m1 = g < 2 ? 0x3F3Fu : 0x0F0Fu, sh_min = g < 2 ? 0u : 4u;
 
     // activations (and gains) of this wave's slices first, the first W quads right behind them
-    u32x4_m xq[NSW][4], gq[PRO ? NSW : 1][4];
+    u32x4_m xq[NSW][4], gq[PRO == 1 ? NSW : 1][4];
+    constexpr int MS = PRO == 2 ? ATTN_MERGE_MAX_SPLITS : 1;
+    u32x4_m pq[PRO == 2 ? 4 : 1][MS];              // attention partials of the lane's four float4s, one per split
+    f32x2_m mlq[2];                                // (max, sum) of the (head, split) pair this lane weighs, two rounds of 8 heads
+    if constexpr (PRO == 2) {
+        // lane = (head of the slice, split): 8 heads per round, heads-per-slice = 1024 / head_dim (4, 8 or 16)
+        const int hd_shift = __builtin_ctz(am.head_dim), hps = 1024 >> hd_shift, sp = lane & 7;
 #pragma unroll
-    for (int t = 0; t < NSW; ++t)
+        for (int r = 0; r < 2; ++r) {
+            const int hh = r * 8 + (lane >> 3);
+            mlq[r] = f32x2_m{-INFINITY, 0.f};
+            if (hh < hps && sp < am.splits) mfma_plain_load8(mlq[r], (uint32_t)(((wave * hps + hh) * am.splits + sp) * 2) * 4u, am.ml);
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t off = (uint32_t)((wave + 4 * t) * 1024 + (i * 64 + lane) * 4) * 4u;
-            mfma_plain_load16(xq[t][i], off, x);
-            if (PRO) mfma_plain_load16(gq[t][i], off, gain);
+            const int e = (i * 64 + lane) * 4, hh = e >> hd_shift, d = e - (hh << hd_shift);
+#pragma unroll
+            for (int sI = 0; sI < MS; ++sI) {
+                pq[i][sI] = u32x4_m{0u, 0u, 0u, 0u};
+                if (sI < am.splits) mfma_plain_load16(pq[i][sI], (uint32_t)(((wave * hps + hh) * am.splits + sI) * am.head_dim + d) * 4u, am.part);
+            }
         }
+    } else {
+#pragma unroll
+        for (int t = 0; t < NSW; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t off = (uint32_t)((wave + 4 * t) * 1024 + (i * 64 + lane) * 4) * 4u;
+                mfma_plain_load16(xq[t][i], off, x);
+                if (PRO == 1) mfma_plain_load16(gq[t][i], off, gain);
+            }
+    }
     uint32_t loff[NLI];
 #pragma unroll
     for (int u = 0; u < NLI; ++u) {
@@ -122,11 +149,44 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
     };
 #pragma unroll
     for (int q = 0; q < W; ++q) issue_quad(min(q, qt - 1));
-    mfma_wait_loads<W * NLI>(xq[0][0]);
+    if constexpr (PRO == 2) {
+        mfma_wait_loads<W * NLI>(mlq[0]); mfma_wait_loads<W * NLI>(mlq[1]);
 #pragma unroll
-    for (int t = 0; t < NSW; ++t)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { mfma_wait_loads<W * NLI>(xq[t][i]); if (PRO) mfma_wait_loads<W * NLI>(gq[t][i]); }
+            for (int sI = 0; sI < MS; ++sI) mfma_wait_loads<W * NLI>(pq[i][sI]);
+        // weights of the splits: per head the maximum over its 8 lanes, 2^(m - max), normalised by the weighted sum of l
+        float* xc = reinterpret_cast<float*>(xa_stage + MFMA_XC_OFFSET);
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            float mm = mlq[r].x;
+            mm = fmaxf(mm, __shfl_xor(mm, 1, 64)); mm = fmaxf(mm, __shfl_xor(mm, 2, 64)); mm = fmaxf(mm, __shfl_xor(mm, 4, 64));
+            const float e = __builtin_amdgcn_exp2f(mlq[r].x - mm);
+            const float wgt = mlq[r].x == -INFINITY ? 0.f : e;
+            float ls = wgt * mlq[r].y;
+            ls += __shfl_xor(ls, 1, 64); ls += __shfl_xor(ls, 2, 64); ls += __shfl_xor(ls, 4, 64);
+            xc[r * 64 + lane] = ls > 0.f ? wgt / ls : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int hh = ((i * 64 + lane) * 4) >> __builtin_ctz(am.head_dim);
+            const float4 c0 = *reinterpret_cast<const float4*>(xc + hh * 8), c1 = *reinterpret_cast<const float4*>(xc + hh * 8 + 4);
+            const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int sI = 0; sI < MS; ++sI) {
+                a.x = fmaf(c[sI], __uint_as_float(pq[i][sI].x), a.x); a.y = fmaf(c[sI], __uint_as_float(pq[i][sI].y), a.y);
+                a.z = fmaf(c[sI], __uint_as_float(pq[i][sI].z), a.z); a.w = fmaf(c[sI], __uint_as_float(pq[i][sI].w), a.w);
+            }
+            xq[0][i] = u32x4_m{__float_as_uint(a.x), __float_as_uint(a.y), __float_as_uint(a.z), __float_as_uint(a.w)};
+        }
+    } else {
+        mfma_wait_loads<W * NLI>(xq[0][0]);
+#pragma unroll
+        for (int t = 0; t < NSW; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { mfma_wait_loads<W * NLI>(xq[t][i]); if (PRO == 1) mfma_wait_loads<W * NLI>(gq[t][i]); }
+    }
 
     // activations of a slice: float4 number f = i * 64 + lane belongs to group f / 16 (the 16 lanes of a DPP row share a
     // group); planes go through LDS into operand order
@@ -140,7 +200,7 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float4 v = make_float4(__uint_as_float(xq[t][i].x), __uint_as_float(xq[t][i].y), __uint_as_float(xq[t][i].z), __uint_as_float(xq[t][i].w));
-            if (PRO) {
+            if (PRO == 1) {
                 ssq = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ssq))));
                 v.x *= __uint_as_float(gq[t][i].x); v.y *= __uint_as_float(gq[t][i].y);
                 v.z *= __uint_as_float(gq[t][i].z); v.w *= __uint_as_float(gq[t][i].w);
@@ -171,7 +231,7 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
         const float4 xsv = xs_lds[blk];
         s_grp[t] = xsv.x; xsl[t] = xsv.y; xsh[t] = xsv.z;
     }
-    if (PRO) *ssq_out = wave_sum(ssq);
+    if (PRO == 1) *ssq_out = wave_sum(ssq);
 
     // lane's read offsets inside a quad slot: header of (row j, super-block blk / 4 of the slice), then its two code pieces
     const uint32_t rd_hdr = (uint32_t)(j * 36 + (blk >> 2) * 9) * 16u, rd_q = rd_hdr + 16u + (uint32_t)g * 32u;
@@ -221,9 +281,10 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
 struct MfmaRowPre { float residual; f32x2_m cs; };
 
 template <int W, int PRO>
-__global__ __launch_bounds__(256, 2) void q4k_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x, float* y,
-                                                             int k, int n, int qt, const float* __restrict__ gain, float eps,
-                                                             const float* residual, int epilogue, RopeQkvEpilogue rope) {
+__global__ __launch_bounds__(256, PRO == 2 ? 1 : 2) void q4k_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x, float* y,
+                                                                            int k, int n, int qt, const float* __restrict__ gain, float eps,
+                                                                            const float* residual, int epilogue, RopeQkvEpilogue rope,
+                                                                            AttnMergePrologue am) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nsl = k >> 10;                                   // slices of 1024 elements
@@ -258,18 +319,18 @@ __global__ __launch_bounds__(256, 2) void q4k_gemv_mfma_kernel(const uint8_t* __
 
     float ssq = 0.f;
     switch (nsw) {
-        case 1: q4k_mfma_wave<1, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 2: q4k_mfma_wave<2, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 3: if constexpr (W <= 2) q4k_mfma_wave<3, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 4: if constexpr (W <= 2) q4k_mfma_wave<4, W, PRO>(w, x, gain, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 1: q4k_mfma_wave<1, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 2: if constexpr (PRO != 2) q4k_mfma_wave<2, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 3: if constexpr (W <= 2 && PRO != 2) q4k_mfma_wave<3, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 4: if constexpr (W <= 2 && PRO != 2) q4k_mfma_wave<4, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
         default:                                               // K below 4 slices: this wave has none
             for (int i = lane; i < qt * 64; i += 64) partials[i] = 0.f;
     }
-    if (PRO && lane == 0) ssq_lds[wave] = ssq;
+    if (PRO == 1 && lane == 0) ssq_lds[wave] = ssq;
     __syncthreads();
 
     float xscale = 1.0f;
-    if (PRO) xscale = 1.0f / sqrtf(((ssq_lds[0] + ssq_lds[1]) + (ssq_lds[2] + ssq_lds[3])) * (1.0f / (float)k) + eps);
+    if (PRO == 1) xscale = 1.0f / sqrtf(((ssq_lds[0] + ssq_lds[1]) + (ssq_lds[2] + ssq_lds[3])) * (1.0f / (float)k) + eps);
     const int u = threadIdx.x & 15, pw = u >> 2, pp = u & 3;
 #pragma unroll
     for (int it = 0; it < ROUNDS; ++it) {
@@ -323,15 +384,24 @@ static size_t mfma_smem_bytes(int k, int qt, int window) {
 }
 
 template <int W>
-static int launch_mfma(bool pro, int grid, size_t smem, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int qt,
-                       const float* gain, float eps, const float* residual, int epilogue, const RopeQkvEpilogue& rope) {
+static int launch_mfma(int pro, int grid, size_t smem, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int qt,
+                       const float* gain, float eps, const float* residual, int epilogue, const RopeQkvEpilogue& rope,
+                       const AttnMergePrologue& am) {
     note_kernel("q4k_gemv_mfma_kernel");
-    if (pro) {
+    if (pro == 2) {
+        if constexpr (W == 3) {
+            note_kernel("q4k_gemv_mfma_kernel (attention-merge prologue)");
+            SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<3, 2>), 160 * 1024);
+            q4k_gemv_mfma_kernel<3, 2><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
+        } else {
+            return 0;
+        }
+    } else if (pro == 1) {
         SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, 1>), 160 * 1024);
-        q4k_gemv_mfma_kernel<W, 1><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
+        q4k_gemv_mfma_kernel<W, 1><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
     } else {
         SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, 0>), 160 * 1024);
-        q4k_gemv_mfma_kernel<W, 0><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
+        q4k_gemv_mfma_kernel<W, 0><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
     }
     SKH_CHECK(hipGetLastError());
     return 1;
@@ -341,9 +411,18 @@ static int launch_mfma(bool pro, int grid, size_t smem, hipStream_t s, const uin
 // row-streaming kernel), -1 on a launch error. One activation row; K a multiple of 1024 up to 16384; the weight below
 // 4 GiB (32-bit byte offsets); operands 16-byte aligned.
 int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n, const float* gain, float eps,
-                         const float* residual, int epilogue, const RopeQkvEpilogue* rope_in) {
+                         const float* residual, int epilogue, const RopeQkvEpilogue* rope_in, const AttnMergePrologue* merge) {
     if (!g_q4k_mfma_enable) return 0;
     if (k < 1024 || (k & 1023) || k > 16384 || n < 4) return 0;
+    AttnMergePrologue am{};
+    if (merge) {
+        // the activations are the merge of attention partials: one slice per wave, heads that tile a slice
+        am = *merge;
+        if (gain || k > 4096 || am.splits < 1 || am.splits > ATTN_MERGE_MAX_SPLITS) return 0;
+        if (am.head_dim != 64 && am.head_dim != 128 && am.head_dim != 256) return 0;
+        if ((reinterpret_cast<uintptr_t>(am.part) & 15) || (reinterpret_cast<uintptr_t>(am.ml) & 7)) return 0;
+        x = am.part;
+    }
     const uint64_t wbytes = (uint64_t)n * (uint64_t)(k >> 8) * Q4K_BYTES;
     if (wbytes >= ((uint64_t)1 << 32) || (uint64_t)n * 4 >= ((uint64_t)1 << 32)) return 0;
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return 0;
@@ -363,13 +442,16 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
     if (qt > MFMA_MAX_QUADS) qt = MFMA_MAX_QUADS;
     if (qt < 1) qt = 1;
     const int grid = (quads + qt - 1) / qt;
-    // measured on 11008 x 4096 with two / three / four quads in flight: 7.06 / 6.52 / 6.68 us
+    // measured on 11008 x 4096 with two / three / four quads in flight: 7.06 / 6.52 / 6.68 us; in a Llama-3-8B decode
+    // step (every Q4_K product) 1.617 / 1.564 / 1.568 / 1.578 ms per token with two / three / four / five
     int window = g_q4k_mfma_window.load() > 0 ? g_q4k_mfma_window.load() : mfma_window(k);
     if (mfma_window(k) == 2) window = 2;                       // long rows: the wave's load counter holds 63
+    if (merge) window = 3;
     const size_t smem = mfma_smem_bytes(k, qt, window);
     if (smem > 160 * 1024) return 0;
-    if (window == 2) return launch_mfma<2>(gain != nullptr, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
-    return launch_mfma<3>(gain != nullptr, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope);
+    const int pro = merge ? 2 : gain ? 1 : 0;
+    if (window == 2) return launch_mfma<2>(pro, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
+    return launch_mfma<3>(pro, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
 }
 
 }  // namespace skh

@@ -14,7 +14,7 @@
 // a 64-key tile of K, then of V, is staged in LDS once and used by all G rows. Each wave keeps a running
 // max / sum (online softmax) and its slice of the output in registers; keys the rules exclude are never
 // loaded unless a mask (or an empty key set) makes their -1e30 score matter.
-#include "common.h"
+#include "gemv_q4k.h"
 
 namespace skh {
 
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) void zero_kernel(float* out, int64_t n) {
 float* sdpa_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown on demand
 int launch_sdpa_decode(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                        int seq_kv, int kv_capacity, int head_dim, float scale, int window, int right_context,
-                       const int32_t* lengths);   // sdpa_decode.hip
+                       const int32_t* lengths, AttnMergePrologue* leave);   // sdpa_decode.hip
 int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                         int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal);   // sdpa_prefill.hip
 
@@ -206,7 +206,7 @@ int launch_sdpa(const float* q, const float* k, const float* v, float* out, int 
     }
     if (seq_q == 1 && !mask) {   // decode shape: the split-K cache-streaming kernel, when the head shape is one it carries
         const int r = launch_sdpa_decode(q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, head_dim, scale, window,
-                                         right_context, lengths);
+                                         right_context, lengths, nullptr);
         if (r != 0) return r < 0 ? -1 : 0;
     }
     if (seq_q > 1 && !mask && !lengths && window == 0) {   // prompt shape: the matrix-core kernel, when it carries the shape

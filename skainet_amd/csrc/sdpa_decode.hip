@@ -20,7 +20,7 @@
 //     no fence at all -- partials as agent-scope atomic stores / loads that bypass the L2s, one relaxed ticket per
 //     workgroup: results identical, but the ticket and the reads behind it are two more trips to memory, about what
 //     the second launch costs at 10 splits and far more at 64 (4096 keys: 21.8 us against 12.3).
-#include "common.h"
+#include "gemv_q4k.h"
 
 namespace skh {
 
@@ -35,7 +35,8 @@ struct SdpaDecodeParams {
     int window, right_context;
     const int32_t* lengths;
     int splits;
-    float* part;          // [batch * heads][splits][D + 2]
+    float* part;          // [batch * heads][splits][D] unnormalised outputs; null: one split, the normalised result goes to out
+    float* ml;            // [batch * heads][splits][2] running maximum (in units of ln 2) and sum of each split
 };
 
 // Scores are kept in units of ln 2 (the query is scaled by scale * log2(e) once), so every exponential of the softmax is
@@ -225,12 +226,11 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
         for (int e = 0; e < EPT; ++e) {
             const int i = i0 + e;
             const int d = ((i & 63) >> 2) * DPL + (i >> 6) * 4 + (i & 3);
-            if (p.splits == 1) {
+            if (!p.part) {
                 p.out[row * D + d] = ls > 0.f ? o[e] / ls : 0.f;
             } else {
-                float* dst = p.part + (row * p.splits + split) * (D + 2);
-                dst[d] = o[e];
-                if (d == 0) { dst[D] = mm; dst[D + 1] = ls; }
+                p.part[(row * p.splits + split) * D + d] = o[e];
+                if (d == 0) *reinterpret_cast<float2*>(p.ml + (row * p.splits + split) * 2) = make_float2(mm, ls);
             }
         }
     }
@@ -241,22 +241,24 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
 // softmax weights of the splits -- exp(max_s - max) / sum -- are worked out once, by the first wave: one split per
 // lane, maximum and sum by wave reductions (splits <= 64), parked in LDS for everyone.
 template <int D>
-__global__ __launch_bounds__(4 * D) void sdpa_decode_combine_kernel(const float* __restrict__ part, float* __restrict__ out, int splits) {
+__global__ __launch_bounds__(4 * D) void sdpa_decode_combine_kernel(const float* __restrict__ part, const float* __restrict__ ml,
+                                                                    float* __restrict__ out, int splits) {
     __shared__ float sw[SDPA_DECODE_MAX_SPLITS];
     __shared__ float so[4][D];
-    const float* src = part + (int64_t)blockIdx.x * splits * (D + 2);
+    const float* src = part + (int64_t)blockIdx.x * splits * D;
+    const float2* src_ml = reinterpret_cast<const float2*>(ml) + (int64_t)blockIdx.x * splits;
     const int d = threadIdx.x % D, j = threadIdx.x / D;
     float pv[SDPA_DECODE_MAX_SPLITS / 4];
 #pragma unroll
     for (int i = 0; i < SDPA_DECODE_MAX_SPLITS / 4; ++i) {
         const int sp = j + 4 * i;
-        pv[i] = src[min(sp, splits - 1) * (D + 2) + d];         // clamped: a split past the end gets weight zero below
+        pv[i] = src[min(sp, splits - 1) * D + d];               // clamped: a split past the end gets weight zero below
     }
     if (threadIdx.x < 64) {
         const int sp = threadIdx.x;
         const bool live = sp < splits;
-        const float m = live ? src[sp * (D + 2) + D] : -INFINITY;
-        const float l = live ? src[sp * (D + 2) + D + 1] : 0.f;
+        const float2 st = live ? src_ml[sp] : make_float2(-INFINITY, 0.f);
+        const float m = st.x, l = st.y;
         float mm = m;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) mm = fmaxf(mm, __shfl_xor(mm, off, 64));
@@ -282,23 +284,33 @@ static std::atomic<int> g_sdpa_decode_split_keys{64};   // least keys per split 
 void set_sdpa_decode_split_keys(int v) { if (v >= 16) g_sdpa_decode_split_keys = (v + 15) & ~15; }
 
 template <int GS, int DPL>
-static int launch_decode_variant(const SdpaDecodeParams& p, int subs) {
+static int launch_decode_variant(const SdpaDecodeParams& p, int subs, bool merge) {
     constexpr int D = 16 * DPL;
     note_kernel("sdpa_decode_kernel");
     sdpa_decode_kernel<GS, DPL><<<dim3(p.splits, p.kv_heads * subs, p.batch), dim3(256), 0, current_stream()>>>(p);
     SKH_CHECK(hipGetLastError());
-    if (p.splits > 1) {
-        sdpa_decode_combine_kernel<D><<<dim3(p.batch * p.heads), dim3(4 * D), 0, current_stream()>>>(p.part, p.out, p.splits);
+    if (merge) {
+        sdpa_decode_combine_kernel<D><<<dim3(p.batch * p.heads), dim3(4 * D), 0, current_stream()>>>(p.part, p.ml, p.out, p.splits);
         SKH_CHECK(hipGetLastError());
     }
     return 1;
 }
 
+static std::atomic<int> g_attn_merge_max_keys{176};    // most keys per split the unmerged form accepts (a multiple of 16)
+void set_attn_merge_max_keys(int v) { if (v >= 16) g_attn_merge_max_keys = (v + 15) & ~15; }
+// most splits the unmerged form uses. Measured in a Llama-3-8B decode step at 520 to 650 keys (ms per token): 2 splits 1.637,
+// 4: 1.565, 6: 1.540, 8: 1.556; the merge in a launch of its own 1.551 -- every split costs each of the projection's 251
+// workgroups another 16 KB of loads, every split less costs the attention workgroups another pass over their keys.
+static std::atomic<int> g_attn_merge_splits{6};
+void set_attn_merge_splits(int v) { if (v >= 1 && v <= ATTN_MERGE_MAX_SPLITS) g_attn_merge_splits = v; }
+
 // Returns 1 when this kernel took the call, 0 when the shape is outside its range (the caller uses the general
-// kernel), -1 on error.
+// kernel), -1 on error. With `leave` the per-split results are left unmerged for a consumer that folds the merge into
+// its own activation load (at most ATTN_MERGE_MAX_SPLITS splits, one sequence): `out` is not written, *leave describes
+// where the partials are; 0 when the key count would need more splits than that.
 int launch_sdpa_decode(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                        int seq_kv, int kv_capacity, int head_dim, float scale, int window, int right_context,
-                       const int32_t* lengths) {
+                       const int32_t* lengths, AttnMergePrologue* leave) {
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return 0;
     if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) & 15) return 0;
     const int per_kv = heads / kv_heads;
@@ -308,30 +320,70 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
     const int subs = per_kv / gs;
     if (batch > 65535) return 0;
     SdpaDecodeParams p{q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, scale, window, right_context, lengths, 1,
-                       nullptr};
+                       nullptr, nullptr};
     // enough workgroups to put every CU on the cache, at least 64 keys per split (measured in the decoder at 500 to 650
     // keys: 32 or 48 keys per split 2.5 % slower per token, 96 and 128 keys the same as 64)
     const int64_t groups = (int64_t)batch * kv_heads * subs;
     int splits = (int)((2 * (int64_t)num_cus() + groups - 1) / groups);
     splits = min(splits, min(SDPA_DECODE_MAX_SPLITS, (seq_kv + g_sdpa_decode_split_keys - 1) / g_sdpa_decode_split_keys));
     if (splits < 1) splits = 1;
-    p.splits = splits;
-    if (splits > 1) {
-        p.part = sdpa_workspace(sizeof(float) * (size_t)batch * heads * splits * (head_dim + 2));
-        if (!p.part) return -1;
+    if (leave) {
+        if (batch != 1) return 0;
+        const int most = g_attn_merge_splits;
+        if (splits > most) {
+            if ((seq_kv + most - 1) / most > g_attn_merge_max_keys) return 0;
+            splits = most;
+        }
     }
+    p.splits = splits;
+    if (splits > 1 || leave) {
+        const size_t rows = (size_t)batch * heads;
+        p.part = sdpa_workspace(sizeof(float) * rows * splits * (head_dim + 2));
+        if (!p.part) return -1;
+        p.ml = p.part + rows * splits * head_dim;
+    }
+    if (leave) *leave = AttnMergePrologue{p.part, p.ml, splits, head_dim};
+    const bool merge = splits > 1 && !leave;
     if (head_dim == 64) {
-        if (gs == 4) return launch_decode_variant<4, 4>(p, subs);
-        if (gs == 2) return launch_decode_variant<2, 4>(p, subs);
-        return launch_decode_variant<1, 4>(p, subs);
+        if (gs == 4) return launch_decode_variant<4, 4>(p, subs, merge);
+        if (gs == 2) return launch_decode_variant<2, 4>(p, subs, merge);
+        return launch_decode_variant<1, 4>(p, subs, merge);
     }
     if (head_dim == 128) {
-        if (gs == 4) return launch_decode_variant<4, 8>(p, subs);
-        if (gs == 2) return launch_decode_variant<2, 8>(p, subs);
-        return launch_decode_variant<1, 8>(p, subs);
+        if (gs == 4) return launch_decode_variant<4, 8>(p, subs, merge);
+        if (gs == 2) return launch_decode_variant<2, 8>(p, subs, merge);
+        return launch_decode_variant<1, 8>(p, subs, merge);
     }
-    if (gs == 2) return launch_decode_variant<2, 16>(p, subs);
-    return launch_decode_variant<1, 16>(p, subs);
+    if (gs == 2) return launch_decode_variant<2, 16>(p, subs, merge);
+    return launch_decode_variant<1, 16>(p, subs, merge);
+}
+
+int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n, const float* gain, float eps,
+                         const float* residual, int epilogue, const RopeQkvEpilogue* rope_in,
+                         const AttnMergePrologue* merge);   // gemv_q4k_mfma.hip
+
+static std::atomic<int> g_attn_merge_enable{1};
+void set_attn_merge_enable(int v) { g_attn_merge_enable = v; }
+
+// One decode token's attention over the cache and the Q4_K output projection behind it as two launches: the attention
+// kernel leaves its per-split results unmerged and the projection's activation load merges them (the merge launch and its
+// round trip through memory disappear). out[n] = (residual ? residual : 0) + Wo[n, heads * head_dim] . attention.
+// Returns 1 when the pair took the call, 0 when the shapes are outside its range (nothing launched), -1 on error.
+int launch_attn_out_proj_q4k(const uint8_t* wo, int n, int k, const float* q, const float* k_cache, const float* v_cache, int heads,
+                             int kv_heads, int head_dim, int seq_kv, int kv_capacity, float scale, int window,
+                             const int32_t* lengths, const float* residual, float* out) {
+    if (!g_attn_merge_enable || k != heads * head_dim || k > 4096 || (k & 1023)) return 0;
+    if (heads % kv_heads != 0 || seq_kv < 1 || kv_capacity < seq_kv) return 0;
+    // dry checks of the projection first: once the attention kernel has run without a merge there is no way back
+    if ((reinterpret_cast<uintptr_t>(wo) & 15) || n < 4 || (uint64_t)n * (uint64_t)(k >> 8) * 144u >= ((uint64_t)1 << 32)) return 0;
+    if (residual && (reinterpret_cast<uintptr_t>(residual) & 3)) return 0;
+    AttnMergePrologue am{};
+    const int r = launch_sdpa_decode(q, k_cache, v_cache, nullptr, 1, heads, kv_heads, seq_kv, kv_capacity, head_dim, scale, window, 0,
+                                     lengths, &am);
+    if (r <= 0) return r;
+    const int g = launch_q4k_gemv_mfma(wo, nullptr, out, k, n, nullptr, 0.f, residual, residual ? EPI_RESIDUAL : EPI_NONE, nullptr, &am);
+    if (g == 0) return set_error("attn_out_proj: the projection refused a shape its checks had passed (n %d, k %d)", n, k);
+    return g;
 }
 
 }  // namespace skh

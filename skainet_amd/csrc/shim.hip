@@ -49,6 +49,9 @@ int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink);
 int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes);
 int launch_fp32_matmul(const float* a, int64_t a_stride, const float* b, int64_t b_stride, float* c, int64_t c_stride,
                        int m, int n, int k, bool b_transposed);
+int launch_attn_out_proj_q4k(const uint8_t* wo, int n, int k, const float* q, const float* k_cache, const float* v_cache, int heads,
+                             int kv_heads, int head_dim, int seq_kv, int kv_capacity, float scale, int window,
+                             const int32_t* lengths, const float* residual, float* out);
 int launch_sdpa(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                 int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window, int right_context,
                 const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k);
@@ -578,6 +581,27 @@ int32_t skainet_hip_f32_sdpa_cache_dev(const float* q, const float* k_cache, con
     if (ensure_device() != 0) return -1;
     return launch_sdpa(q, k_cache, v_cache, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale, causal,
                        window, right_context, lengths, nullptr, 0, 0, 0, 0);
+}
+// One decode token: out = (residual ? residual : 0) + Wo . sdpa(q, cache). Q4_K projections whose input is at most 4096
+// wide run as two launches (attention leaving its key splits unmerged, the projection merging them as it loads its
+// activations); everything else as attention into `attn_tmp` followed by the fused product.
+int32_t skainet_hip_attn_out_proj_dev(const skainet_hip_weight* wo, const float* q, const float* k_cache, const float* v_cache,
+                                      int32_t heads, int32_t kv_heads, int32_t head_dim, int32_t seq_kv, int32_t kv_capacity,
+                                      float scale, int32_t window, const int32_t* lengths, const float* residual, float* out,
+                                      float* attn_tmp) {
+    if (ensure_device() != 0) return -1;
+    if (!wo) return set_error("attn_out_proj: null weight handle");
+    if (!q || !k_cache || !v_cache || !out || !attn_tmp) return set_error("attn_out_proj: null pointer");
+    if (heads <= 0 || kv_heads <= 0 || head_dim <= 0) return set_error("attn_out_proj: heads, kv_heads and head_dim must be positive");
+    if (wo->cols != heads * head_dim) return set_error("attn_out_proj: the weight takes %d inputs, the attention gives %d", wo->cols, heads * head_dim);
+    if (wo->encoding == ENC_Q4_K) {
+        const int r = launch_attn_out_proj_q4k(wo->data, wo->rows, wo->cols, q, k_cache, v_cache, heads, kv_heads, head_dim, seq_kv,
+                                               kv_capacity, scale, window, lengths, residual, out);
+        if (r != 0) return r < 0 ? -1 : 0;
+    }
+    if (launch_sdpa(q, k_cache, v_cache, attn_tmp, 1, heads, kv_heads, 1, seq_kv, kv_capacity, head_dim, scale, 1, window, 0, lengths,
+                    nullptr, 0, 0, 0, 0) != 0) return -1;
+    return skainet_hip_matmul_fused_dev(wo, attn_tmp, 1, out, nullptr, 0.f, residual, residual ? 1 : 0);
 }
 int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* out, int64_t n) {
     if (ensure_device() != 0) return -1;

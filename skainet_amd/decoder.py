@@ -336,6 +336,8 @@ class LlamaDecoder:
         self.generated = DeviceBuffer(4 * (c.ctx_max + 1))   # generated[p] = the token predicted for position p
         self.prompt_len = 0
         self._graph: Optional[kernels.Graph] = None
+        self._graph_bound = 0          # key count the recorded step was laid out for (its attention splits that many keys)
+        self._host_pos = 0             # the device-side position, tracked on the host so a replay needs no read-back
 
     # ------------------------------------------------------------------ building blocks
     def _block(self, li: int, rows: int, pos_start: int, pos_dev, seq_kv: int, kv_len_dev) -> None:
@@ -357,14 +359,16 @@ class LlamaDecoder:
             kx.rope_qkv_dev(self.qkv, self.q, kc, vc, rows, c.heads, c.kv_heads, c.head_dim, c.ctx_max, pos_start, pos_dev,
                             c.rope_theta)
         scale = float(1.0 / np.sqrt(c.head_dim))
-        kx.sdpa_cache_dev(self.q, kc, vc, self.attn, 1, c.heads, c.kv_heads, rows, seq_kv, c.ctx_max, c.head_dim, scale,
-                          True, 0, 0, kv_len_dev)
-        if rows > 1:
-            kx.heads_to_rows_dev(self.attn, self.attn_rows, c.heads, rows, c.head_dim)
-            attn_rows = self.attn_rows
+        if rows == 1 and pos_dev is not None:
+            # one token: [heads, 1, head_dim] is already the projection's input row; attention and projection as a pair
+            L.wo.attn_out_proj(self.q, kc, vc, c.heads, c.kv_heads, c.head_dim, seq_kv, c.ctx_max, scale, self.h, self.attn,
+                               residual=self.h, lengths=kv_len_dev)
         else:
-            attn_rows = self.attn                  # one token: [heads, 1, head_dim] is already the row
-        L.wo.matmul_fused(attn_rows, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
+            kx.sdpa_cache_dev(self.q, kc, vc, self.attn, 1, c.heads, c.kv_heads, rows, seq_kv, c.ctx_max, c.head_dim, scale,
+                              True, 0, 0, kv_len_dev)
+            if rows > 1:
+                kx.heads_to_rows_dev(self.attn, self.attn_rows, c.heads, rows, c.head_dim)
+            L.wo.matmul_fused(self.attn_rows if rows > 1 else self.attn, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
         L.w_gate_up.matmul_fused(self.h, rows, self.act, gain=L.ffn_norm, eps=c.rms_eps, epilogue=kx.EPI_SWIGLU)
         L.w_down.matmul_fused(self.act, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
 
@@ -395,66 +399,86 @@ class LlamaDecoder:
         self.pos.upload(np.array([rows], np.int32))
         self.kv_len.upload(np.array([rows + 1], np.int32))
         self.prompt_len = rows
+        self._host_pos = rows
         kernels.i32_store_at_dev(self.generated, self.pos, 0, self.token)
         kernels.sync()
         ids_dev.close()
         return int(self.token.download(np.int32, 1)[0])
 
-    def _decode_step(self) -> None:
+    KEY_BUCKET = 512
+
+    def _key_bound(self, keys: int) -> int:
+        """The key count a step is laid out for: the next multiple of KEY_BUCKET (the device-side length picks the keys
+        that exist, the bound decides how attention splits them)."""
+        b = self.KEY_BUCKET
+        return min(self.cfg.ctx_max, (keys + b - 1) // b * b)
+
+    def _decode_step(self, bound: Optional[int] = None) -> None:
         """Consumes self.token at device position self.pos, leaves the next token in self.token, advances the position."""
         c = self.cfg
+        if bound is None:
+            bound = self._key_bound(self._host_pos + 1)
         self.w.tok_embd.dequantize_rows(self.token, 1, self.h)
         kernels.rope_table_dev(self.pos, c.rope_theta, c.head_dim, self.rope_table)     # once per token, shared by all layers
         for li in range(c.layers):
-            self._block(li, 1, 0, self.pos, c.ctx_max, self.kv_len)
+            self._block(li, 1, 0, self.pos, bound, self.kv_len)
         self._head(0)
         kernels.decode_advance_dev(self.pos, self.kv_len, self.token, self.generated, c.ctx_max)
 
-    def decode(self, steps: int, use_graph: bool = True) -> np.ndarray:
-        """Greedy-decode `steps` tokens after prefill(); returns them. With use_graph the step is recorded once and replayed."""
-        c = self.cfg
-        if self.position() + steps > c.ctx_max:
-            raise ValueError(f"{steps} more tokens would pass the context limit {c.ctx_max}")
-        out = np.empty(steps, np.int32)
-        if use_graph and self._graph is not None and not self._graph.valid():
-            self._graph.close()                       # scratch moved since the recording (e.g. a longer prompt): record again
+    def _graph_step(self) -> None:
+        """One decode step through the recorded graph; records it first (one eager step, then the recording, which runs
+        nothing) when there is none, when the library's scratch moved since, or when the cache outgrew its key bound."""
+        keys = self._host_pos + 1
+        if self._graph is not None and (not self._graph.valid() or keys > self._graph_bound):
+            self._graph.close()
             self._graph = None
-        if use_graph and self._graph is None:
-            self._decode_step()                       # eager once: sizes every scratch buffer
+        if self._graph is None:
+            bound = self._key_bound(keys + 1)          # the recording serves the steps after this one
+            self._decode_step(bound)                   # eager once: sizes every scratch buffer
             kernels.sync()
-            out0 = int(self.token.download(np.int32, 1)[0])
-            with kernels.Graph() as g:
-                self._decode_step()
-            self._graph = g
-            first = 1
-            out[0] = out0
-        else:
-            first = 0
-        for i in range(first, steps):
+            self._host_pos += 1
+            if self._host_pos < self.cfg.ctx_max:      # at the limit there is no next step to record
+                with kernels.Graph() as g:
+                    self._decode_step(bound)
+                self._graph, self._graph_bound = g, bound
+            return
+        self._graph.launch()
+        self._host_pos += 1
+
+    def run_steps(self, steps: int, use_graph: bool = True) -> None:
+        """`steps` decode steps back to back without reading anything back (tokens feed back on the device)."""
+        if self._host_pos + steps > self.cfg.ctx_max:
+            raise ValueError(f"{steps} more tokens would pass the context limit {self.cfg.ctx_max}")
+        for _ in range(steps):
             if use_graph:
-                self._graph.launch()
-                self._graph.sync()
+                self._graph_step()
             else:
                 self._decode_step()
-                kernels.sync()
+                self._host_pos += 1
+
+    def decode(self, steps: int, use_graph: bool = True) -> np.ndarray:
+        """Greedy-decode `steps` tokens after prefill(); returns them. With use_graph the step is recorded once per key
+        bucket and replayed."""
+        c = self.cfg
+        if self._host_pos + steps > c.ctx_max:
+            raise ValueError(f"{steps} more tokens would pass the context limit {c.ctx_max}")
+        out = np.empty(steps, np.int32)
+        for i in range(steps):
+            self.run_steps(1, use_graph)
+            kernels.sync()
             out[i] = int(self.token.download(np.int32, 1)[0])
         return out
 
     def decode_timed(self, steps: int) -> float:
-        """Replay the recorded step `steps` times without reading tokens back; returns seconds (host clock around
-        launch + sync). Tokens stay on the device (greedy feedback happens there)."""
+        """`steps` recorded steps without reading tokens back; returns seconds (host clock around launch + sync). Tokens
+        stay on the device (greedy feedback happens there)."""
         import time
-        record = self._graph is None or not self._graph.valid()      # recording costs one (eager) step of its own
-        if self.position() + steps + int(record) > self.cfg.ctx_max:
+        if self._host_pos + steps > self.cfg.ctx_max:
             raise ValueError(f"{steps} more tokens would pass the context limit {self.cfg.ctx_max}")
-        if record:
-            self.decode(1, use_graph=True)
         kernels.sync()
-        self._graph.sync()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            self._graph.launch()
-        self._graph.sync()
+        self.run_steps(steps)
+        kernels.sync()
         return time.perf_counter() - t0
 
     def close(self) -> None:

@@ -174,6 +174,13 @@ class DeviceWeight:
                                                          _ptr(v_cache), heads, kv_heads, head_dim, kv_capacity,
                                                          _ptr(pos_dev), theta, _ptr(rope_table)), "matmul_qkv_rope")
 
+    def attn_out_proj(self, q, k_cache, v_cache, heads, kv_heads, head_dim, seq_kv, kv_capacity, scale, out, attn_tmp,
+                      residual=None, window: int = 0, lengths=None) -> None:
+        """out = (residual or 0) + W . sdpa(q, cache) for one decode token (skainet_hip_attn_out_proj_dev)."""
+        check(_lib.hip().skainet_hip_attn_out_proj_dev(self._h, _ptr(q), _ptr(k_cache), _ptr(v_cache), heads, kv_heads, head_dim,
+                                                       seq_kv, kv_capacity, scale, window, _ptr(lengths), _ptr(residual),
+                                                       _ptr(out), _ptr(attn_tmp)), "attn_out_proj")
+
     def dequantize(self, out) -> None:
         check(_lib.hip().skainet_hip_dequantize_dev(self._h, _ptr(out)), "dequantize")
 

@@ -619,3 +619,87 @@ def test_spi_route_decoder_follows_the_resident_decoder(small_model):
     with pytest.raises(ValueError):
         spi.step(cfg.vocab)
     spi.close()
+
+
+# ---- attention + output projection as a pair (the projection merges the attention's key splits) ---------------------
+@pytest.mark.parametrize("heads,kvh,hd,n,keys,bound,window,merged", [
+    (32, 8, 128, 512, 576, 1024, 0, True),      # the Llama-3 head shape: 6 splits of 96 keys
+    (32, 8, 128, 260, 1, 512, 0, True),         # one key
+    (32, 8, 128, 512, 37, 64, 0, True),         # one split
+    (32, 8, 128, 512, 1000, 1024, 256, True),   # sliding window inside the cache
+    (16, 4, 64, 128, 200, 512, 0, True),        # 16 heads per K slice
+    (4, 2, 256, 64, 130, 512, 0, True),         # 4 heads per K slice
+    (32, 8, 128, 512, 1500, 2048, 0, False),    # more keys per split than the pair accepts: merge launch + product
+    (8, 2, 64, 128, 100, 512, 0, False),        # 512 inputs: not a whole K slice
+])
+def test_attention_projection_pair_equals_its_parts(hip_backend, torch_cuda, heads, kvh, hd, n, keys, bound, window, merged):
+    """skainet_hip_attn_out_proj_dev against attention into a buffer followed by the fused product, with and without a
+    residual that aliases the output; the key count comes from the device, the bound from the host. Both routes
+    accumulate in fp32 in different orders: 2e-5 of the largest output."""
+    import oracle.golden as G
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(heads * 1000 + keys)
+    k = heads * hd
+    cap = bound + 16
+    blocks = G.weight_blocks("Q4_K", n, k // 256, 0xA77E)
+    w = kx.DeviceWeight.upload("Q4_K", G.row_major(blocks), n, k)
+    q = dev(torch, rng.standard_normal((heads, hd)).astype(np.float32))
+    kc = dev(torch, rng.standard_normal((kvh, cap, hd)).astype(np.float32))
+    vc = dev(torch, rng.standard_normal((kvh, cap, hd)).astype(np.float32))
+    lens = dev(torch, np.array([keys], np.int32))
+    res = rng.standard_normal(n).astype(np.float32)
+    scale = float(1.0 / np.sqrt(hd))
+    attn = torch.empty(k, dtype=torch.float32, device="cuda")
+    tmp = torch.full((k,), float("nan"), dtype=torch.float32, device="cuda")
+    for residual in (False, True):
+        want = dev(torch, res.copy())
+        kx.sdpa_cache_dev(q, kc, vc, attn, 1, heads, kvh, 1, bound, cap, hd, scale, True, window, 0, lens)
+        w.matmul_fused(attn, 1, want, residual=want if residual else None, epilogue=kx.EPI_RESIDUAL if residual else kx.EPI_NONE)
+        got = dev(torch, res.copy())
+        w.attn_out_proj(q, kc, vc, heads, kvh, hd, bound, cap, scale, got, tmp, residual=got if residual else None,
+                        window=window, lengths=lens)
+        kx.sync()
+        assert ("attention-merge" in kx.last_kernel()) == merged
+        a, b = got.cpu().numpy(), want.cpu().numpy()
+        assert np.isfinite(a).all()
+        assert np.abs(a - b).max() <= 2e-5 * np.abs(b).max(), (residual, np.abs(a - b).max(), np.abs(b).max())
+    # the switch takes the pair back to its parts, bit for bit
+    kx.set_tuning("attn_merge_enable", 0)
+    try:
+        got = torch.empty(n, dtype=torch.float32, device="cuda")
+        w.attn_out_proj(q, kc, vc, heads, kvh, hd, bound, cap, scale, got, tmp, lengths=lens, window=window)
+        want = torch.empty(n, dtype=torch.float32, device="cuda")
+        kx.sdpa_cache_dev(q, kc, vc, attn, 1, heads, kvh, 1, bound, cap, hd, scale, True, window, 0, lens)
+        w.matmul_fused(attn, 1, want)
+        kx.sync()
+        assert "attention-merge" not in kx.last_kernel()
+        assert np.array_equal(got.cpu().numpy(), want.cpu().numpy())
+    finally:
+        kx.set_tuning("attn_merge_enable", 1)
+    from skainet_amd._lib import HipError
+    with pytest.raises(HipError):
+        w.attn_out_proj(q, kc, vc, heads + 1, kvh, hd, bound, cap, scale, got, tmp)
+    w.close()
+
+
+def test_decoder_crosses_a_key_bucket_with_its_graph(hip_backend):
+    """The recorded step is laid out for a bound on the key count; when the cache outgrows it the decoder records
+    again, and the tokens are the ones the eager route emits."""
+    from skainet_amd.decoder import LlamaConfig, LlamaDecoder, LlamaWeights
+    cfg = LlamaConfig(layers=2, hidden=1024, heads=8, kv_heads=2, head_dim=128, ffn=1024, vocab=512, ctx_max=96, rope_theta=10000.0)
+    w = LlamaWeights(cfg, seed=5, sigma=0.05)
+    prompt = np.random.default_rng(9).integers(0, cfg.vocab, 7)
+    outs = []
+    for use_graph in (False, True):
+        dec = LlamaDecoder(w, max_prefill=8)
+        dec.KEY_BUCKET = 16                      # buckets of 16 keys: the 40 steps cross two edges
+        first = dec.prefill(prompt)
+        toks = dec.decode(40, use_graph=use_graph)
+        assert dec.position() == 47
+        if use_graph:
+            assert dec._graph_bound == 48
+        outs.append((first, toks, dec.last_logits()))
+        dec.close()
+    assert outs[0][0] == outs[1][0]
+    assert np.array_equal(outs[0][1], outs[1][1])
+    assert np.array_equal(outs[0][2], outs[1][2])
