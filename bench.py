@@ -223,6 +223,8 @@ def cpu_baseline_decode(cfg, host, ctx):
 ATTENTION_WORKLOADS = {
     # name -> (batch, seq_q, seq_kv); 32 query heads, 8 KV heads, head_dim 128, fp32, scale 1/sqrt(128), causal
     "sdpa_prefill_2048": (1, 2048, 2048),
+    # the same prompt under a 512-key sliding window (a fourth field: the window)
+    "sdpa_prefill_2048_w512": (1, 2048, 2048, 512),
     "sdpa_decode_576_b1": (1, 1, 576),
     "sdpa_decode_4096_b1": (1, 1, 4096),
     "sdpa_decode_4096_b8": (8, 1, 4096),
@@ -230,7 +232,7 @@ ATTENTION_WORKLOADS = {
 FP32_VECTOR_PEAK_TFLOPS = 157.3
 
 
-def cpu_baseline_attention(batch, seq_q, seq_kv, heads, kv_heads, d, scale, budget_s=15.0):
+def cpu_baseline_attention(batch, seq_q, seq_kv, heads, kv_heads, d, scale, window=0, budget_s=15.0):
     """The reference's skainet_f32_sdpa on this host. Prefill is sampled on one KV head's group (heads / kv_heads
     query heads) and scaled to all groups; decode runs the whole call."""
     from oracle import lib as L
@@ -244,7 +246,7 @@ def cpu_baseline_attention(batch, seq_q, seq_kv, heads, kv_heads, d, scale, budg
     o = np.empty_like(q)
 
     def call():
-        fn(L.fp(q), L.fp(k), L.fp(v), L.fp(o), batch, h, hkv, seq_q, seq_kv, d, scale, 1, 0, 0, None, None, 0, 0, 0, 0)
+        fn(L.fp(q), L.fp(k), L.fp(v), L.fp(o), batch, h, hkv, seq_q, seq_kv, d, scale, 1, window, 0, None, None, 0, 0, 0, 0)
 
     t0 = time.perf_counter()
     call()
@@ -265,7 +267,8 @@ def bench_attention(a):
     scenarios do) and one-token decode against a 4096-long KV cache (HBM-bound: K and V are read once)."""
     import torch
     from skainet_amd import _lib, kernels
-    batch, sq, skv = ATTENTION_WORKLOADS[a.workload]
+    batch, sq, skv = ATTENTION_WORKLOADS[a.workload][:3]
+    window = ATTENTION_WORKLOADS[a.workload][3] if len(ATTENTION_WORKLOADS[a.workload]) > 3 else 0
     heads, kvh, d = 32, 8, 128
     scale = float(1.0 / np.sqrt(d))
     decode = sq == 1
@@ -280,7 +283,7 @@ def bench_attention(a):
     out = torch.empty_like(q)
 
     def call(i):
-        kernels.sdpa_dev(q, ks[i % copies], vs[i % copies], out, batch, heads, kvh, sq, skv, d, scale, True)
+        kernels.sdpa_dev(q, ks[i % copies], vs[i % copies], out, batch, heads, kvh, sq, skv, d, scale, True, window)
 
     call(0)                                   # sizes the library's scratch before any capture
     kernels.sync()
@@ -312,7 +315,10 @@ def bench_attention(a):
     kk, vv = ks[0].repeat_interleave(heads // kvh, 1), vs[0].repeat_interleave(heads // kvh, 1)
     sc = torch.matmul(q.double(), kk.double().transpose(-1, -2)) * scale
     if not decode:
-        sc = sc.masked_fill(~torch.ones(sq, skv, dtype=torch.bool, device="cuda").tril(skv - sq), -1e30)
+        keep = torch.ones(sq, skv, dtype=torch.bool, device="cuda").tril(skv - sq)
+        if window > 0:
+            keep &= torch.ones(sq, skv, dtype=torch.bool, device="cuda").triu(skv - sq - window + 1)
+        sc = sc.masked_fill(~keep, -1e30)
     want = torch.matmul(torch.softmax(sc, -1), vv.double())
     err = float(((out.double() - want).abs().max() / want.abs().max()).cpu())
     tol = 2e-2
@@ -326,6 +332,8 @@ def bench_attention(a):
                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": measured_traffic(a.workload, kernels.last_kernel())}
     else:
         tf = flops_dense / (ms_per_step * 1e-3) / 1e12
+        # attended (query, key) pairs under the causal rule and the window: what a kernel that skips the rest has to do
+        useful_pairs = sum(min(qi + skv - sq + 1, window if window > 0 else skv) for qi in range(sq))
         value, unit, metric = tf, "TFLOP/s", "prefill attention TFLOP/s (dense-counted)"
         peak = MFMA_BF16_PEAK_TFLOPS if ATTENTION_PREFILL_USES_MFMA else FP32_VECTOR_PEAK_TFLOPS
         roof = {"bound": "mfma", "achieved": round(tf, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(tf / peak, 4),
@@ -335,18 +343,18 @@ def bench_attention(a):
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if decode or not ATTENTION_PREFILL_USES_MFMA else "bf16 x bf16 -> f32", "data": "synthetic",
         "config": {"workload": a.workload, "batch": batch, "heads": heads, "kv_heads": kvh, "head_dim": d, "seq_q": sq,
-                   "seq_kv": skv, "causal": True, "kv_copies_rotated": copies,
+                   "seq_kv": skv, "causal": True, "window": window, "kv_copies_rotated": copies,
                    "launch": "host loop" if a.no_graph else "hip-graph replay"},
         "roofline": roof,
         "extra": {"algorithmic_bytes_per_step": alg_bytes, "flops_dense_per_step": flops_dense,
-                  "flops_causal_useful_per_step": flops_dense if decode else flops_dense * (skv + 1) / (2 * skv),
+                  "flops_causal_useful_per_step": flops_dense if decode else 4.0 * batch * heads * d * useful_pairs,
                   "wall_s_timed_region": round(wall, 4), "max_err_over_max_vs_torch_fp64": err,
                   "device": _lib.hip().skainet_hip_device_name().decode()},
     }
     if err > tol:
         out_json["extra"]["PARITY_FAILED"] = True
     if not a.skip_cpu:
-        med, kind, sample = cpu_baseline_attention(batch, sq, skv, heads, kvh, d, scale)
+        med, kind, sample = cpu_baseline_attention(batch, sq, skv, heads, kvh, d, scale, window)
         cpu_val = alg_bytes / med / 1e9 if decode else flops_dense / med / 1e12
         # the reference threads its attention rows over at most 4 pool participants once there are >= 512 rows
         cores = 4 if (kind == "reference" and not decode) else 1

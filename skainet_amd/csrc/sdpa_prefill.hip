@@ -3,10 +3,12 @@
 //
 // Contract: the reference's skainet_f32_sdpa
 //   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/f32_fused.c:290-396
-// restricted to what a prompt pass uses: no additive mask, no key lengths, no window, seq_q <= seq_kv, causal or
-// full; head_dim 64 or 128. Every other call stays on the general fp32 kernel (sdpa.hip). Within these shapes
-// every query attends at least one key, so the reference's "-1e30 on excluded keys" and "excluded keys do not
-// take part" are the same function.
+// restricted to what a prompt pass uses: no additive mask, seq_q <= seq_kv, head_dim 64 or 128; causal or full, with
+// or without a sliding window (window, rightContext) and per-sequence key lengths, by the rules of
+//   /root/reference/skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/ops/AttentionMask.kt:24-104
+// Every other call stays on the general fp32 kernel (sdpa.hip). A query whose rules leave it at least one key gives
+// the same result whether excluded keys score -1e30 (the reference) or take no part (here); a query they leave none
+// weighs every key of the sequence equally, as the reference's row of equal scores does.
 //
 // Two launches:
 //   1. kv_to_bf16_kernel: K -> bf16 [kv head][key][D], V -> bf16 transposed [kv head][D][key], keys padded with
@@ -75,7 +77,8 @@ struct PrefillParams {
     float* out;
     int heads, kv_heads, seq_q, seq_kv, spad;
     float scale_log2e;
-    int causal;
+    int causal, window, right_context;
+    const int32_t* lengths;    // per-sequence key counts on the device, or null
     int heads_per_wg;      // 1, 2 or 4 query heads of one KV head per workgroup
 };
 
@@ -136,14 +139,35 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
     // causal: the workgroups with the most keys start first
     const int qb_wg = p.causal ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
     const int q0 = (qb_wg * qblocks_per_wg + wave / hpw) * PF_QW;          // first query position of this wave
+    const int q_wg_first = qb_wg * qblocks_per_wg * PF_QW;
     const int q_wg_last = min(p.seq_q, (qb_wg + 1) * qblocks_per_wg * PF_QW) - 1;
     const int shift = p.seq_kv - p.seq_q;                                   // absolute position of query 0
-    // keys any wave of this workgroup needs: [0, kend)
-    const int kend = p.causal ? min(p.seq_kv, q_wg_last + shift + 1) : p.seq_kv;
-    const int nblocks = (kend + PF_KB - 1) / PF_KB;
+    const int len = p.lengths ? p.lengths[b] : p.seq_kv;
+    // attended keys [first, end) of a query position: both bounds grow with the position
+    auto first_of = [&](int qi) { return p.window > 0 ? max(0, qi + shift - p.window + 1) : 0; };
+    auto end_of = [&](int qi) {
+        int e = p.seq_kv;
+        if (p.window > 0) e = min(e, qi + shift + p.right_context + 1);
+        if (p.causal) e = min(e, qi + shift + 1);
+        return max(min(e, len), 0);
+    };
     const int my_q = q0 + col;
-    const int my_last_key = p.causal ? my_q + shift : p.seq_kv - 1;         // last key this lane's query attends
-    const int wave_last_key = p.causal ? min(p.seq_kv - 1, q0 + PF_QW - 1 + shift) : p.seq_kv - 1;
+    const int my_qc = min(my_q, p.seq_q - 1);
+    const bool my_uniform = first_of(my_qc) >= end_of(my_qc);               // no key left: every key of the sequence, equally
+    const int my_first_key = my_uniform ? 0 : first_of(my_qc);
+    const int my_last_key = my_uniform ? p.seq_kv - 1 : end_of(my_qc) - 1;
+    const bool wave_uniform = __ballot(my_uniform) != 0;
+    const bool wg_uniform = __syncthreads_or(my_uniform) != 0;
+    // keys any wave of this workgroup needs: [kbeg, kend), whole blocks
+    const int kbeg = wg_uniform ? 0 : first_of(q_wg_first);
+    const int kend = wg_uniform ? p.seq_kv : end_of(q_wg_last);
+    const int blk_begin = kbeg / PF_KB;
+    const int nblocks = kend > kbeg ? (kend + PF_KB - 1) / PF_KB : blk_begin;
+    // this wave's 32 positions: the keys any of them attends, and the keys all of them attend
+    const int q_wave_last = min(q0 + PF_QW - 1, p.seq_q - 1), q_wave_first = min(q0, p.seq_q - 1);
+    const int wave_first_key = wave_uniform ? 0 : first_of(q_wave_first);
+    const int wave_last_key = wave_uniform ? p.seq_kv - 1 : end_of(q_wave_last) - 1;
+    const int wave_common_first = first_of(q_wave_last), wave_common_last = end_of(q_wave_first) - 1;
 
     // Q fragment: lane (query col, half h) holds q[16 t + 8 h .. + 7] for every t, times scale * log2(e)
     pf_bf16x8 qf[NT];
@@ -171,17 +195,17 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
         for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;     // per query (column); l_run is this lane's half of the keys
 
-    if (nblocks > 0) {
-        pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, 0, tid);
-        pf_store_block<D>(kreg, vreg, ktile0, vtile0, tid);
+    if (nblocks > blk_begin) {
+        pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, blk_begin * PF_KB, tid);
+        pf_store_block<D>(kreg, vreg, ktile0 + (blk_begin & 1) * (PF_KB * KP), vtile0 + (blk_begin & 1) * (D * VP), tid);
     }
     __syncthreads();
 
-    for (int blk = 0; blk < nblocks; ++blk) {
+    for (int blk = blk_begin; blk < nblocks; ++blk) {
         const int buf = blk & 1;
         const int k0 = blk * PF_KB;
         if (blk + 1 < nblocks) pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, k0 + PF_KB, tid);
-        if (k0 <= wave_last_key) {                                   // wave-uniform: this wave has keys in the block
+        if (k0 <= wave_last_key && k0 + PF_KB > wave_first_key) {     // wave-uniform: this wave has keys in the block
             // S^T tiles: s[j] covers keys k0 + 32 j .. + 31 (rows) x this wave's 32 queries (columns)
             pf_f32x16 s[2];
 #pragma unroll
@@ -195,15 +219,15 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
                     s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s[j], 0, 0, 0);
                 }
             }
-            // keys past this query's last key score -inf (they take no part)
-            const int first_last = p.causal ? q0 + shift : p.seq_kv - 1;     // the smallest last-key among this wave's queries
-            if (k0 + PF_KB - 1 > first_last || k0 + PF_KB > p.seq_kv) {      // wave-uniform: the block crosses a boundary
+            // keys outside this query's range score -inf (they take no part); a query without a range scores every key 0
+            if (wave_uniform || k0 < wave_common_first || k0 + PF_KB - 1 > wave_common_last) {   // wave-uniform: the block crosses a boundary
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int key = k0 + 32 * j + 8 * (e >> 2) + 4 * h + (e & 3);
-                        if (key > my_last_key) s[j][e] = -INFINITY;
+                        if (my_uniform) s[j][e] = 0.f;
+                        if (key > my_last_key || key < my_first_key) s[j][e] = -INFINITY;
                     }
             }
             float mx = s[0][0];
@@ -273,7 +297,8 @@ void set_sdpa_prefill_mfma(int v) { g_prefill_mfma = v; }
 
 template <int D>
 static int launch_prefill_d(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
-                            int seq_q, int seq_kv, int kv_capacity, float scale, int causal) {
+                            int seq_q, int seq_kv, int kv_capacity, float scale, int causal, int window, int right_context,
+                            const int32_t* lengths) {
     const int spad = (seq_kv + PF_KB - 1) / PF_KB * PF_KB;
     const size_t elems = (size_t)batch * kv_heads * spad * D;
     __bf16* ws = static_cast<__bf16*>(kernel_workspace(2 * elems * sizeof(__bf16)));
@@ -285,7 +310,7 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
     const int per_kv = heads / kv_heads;
     const int hpw = per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1);
     const int q_per_wg = (4 / hpw) * PF_QW;
-    PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, hpw};
+    PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, window, right_context, lengths, hpw};
     const dim3 grid((seq_q + q_per_wg - 1) / q_per_wg, kv_heads * (per_kv / hpw), batch);
     constexpr size_t smem = sizeof(__bf16) * (2 * PF_KB * (D + 8) + 2 * D * (PF_KB + 8));
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D>), smem);
@@ -297,15 +322,16 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
 
 // Returns 1 when the MFMA path took the call, 0 when the shape is outside its range, -1 on error.
 int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
-                        int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal) {
+                        int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window,
+                        int right_context, const int32_t* lengths) {
     if (!g_prefill_mfma) return 0;
     if (head_dim != 64 && head_dim != 128) return 0;
     if (seq_q < 16 || seq_q > seq_kv) return 0;          // a handful of rows is the row kernel's business
     if (batch > 65535 || (int64_t)kv_heads * heads > 65535) return 0;
     if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
          reinterpret_cast<uintptr_t>(out)) & 15) return 0;
-    if (head_dim == 64) return launch_prefill_d<64>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal);
-    return launch_prefill_d<128>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal);
+    if (head_dim == 64) return launch_prefill_d<64>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths);
+    return launch_prefill_d<128>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths);
 }
 
 }  // namespace skh

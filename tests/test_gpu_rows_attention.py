@@ -184,6 +184,44 @@ def test_attention_prefill_mfma_shapes(hip_backend, torch_cuda, batch, heads, kv
     assert np.abs(gpu_sdpa(hip_backend, torch_cuda, q, k, ones, scale, causal) - 1.0).max() <= 1e-2
 
 
+@pytest.mark.parametrize("batch,heads,kv_heads,d,sq,skv,causal,window,rc,lengths", [
+    (1, 8, 2, 128, 300, 300, True, 64, 0, None),            # sliding window shorter than a key block ... 
+    (1, 8, 2, 128, 300, 300, True, 100, 0, None),           # ... and one that straddles blocks
+    (2, 4, 2, 64, 200, 200, True, 0, 0, [200, 77]),         # key lengths: the second sequence ends inside a block
+    (3, 4, 4, 64, 130, 130, True, 50, 0, [130, 40, 0]),     # window + lengths: late queries of sequence 1 and all of 2 keep no key
+    (1, 4, 1, 128, 96, 400, True, 128, 0, None),            # a later prompt chunk with a window
+    (1, 6, 3, 128, 150, 150, False, 40, 7, None),           # bidirectional window with right context
+    (2, 2, 2, 64, 64, 64, False, 0, 0, [1, 64]),            # full attention, one key
+    (1, 32, 8, 128, 512, 512, True, 256, 0, None),          # the Llama-3 head shape with a 256-key window
+])
+def test_attention_prefill_mfma_window_and_key_lengths(hip_backend, torch_cuda, batch, heads, kv_heads, d, sq, skv, causal, window,
+                                                       rc, lengths):
+    """The matrix-core prompt kernel under the structured rules (sliding window, right context, per-sequence key
+    lengths), including queries the rules leave without a key (equal weight on every key, as the reference's row of
+    equal -1e30 scores). Against the oracle, 2e-2 of the largest reference magnitude; the fp32 kernel on the same call
+    stays within the reference's own tolerance."""
+    rng = np.random.default_rng(sq * skv + d + window)
+    q = rng.standard_normal((batch, heads, sq, d)).astype(np.float32)
+    k = rng.standard_normal((batch, kv_heads, skv, d)).astype(np.float32)
+    v = rng.standard_normal((batch, kv_heads, skv, d)).astype(np.float32)
+    scale = float(1 / np.sqrt(d))
+    ln = None if lengths is None else np.asarray(lengths, np.int32)
+    got = gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, rc, ln)
+    assert hip_backend.last_kernel() == "sdpa_prefill_kernel"
+    want = L.sdpa(q, k, v, scale, causal, window, rc, ln)
+    assert np.isfinite(got).all()
+    assert normalized_err(got, want, eps=1.0) <= 2e-2
+    assert np.sqrt(np.mean((got - want) ** 2)) <= 5e-3 * np.abs(want).max()
+    ones = np.ones_like(v)
+    assert np.abs(gpu_sdpa(hip_backend, torch_cuda, q, k, ones, scale, causal, window, rc, ln) - 1.0).max() <= 1e-2
+    hip_backend.set_tuning("sdpa_prefill_mfma", 0)
+    try:
+        close(gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, rc, ln), want)
+        assert hip_backend.last_kernel() != "sdpa_prefill_kernel"
+    finally:
+        hip_backend.set_tuning("sdpa_prefill_mfma", 1)
+
+
 def test_norms_softmax_and_glue(hip_backend, torch_cuda):
     torch = torch_cuda
     kx = hip_backend
