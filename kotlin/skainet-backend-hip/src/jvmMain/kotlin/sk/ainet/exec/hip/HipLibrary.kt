@@ -1,0 +1,97 @@
+package sk.ainet.exec.hip
+
+import java.lang.foreign.Arena
+import java.lang.foreign.FunctionDescriptor
+import java.lang.foreign.Linker
+import java.lang.foreign.MemorySegment
+import java.lang.foreign.SymbolLookup
+import java.lang.foreign.ValueLayout
+import java.lang.invoke.MethodHandle
+
+/**
+ * libskainet_hip.so, loaded once. Every failure on the way (property switch, missing library, missing symbol, no
+ * gfx950 device) ends in "unavailable", never in an exception: the registry then keeps the CPU tiers.
+ *
+ * Properties: `skainet.hip.enabled` (default true), `skainet.hip.device` (default 0).
+ */
+internal object HipLibrary {
+    private val linker: Linker = Linker.nativeLinker()
+
+    val lookup: SymbolLookup? = runCatching {
+        if (System.getProperty("skainet.hip.enabled", "true") != "true") null
+        else SymbolLookup.libraryLookup(System.mapLibraryName("skainet_hip"), Arena.global())
+    }.getOrNull()
+
+    private val I = ValueLayout.JAVA_INT
+    private val L = ValueLayout.JAVA_LONG
+    private val F = ValueLayout.JAVA_FLOAT
+    private val P = ValueLayout.ADDRESS
+
+    private fun bind(name: String, descriptor: FunctionDescriptor): MethodHandle? =
+        lookup?.find(name)?.orElse(null)?.let { runCatching { linker.downcallHandle(it, descriptor) }.getOrNull() }
+
+    // ---- runtime
+    val available: MethodHandle? = bind("skainet_hip_available", FunctionDescriptor.of(I))
+    val init: MethodHandle? = bind("skainet_hip_init", FunctionDescriptor.of(I, I))
+    val lastError: MethodHandle? = bind("skainet_hip_last_error", FunctionDescriptor.of(P))
+    val sync: MethodHandle? = bind("skainet_hip_sync", FunctionDescriptor.of(I))
+    val threadRelease: MethodHandle? = bind("skainet_hip_thread_release", FunctionDescriptor.of(I))
+
+    // ---- device memory (size_t == long on LP64)
+    val malloc: MethodHandle? = bind("skainet_hip_malloc", FunctionDescriptor.of(P, L))
+    val free: MethodHandle? = bind("skainet_hip_free", FunctionDescriptor.of(I, P))
+    val h2d: MethodHandle? = bind("skainet_hip_memcpy_h2d", FunctionDescriptor.of(I, P, P, L))
+    val d2h: MethodHandle? = bind("skainet_hip_memcpy_d2h", FunctionDescriptor.of(I, P, P, L))
+    val d2d: MethodHandle? = bind("skainet_hip_memcpy_d2d", FunctionDescriptor.of(I, P, P, L))
+
+    // ---- resident weights
+    val weightUpload: MethodHandle? = bind("skainet_hip_weight_upload", FunctionDescriptor.of(P, P, L, I, I, I, I))
+    val weightFree: MethodHandle? = bind("skainet_hip_weight_free", FunctionDescriptor.ofVoid(P))
+    val matmulHost: MethodHandle? = bind("skainet_hip_matmul_host", FunctionDescriptor.of(I, P, P, I, P))
+    val matmulDev: MethodHandle? = bind("skainet_hip_matmul_dev", FunctionDescriptor.of(I, P, P, I, P))
+
+    // ---- host entries with the CPU library's signatures
+    /** (input, input_offset, weight, weight_byte_offset, input_dim, output_dim, output, output_offset) */
+    private val GEMV: FunctionDescriptor = FunctionDescriptor.ofVoid(P, I, P, I, I, I, P, I)
+    val q4k: MethodHandle? = bind("skainet_hip_q4k_matmul", GEMV)
+    val q6k: MethodHandle? = bind("skainet_hip_q6k_matmul", GEMV)
+    val q5k: MethodHandle? = bind("skainet_hip_q5k_matmul", GEMV)
+    val q80: MethodHandle? = bind("skainet_hip_q8_0_matmul", GEMV)
+    val q40: MethodHandle? = bind("skainet_hip_q4_0_matmul", GEMV)
+    val q50: MethodHandle? = bind("skainet_hip_q5_0_matmul", GEMV)
+    val q51: MethodHandle? = bind("skainet_hip_q5_1_matmul", GEMV)
+
+    /** (a, a_offset, a_stride, b, b_offset, b_stride, c, c_offset, c_stride, m, n, k); b is bytes for the narrow floats */
+    private val GEMM: FunctionDescriptor = FunctionDescriptor.ofVoid(P, I, I, P, I, I, P, I, I, I, I, I)
+    val sgemm: MethodHandle? = bind("skainet_hip_fp32_matmul", GEMM)
+    val bf16Gemm: MethodHandle? = bind("skainet_hip_bf16_matmul", GEMM)
+    val fp16Gemm: MethodHandle? = bind("skainet_hip_fp16_matmul", GEMM)
+    val sgemmWt: MethodHandle? = bind("skainet_hip_fp32_matmul_wt", FunctionDescriptor.ofVoid(P, I, P, I, P, I, I, I, I))
+
+    val rmsNorm: MethodHandle? = bind("skainet_hip_f32_rms_norm", FunctionDescriptor.ofVoid(P, P, P, I, I, F))
+    val layerNorm: MethodHandle? = bind("skainet_hip_f32_layer_norm", FunctionDescriptor.ofVoid(P, P, P, P, I, I, F))
+    val softmax: MethodHandle? = bind("skainet_hip_f32_softmax_rows", FunctionDescriptor.ofVoid(P, P, I, I, I))
+    val sdpa: MethodHandle? = bind(
+        "skainet_hip_f32_sdpa",
+        FunctionDescriptor.ofVoid(P, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P, I, I, I, I),
+    )
+
+    /** Cheap, cached, false (not throwing) when the library or a gfx950 device is missing. */
+    val usable: Boolean by lazy {
+        runCatching {
+            (available?.invoke() as? Int) == 1 &&
+                (init?.invoke(Integer.getInteger("skainet.hip.device", 0)) as? Int) == 0
+        }.getOrDefault(false)
+    }
+
+    /** The calling thread's last failure ("" when its last call succeeded). */
+    fun error(): String = runCatching {
+        (lastError!!.invoke() as MemorySegment).reinterpret(1024).getString(0)
+    }.getOrDefault("")
+
+    /** After a `void` host entry: those clear the thread's error text on entry and set it on failure. */
+    fun checkHostCall(who: String) {
+        val message = error()
+        check(message.isEmpty()) { "$who: $message" }
+    }
+}

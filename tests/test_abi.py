@@ -81,3 +81,63 @@ def test_unavailable_is_an_answer_and_calls_fail_loudly():
     y[:] = 7
     _lib.hip().skainet_hip_q4k_matmul_rm(x.ctypes.data, 0, w.ctypes.data, 0, 256, 2, y.ctypes.data, 0)
     assert (y == 7).all() and _lib.last_error()
+
+
+def _c_parameter_kinds():
+    """name -> (return kind, [parameter kinds]) of every declaration of the header; kinds are the FFM layout letters the
+    Kotlin module uses: I int32, L int64 / size_t, F float, P pointer, V void."""
+    text = open(os.path.join(ROOT, "include", "skainet_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+
+    def kind(decl):
+        decl = decl.strip()
+        if "*" in decl:
+            return "P"
+        base = decl.split()
+        if not base or decl == "void":
+            return "V"
+        if "float" in base:
+            return "F"
+        if "int64_t" in base or "size_t" in base:
+            return "L"
+        if "int32_t" in base:
+            return "I"
+        raise AssertionError(f"unclassified C type in {decl!r}")
+
+    out = {}
+    for m in re.finditer(r"SKAINET_HIP_API\s+([^;]*?)\b(skainet_hip_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        ret, name, params = m.group(1), m.group(2), m.group(3)
+        plist = [] if params.strip() in ("", "void") else [kind(p) for p in params.split(",")]
+        out[name] = (kind(ret + " x") if "*" in ret else kind(ret), plist)
+    return out
+
+
+def test_kotlin_module_binds_the_header_as_declared():
+    """The Kotlin module text is not compiled here, so its native descriptors are held against the header: every symbol
+    it binds is declared, with the same return and parameter layouts; both ServiceLoader files name classes that exist."""
+    kdir = os.path.join(ROOT, "kotlin", "skainet-backend-hip", "src", "jvmMain")
+    src = open(os.path.join(kdir, "kotlin", "sk", "ainet", "exec", "hip", "HipLibrary.kt")).read()
+    decls = _c_parameter_kinds()
+    named = {m.group(1): m.group(2) for m in re.finditer(r"private val (\w+): FunctionDescriptor = (FunctionDescriptor\.\w+\([^)]*\))", src)}
+    bound = re.findall(r'bind\(\s*"(skainet_hip_\w+)",\s*(FunctionDescriptor\.\w+\([^)]*\)|\w+)', src)
+    assert len(bound) >= 29
+    for name, desc in bound:
+        assert name in decls, f"{name} is not declared in the header"
+        desc = named.get(desc, desc)
+        m = re.match(r"FunctionDescriptor\.(of|ofVoid)\(([^)]*)\)", desc)
+        assert m, (name, desc)
+        letters = [t.strip() for t in m.group(2).split(",") if t.strip()]
+        ret, params = ("V", letters) if m.group(1) == "ofVoid" else (letters[0], letters[1:])
+        assert (ret, params) == decls[name], (name, ret, params, decls[name])
+    all_kt = "".join(open(os.path.join(kdir, "kotlin", "sk", "ainet", "exec", "hip", f)).read()
+                     for f in sorted(os.listdir(os.path.join(kdir, "kotlin", "sk", "ainet", "exec", "hip"))))
+    assert "TODO" not in all_kt
+    services = os.path.join(kdir, "resources", "META-INF", "services")
+    for iface in ("sk.ainet.backend.api.kernel.KernelProvider", "sk.ainet.backend.api.kernel.ViewKernelPack"):
+        cls = open(os.path.join(services, iface)).read().strip()
+        assert cls.startswith("sk.ainet.exec.hip.") and f"class {cls.rsplit('.', 1)[1]} " in all_kt
+    # every accessor of the provider interface the Python mirror serves is served by the Kotlin provider as well
+    provider = open(os.path.join(kdir, "kotlin", "sk", "ainet", "exec", "hip", "HipKernelProvider.kt")).read()
+    for accessor in ("matmulFp32", "matmulFp32Wt", "matmulBf16", "matmulFp16", "matmulQ4K", "matmulQ6K", "matmulQ5K", "matmulQ8_0",
+                     "matmulQ4_0", "matmulQ5_0", "matmulQ5_1", "softmaxFp32", "normFp32", "attentionFp32"):
+        assert f"override fun {accessor}()" in provider
