@@ -286,6 +286,21 @@ SKAINET_HIP_API int32_t skainet_hip_attn_out_proj_dev(const skainet_hip_weight* 
  *             REF/../skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/ops/TensorOps.kt:263-277) */
 SKAINET_HIP_API int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* out, int64_t n);
 SKAINET_HIP_API int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int64_t n);
+/* Dense elementwise, activation and reduction kernels on device operands: the resident-activation set of
+ * REF/skainet-backend-wasm-simd/src/wasmJsMain/kotlin/sk/ainet/exec/wasm/WasmCpuOps.kt:30-40 with the contracts of the CPU
+ * library (NAT:515-546, REF/skainet-backend-native-cpu/native/src/f32_ops.c:130-330):
+ *   binary: out[i] = a[ia] op b[ib]; op 0 add, 1 sub, 2 mul, 3 div; a_mode / b_mode 0 full (ia = i), 1 scalar (ia = 0),
+ *           2 bias (ia = i % inner); inner <= 0 counts as 1;
+ *   unary:  op 0 relu, 1 sigmoid, 2 silu, 3 gelu (tanh form), 4 gelu (erf form, evaluated in double), 5 erf, 6 tanh;
+ *   reduce_all: *out = sum of in[0..n) (divided by n when mean != 0; n <= 0 gives 0);
+ *   reduce_axis: out[o * inner + x] = sum over k < red of in[(o * red + k) * inner + x] (divided by red when mean != 0).
+ * n <= 0 (outer or inner <= 0) is a no-op; unknown ops or modes return -1. */
+SKAINET_HIP_API int32_t skainet_hip_f32_binary_dev(int32_t op, const float* a, int32_t a_mode, const float* b, int32_t b_mode,
+    float* out, int64_t n, int32_t inner);
+SKAINET_HIP_API int32_t skainet_hip_f32_unary_dev(int32_t op, const float* in, float* out, int64_t n);
+SKAINET_HIP_API int32_t skainet_hip_f32_reduce_all_dev(const float* in, int64_t n, int32_t mean, float* out);
+SKAINET_HIP_API int32_t skainet_hip_f32_reduce_axis_dev(const float* in, int32_t outer, int32_t red, int32_t inner, int32_t mean,
+    float* out);
 SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
 /* skainet_hip_f32_argmax_rows_dev for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid it). No counterpart in the reference. Same result (first maximum of each row);

@@ -49,6 +49,10 @@ int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink);
 int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes);
 int launch_fp32_matmul(const float* a, int64_t a_stride, const float* b, int64_t b_stride, float* c, int64_t c_stride,
                        int m, int n, int k, bool b_transposed);
+int launch_f32_binary(int op, const float* a, int a_mode, const float* b, int b_mode, float* out, int64_t n, int inner);   // elementwise.hip
+int launch_f32_unary(int op, const float* in, float* out, int64_t n);
+int launch_f32_reduce_all(const float* in, int64_t n, int mean, float* out);
+int launch_f32_reduce_axis(const float* in, int outer, int red, int inner, int mean, float* out);
 int launch_attn_out_proj_q4k(const uint8_t* wo, int n, int k, const float* q, const float* k_cache, const float* v_cache, int heads,
                              int kv_heads, int head_dim, int seq_kv, int kv_capacity, float scale, int window,
                              const int32_t* lengths, const float* residual, float* out);
@@ -610,6 +614,23 @@ int32_t skainet_hip_f32_silu_mul_dev(const float* gate, const float* up, float* 
 int32_t skainet_hip_f32_add_dev(const float* a, const float* b, float* out, int64_t n) {
     if (ensure_device() != 0) return -1;
     return launch_add(a, b, out, n);
+}
+int32_t skainet_hip_f32_binary_dev(int32_t op, const float* a, int32_t a_mode, const float* b, int32_t b_mode, float* out,
+                                   int64_t n, int32_t inner) {
+    if (ensure_device() != 0) return -1;
+    return launch_f32_binary(op, a, a_mode, b, b_mode, out, n, inner);
+}
+int32_t skainet_hip_f32_unary_dev(int32_t op, const float* in, float* out, int64_t n) {
+    if (ensure_device() != 0) return -1;
+    return launch_f32_unary(op, in, out, n);
+}
+int32_t skainet_hip_f32_reduce_all_dev(const float* in, int64_t n, int32_t mean, float* out) {
+    if (ensure_device() != 0) return -1;
+    return launch_f32_reduce_all(in, n, mean, out);
+}
+int32_t skainet_hip_f32_reduce_axis_dev(const float* in, int32_t outer, int32_t red, int32_t inner, int32_t mean, float* out) {
+    if (ensure_device() != 0) return -1;
+    return launch_f32_reduce_axis(in, outer, red, inner, mean, out);
 }
 int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out) {
     if (ensure_device() != 0) return -1;

@@ -275,6 +275,28 @@ def add_dev(a, b, out, n: int) -> None:
     check(_lib.hip().skainet_hip_f32_add_dev(_ptr(a), _ptr(b), _ptr(out), n), "add")
 
 
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+UNARY_OPS = {"relu": 0, "sigmoid": 1, "silu": 2, "gelu_tanh": 3, "gelu": 4, "erf": 5, "tanh": 6}
+MODE_FULL, MODE_SCALAR, MODE_BIAS = 0, 1, 2
+
+
+def binary_dev(op: str, a, b, out, n: int, a_mode: int = MODE_FULL, b_mode: int = MODE_FULL, inner: int = 1) -> None:
+    """out[i] = a[ia] op b[ib] on device operands (skainet_f32_binary's contract: full / scalar / bias operand modes)."""
+    check(_lib.hip().skainet_hip_f32_binary_dev(BINARY_OPS[op], _ptr(a), a_mode, _ptr(b), b_mode, _ptr(out), n, inner), "binary")
+
+
+def unary_dev(op: str, x, out, n: int) -> None:
+    check(_lib.hip().skainet_hip_f32_unary_dev(UNARY_OPS[op], _ptr(x), _ptr(out), n), "unary")
+
+
+def reduce_all_dev(x, n: int, out, mean: bool = False) -> None:
+    check(_lib.hip().skainet_hip_f32_reduce_all_dev(_ptr(x), n, int(mean), _ptr(out)), "reduce_all")
+
+
+def reduce_axis_dev(x, outer: int, red: int, inner: int, out, mean: bool = False) -> None:
+    check(_lib.hip().skainet_hip_f32_reduce_axis_dev(_ptr(x), outer, red, inner, int(mean), _ptr(out)), "reduce_axis")
+
+
 def argmax_rows_dev(x, rows: int, cols: int, out) -> None:
     check(_lib.hip().skainet_hip_f32_argmax_rows_dev(_ptr(x), rows, cols, _ptr(out)), "argmax_rows")
 
