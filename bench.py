@@ -57,6 +57,12 @@ WORKLOADS = {
     "q5k_gemv_11008x4096_b1": ("Q5_K", 11008, 4096, 1),
     # prefill: batch > 8 goes to the MFMA dequant-GEMM and is reported in TFLOP/s against the bf16 MFMA peak
     "q4k_gemm_512x4096x4096": ("Q4_K", 4096, 4096, 512),
+    # short prompts and speculative batches: more rows than the GEMV kernels take, fewer than a 256-row tile
+    "q4k_gemm_16x4096x4096": ("Q4_K", 4096, 4096, 16),
+    "q4k_gemm_32x4096x4096": ("Q4_K", 4096, 4096, 32),
+    "q4k_gemm_64x4096x4096": ("Q4_K", 4096, 4096, 64),
+    "q4k_gemm_128x4096x4096": ("Q4_K", 4096, 4096, 128),
+    "q4k_gemm_128x14336x4096": ("Q4_K", 14336, 4096, 128),
     "q6k_gemm_512x32000x4096": ("Q6_K", 32000, 4096, 512),
     "q4k_gemm_512x14336x4096": ("Q4_K", 14336, 4096, 512),
     "q5k_gemm_512x4096x4096": ("Q5_K", 4096, 4096, 512),

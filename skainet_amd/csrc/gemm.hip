@@ -31,13 +31,14 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // twice the MFMAs, so the wide tile is the one that can keep the matrix cores busy; it needs 32 tiles per CU round
 // fewer to fill the chip, so it serves the wide weights (N >= 128 rows per CU) and the narrow one the rest.
 constexpr int G_WAVES_M = 2, G_WAVES_N = 2;
-constexpr int GM = 128 * G_WAVES_M, GK = 64;
+constexpr int GK = 64;
 constexpr int G_THREADS = G_WAVES_M * G_WAVES_N * 64;
-constexpr int G_A_LOADS = GM * (GK / 8) / G_THREADS;          // 16-byte chunks of the activation tile per thread
 constexpr int GSTRIDE = GK + 8;                               // bf16 elements per LDS row (144 bytes)
-constexpr int G_A_ELEMS = GM * GSTRIDE;
+// A wave owns WTM x WTN MFMA tiles of 32 x 32: WTM = 4 row tiles (workgroup tile 256 rows) for prompts, WTM = 2 (128 rows)
+// where at most 128 activation rows exist or where the taller tile would leave most of the chip idle.
+constexpr int gemm_gm(int wtm) { return 32 * wtm * G_WAVES_M; }
 constexpr int gemm_gn(int wtn) { return 32 * wtn * G_WAVES_N; }
-constexpr size_t gemm_smem(int wtn) { return 2 * (size_t)(G_A_ELEMS + gemm_gn(wtn) * GSTRIDE) * sizeof(__bf16); }   // two stages
+constexpr size_t gemm_smem(int wtm, int wtn) { return 2 * (size_t)(gemm_gm(wtm) + gemm_gn(wtn)) * GSTRIDE * sizeof(__bf16); }   // two stages
 
 void* kernel_workspace(size_t bytes);   // shim.hip
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);   // gemv.hip
@@ -359,17 +360,19 @@ __device__ __forceinline__ uint32_t decode_item_at(int h, const Raw& r, const De
     }
 }
 
-template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES, int WTN>
+template <class Raw, int BLOCK_ELEMS, int BLOCK_BYTES, int WTM, int WTN>
 __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
                                                            float* __restrict__ c, int m, int n, int k, int k_chunk,
                                                            int64_t split_stride) {
-    constexpr int G_WTN = WTN, GN = gemm_gn(WTN);
+    constexpr int G_WTN = WTN, GN = gemm_gn(WTN), GM = gemm_gm(WTM);
+    constexpr int G_A_LOADS = GM * (GK / 8) / G_THREADS;      // 16-byte chunks of the activation tile per thread
+    constexpr int G_A_ELEMS = GM * GSTRIDE;
     constexpr int G_W_TASKS = GN * 2 / G_THREADS;             // 32-weight decode tasks per thread and step
     constexpr int G_W_ELEMS = GN * GSTRIDE;
     // Register slots of the activation ring. Narrow tile: two (requested two steps ahead, like the weights). Wide tile:
     // one -- the second slot's 32 registers are what the 256 accumulators leave no room for: a step parks the slot in
     // LDS at its end and requests the step after next into it right away, a full step ahead of its own parking.
-    constexpr int A_SLOTS = WTN == 2 ? 2 : 1;
+    constexpr int A_SLOTS = WTM * WTN <= 8 ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) __bf16 smem[];
     // stage `buf` (0 / 1): activation tile, then weight tile
     auto a_tile = [&](int buf) { return smem + buf * (G_A_ELEMS + G_W_ELEMS); };
@@ -423,9 +426,9 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
         *reinterpret_cast<u32x4*>(dst + 8 * i) = u32x4{wp[t][4 * i], wp[t][4 * i + 1], wp[t][4 * i + 2], wp[t][4 * i + 3]};
     };
 
-    f32x16 acc[4][G_WTN];
+    f32x16 acc[WTM][G_WTN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < G_WTN; ++j)
 #pragma unroll
@@ -452,16 +455,16 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     auto step_body = [&](int stage, int slot_next, int step_next, int load_slot, int load_step) __attribute__((always_inline)) {
         const int a_slot_next = A_SLOTS == 2 ? slot_next : 0;
         const int a_load_slot = A_SLOTS == 2 ? load_slot : 0, a_load_step = A_SLOTS == 2 ? load_step : step_next + 1;
-        constexpr int N_MFMA = 4 * G_WTN * (GK / 16), N_HALVES = 16 * G_W_TASKS, N_STORES = G_A_LOADS + 4 * G_W_TASKS;
+        constexpr int N_MFMA = WTM * G_WTN * (GK / 16), N_HALVES = 16 * G_W_TASKS, N_STORES = G_A_LOADS + 4 * G_W_TASKS;
         constexpr int FIRST_ITEM = 2 * G_W_TASKS;                  // MFMAs whose slots hold the loads and the headers
         constexpr int N_GAPS = N_MFMA - N_STORES - FIRST_ITEM;      // MFMAs with a decode slot behind them
-        static_assert(N_GAPS >= N_HALVES, "more decode items than slots between the MFMAs");
-        const __bf16* at = a_tile(stage) + (128 * wm + fr) * GSTRIDE + fk;
+        static_assert(N_GAPS >= 1, "no slot between the MFMAs for the decode");   // the 128-row tiles put several items in a slot
+        const __bf16* at = a_tile(stage) + (32 * WTM * wm + fr) * GSTRIDE + fk;
         const __bf16* wt = w_tile(stage) + (32 * G_WTN * wn + fr) * GSTRIDE + fk;
-        bf16x8 af[2][4], bf[2][G_WTN];
+        bf16x8 af[2][WTM], bf[2][G_WTN];
         auto frags = [&](int set, int kk) __attribute__((always_inline)) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) af[set][i] = *reinterpret_cast<const bf16x8*>(at + 32 * i * GSTRIDE + kk);
+            for (int i = 0; i < WTM; ++i) af[set][i] = *reinterpret_cast<const bf16x8*>(at + 32 * i * GSTRIDE + kk);
 #pragma unroll
             for (int j = 0; j < G_WTN; ++j) bf[set][j] = *reinterpret_cast<const bf16x8*>(wt + 32 * j * GSTRIDE + kk);
         };
@@ -471,7 +474,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
         __builtin_amdgcn_sched_barrier(0);
 #pragma clang loop unroll(full)
         for (int q = 0; q < N_MFMA; ++q) {
-            const int kk = q / (4 * G_WTN), r = q % (4 * G_WTN), i = r / G_WTN, j = r % G_WTN, set = kk & 1;
+            const int kk = q / (WTM * G_WTN), r = q % (WTM * G_WTN), i = r / G_WTN, j = r % G_WTN, set = kk & 1;
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             if (r == 0 && kk + 1 < GK / 16) {                   // behind the slice's first MFMA: its wait covers only its own reads
@@ -486,11 +489,13 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
                 decode_prepare(wring[slot_next][t], step_k(step_next) + 32 * wsub, dc[t]);
                 __builtin_amdgcn_sched_barrier(0);
             } else if (q < FIRST_ITEM + N_GAPS) {
-                // decode item h sits behind MFMA FIRST_ITEM + h * N_GAPS / N_HALVES: evenly spread, at most one per slot
+                // decode item h sits behind MFMA FIRST_ITEM + h * N_GAPS / N_HALVES: evenly spread (the 256-row tiles have
+                // more slots than items: at most one per slot)
                 const int g = q - FIRST_ITEM;
                 const int h0 = (g * N_HALVES + N_GAPS - 1) / N_GAPS, h1 = ((g + 1) * N_HALVES + N_GAPS - 1) / N_GAPS;
-                if (h0 < h1 && h0 < N_HALVES) {
-                    wp[h0 / 16][h0 % 16] = decode_item_at(h0 % 16, wring[slot_next][h0 / 16], dc[h0 / 16], codes[h0 / 16]);
+#pragma clang loop unroll(full)
+                for (int hh = h0; hh < h1 && hh < N_HALVES; ++hh) {
+                    wp[hh / 16][hh % 16] = decode_item_at(hh % 16, wring[slot_next][hh / 16], dc[hh / 16], codes[hh / 16]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
@@ -547,24 +552,24 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     // the stores queue one behind the other (the compiler waits for everything in flight there).
     if (m0 + GM <= m && n0 + GN <= n) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < WTM; ++i)
 #pragma unroll
             for (int j = 0; j < G_WTN; ++j) {
-                float* dst = cz + (int64_t)(m0 + 128 * wm + 32 * i + 4 * (lane >> 5)) * n + n0 + 32 * G_WTN * wn + 32 * j + (lane & 31);
+                float* dst = cz + (int64_t)(m0 + 32 * WTM * wm + 32 * i + 4 * (lane >> 5)) * n + n0 + 32 * G_WTN * wn + 32 * j + (lane & 31);
 #pragma unroll
                 for (int e = 0; e < 16; ++e) dst[(int64_t)(8 * (e >> 2) + (e & 3)) * n] = acc[i][j][e];
             }
         return;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < G_WTN; ++j) {
             const int col = n0 + 32 * G_WTN * wn + 32 * j + (lane & 31);
             if (col >= n) continue;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int row = m0 + 128 * wm + 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                const int row = m0 + 32 * WTM * wm + 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (row < m) {
                     cz[(int64_t)row * n + col] = acc[i][j][e];
                 }
@@ -572,26 +577,32 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
         }
 }
 
-template <class Raw, int BE, int BB, int WTN>
+template <class Raw, int BE, int BB, int WTM, int WTN>
 static int launch_gemm_tile(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
                             int64_t split_stride, hipStream_t s) {
-    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&dequant_gemm_kernel<Raw, BE, BB, WTN>), gemm_smem(WTN));
+    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&dequant_gemm_kernel<Raw, BE, BB, WTM, WTN>), gemm_smem(WTM, WTN));
     note_kernel("dequant_gemm_kernel");
-    dequant_gemm_kernel<Raw, BE, BB, WTN><<<grid, dim3(G_THREADS), gemm_smem(WTN), s>>>(a, w, c, m, n, k, k_chunk, split_stride);
+    dequant_gemm_kernel<Raw, BE, BB, WTM, WTN><<<grid, dim3(G_THREADS), gemm_smem(WTM, WTN), s>>>(a, w, c, m, n, k, k_chunk, split_stride);
     SKH_CHECK(hipGetLastError());
     return 0;
 }
 template <class Raw, int BE, int BB>
-static int launch_gemm_enc(int wtn, const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
+static int launch_gemm_enc(int wtm, int wtn, const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, dim3 grid, int k_chunk,
                            int64_t split_stride, hipStream_t s) {
-    if (wtn == 4) return launch_gemm_tile<Raw, BE, BB, 4>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    return launch_gemm_tile<Raw, BE, BB, 2>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    if (wtm == 2) {
+        if (wtn == 4) return launch_gemm_tile<Raw, BE, BB, 2, 4>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+        return launch_gemm_tile<Raw, BE, BB, 2, 2>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    }
+    if (wtn == 4) return launch_gemm_tile<Raw, BE, BB, 4, 4>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    return launch_gemm_tile<Raw, BE, BB, 4, 2>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
 }
 
 static std::atomic<int> g_gemm_ksplit{0};   // 0 = choose from the tile count
 void set_gemm_ksplit(int v) { g_gemm_ksplit = v; }
 static std::atomic<int> g_gemm_wide{-1};    // -1 = choose from the shape, 0 / 1 = narrow / wide tile
 void set_gemm_wide(int v) { g_gemm_wide = v; }
+static std::atomic<int> g_gemm_rows{0};     // 0 = choose from the shape, 2 / 4 = 128 / 256 activation rows per tile
+void set_gemm_rows(int v) { if (v == 0 || v == 2 || v == 4) g_gemm_rows = v; }
 
 // y = epilogue(prologue(x) . W^T): gain != null normalises every activation row first (RMSNorm, folded into the pass that
 // rounds the activations to bf16); epilogue is one of GEMM_EPI_* (residual [m, n] may be y; SwiGLU: y is [m, n / 2]).
@@ -613,8 +624,11 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         (epilogue != GEMM_EPI_NONE && !tmp))
         return fused ? 1 : launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
-    // the wide tile where it alone fills most of the chip in one round
-    const int tiles_m = (m + GM - 1) / GM;
+    // 128 activation rows per tile where there are no more than that (the weight is then decoded once, and half the
+    // matrix work of the taller tile is not spent on rows that do not exist); the wide tile where it alone fills most of
+    // the chip in one round
+    const int wtm = g_gemm_rows.load() != 0 ? g_gemm_rows.load() : (m <= 128 ? 2 : 4);
+    const int tiles_m = (m + gemm_gm(wtm) - 1) / gemm_gm(wtm);
     const int wide_tiles = tiles_m * ((n + gemm_gn(4) - 1) / gemm_gn(4));
     const bool wide = g_gemm_wide.load() >= 0 ? g_gemm_wide.load() != 0 : 4 * wide_tiles >= 3 * num_cus();
     const int wtn = wide ? 4 : 2;
@@ -633,7 +647,8 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         for (int ks = 1; ks <= 8 && ks <= kgroups; ++ks) {
             const int rounds = (tiles * ks + cus - 1) / cus;
             const int steps = ((kgroups + ks - 1) / ks) * (256 / GK);
-            double t = rounds * (8.0 + (wide ? 2.0 : 1.04) * steps);
+            const double step_us = wtm == 4 ? (wide ? 2.0 : 1.04) : (wide ? 1.13 : 0.65);   // measured per tile shape
+            double t = rounds * (8.0 + step_us * steps);
             if (ks > 1) t += 2.3 + (double)(ks + 1) * m * n * 4.0 / 8.0e6;
             if (ks == 1 || t < best) { best = t; ksplit = ks; }
         }
@@ -656,13 +671,13 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     const dim3 grid(tiles_n, tiles_m, ksplit);
     float* c = ksplit > 1 ? part : (epilogue != GEMM_EPI_NONE ? tmp : y);
     int rc;
-    if (enc == ENC_Q4_K) rc = launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q6_K) rc = launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q5_K) rc = launch_gemm_enc<RawQ5K, QK_ELEMS, Q5K_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q4_0) rc = launch_gemm_enc<RawQ45<0>, Q80_ELEMS, Q40_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q5_0) rc = launch_gemm_enc<RawQ45<1>, Q80_ELEMS, Q50_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else if (enc == ENC_Q5_1) rc = launch_gemm_enc<RawQ45<2>, Q80_ELEMS, Q51_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
-    else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    if (enc == ENC_Q4_K) rc = launch_gemm_enc<RawQ4K, QK_ELEMS, Q4K_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q6_K) rc = launch_gemm_enc<RawQ6K, QK_ELEMS, Q6K_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_K) rc = launch_gemm_enc<RawQ5K, QK_ELEMS, Q5K_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q4_0) rc = launch_gemm_enc<RawQ45<0>, Q80_ELEMS, Q40_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_0) rc = launch_gemm_enc<RawQ45<1>, Q80_ELEMS, Q50_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else if (enc == ENC_Q5_1) rc = launch_gemm_enc<RawQ45<2>, Q80_ELEMS, Q51_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
+    else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     if (rc != 0) return rc;
     if (ksplit == 1) {
         if (epilogue == GEMM_EPI_RESIDUAL) return launch_add(residual, tmp, y, (int64_t)m * n);

@@ -81,16 +81,19 @@ def test_gemm_on_random_valid_blocks_and_forced_k_splits(hip_backend, torch_cuda
     x = np.random.default_rng(5).standard_normal((m, k)).astype(np.float32)
     want = L.gemv(enc, x, packed, n)
     try:
-        for wide in (0, 1):
-            hip_backend.set_tuning("gemm_wide", wide)
-            for ks in (1, 2, 3, 8):
-                hip_backend.set_tuning("gemm_ksplit", ks)
-                got = gpu_gemm(hip_backend, torch_cuda, enc, packed, n, k, x)
-                check(got, want)
-                check_exact(torch_cuda, enc, got, x, packed, n)
+        for rows in (2, 4):                      # 128 / 256 activation rows per tile (40 rows would pick 128 by itself)
+            hip_backend.set_tuning("gemm_rows", rows)
+            for wide in (0, 1):
+                hip_backend.set_tuning("gemm_wide", wide)
+                for ks in (1, 2, 3, 8):
+                    hip_backend.set_tuning("gemm_ksplit", ks)
+                    got = gpu_gemm(hip_backend, torch_cuda, enc, packed, n, k, x)
+                    check(got, want)
+                    check_exact(torch_cuda, enc, got, x, packed, n)
     finally:
         hip_backend.set_tuning("gemm_ksplit", 0)
         hip_backend.set_tuning("gemm_wide", -1)
+        hip_backend.set_tuning("gemm_rows", 0)
 
 
 @pytest.mark.parametrize("k", [96, 192, 320, 448])
