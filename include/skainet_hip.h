@@ -369,7 +369,8 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * kernel and run the fp32 row-streaming one), "q4k_mfma_window" (row quads that kernel keeps in flight per wave: 2 or 3,
  * 0 = chosen from K), "gemm_ksplit" (K splits of the MFMA GEMM,
  * 0 = automatic), "gemm_wide" (1 / 0: force the 256-column / 128-column tile, -1 = chosen from the shape), "gemm_rows" (2 / 4: 128 / 256
- * activation rows per tile, 0 = 128 up to 128 rows and 256 above),
+ * activation rows per tile, 0 = 128 up to 128 rows and 256 above), "gemm_ksw" (the Q4_K kernel that splits K over the
+ * waves of a workgroup: 0 never, 1 where the launcher's estimate favours it, 2 wherever it fits),
  * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_decode_split_keys" (least keys per split of
  * decode-shape attention, default 64), "attn_merge_enable" (0: skainet_hip_attn_out_proj_dev always merges the key
  * splits in a launch of its own), "attn_merge_max_keys" (most keys per split for which that entry leaves the merge to

@@ -597,6 +597,11 @@ static int launch_gemm_enc(int wtm, int wtn, const __bf16* a, const uint8_t* w, 
     return launch_gemm_tile<Raw, BE, BB, 4, 2>(a, w, c, m, n, k, grid, k_chunk, split_stride, s);
 }
 
+int launch_q4k_gemm_ksw(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s);   // gemm_q4k_ksw.hip
+bool gemm_ksw_enabled();
+bool gemm_ksw_fits(int m, int n, int k);
+bool gemm_ksw_forced();
+
 static std::atomic<int> g_gemm_ksplit{0};   // 0 = choose from the tile count
 void set_gemm_ksplit(int v) { g_gemm_ksplit = v; }
 static std::atomic<int> g_gemm_wide{-1};    // -1 = choose from the shape, 0 / 1 = narrow / wide tile
@@ -624,6 +629,28 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         (epilogue != GEMM_EPI_NONE && !tmp))
         return fused ? 1 : launch_gemv(enc, w, x, m, k, n, y);
     hipStream_t s = current_stream();
+    auto round_activations = [&](__bf16* a) -> int {            // fp32 -> bf16, with the RMSNorm of a fused call folded in
+        const int64_t n4 = (int64_t)m * k / 4;                  // k is a multiple of 64
+        if (!gain) gemm_prepass_kernel<<<dim3((unsigned)((n4 + 256 * PREPASS_UNROLL - 1) / (256 * PREPASS_UNROLL))), dim3(256), 0, s>>>(x, a, n4);
+        else if (k <= 256 * 4 * 4) gemm_prepass_rmsnorm_kernel<4><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
+        else gemm_prepass_rmsnorm_kernel<16><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
+        SKH_CHECK(hipGetLastError());
+        return 0;
+    };
+    auto finish = [&]() -> int {                                 // the epilogue of a product parked whole in tmp
+        if (epilogue == GEMM_EPI_RESIDUAL) return launch_add(residual, tmp, y, (int64_t)m * n);
+        if (epilogue == GEMM_EPI_SWIGLU) return launch_swiglu_pairs(tmp, y, (int64_t)m * (n / 2));
+        return 0;
+    };
+    auto run_ksw = [&]() -> int {                                // Q4_K: K split over the waves of a workgroup, 128 x 64 tiles
+        __bf16* a = static_cast<__bf16*>(kernel_workspace((size_t)m * k * sizeof(__bf16)));
+        if (!a) return -1;
+        if (round_activations(a) != 0) return -1;
+        if (launch_q4k_gemm_ksw(a, w, epilogue != GEMM_EPI_NONE ? tmp : y, m, n, k, s) != 0) return -1;
+        return finish();
+    };
+    const bool ksw_ok = enc == ENC_Q4_K && gemm_ksw_fits(m, n, k) && g_gemm_wide.load() < 0 && g_gemm_rows.load() == 0;
+    if (ksw_ok && gemm_ksw_forced()) return run_ksw();
     // 128 activation rows per tile where there are no more than that (the weight is then decoded once, and half the
     // matrix work of the taller tile is not spent on rows that do not exist); the wide tile where it alone fills most of
     // the chip in one round
@@ -637,6 +664,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     // K chunks are whole 256-element groups so every encoding's blocks stay intact
     const int kgroups = (k + 255) / 256;
     int ksplit = g_gemm_ksplit;
+    double tile_estimate = 0.0;
     if (ksplit <= 0) {
         // One workgroup is resident per CU, so the tile grid runs in rounds of num_cus() workgroups. Measured on this
         // kernel: about 8 us per round outside the K loop, 1.04 us per 64-element K step, and for the launch that sums
@@ -652,6 +680,14 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
             if (ks > 1) t += 2.3 + (double)(ks + 1) * m * n * 4.0 / 8.0e6;
             if (ks == 1 || t < best) { best = t; ksplit = ks; }
         }
+        tile_estimate = best;
+    }
+    if (ksw_ok && gemm_ksw_enabled() && g_gemm_ksplit.load() <= 0) {
+        // The kernel that splits K over the waves of a workgroup fills the chip with 128 x 64 tiles and parks no partial
+        // products; its step is slower (0.46 us per 64 elements of K measured, about 2 us per round outside the loop).
+        // It wins where the tile kernel would have to split K across workgroups: 512 x 4096 x 4096 is such a shape.
+        const int rounds = (((m + 127) / 128) * ((n + 63) / 64) + num_cus() - 1) / num_cus();
+        if (rounds * (2.0 + 0.46 * (k / GK)) < tile_estimate) return run_ksw();
     }
     if (ksplit > kgroups) ksplit = kgroups;
     const int k_chunk = ((kgroups + ksplit - 1) / ksplit) * 256;
@@ -663,11 +699,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     if (!ws) return -1;
     __bf16* a = reinterpret_cast<__bf16*>(ws);
     float* part = reinterpret_cast<float*>(ws + a_bytes);
-    const int64_t n4 = (int64_t)m * k / 4;                      // k is a multiple of 64
-    if (!gain) gemm_prepass_kernel<<<dim3((unsigned)((n4 + 256 * PREPASS_UNROLL - 1) / (256 * PREPASS_UNROLL))), dim3(256), 0, s>>>(x, a, n4);
-    else if (k <= 256 * 4 * 4) gemm_prepass_rmsnorm_kernel<4><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
-    else gemm_prepass_rmsnorm_kernel<16><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
-    SKH_CHECK(hipGetLastError());
+    if (round_activations(a) != 0) return -1;
     const dim3 grid(tiles_n, tiles_m, ksplit);
     float* c = ksplit > 1 ? part : (epilogue != GEMM_EPI_NONE ? tmp : y);
     int rc;
@@ -679,11 +711,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     else if (enc == ENC_Q5_1) rc = launch_gemm_enc<RawQ45<2>, Q80_ELEMS, Q51_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     else rc = launch_gemm_enc<RawQ80, Q80_ELEMS, Q80_BYTES>(wtm, wtn, a, w, c, m, n, k, grid, k_chunk, split_stride, s);
     if (rc != 0) return rc;
-    if (ksplit == 1) {
-        if (epilogue == GEMM_EPI_RESIDUAL) return launch_add(residual, tmp, y, (int64_t)m * n);
-        if (epilogue == GEMM_EPI_SWIGLU) return launch_swiglu_pairs(tmp, y, (int64_t)m * (n / 2));
-        return 0;
-    }
+    if (ksplit == 1) return finish();
     const int64_t total = (int64_t)m * n;
     gemm_splitk_sum_kernel<<<dim3((unsigned)((total / 4 + 256) / 256)), dim3(256), 0, s>>>(
         part, split_stride, ksplit, y, total, (reinterpret_cast<uintptr_t>(y) & 15) == 0, residual, epilogue);

@@ -128,3 +128,30 @@ def test_gemm_at_config_sizes(hip_backend, torch_cuda, enc, n, k):
     # and the GEMM agrees with the fp32 row kernels on the same device
     few = gpu_gemm(hip_backend, torch_cuda, enc, packed, n, k, x[:4].copy(), kind=0)
     check(got[:4], few)
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (9, 64, 256), (130, 70, 512), (128, 129, 1024), (300, 1000, 2304), (40, 200, 14336),
+                                   (257, 63, 768)])
+def test_q4k_gemm_with_k_split_over_the_waves(hip_backend, torch_cuda, m, n, k):
+    """The Q4_K kernel that gives every wave the whole 128 x 64 tile and a quarter of K, forced on shapes with ragged row
+    and column tiles, one and many super-blocks per row, and the shape the launcher picks it for by itself; against the
+    oracle (2e-2) and against the same product with both operands rounded to bf16 first (2e-4)."""
+    packed = gaussian_weight(hip_backend, "Q4_K", n, k, 900 + n)
+    x = np.random.default_rng(m * 7 + k).standard_normal((m, k)).astype(np.float32)
+    want = L.gemv("Q4_K", x, packed, n)
+    try:
+        hip_backend.set_tuning("gemm_ksw", 2)
+        got = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemm_ksw_kernel"
+        assert not np.isnan(got).any()
+        check(got, want)
+        check_exact(torch_cuda, "Q4_K", got, x, packed, n)
+        hip_backend.set_tuning("gemm_ksw", 0)
+        tiles = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "dequant_gemm_kernel"
+        assert normalized_err(got, tiles) <= 1e-4          # same operands, another fp32 summation order
+    finally:
+        hip_backend.set_tuning("gemm_ksw", 1)
+    if (m, n, k) == (512, 4096, 4096):
+        gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemm_ksw_kernel"      # the launcher's own choice for this shape
