@@ -372,7 +372,8 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * activation rows per tile, 0 = 128 up to 128 rows and 256 above), "gemm_ksw" (the Q4_K kernel that splits K over the
  * waves of a workgroup: 0 never, 1 where the launcher's estimate favours it, 2 wherever it fits),
  * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_decode_split_keys" (least keys per split of
- * decode-shape attention, default 64), "attn_merge_enable" (0: skainet_hip_attn_out_proj_dev always merges the key
+ * decode-shape attention, default 64), "sdpa_decode_gs" (query heads per workgroup of decode-shape attention: 1, 2 or 4, 0 = chosen from
+ * the shape), "attn_merge_enable" (0: skainet_hip_attn_out_proj_dev always merges the key
  * splits in a launch of its own), "attn_merge_max_keys" (most keys per split for which that entry leaves the merge to
  * the projection, default 176), "attn_merge_splits" (most key splits it then uses, 1 to 8, default 6).
  * 0 when the key is known. No reference counterpart. */

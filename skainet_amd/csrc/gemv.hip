@@ -575,6 +575,7 @@ void set_q4k_ksplit_enable(int v);
 void set_q4k_mfma_enable(int v);
 void set_q4k_mfma_window(int v);
 void set_attn_merge_enable(int v);
+void set_sdpa_decode_gs(int v);
 void set_attn_merge_max_keys(int v);
 void set_attn_merge_splits(int v);
 int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int n, int batch);   // gemv_q4k.hip
@@ -596,6 +597,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q4k_mfma_window")) { set_q4k_mfma_window(value); return 0; }
     if (!strcmp(key, "sdpa_decode_split_keys")) { set_sdpa_decode_split_keys(value); return 0; }
     if (!strcmp(key, "attn_merge_enable")) { set_attn_merge_enable(value); return 0; }
+    if (!strcmp(key, "sdpa_decode_gs")) { set_sdpa_decode_gs(value); return 0; }
     if (!strcmp(key, "attn_merge_max_keys")) { set_attn_merge_max_keys(value); return 0; }
     if (!strcmp(key, "attn_merge_splits")) { set_attn_merge_splits(value); return 0; }
     return -1;

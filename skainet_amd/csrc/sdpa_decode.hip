@@ -296,6 +296,8 @@ static int launch_decode_variant(const SdpaDecodeParams& p, int subs, bool merge
     return 1;
 }
 
+static std::atomic<int> g_sdpa_decode_gs{0};            // query heads per workgroup: 0 = chosen from the shape, else 1 / 2 / 4
+void set_sdpa_decode_gs(int v) { if (v == 0 || v == 1 || v == 2 || v == 4) g_sdpa_decode_gs = v; }
 static std::atomic<int> g_attn_merge_max_keys{176};    // most keys per split the unmerged form accepts (a multiple of 16)
 void set_attn_merge_max_keys(int v) { if (v >= 16) g_attn_merge_max_keys = (v + 15) & ~15; }
 // most splits the unmerged form uses. Measured in a Llama-3-8B decode step at 520 to 650 keys (ms per token): 2 splits 1.637,
@@ -315,8 +317,18 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
     if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) & 15) return 0;
     const int per_kv = heads / kv_heads;
     const int gs_max = head_dim == 256 ? 2 : 4;
-    int gs = gs_max;
+    int gs = g_sdpa_decode_gs.load() > 0 ? min(g_sdpa_decode_gs.load(), gs_max) : gs_max;
     while (per_kv % gs != 0) gs >>= 1;
+    // Few workgroups (one sequence at a short context, or splits capped for the projection that merges them): two query
+    // heads per workgroup instead of four. The K / V rows are then fetched by two workgroups (the second from L2), each
+    // with half the arithmetic per pass, and twice as many CUs take part: 1.502 against 1.526 ms per token in a
+    // Llama-3-8B decode step at 520 to 650 keys (one head per workgroup: 1.529).
+    if (g_sdpa_decode_gs.load() == 0 && gs == 4) {
+        const int64_t groups4 = (int64_t)batch * kv_heads * (per_kv / 4);
+        const int most = leave ? g_attn_merge_splits.load() : SDPA_DECODE_MAX_SPLITS;
+        const int splits4 = min(most, (seq_kv + g_sdpa_decode_split_keys - 1) / g_sdpa_decode_split_keys);
+        if (groups4 * splits4 < num_cus()) gs = 2;
+    }
     const int subs = per_kv / gs;
     if (batch > 65535) return 0;
     SdpaDecodeParams p{q, k, v, out, batch, heads, kv_heads, seq_kv, kv_capacity, scale, window, right_context, lengths, 1,
