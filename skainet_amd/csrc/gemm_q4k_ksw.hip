@@ -35,7 +35,8 @@ typedef uint32_t ksw_u32x2 __attribute__((ext_vector_type(2)));
 constexpr int KSW_M = 128, KSW_N = 64, KSW_K = 64;
 constexpr int KSW_ASTRIDE = KSW_K + 8;                        // bf16 elements per LDS row of the activation tile (144 bytes)
 constexpr int KSW_A_BYTES = KSW_M * KSW_ASTRIDE * 2;          // one stage of the activation tile
-constexpr int KSW_W_BYTES = KSW_N * 144;                      // one stage of raw super-blocks: 64 rows x 144 bytes
+constexpr int KSW_W_BYTES = 768 * 16;                         // one stage of raw super-blocks: 64 rows x 144 bytes = 576 pieces of 16
+                                                              // bytes, padded to three pieces per thread (the padding takes copies)
 constexpr int KSW_RED_PITCH = KSW_N + 4;                      // floats per row of a partial tile in the final exchange
 constexpr size_t KSW_LOOP_BYTES = 4 * (size_t)KSW_A_BYTES + 2 * (size_t)KSW_W_BYTES;
 constexpr size_t KSW_RED_BYTES = (size_t)4 * KSW_M * KSW_RED_PITCH * sizeof(float);
@@ -87,44 +88,44 @@ __global__ __launch_bounds__(256) void q4k_gemm_ksw_kernel(const __bf16* __restr
     const int64_t row_bytes = (int64_t)nsb * 144;
 
     // activation tile: thread t copies chunks t, t + 256, ... (4 of them): row = chunk / 8, 16-byte piece = chunk % 8
-    // (element offsets from `a` fit 32 bits: the launcher checks m * k)
+    // Both operands are read through buffer descriptors: a lane's byte offset is a constant register, the step's offset a
+    // scalar, so a load costs no address arithmetic (offsets fit 32 bits: the launcher checks the operand sizes).
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(a), 0, (int)0x7FFFFFFF, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(w), 0, (int)0x7FFFFFFF, 0x00020000);
     uint32_t a_off[4];
     int a_dst[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int p = tid + 256 * j, row = p >> 3, kp = p & 7;
-        a_off[j] = (uint32_t)min(m0 + row, m - 1) * (uint32_t)k + 8u * kp;   // rows past M: a valid copy, never stored
+        a_off[j] = ((uint32_t)min(m0 + row, m - 1) * (uint32_t)k + 8u * kp) * 2u;   // bytes; rows past M: a valid copy, never stored
         a_dst[j] = row * KSW_ASTRIDE + 8 * kp;
     }
     // raw super-blocks: 64 rows x 9 pieces of 16 bytes = 576 pieces, thread t copies pieces t, t + 256 and (t < 64) t + 512
-    // (byte offsets from `w` fit 32 bits: the launcher checks n * row_bytes)
     uint32_t w_off[3];
     int w_dst[3];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
         const int p = min(tid + 256 * j, 575), row = p / 9, pc = p - 9 * row;
         w_off[j] = (uint32_t)min(n0 + row, n - 1) * (uint32_t)row_bytes + pc * 16u;   // rows past N: a valid copy, never stored
-        w_dst[j] = p * 16;
+        w_dst[j] = (tid + 256 * j) * 16;                                             // pieces 576 .. 767: padding
     }
-    const bool w_third = tid < 64;
 
     ksw_u32x4 aring[2][4], wring[3];
     auto load_a_chunk = [&](int slot, int step, int j) __attribute__((always_inline)) {
-        const __bf16* base = a + (size_t)(min(step, nsteps - 1) * KSW_K);                                  // uniform; past the end: the last step again
-        aring[slot][j] = *reinterpret_cast<const ksw_u32x4*>(base + a_off[j]);
+        const int soff = min(step, nsteps - 1) * (KSW_K * 2);                                              // uniform; past the end: the last step again
+        aring[slot][j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)a_off[j], soff, 0);
     };
     auto park_a_chunk = [&](int slot, int stage, int j) __attribute__((always_inline)) {
         *reinterpret_cast<ksw_u32x4*>(a_stage(stage) + a_dst[j]) = aring[slot][j];
     };
     auto load_w = [&](int sb) __attribute__((always_inline)) {
-        const uint8_t* base = w + (size_t)(min(sb, nsb - 1) * 144);          // uniform
+        const int soff = min(sb, nsb - 1) * 144;                             // uniform
 #pragma unroll
-        for (int j = 0; j < 3; ++j) wring[j] = *reinterpret_cast<const ksw_u32x4*>(base + w_off[j]);
+        for (int j = 0; j < 3; ++j) wring[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)w_off[j], soff, 0);
     };
     auto park_w = [&](int stage) __attribute__((always_inline)) {
-        *reinterpret_cast<ksw_u32x4*>(w_stage(stage) + w_dst[0]) = wring[0];
-        *reinterpret_cast<ksw_u32x4*>(w_stage(stage) + w_dst[1]) = wring[1];
-        if (w_third) *reinterpret_cast<ksw_u32x4*>(w_stage(stage) + w_dst[2]) = wring[2];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) *reinterpret_cast<ksw_u32x4*>(w_stage(stage) + w_dst[j]) = wring[j];
     };
 
     ksw_f32x16 acc[4][2];
@@ -278,13 +279,13 @@ void set_gemm_ksw(int v) { if (v >= 0 && v <= 2) g_gemm_ksw = v; }
 bool gemm_ksw_enabled() { return g_gemm_ksw.load() != 0; }
 bool gemm_ksw_forced() { return g_gemm_ksw.load() == 2; }
 bool gemm_ksw_fits(int m, int n, int k) {
-    return (uint64_t)m * (uint64_t)k < ((uint64_t)1 << 32) && (uint64_t)n * (uint64_t)(k >> 8) * 144u < ((uint64_t)1 << 32);
+    return (uint64_t)m * (uint64_t)k < ((uint64_t)1 << 30) && (uint64_t)n * (uint64_t)(k >> 8) * 144u < ((uint64_t)1 << 31);   // 2 GiB each
 }
 
 // C = A . W^T for bf16 activations already in `a`; k a multiple of 256, operands 16-byte aligned, both operands below
 // 4 G elements / bytes (the caller checks, see gemm_ksw_fits). 0 on success.
 int launch_q4k_gemm_ksw(const __bf16* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s) {
-    if ((uint64_t)m * (uint64_t)k >= ((uint64_t)1 << 32) || (uint64_t)n * (uint64_t)(k >> 8) * 144u >= ((uint64_t)1 << 32))
+    if ((uint64_t)m * (uint64_t)k >= ((uint64_t)1 << 30) || (uint64_t)n * (uint64_t)(k >> 8) * 144u >= ((uint64_t)1 << 31))
         return set_error("gemm: operands of %d x %d x %d exceed the 32-bit offsets of this kernel", m, n, k);
     const dim3 grid((n + KSW_N - 1) / KSW_N, (m + KSW_M - 1) / KSW_M);
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_ksw_kernel), KSW_SMEM);
