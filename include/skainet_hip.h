@@ -370,7 +370,10 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * 0 = chosen from K), "gemm_ksplit" (K splits of the MFMA GEMM,
  * 0 = automatic), "gemm_wide" (1 / 0: force the 256-column / 128-column tile, -1 = chosen from the shape), "gemm_rows" (2 / 4: 128 / 256
  * activation rows per tile, 0 = 128 up to 128 rows and 256 above), "gemm_ksw" (the Q4_K kernel that splits K over the
- * waves of a workgroup: 0 never, 1 where the launcher's estimate favours it, 2 wherever it fits),
+ * waves of a workgroup: 0 never, 1 where the launcher's estimate favours it, 2 wherever it fits), "gemm_ksw_teams" (teams
+ * of four waves per workgroup of that kernel, each with its own share of K: 1 or 2, default 2; rows with an odd number
+ * of 256-element super-blocks always run one team), "gemm_ksw_stages" (activation tiles the one-team form keeps in LDS: 3 to 7,
+ * default 5),
  * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_decode_split_keys" (least keys per split of
  * decode-shape attention, default 64), "sdpa_decode_gs" (query heads per workgroup of decode-shape attention: 1, 2 or 4, 0 = chosen from
  * the shape), "attn_merge_enable" (0: skainet_hip_attn_out_proj_dev always merges the key

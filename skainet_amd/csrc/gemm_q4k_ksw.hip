@@ -7,19 +7,26 @@
 //   * workgroup tile 128 (M) x 64 (N): 512 x 4096 outputs are 256 tiles, one per CU, so the chip is full without
 //     splitting K across workgroups (no partial tiles parked in memory, no launch that sums them);
 //   * every wave owns the WHOLE tile (4 x 2 MFMA tiles of 32 x 32: 128 accumulator registers, each fragment read from
-//     LDS feeds two or four matrix instructions) and a quarter of K: in every 64-element step wave w takes the
-//     16-element slice w. The four partial tiles meet once, at the end, through LDS;
+//     LDS feeds two or four matrix instructions) and a share of K: in every 64-element step wave w of a team of four
+//     takes the 16-element slice w. The partial tiles meet once, at the end, through LDS;
 //   * a 16-element slice of a Q4_K row is one nibble plane (low for slices 0 and 1, high for 2 and 3) of 16 consecutive
 //     bytes, and lane (column n, half h) of the matrix instruction's B operand needs 8 of them: so a lane decodes exactly
 //     the 8 weights of each of its two columns that its own operand holds, straight into registers. Decoded weights never
-//     pass through LDS and nothing is decoded twice. The raw super-blocks (144 bytes per row and 256 elements) are copied
-//     into LDS once per four steps with plain coalesced 16-byte loads, so the lanes' 8-byte picks come out of LDS, not out
-//     of the cache hierarchy;
-//   * the activation tile of a step (128 rows x 64 elements, bf16) goes global -> registers -> LDS as in the other
-//     kernel, parked two steps ahead of its use (three LDS stages), so that a step's fragments are read while the
-//     previous step multiplies; one barrier per step. A step's weights are decoded during the previous step as well:
-//     between the 8 matrix instructions of a step sit, in pinned program order, the reads, the parking and the decode
-//     for the steps behind it.
+//     pass through LDS and nothing is decoded twice;
+//   * both operands come in by loads that write LDS directly (global_load_lds_dwordx4: no staging registers, no LDS
+//     store instructions; inline assembly with explicit wait counts, since the loads complete in issue order): the raw
+//     super-blocks (144 bytes per row and 256 elements, once per four steps) so that the lanes' 8-byte picks come out of
+//     LDS, and the activation tile of a step (128 rows x 64 elements, bf16) S - 1 steps ahead of the step that reads it.
+//     The lane chooses the source address, so the LDS layout is free: activation rows are 128 bytes with their 16-byte
+//     pieces XOR-swizzled by the row, which the fragment reads take without bank conflicts and without padding;
+//   * a step's fragments are read, and its weights decoded, during the previous step: between the 8 matrix
+//     instructions of a step sit, in pinned program order, the reads, the loads and the decode for the steps behind it;
+//     one barrier per step.
+// What bounds it (measured by compiling pieces out, 512 x 4096 x 4096, one launch 26 us): the launch, the prologue and
+// the final exchange and store 6.5 us; the matrix instructions alone 8.5 us on top; the loads alone 12 us on top (every
+// workgroup pulls its whole 1 MB row block of activations through L2: 311 MB per launch, 2/3 of what the L2s deliver);
+// decode and matrix instructions do not overlap on a SIMD (a vector instruction issued behind a matrix instruction
+// waits for it, also from another wave), so the decode's 44 vector instructions per step add their full time.
 #include "common.h"
 
 #include <type_traits>
@@ -33,14 +40,28 @@ typedef uint32_t ksw_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t ksw_u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int KSW_M = 128, KSW_N = 64, KSW_K = 64;
-constexpr int KSW_ASTRIDE = KSW_K + 8;                        // bf16 elements per LDS row of the activation tile (144 bytes)
-constexpr int KSW_A_BYTES = KSW_M * KSW_ASTRIDE * 2;          // one stage of the activation tile
-constexpr int KSW_W_BYTES = 768 * 16;                         // one stage of raw super-blocks: 64 rows x 144 bytes = 576 pieces of 16
-                                                              // bytes, padded to three pieces per thread (the padding takes copies)
+constexpr int KSW_A_BYTES = KSW_M * KSW_K * 2;                // one stage of the activation tile: rows of 128 bytes, no padding; the
+                                                              // 16-byte piece p of row r sits in slot p ^ ((r >> 1) & 7) of its row
+constexpr int KSW_W_BYTES = KSW_N * 144;                      // one stage of raw super-blocks: 64 rows x 144 bytes = 9 wave loads
+// Activation stages (template argument S, 3 .. 7): step s multiplies from registers, reads step s + 1 out of LDS and has
+// step s + S land in the stage step s has left: S - 2 steps between a load's issue and the barrier it must have landed by.
 constexpr int KSW_RED_PITCH = KSW_N + 4;                      // floats per row of a partial tile in the final exchange
-constexpr size_t KSW_LOOP_BYTES = 4 * (size_t)KSW_A_BYTES + 2 * (size_t)KSW_W_BYTES;
+constexpr size_t ksw_team_bytes(int stages) { return stages * (size_t)KSW_A_BYTES + 2 * (size_t)KSW_W_BYTES; }   // the loop's LDS of one team of four waves
 constexpr size_t KSW_RED_BYTES = (size_t)4 * KSW_M * KSW_RED_PITCH * sizeof(float);
-constexpr size_t KSW_SMEM = KSW_RED_BYTES > KSW_LOOP_BYTES ? KSW_RED_BYTES : KSW_LOOP_BYTES;
+constexpr size_t ksw_smem_bytes(int teams, int stages) { return KSW_RED_BYTES > teams * ksw_team_bytes(stages) ? KSW_RED_BYTES : teams * ksw_team_bytes(stages); }
+
+// 16 bytes per lane from base + off straight into LDS at lds_addr + 16 * lane (M0 carries the LDS address); counted by
+// vmcnt like any other load, in issue order
+__device__ __forceinline__ void ksw_dma16(uint32_t lds_addr, uint32_t off, const uint8_t* base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory");
+}
+// of the `steps` steps that end with step p of a super-block, how many are a step 3
+constexpr int ksw_count_p3(int p, int steps) {
+    int c = 0;
+    for (int d = 0; d < steps; ++d) c += (((p - d) % 4 + 4) % 4) == 3;
+    return c;
+}
+template <int N> __device__ __forceinline__ void ksw_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
 // The eight 6-bit scales and minima of a super-block header (ggml get_scale_min_k4) as bytes of four dwords: low four
 // sub-blocks, high four sub-blocks, each for scales and minima. `pre` shifts a wave's own sub-blocks (even or odd ones:
@@ -71,61 +92,55 @@ __device__ __forceinline__ void ksw_decode4(uint32_t c, float scale, float offse
     hi = __builtin_bit_cast(uint32_t, ksw_bf16x2{(__bf16)w2, (__bf16)w3});
 }
 
-constexpr int KSW_STAGES = 4;                                 // activation stages: parked two steps ahead of their use; four, so
-                                                              // that a step's stages are compile-time constants (step % 4)
+// TEAMS teams of four waves share a workgroup and its tile; team t runs the loop above on its own share of K (whole
+// super-blocks, TEAMS equal shares) out of its own part of LDS. With two teams a SIMD holds two waves, so one team's
+// decode and LDS traffic issue under the other's matrix instructions; the price is 256 registers per wave instead of 512
+// and one more exchange of partial tiles at the end.
+template <int TEAMS, int S>
+__global__ __launch_bounds__(256 * TEAMS) void q4k_gemm_ksw_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
+                                                                   float* __restrict__ c, int m, int n, int k) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t ksw_smem[];   // the kernel has no other LDS: offsets into it are LDS addresses
+    const int lane = threadIdx.x & 63;
+    const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int team = TEAMS == 1 ? 0 : wave_all >> 2, wave = wave_all & 3;
+    const uint32_t team_lds = (uint32_t)team * (uint32_t)ksw_team_bytes(S);
+    auto w_stage_off = [&](int s) { return team_lds + (uint32_t)(S * KSW_A_BYTES + s * KSW_W_BYTES); };
 
-__global__ __launch_bounds__(256) void q4k_gemm_ksw_kernel(const __bf16* __restrict__ a, const uint8_t* __restrict__ w,
-                                                           float* __restrict__ c, int m, int n, int k) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t ksw_smem[];
-    auto a_stage = [&](int s) { return reinterpret_cast<__bf16*>(ksw_smem + s * KSW_A_BYTES); };
-    auto w_stage = [&](int s) { return ksw_smem + KSW_STAGES * KSW_A_BYTES + s * KSW_W_BYTES; };
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, kh = lane >> 5;
     const int m0 = blockIdx.y * KSW_M, n0 = blockIdx.x * KSW_N;
-    const int nsteps = k / KSW_K;                              // k is a multiple of 256: whole super-blocks
-    const int nsb = k >> 8;
-    const int64_t row_bytes = (int64_t)nsb * 144;
+    const int nsb = (k >> 8) / TEAMS;                          // this team's super-blocks (the launcher checks divisibility)
+    const int nsteps = nsb * 4;
+    const uint32_t row_bytes = (uint32_t)(k >> 8) * 144u;
+    const uint8_t* const a_team = reinterpret_cast<const uint8_t*>(a) + (size_t)team * nsb * 512;   // the team's first column, bytes
+    const uint8_t* const w_team = w + (size_t)team * nsb * 144;
 
-    // activation tile: thread t copies chunks t, t + 256, ... (4 of them): row = chunk / 8, 16-byte piece = chunk % 8
-    // Both operands are read through buffer descriptors: a lane's byte offset is a constant register, the step's offset a
-    // scalar, so a load costs no address arithmetic (offsets fit 32 bits: the launcher checks the operand sizes).
-    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(a), 0, (int)0x7FFFFFFF, 0x00020000);
-    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(w), 0, (int)0x7FFFFFFF, 0x00020000);
-    uint32_t a_off[4];
-    int a_dst[4];
+    // Both operands come in by loads that write LDS directly (no registers, no store instruction). A wave load fills
+    // 1 KB of consecutive LDS, lane l the 16 bytes at 16 l, from whatever address the lane gives: so the LDS layout is
+    // chosen by the lane's source address. Offsets fit 32 bits (the launcher checks the operand sizes).
+    //   activation stage: wave load q = 4 j + wave covers rows 8 q .. 8 q + 7 (8 slots of 16 bytes each)
+    uint32_t a_voff[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int p = tid + 256 * j, row = p >> 3, kp = p & 7;
-        a_off[j] = ((uint32_t)min(m0 + row, m - 1) * (uint32_t)k + 8u * kp) * 2u;   // bytes; rows past M: a valid copy, never stored
-        a_dst[j] = row * KSW_ASTRIDE + 8 * kp;
+        const int row = 8 * (4 * j + wave) + (lane >> 3), piece = (lane & 7) ^ ((row >> 1) & 7);
+        a_voff[j] = (uint32_t)min(m0 + row, m - 1) * (uint32_t)k * 2u + 16u * piece;   // rows past M: a valid copy, never stored
     }
-    // raw super-blocks: 64 rows x 9 pieces of 16 bytes = 576 pieces, thread t copies pieces t, t + 256 and (t < 64) t + 512
-    uint32_t w_off[3];
-    int w_dst[3];
+    //   raw super-blocks: 576 pieces of 16 bytes in row order = 9 wave loads; wave w issues loads w, w + 4 and (all four
+    //   waves, so that every wave counts the same number of loads) 8
+    uint32_t w_voff[3];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-        const int p = min(tid + 256 * j, 575), row = p / 9, pc = p - 9 * row;
-        w_off[j] = (uint32_t)min(n0 + row, n - 1) * (uint32_t)row_bytes + pc * 16u;   // rows past N: a valid copy, never stored
-        w_dst[j] = (tid + 256 * j) * 16;                                             // pieces 576 .. 767: padding
+        const int p = 64 * (j < 2 ? wave + 4 * j : 8) + lane, row = p / 9, pc = p - 9 * row;
+        w_voff[j] = (uint32_t)min(n0 + row, n - 1) * row_bytes + 16u * pc;              // rows past N: a valid copy, never stored
     }
-
-    ksw_u32x4 aring[2][4], wring[3];
-    auto load_a_chunk = [&](int slot, int step, int j) __attribute__((always_inline)) {
-        const int soff = min(step, nsteps - 1) * (KSW_K * 2);                                              // uniform; past the end: the last step again
-        aring[slot][j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)a_off[j], soff, 0);
-    };
-    auto park_a_chunk = [&](int slot, int stage, int j) __attribute__((always_inline)) {
-        *reinterpret_cast<ksw_u32x4*>(a_stage(stage) + a_dst[j]) = aring[slot][j];
-    };
-    auto load_w = [&](int sb) __attribute__((always_inline)) {
-        const int soff = min(sb, nsb - 1) * 144;                             // uniform
+    auto dma_a = [&](uint32_t stage_off, int step) __attribute__((always_inline)) {
+        const uint8_t* base = a_team + (size_t)min(step, nsteps - 1) * (KSW_K * 2);     // uniform; past the end: the last step again
 #pragma unroll
-        for (int j = 0; j < 3; ++j) wring[j] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)w_off[j], soff, 0);
+        for (int j = 0; j < 4; ++j) ksw_dma16(stage_off + 1024u * (4 * j + wave), a_voff[j], base);
     };
-    auto park_w = [&](int stage) __attribute__((always_inline)) {
+    auto dma_w = [&](uint32_t stage_off, int sb) __attribute__((always_inline)) {
+        const uint8_t* base = w_team + (size_t)min(sb, nsb - 1) * 144;                 // uniform
 #pragma unroll
-        for (int j = 0; j < 3; ++j) *reinterpret_cast<ksw_u32x4*>(w_stage(stage) + w_dst[j]) = wring[j];
+        for (int j = 0; j < 3; ++j) ksw_dma16(stage_off + 1024u * (j < 2 ? wave + 4 * j : 8), w_voff[j], base);
     };
 
     ksw_f32x16 acc[4][2];
@@ -139,43 +154,43 @@ __global__ __launch_bounds__(256) void q4k_gemm_ksw_kernel(const __bf16* __restr
     // this lane's picks: rows col and col + 32 of the weight tile; in step p of a super-block the 8 bytes at
     // 16 + 32 p + 16 (wave & 1) + 8 kh of the block, low nibbles for waves 0 and 1, high nibbles for waves 2 and 3
     const int hi_plane = wave >> 1;
-    const int w_row0 = col * 144, w_row1 = (col + 32) * 144;
-    const int w_pick = 16 + 16 * (wave & 1) + 8 * kh;
+    const int w_pick = col * 144 + 16 + 16 * (wave & 1) + 8 * kh;          // row col + 32: 32 * 144 bytes further
+    const int w_hdr = col * 144;
     const uint32_t nib_mask = 0x0F0F0F0Fu << (4 * hi_plane);
     const float nib_scale = hi_plane ? 0.0625f : 1.0f;
-    const int a_frag = col * KSW_ASTRIDE + 16 * wave + 8 * kh;              // + 32 i rows per MFMA row tile
+    // fragment of MFMA row tile i: row col + 32 i, elements 16 wave + 8 kh ..: piece 2 wave + kh, swizzled by the row
+    const int a_frag = col * (KSW_K * 2) + 16 * ((2 * wave + kh) ^ ((col >> 1) & 7));
 
-    auto read_frags = [&](ksw_bf16x8 (&af)[4], int stage) __attribute__((always_inline)) {
+    auto read_frags = [&](ksw_bf16x8 (&af)[4], uint32_t stage_off) __attribute__((always_inline)) {
+        const uint8_t* p = ksw_smem + (stage_off + (uint32_t)a_frag);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const ksw_bf16x8*>(a_stage(stage) + a_frag + 32 * i * KSW_ASTRIDE);
+        for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const ksw_bf16x8*>(p + 32 * i * (KSW_K * 2));
     };
     auto read_raw = [&](ksw_u32x2 (&raw)[2], int wstage, int p) __attribute__((always_inline)) {
-        raw[0] = *reinterpret_cast<const ksw_u32x2*>(w_stage(wstage) + w_row0 + w_pick + 32 * p);
-        raw[1] = *reinterpret_cast<const ksw_u32x2*>(w_stage(wstage) + w_row1 + w_pick + 32 * p);
+        const uint8_t* q = ksw_smem + (w_stage_off(wstage) + (uint32_t)w_pick);
+        raw[0] = *reinterpret_cast<const ksw_u32x2*>(q + 32 * p);
+        raw[1] = *reinterpret_cast<const ksw_u32x2*>(q + 32 * p + 32 * 144);
     };
     auto read_scales = [&](KswScales (&ks)[2], int wstage) __attribute__((always_inline)) {
-        ks[0] = ksw_unpack(*reinterpret_cast<const ksw_u32x4*>(w_stage(wstage) + w_row0), 8 * hi_plane, nib_scale);
-        ks[1] = ksw_unpack(*reinterpret_cast<const ksw_u32x4*>(w_stage(wstage) + w_row1), 8 * hi_plane, nib_scale);
+        const uint8_t* q = ksw_smem + (w_stage_off(wstage) + (uint32_t)w_hdr);
+        ks[0] = ksw_unpack(*reinterpret_cast<const ksw_u32x4*>(q), 8 * hi_plane, nib_scale);
+        ks[1] = ksw_unpack(*reinterpret_cast<const ksw_u32x4*>(q + 32 * 144), 8 * hi_plane, nib_scale);
     };
 
-    // Prologue: steps 0 and 1 parked, steps 2 and 3 on their way in the ring, super-block 0 parked and 1 on its way;
-    // fragments, scales and decoded weights of step 0 in registers.
+    // Prologue: steps 0 .. S - 1 and super-blocks 0 and 1 in LDS; fragments, scales and decoded weights of step 0 in
+    // registers. st[i]: the stage of the step i after the current one (they rotate).
+    uint32_t st[S];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) { load_a_chunk(0, 0, j); load_a_chunk(1, 1, j); }
-    load_w(0);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) { park_a_chunk(0, 0, j); park_a_chunk(1, 1, j); }
-    park_w(0);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) { load_a_chunk(0, 2, j); load_a_chunk(1, 3, j); }
-    load_w(1);
+    for (int i = 0; i < S; ++i) { st[i] = team_lds + i * KSW_A_BYTES; dma_a(st[i], i); }
+    dma_w(w_stage_off(0), 0); dma_w(w_stage_off(1), 1);
+    ksw_wait_loads<0>();
     __syncthreads();
 
     ksw_bf16x8 af[2][4];                       // fragments of the step being multiplied and of the next one
     uint32_t bw[2][2][4];                      // [set][column tile][dword]: decoded B operands
     ksw_u32x2 raw[2];
-    KswScales ks[2], ks_next[2];
-    read_frags(af[0], 0);
+    KswScales ks[2];
+    read_frags(af[0], st[0]);
     read_raw(raw, 0, 0);
     read_scales(ks, 0);
     {
@@ -187,18 +202,21 @@ __global__ __launch_bounds__(256) void q4k_gemm_ksw_kernel(const __bf16* __restr
             ksw_decode4(raw[j].y & nib_mask, sc, of, bw[0][j][2], bw[0][j][3]);
         }
     }
+    __syncthreads();                           // every wave has read stage 0 before step 0 lets step 3 land in it
 
     // One step: the 8 matrix instructions of step `step` (fragments and weights already in registers, set `P & 1`), and
     // between them, in program order, everything that prepares later steps:
-    //   behind MFMA 0   the LDS reads of the next step's fragments and raw codes
-    //   behind MFMA 1-2 the activation tile of step + 2 parked (two chunks each), each ring register refilled with step + 4
-    //   behind MFMA 3   the next step's scales (and, in step 2 of a super-block, the next super-block's header unpacked)
+    //   behind MFMA 0   the LDS reads of the next step's fragments and raw codes (in step 3 of a super-block: the next
+    //                   super-block's header as well)
+    //   behind MFMA 1   the loads of step + S into the stage this step has left (its fragments were read a step ago),
+    //                   and in step 3 of a super-block the loads of super-block + 2 into the stage this one has left
+    //   behind MFMA 3   the next step's scales
     //   behind MFMA 4-7 the next step's weights decoded, four at a time
-    // then one barrier. sched_barrier(0) pins the order.
+    // then a wait for the loads issued a step ago (step + 2 must be readable in the next step) and one barrier.
+    // sched_barrier(0) pins the order.
     auto step_body = [&](auto pc, int s0) __attribute__((always_inline)) {
         constexpr int P = decltype(pc)::value, SET = P & 1, NP = (P + 1) & 3;
         const int step = s0 + P, sb = s0 >> 2, ws = sb & 1;
-        constexpr int st_next = (P + 1) % KSW_STAGES, st_park = (P + 2) % KSW_STAGES;   // s0 is a multiple of 4
         float sc[2], of[2];
         ksw_bf16x8 b[2];
 #pragma unroll
@@ -209,26 +227,30 @@ __global__ __launch_bounds__(256) void q4k_gemm_ksw_kernel(const __bf16* __restr
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[SET][i], b[j], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             if (q == 0) {
-                read_frags(af[SET ^ 1], st_next);
+                read_frags(af[SET ^ 1], st[1]);
                 read_raw(raw, P == 3 ? ws ^ 1 : ws, NP);
-                if (P == 2) read_scales(ks_next, ws ^ 1);                   // parked during step 1, behind that step's barrier
-            } else if (q == 1 || q == 2) {
-                const int j0 = 2 * (q - 1);
-                park_a_chunk(P & 1, st_park, j0); park_a_chunk(P & 1, st_park, j0 + 1);
-                load_a_chunk(P & 1, step + 4, j0); load_a_chunk(P & 1, step + 4, j0 + 1);
+                if (P == 3) read_scales(ks, ws ^ 1);                        // this block's last use of ks was in step 2
+            } else if (q == 1) {
+                dma_a(st[0], step + S);
+                if (P == 3) dma_w(w_stage_off(ws), sb + 2);                 // read for the last time a step ago
             } else if (q == 3) {
-                if (P == 3) { ks[0] = ks_next[0]; ks[1] = ks_next[1]; }
                 ksw_step_scale<NP>(ks[0], sc[0], of[0]);
                 ksw_step_scale<NP>(ks[1], sc[1], of[1]);
-                if (P == 1) park_w(ws ^ 1);                                 // the next super-block's raw bytes, loaded a trip ago
-                if (P == 2) load_w(sb + 2);
-            } else {
+            } else if (q >= 4) {
                 const int jj = (q - 4) >> 1, half = (q - 4) & 1;
                 ksw_decode4((half ? raw[jj].y : raw[jj].x) & nib_mask, sc[jj], of[jj], bw[SET ^ 1][jj][2 * half], bw[SET ^ 1][jj][2 * half + 1]);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        // Loads complete in issue order: step + 2 (issued S - 2 steps ago) must have landed, so everything issued in the
+        // S - 2 steps up to this one may still fly: 4 activation loads a step and the 3 of a super-block in its step 3.
+        constexpr int in_flight = 4 * (S - 2) + 3 * ksw_count_p3(P, S - 2);
+        ksw_wait_loads<in_flight>();
         __syncthreads();
+        const uint32_t t = st[0];
+#pragma unroll
+        for (int i = 0; i + 1 < S; ++i) st[i] = st[i + 1];
+        st[S - 1] = t;
     };
 
     for (int s0 = 0; s0 < nsteps; s0 += 4) {                               // one super-block (four steps) per trip
@@ -237,23 +259,50 @@ __global__ __launch_bounds__(256) void q4k_gemm_ksw_kernel(const __bf16* __restr
         step_body(std::integral_constant<int, 2>{}, s0);
         step_body(std::integral_constant<int, 3>{}, s0);
     }
+    ksw_wait_loads<0>();                       // the loads past the end still write LDS
+    __syncthreads();
 
-    // The four waves hold partial sums of the same 128 x 64 tile: park them, then wave v adds up rows 32 v .. 32 v + 31.
+    // The waves hold partial sums of the same 128 x 64 tile: park them, then every wave adds up its share of the rows.
     // Accumulator element e of lane l: row 8 (e / 4) + 4 (l / 32) + e % 4, column l % 32 of its 32 x 32 tile.
+    // With two teams the second team's tiles go through LDS first, each into the accumulators of the first team's wave
+    // of the same number (same lane, same element: the addresses a lane reads are the ones its twin wrote).
     float* red = reinterpret_cast<float*>(ksw_smem);
     float* mine = red + (size_t)wave * KSW_M * KSW_RED_PITCH;
+    auto tile_at = [&](int i, int j, int e) -> float& { return mine[(32 * i + 8 * (e >> 2) + 4 * kh + (e & 3)) * KSW_RED_PITCH + 32 * j + col]; };
+    if (TEAMS == 2) {
+        if (team == 1) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
-                mine[(32 * i + 8 * (e >> 2) + 4 * kh + (e & 3)) * KSW_RED_PITCH + 32 * j + col] = acc[i][j][e];
+                    for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
+        }
+        __syncthreads();
+        if (team == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[i][j][e] += tile_at(i, j, e);
+        }
+        __syncthreads();
+    }
+    if (team == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
+    }
     __syncthreads();
     const int c4 = (lane & 15) * 4;
+    constexpr int ROWS_PER_WAVE = KSW_M / (4 * TEAMS);
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int row = 32 * wave + 4 * it + (lane >> 4);
+    for (int it = 0; it < ROWS_PER_WAVE / 4; ++it) {
+        const int row = ROWS_PER_WAVE * wave_all + 4 * it + (lane >> 4);
         float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -276,6 +325,10 @@ __global__ __launch_bounds__(256) void q4k_gemm_ksw_kernel(const __bf16* __restr
 
 static std::atomic<int> g_gemm_ksw{1};      // 0 never, 1 where the launcher's estimate favours it, 2 wherever it fits
 void set_gemm_ksw(int v) { if (v >= 0 && v <= 2) g_gemm_ksw = v; }
+static std::atomic<int> g_gemm_ksw_teams{2};   // teams of four waves per workgroup (1 or 2)
+void set_gemm_ksw_teams(int v) { if (v == 1 || v == 2) g_gemm_ksw_teams = v; }
+static std::atomic<int> g_gemm_ksw_stages{5};  // activation stages of the one-team form (3 .. 7)
+void set_gemm_ksw_stages(int v) { if (v >= 3 && v <= 7) g_gemm_ksw_stages = v; }
 bool gemm_ksw_enabled() { return g_gemm_ksw.load() != 0; }
 bool gemm_ksw_forced() { return g_gemm_ksw.load() == 2; }
 bool gemm_ksw_fits(int m, int n, int k) {
@@ -288,9 +341,20 @@ int launch_q4k_gemm_ksw(const __bf16* a, const uint8_t* w, float* c, int m, int 
     if ((uint64_t)m * (uint64_t)k >= ((uint64_t)1 << 30) || (uint64_t)n * (uint64_t)(k >> 8) * 144u >= ((uint64_t)1 << 31))
         return set_error("gemm: operands of %d x %d x %d exceed the 32-bit offsets of this kernel", m, n, k);
     const dim3 grid((n + KSW_N - 1) / KSW_N, (m + KSW_M - 1) / KSW_M);
-    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_ksw_kernel), KSW_SMEM);
     note_kernel("q4k_gemm_ksw_kernel");
-    q4k_gemm_ksw_kernel<<<grid, dim3(256), KSW_SMEM, s>>>(a, w, c, m, n, k);
+    const int teams = g_gemm_ksw_teams.load(), stages = g_gemm_ksw_stages.load();
+#define SKH_KSW_LAUNCH(T, ST)                                                                              \
+    do {                                                                                                   \
+        SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_ksw_kernel<T, ST>), ksw_smem_bytes(T, ST));                \
+        q4k_gemm_ksw_kernel<T, ST><<<grid, dim3(256 * T), ksw_smem_bytes(T, ST), s>>>(a, w, c, m, n, k);   \
+    } while (0)
+    if (teams == 2 && ((k >> 8) & 1) == 0) SKH_KSW_LAUNCH(2, 3);   // two teams take half of K each: an even number of super-blocks
+    else if (stages <= 3) SKH_KSW_LAUNCH(1, 3);
+    else if (stages == 4) SKH_KSW_LAUNCH(1, 4);
+    else if (stages == 5) SKH_KSW_LAUNCH(1, 5);
+    else if (stages == 6) SKH_KSW_LAUNCH(1, 6);
+    else SKH_KSW_LAUNCH(1, 7);
+#undef SKH_KSW_LAUNCH
     SKH_CHECK(hipGetLastError());
     return 0;
 }

@@ -569,6 +569,8 @@ void set_gemm_wide(int v);
 void set_gemm_ksplit(int v);
 void set_gemm_rows(int v);
 void set_gemm_ksw(int v);
+void set_gemm_ksw_teams(int v);
+void set_gemm_ksw_stages(int v);
 void set_sdpa_prefill_mfma(int v);
 void set_sdpa_decode_split_keys(int v);
 void set_q4k_ksplit_enable(int v);
@@ -591,6 +593,8 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "gemm_ksplit")) { set_gemm_ksplit(value); return 0; }
     if (!strcmp(key, "gemm_rows")) { set_gemm_rows(value); return 0; }
     if (!strcmp(key, "gemm_ksw")) { set_gemm_ksw(value); return 0; }
+    if (!strcmp(key, "gemm_ksw_teams")) { set_gemm_ksw_teams(value); return 0; }
+    if (!strcmp(key, "gemm_ksw_stages")) { set_gemm_ksw_stages(value); return 0; }
     if (!strcmp(key, "sdpa_prefill_mfma")) { set_sdpa_prefill_mfma(value); return 0; }
     if (!strcmp(key, "q4k_ksplit_enable")) { set_q4k_ksplit_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_enable")) { set_q4k_mfma_enable(value); return 0; }

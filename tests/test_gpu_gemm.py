@@ -133,7 +133,7 @@ def test_gemm_at_config_sizes(hip_backend, torch_cuda, enc, n, k):
 @pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (9, 64, 256), (130, 70, 512), (128, 129, 1024), (300, 1000, 2304), (40, 200, 14336),
                                    (257, 63, 768)])
 def test_q4k_gemm_with_k_split_over_the_waves(hip_backend, torch_cuda, m, n, k):
-    """The Q4_K kernel that gives every wave the whole 128 x 64 tile and a quarter of K, forced on shapes with ragged row
+    """The Q4_K kernel that gives every wave the whole 128 x 64 tile and a share of K, forced on shapes with ragged row
     and column tiles, one and many super-blocks per row, and the shape the launcher picks it for by itself; against the
     oracle (2e-2) and against the same product with both operands rounded to bf16 first (2e-4)."""
     packed = gaussian_weight(hip_backend, "Q4_K", n, k, 900 + n)
@@ -146,12 +146,22 @@ def test_q4k_gemm_with_k_split_over_the_waves(hip_backend, torch_cuda, m, n, k):
         assert not np.isnan(got).any()
         check(got, want)
         check_exact(torch_cuda, "Q4_K", got, x, packed, n)
+        # one team of four waves per workgroup instead of two (each team takes half of K where the super-blocks split
+        # evenly), with the fewest and the most activation stages in LDS: same operands, another fp32 summation order
+        for stages in (3, 7):
+            hip_backend.set_tuning("gemm_ksw_teams", 1)
+            hip_backend.set_tuning("gemm_ksw_stages", stages)
+            one_team = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+            assert hip_backend.last_kernel() == "q4k_gemm_ksw_kernel"
+            assert normalized_err(got, one_team) <= 1e-4
         hip_backend.set_tuning("gemm_ksw", 0)
         tiles = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
         assert hip_backend.last_kernel() == "dequant_gemm_kernel"
         assert normalized_err(got, tiles) <= 1e-4          # same operands, another fp32 summation order
     finally:
         hip_backend.set_tuning("gemm_ksw", 1)
+        hip_backend.set_tuning("gemm_ksw_teams", 2)
+        hip_backend.set_tuning("gemm_ksw_stages", 5)
     if (m, n, k) == (512, 4096, 4096):
         gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
         assert hip_backend.last_kernel() == "q4k_gemm_ksw_kernel"      # the launcher's own choice for this shape
