@@ -684,10 +684,10 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     }
     if (ksw_ok && gemm_ksw_enabled() && g_gemm_ksplit.load() <= 0) {
         // The kernel that splits K over the waves of a workgroup fills the chip with 128 x 64 tiles and parks no partial
-        // products; its step is slower (0.46 us per 64 elements of K measured, about 2 us per round outside the loop).
+        // products; its step is slower per tile row (0.31 us per 64 elements of K measured, 6.5 us per round outside the loop).
         // It wins where the tile kernel would have to split K across workgroups: 512 x 4096 x 4096 is such a shape.
         const int rounds = (((m + 127) / 128) * ((n + 63) / 64) + num_cus() - 1) / num_cus();
-        if (rounds * (2.0 + 0.46 * (k / GK)) < tile_estimate) return run_ksw();
+        if (rounds * (6.5 + 0.31 * (k / GK)) < tile_estimate) return run_ksw();
     }
     if (ksplit > kgroups) ksplit = kgroups;
     const int k_chunk = ((kgroups + ksplit - 1) / ksplit) * 256;

@@ -149,6 +149,7 @@ def test_q6k_batch1_slot_variants_agree_with_the_oracle(hip_backend, torch_cuda,
     batched kernel: the same bound against the exact-fp32 oracle, on quantised Gaussian weights and on random valid
     blocks; rows of one super-block, rows longer than one wave pass, ragged last workgroups."""
     hip_backend.set_tuning("q6k_slot64", slot64)
+    hip_backend.set_tuning("gemv_stream_enable", 0)      # the row kernel's two slot shapes are what this test compares
     try:
         for packed in (gaussian_weight(hip_backend, "Q6_K", n, k, 81), random_valid_blocks("Q6_K", n * k // 256, 82)):
             x = np.random.default_rng(83).standard_normal((1, k)).astype(np.float32)
@@ -160,6 +161,39 @@ def test_q6k_batch1_slot_variants_agree_with_the_oracle(hip_backend, torch_cuda,
             assert err <= GEMV_TOL
     finally:
         hip_backend.set_tuning("q6k_slot64", 1)
+        hip_backend.set_tuning("gemv_stream_enable", 1)
+
+
+STREAM_ENCS = ["Q8_0", "Q4_0", "Q5_0", "Q5_1"]
+
+
+@pytest.mark.parametrize("enc", STREAM_ENCS)
+@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (1000, 4096), (1027, 2048), (70, 768), (33, 256), (5000, 1024), (3, 4096),
+                                 (2100, 8192)])
+def test_one_row_products_streamed_through_lds(hip_backend, torch_cuda, enc, n, k):
+    """One activation row against the formats of 32-element blocks: rows whose byte length is a multiple of 16 and
+    that have at most 128 blocks take the kernel that streams each wave's rows through LDS; the others stay on the row
+    kernel. Both against the exact-fp32 oracle (1e-3), and against each other (same products, another
+    summation order). Shapes: one, two and many units per wave, ragged last waves and workgroups, fewer rows than waves,
+    rows shorter than a wave's 64 slots."""
+    bs, bb = G.PACKED[enc][0], G.PACKED[enc][1]
+    row_bytes = k // bs * bb
+    eligible = row_bytes % 16 == 0 and k // 32 <= 128
+    packed = gaussian_weight(hip_backend, enc, n, k, 61) if n * k >= 1 << 22 else random_valid_blocks(enc, n * k // bs, 62 + n)
+    x = np.random.default_rng(63 + k).standard_normal((1, k)).astype(np.float32)
+    x[0, 5] = -41.0
+    want = L.gemv(enc, x, packed, n)
+    got = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x)
+    assert hip_backend.last_kernel() == ("gemv_stream_kernel" if eligible else "gemv_kernel")
+    assert not np.isnan(got).any()
+    assert normalized_err(got, want) <= GEMV_TOL
+    try:
+        hip_backend.set_tuning("gemv_stream_enable", 0)
+        rows = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x)
+        assert hip_backend.last_kernel() == "gemv_kernel"
+    finally:
+        hip_backend.set_tuning("gemv_stream_enable", 1)
+    assert normalized_err(got, rows) <= 2e-5
 
 
 @pytest.mark.parametrize("n,k,m", [(5, 256, 3), (25, 1280, 8), (77, 2304, 7), (1000, 11008, 4), (11008, 4096, 6), (4096, 14336, 8),
