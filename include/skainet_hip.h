@@ -363,6 +363,8 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
 
 /* Launch-shape knobs for experiments (defaults are the measured best). Keys: "gemv_waves_per_cu",
  * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares, 0 = chosen from the shape),
+ * "gemv_stream_enable" (0: one-row Q8_0 / Q4_0 / Q5_0 / Q5_1 products stay on the row kernel instead of the one that
+ * streams each wave's rows through LDS),
  * "q4k_rows_enable" (0: Q4_K decode shapes take the generic slot kernel), "q6k_slot64" (0: Q6_K at batch 1 keeps the
  * 32-weight slot of the batched kernel), "q4k_ksplit_enable" (0: long Q4_K rows are not
  * split over the waves of a workgroup), "q4k_mfma_enable" (0: one-row Q4_K products stay off the integer matrix-core

@@ -62,6 +62,9 @@ constexpr int ksw_count_p3(int p, int steps) {
     return c;
 }
 template <int N> __device__ __forceinline__ void ksw_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// the same, and this wave's LDS reads have returned as well: behind the barrier that follows, another wave's loads may
+// overwrite the stage they read
+template <int N> __device__ __forceinline__ void ksw_wait_loads_and_reads() { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(N) : "memory"); }
 
 // The eight 6-bit scales and minima of a super-block header (ggml get_scale_min_k4) as bytes of four dwords: low four
 // sub-blocks, high four sub-blocks, each for scales and minima. `pre` shifts a wave's own sub-blocks (even or odd ones:
@@ -244,8 +247,11 @@ __global__ __launch_bounds__(256 * TEAMS) void q4k_gemm_ksw_kernel(const __bf16*
         }
         // Loads complete in issue order: step + 2 (issued S - 2 steps ago) must have landed, so everything issued in the
         // S - 2 steps up to this one may still fly: 4 activation loads a step and the 3 of a super-block in its step 3.
-        constexpr int in_flight = 4 * (S - 2) + 3 * ksw_count_p3(P, S - 2);
-        ksw_wait_loads<in_flight>();
+        // The raw super-block requested in step 3 of the previous super-block is read from step 3 of this one on: at the
+        // end of step 2 only the 12 activation loads issued since may still fly.
+        constexpr int in_flight_a = 4 * (S - 2) + 3 * ksw_count_p3(P, S - 2);
+        constexpr int in_flight = P == 2 && in_flight_a > 12 ? 12 : in_flight_a;
+        ksw_wait_loads_and_reads<in_flight>();
         __syncthreads();
         const uint32_t t = st[0];
 #pragma unroll
