@@ -3,12 +3,15 @@
 //
 // Contract: the reference's skainet_f32_sdpa
 //   /root/reference/skainet-backends/skainet-backend-native-cpu/native/src/f32_fused.c:290-396
-// restricted to what a prompt pass uses: no additive mask, seq_q <= seq_kv, head_dim 64 or 128; causal or full, with
-// or without a sliding window (window, rightContext) and per-sequence key lengths, by the rules of
+// restricted to what a prompt pass uses: seq_q <= seq_kv, head_dim 64 or 128; causal or full, with or without a
+// sliding window (window, rightContext) and per-sequence key lengths, by the rules of
 //   /root/reference/skainet-lang/skainet-lang-core/src/commonMain/kotlin/sk/ainet/lang/tensor/ops/AttentionMask.kt:24-104
-// Every other call stays on the general fp32 kernel (sdpa.hip). A query whose rules leave it at least one key gives
-// the same result whether excluded keys score -1e30 (the reference) or take no part (here); a query they leave none
-// weighs every key of the sequence equally, as the reference's row of equal scores does.
+// and with or without an additive mask broadcast over [B|1, H|Hkv|1, Sq|1, Skv|1] (f32_fused.c:312-331).
+// Every other call stays on the general fp32 kernel (sdpa.hip). Without a mask, a query whose rules leave it at least
+// one key gives the same result whether excluded keys score -1e30 (the reference) or take no part (here), and a query
+// they leave none weighs every key of the sequence equally, as the reference's row of equal scores does. With a mask
+// the reference's arithmetic is kept as it stands: every key of the sequence takes part, an excluded one at -1e30
+// plus its mask value (the mask is added to every score), so no key block is skipped.
 //
 // Two launches:
 //   1. kv_to_bf16_kernel: K -> bf16 [kv head][key][D], V -> bf16 transposed [kv head][D][key], keys padded with
@@ -80,6 +83,8 @@ struct PrefillParams {
     int causal, window, right_context;
     const int32_t* lengths;    // per-sequence key counts on the device, or null
     int heads_per_wg;      // 1, 2 or 4 query heads of one KV head per workgroup
+    const float* mask;         // additive mask or null; dims 1 or the full extent (heads: 1, kv_heads or heads)
+    int mask_b, mask_h, mask_q, mask_k;
 };
 
 // One 64-key block of the bf16 K and V^T copies: global -> registers, and registers -> the LDS tiles.
@@ -153,20 +158,23 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
     };
     const int my_q = q0 + col;
     const int my_qc = min(my_q, p.seq_q - 1);
-    const bool my_uniform = first_of(my_qc) >= end_of(my_qc);               // no key left: every key of the sequence, equally
+    const bool masked = p.mask != nullptr;                                  // uniform
+    const int real_first = first_of(my_qc), real_last = end_of(my_qc) - 1;  // the rules' own range (may be empty)
+    // no key left: every key of the sequence, equally (with a mask the -1e30 scores do that by themselves)
+    const bool my_uniform = !masked && first_of(my_qc) >= end_of(my_qc);
     const int my_first_key = my_uniform ? 0 : first_of(my_qc);
     const int my_last_key = my_uniform ? p.seq_kv - 1 : end_of(my_qc) - 1;
     const bool wave_uniform = __ballot(my_uniform) != 0;
     const bool wg_uniform = __syncthreads_or(my_uniform) != 0;
     // keys any wave of this workgroup needs: [kbeg, kend), whole blocks
-    const int kbeg = wg_uniform ? 0 : first_of(q_wg_first);
-    const int kend = wg_uniform ? p.seq_kv : end_of(q_wg_last);
+    const int kbeg = (wg_uniform || masked) ? 0 : first_of(q_wg_first);
+    const int kend = (wg_uniform || masked) ? p.seq_kv : end_of(q_wg_last);
     const int blk_begin = kbeg / PF_KB;
     const int nblocks = kend > kbeg ? (kend + PF_KB - 1) / PF_KB : blk_begin;
     // this wave's 32 positions: the keys any of them attends, and the keys all of them attend
     const int q_wave_last = min(q0 + PF_QW - 1, p.seq_q - 1), q_wave_first = min(q0, p.seq_q - 1);
-    const int wave_first_key = wave_uniform ? 0 : first_of(q_wave_first);
-    const int wave_last_key = wave_uniform ? p.seq_kv - 1 : end_of(q_wave_last) - 1;
+    const int wave_first_key = (wave_uniform || masked) ? 0 : first_of(q_wave_first);
+    const int wave_last_key = (wave_uniform || masked) ? p.seq_kv - 1 : end_of(q_wave_last) - 1;
     const int wave_common_first = first_of(q_wave_last), wave_common_last = end_of(q_wave_first) - 1;
 
     // Q fragment: lane (query col, half h) holds q[16 t + 8 h .. + 7] for every t, times scale * log2(e)
@@ -184,6 +192,13 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
         }
     }
 
+    // this lane's row of the mask (one query position; the key index is added per score), in units of ln 2 later
+    const float* mrow = nullptr;
+    if (masked) {
+        const int bi = p.mask_b == 1 ? 0 : b;
+        const int hi = p.mask_h == 1 ? 0 : (p.mask_h == p.heads ? head : kvh);
+        mrow = p.mask + (((int64_t)bi * p.mask_h + hi) * p.mask_q + (p.mask_q == 1 ? 0 : my_qc)) * p.mask_k;
+    }
     const int64_t kvhead = (int64_t)b * p.kv_heads + kvh;
     const __bf16* kbase = p.kb + kvhead * p.spad * D;
     const __bf16* vbase = p.vt + kvhead * D * p.spad;
@@ -219,6 +234,28 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
                     s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s[j], 0, 0, 0);
                 }
             }
+            if (masked) {
+                // the reference's arithmetic: an excluded key scores -1e30, the mask is added to every score; keys past
+                // the sequence (padding of the last block) take no part. Four adjacent keys per 16-byte mask load.
+                constexpr float LOG2E = 1.4426950408889634f;
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const int key4 = k0 + 32 * j + 8 * e4 + 4 * h;
+                        float4 mv;
+                        if (p.mask_k == 1) { const float m1 = mrow[0]; mv = make_float4(m1, m1, m1, m1); }
+                        else mv = *reinterpret_cast<const float4*>(mrow + min(key4, p.seq_kv - 4));     // seq_kv is a multiple of 4 here
+                        const float m4[4] = {mv.x, mv.y, mv.z, mv.w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int key = key4 + i;
+                            float sc = (key > real_last || key < real_first) ? -1.0e30f * LOG2E : s[j][4 * e4 + i];
+                            sc = fmaf(m4[i], LOG2E, sc);
+                            s[j][4 * e4 + i] = key < p.seq_kv ? sc : -INFINITY;
+                        }
+                    }
+            } else
             // keys outside this query's range score -inf (they take no part); a query without a range scores every key 0
             if (wave_uniform || k0 < wave_common_first || k0 + PF_KB - 1 > wave_common_last) {   // wave-uniform: the block crosses a boundary
 #pragma unroll
@@ -298,7 +335,7 @@ void set_sdpa_prefill_mfma(int v) { g_prefill_mfma = v; }
 template <int D>
 static int launch_prefill_d(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                             int seq_q, int seq_kv, int kv_capacity, float scale, int causal, int window, int right_context,
-                            const int32_t* lengths) {
+                            const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k) {
     const int spad = (seq_kv + PF_KB - 1) / PF_KB * PF_KB;
     const size_t elems = (size_t)batch * kv_heads * spad * D;
     __bf16* ws = static_cast<__bf16*>(kernel_workspace(2 * elems * sizeof(__bf16)));
@@ -310,7 +347,8 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
     const int per_kv = heads / kv_heads;
     const int hpw = per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1);
     const int q_per_wg = (4 / hpw) * PF_QW;
-    PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, window, right_context, lengths, hpw};
+    PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, window, right_context, lengths, hpw,
+                    mask, mask_b, mask_h, mask_q, mask_k};
     const dim3 grid((seq_q + q_per_wg - 1) / q_per_wg, kv_heads * (per_kv / hpw), batch);
     constexpr size_t smem = sizeof(__bf16) * (2 * PF_KB * (D + 8) + 2 * D * (PF_KB + 8));
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D>), smem);
@@ -323,15 +361,18 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
 // Returns 1 when the MFMA path took the call, 0 when the shape is outside its range, -1 on error.
 int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                         int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window,
-                        int right_context, const int32_t* lengths) {
+                        int right_context, const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q,
+                        int mask_k) {
     if (!g_prefill_mfma) return 0;
+    // a mask row is read four keys at a time: rows of a multiple of four keys from a 16-byte aligned base (or one value per row)
+    if (mask && mask_k != 1 && ((mask_k & 3) || (reinterpret_cast<uintptr_t>(mask) & 15))) return 0;
     if (head_dim != 64 && head_dim != 128) return 0;
     if (seq_q < 16 || seq_q > seq_kv) return 0;          // a handful of rows is the row kernel's business
     if (batch > 65535 || (int64_t)kv_heads * heads > 65535) return 0;
     if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
          reinterpret_cast<uintptr_t>(out)) & 15) return 0;
-    if (head_dim == 64) return launch_prefill_d<64>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths);
-    return launch_prefill_d<128>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths);
+    if (head_dim == 64) return launch_prefill_d<64>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k);
+    return launch_prefill_d<128>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k);
 }
 
 }  // namespace skh

@@ -222,6 +222,54 @@ def test_attention_prefill_mfma_window_and_key_lengths(hip_backend, torch_cuda, 
         hip_backend.set_tuning("sdpa_prefill_mfma", 1)
 
 
+@pytest.mark.parametrize("batch,heads,kv_heads,d,sq,skv,causal,window,lengths,mask_dims", [
+    (2, 8, 2, 64, 200, 200, True, 0, None, (1, 1, 200, 200)),        # one bias matrix for every head (ALiBi-like), causal
+    (2, 8, 2, 128, 96, 160, False, 0, [160, 70], (2, 8, 96, 160)),   # a bias per batch and head, ragged key lengths, a prompt chunk
+    (1, 4, 4, 64, 130, 132, True, 48, None, (1, 4, 1, 132)),         # per-head key bias broadcast over queries, window (late queries lose keys)
+    (3, 6, 3, 128, 64, 64, True, 0, [64, 10, 0], (3, 3, 64, 64)),    # a bias per KV head; sequence 2 has no key at all
+    (2, 4, 2, 64, 80, 80, False, 0, None, (2, 1, 80, 1)),            # one value per query row: shifts every score of the row alike
+    (1, 32, 8, 128, 512, 512, True, 0, None, (1, 1, 512, 512)),      # the Llama-3 head shape with a padding-style mask of -1e9 entries
+])
+def test_attention_prefill_mfma_with_an_additive_mask(hip_backend, torch_cuda, batch, heads, kv_heads, d, sq, skv, causal, window,
+                                                      lengths, mask_dims):
+    """The matrix-core prompt kernel with an additive mask in every broadcast form the reference accepts, alone and on
+    top of the structured rules: the mask is added to every score, an excluded key's -1e30 included, so a row the rules
+    leave without a key weighs the keys by its mask values' softmax only if those differ by less than fp32 resolves at
+    1e30 -- i.e. equally. Against the oracle, 2e-2 of the largest reference magnitude; masks whose rows are not a
+    multiple of four keys stay on the fp32 kernel."""
+    rng = np.random.default_rng(sq * skv + d + mask_dims[0])
+    q = rng.standard_normal((batch, heads, sq, d)).astype(np.float32)
+    k = rng.standard_normal((batch, kv_heads, skv, d)).astype(np.float32)
+    v = rng.standard_normal((batch, kv_heads, skv, d)).astype(np.float32)
+    scale = float(1 / np.sqrt(d))
+    mask = (rng.standard_normal(mask_dims) * 2).astype(np.float32)
+    if mask_dims[3] > 1:
+        mask[..., rng.random(mask_dims[3]) < 0.2] = -1e9              # some keys switched off for everyone, as a padding mask does
+        mask[..., 0] = np.minimum(mask[..., 0], 3.0)                   # and key 0 stays available
+        mask[..., 0] = np.maximum(mask[..., 0], -3.0)
+    ln = None if lengths is None else np.asarray(lengths, np.int32)
+    got = gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, 0, ln, mask)
+    assert hip_backend.last_kernel() == "sdpa_prefill_kernel"
+    want = L.sdpa(q, k, v, scale, causal, window, 0, ln, mask)
+    assert np.isfinite(got).all()
+    assert normalized_err(got, want, eps=1.0) <= 2e-2
+    assert np.sqrt(np.mean((got - want) ** 2)) <= 5e-3 * np.abs(want).max()
+    hip_backend.set_tuning("sdpa_prefill_mfma", 0)
+    try:
+        close(gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, 0, ln, mask), want)
+        assert hip_backend.last_kernel() != "sdpa_prefill_kernel"
+    finally:
+        hip_backend.set_tuning("sdpa_prefill_mfma", 1)
+    if mask_dims[3] > 4:
+        odd = np.ascontiguousarray(mask[..., : mask_dims[3] - 1])     # rows of skv - 1 keys: not the layout the kernel reads
+        got_odd = gpu_sdpa(hip_backend, torch_cuda, q, k[:, :, : skv - 1], v[:, :, : skv - 1], scale, causal, window, 0,
+                           None if ln is None else np.minimum(ln, skv - 1), odd) if sq <= skv - 1 else None
+        if got_odd is not None:
+            assert hip_backend.last_kernel() != "sdpa_prefill_kernel" or (skv - 1) % 4 == 0
+            close(got_odd, L.sdpa(q, k[:, :, : skv - 1], v[:, :, : skv - 1], scale, causal, window, 0,
+                                  None if ln is None else np.minimum(ln, skv - 1), odd))
+
+
 def test_norms_softmax_and_glue(hip_backend, torch_cuda):
     torch = torch_cuda
     kx = hip_backend
