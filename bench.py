@@ -268,6 +268,98 @@ def cpu_baseline_attention(batch, seq_q, seq_kv, heads, kv_heads, d, scale, wind
                       f"median of {reps} after 1 warm-up ({med * 1e3:.2f} ms per call, host has {os.cpu_count()} logical cores)"
 
 
+DENSE_WORKLOADS = {   # name: (m, n, k, B given as [n, k] (x . W^T)); fp32 operands on the fp32 matrix instruction
+    "dense_f32_4096x4096x4096": (4096, 4096, 4096, False),
+    "dense_f32_wt_512x4096x4096": (512, 4096, 4096, True),
+    "dense_f32_wt_2048x11008x4096": (2048, 11008, 4096, True),
+}
+MFMA_F32_PEAK_TFLOPS = 157.3
+
+
+def bench_dense(a):
+    """Dense fp32 matmul of the kernel SPI (Fp32MatmulKernel / Fp32MatmulWtKernel) on resident operands."""
+    import torch
+    from skainet_amd import _lib, kernels
+    m, n, k, wt = DENSE_WORKLOADS[a.workload]
+    steps = 20 if a.steps == 2000 else a.steps
+    warmup = 3 if a.warmup == 200 else a.warmup
+    gen = torch.Generator(device="cuda").manual_seed(20251125)
+    x = torch.randn((m, k), device="cuda", generator=gen)
+    w = torch.randn((n, k) if wt else (k, n), device="cuda", generator=gen)
+    out = torch.empty((m, n), device="cuda")
+
+    def call():
+        if wt:
+            kernels.fp32_matmul_wt_dev(x, 0, w, 0, out, 0, m, n, k)
+        else:
+            kernels.fp32_matmul_dev(x, 0, k, w, 0, n, out, 0, n, m, n, k)
+
+    call()
+    kernels.sync()
+    kernel = kernels.last_kernel()
+
+    def timed(count):
+        if a.no_graph:
+            with kernels.Timer() as t:
+                for _ in range(count):
+                    call()
+            return t.ms
+        with kernels.Graph() as g:
+            for _ in range(count):
+                call()
+        g.launch(); g.sync()
+        with kernels.Timer() as t:
+            g.launch()
+        g.close()
+        return t.ms
+
+    if warmup > 0:
+        timed(warmup)
+    t0 = time.perf_counter()
+    ms_per_step = timed(steps) / steps
+    wall = time.perf_counter() - t0
+    rows = torch.arange(0, m, max(1, m // 64), device="cuda")
+    want = x[rows].double() @ (w.double().T if wt else w.double())
+    err = float(((out[rows].double() - want).abs().max() / want.abs().max()).cpu())
+    tol = 1e-5
+    flops = 2.0 * m * n * k
+    tf = flops / (ms_per_step * 1e-3) / 1e12
+    out_json = {
+        "metric": "dense fp32 matmul TFLOP/s", "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": a.workload, "m": m, "n": n, "k": k, "b_layout": "[n, k]" if wt else "[k, n]",
+                   "launch": "host loop" if a.no_graph else "hip-graph replay"},
+        "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / MFMA_F32_PEAK_TFLOPS, 4), "traffic": None},
+        "extra": {"flops_per_step": flops, "kernel": kernel, "wall_s_timed_region": round(wall, 4),
+                  "max_err_over_max_vs_torch_fp64_on_sampled_rows": err, "device": _lib.hip().skainet_hip_device_name().decode()},
+    }
+    if err > tol:
+        out_json["extra"]["PARITY_FAILED"] = True
+    if not a.skip_cpu:
+        # the reference's own C library on a bounded sample of the same product: the first rows of A, all of B
+        from oracle import lib as L
+        ref = L.ref()
+        if ref is not None:
+            ms_ = max(8, min(m, int(2.0e9 / (n * k)) or 1))
+            xa = np.ascontiguousarray(x[:ms_].cpu().numpy())
+            wa = np.ascontiguousarray(w.cpu().numpy())
+            oa = np.empty((ms_, n), np.float32)
+            fn = (lambda: ref.skainet_fp32_matmul_wt(L.fp(xa), 0, L.fp(wa), 0, L.fp(oa), 0, ms_, n, k)) if wt else \
+                 (lambda: ref.skainet_fp32_matmul(L.fp(xa), 0, k, L.fp(wa), 0, n, L.fp(oa), 0, n, ms_, n, k))
+            fn()
+            ts = []
+            t_end = time.perf_counter() + 10.0
+            while len(ts) < 3 or (time.perf_counter() < t_end and len(ts) < 20):
+                t1 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t1)
+            med = float(np.median(ts))
+            out_json["cpu_baseline"] = {"value": round(2.0 * ms_ * n * k / med / 1e12, 4), "unit": "TFLOP/s", "cores": 4, "kind": "reference",
+                                        "sample": f"the first {ms_} rows of A against all of B, median of {len(ts)} calls of the reference's C entry ({med * 1e3:.1f} ms)"}
+    print(json.dumps(out_json).replace("NaN", "null"))
+    sys.exit(0 if err <= tol else 1)
+
+
 def bench_attention(a):
     """Fused causal GQA attention, fp32 operands: prefill at 2048 (MFMA-class, flops counted dense as the reference's
     scenarios do) and one-token decode against a 4096-long KV cache (HBM-bound: K and V are read once)."""
@@ -538,7 +630,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000, help="timed steps (default 2000; 200 for the GEMM workloads)")
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(SPI_DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS))
+    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(SPI_DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS) + sorted(DENSE_WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
     ap.add_argument("--hbm-only", action="store_true", help="skip the cache-warm pass and the read probe, so every launch of the "
@@ -562,6 +654,8 @@ def main():
 
     if a.workload in DECODER_WORKLOADS or a.workload in SPI_DECODER_WORKLOADS:
         bench_decoder(a)
+    if a.workload in DENSE_WORKLOADS:
+        return bench_dense(a)
     if a.workload in ATTENTION_WORKLOADS:
         bench_attention(a)
     default_run = a.workload == "q4k_gemv_11008x4096_b1" and not a.no_headline

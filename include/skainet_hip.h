@@ -363,6 +363,7 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
 
 /* Launch-shape knobs for experiments (defaults are the measured best). Keys: "gemv_waves_per_cu",
  * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares, 0 = chosen from the shape),
+ * "dense_mfma" (0: dense fp32 products stay on the vector-ALU tile kernel instead of the fp32 matrix instruction),
  * "gemv_stream_enable" (0: one-row Q8_0 / Q4_0 / Q5_0 / Q5_1 products stay on the row kernel instead of the one that
  * streams each wave's rows through LDS),
  * "q4k_rows_enable" (0: Q4_K decode shapes take the generic slot kernel), "q6k_slot64" (0: Q6_K at batch 1 keeps the

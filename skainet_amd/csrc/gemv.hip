@@ -180,6 +180,7 @@ int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int 
 int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int n, int batch);  // gemv_q4k_quads.hip
 int launch_gemv_stream(int enc, const uint8_t* w, const float* x, float* y, int k, int n);        // gemv_stream.hip
 void set_gemv_stream_enable(int v);
+void set_dense_mfma(int v);
 
 // Experiment knobs (defaults are the measured best): returns 0 when the key is known.
 int set_tuning(const char* key, int value) {
@@ -187,6 +188,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q4k_rows_waves_per_cu")) { set_q4k_rows_waves_per_cu(value); return 0; }
     if (!strcmp(key, "q6k_slot64")) { g_q6k_slot64 = value != 0; return 0; }
     if (!strcmp(key, "gemv_stream_enable")) { set_gemv_stream_enable(value); return 0; }
+    if (!strcmp(key, "dense_mfma")) { set_dense_mfma(value); return 0; }
     if (!strcmp(key, "gemm_wide")) { set_gemm_wide(value); return 0; }
     if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }
     if (!strcmp(key, "gemm_ksplit")) { set_gemm_ksplit(value); return 0; }

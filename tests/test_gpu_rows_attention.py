@@ -389,6 +389,48 @@ def test_dense_matmuls(hip_backend, torch_cuda):
     close(o, a.astype(np.float64) @ w.T, rel=1e-5, abs_=1e-4)
 
 
+@pytest.mark.parametrize("m,n,k,wt", [(512, 1024, 768, False), (200, 300, 260, False), (64, 32, 4, True), (130, 4096, 516, True),
+                                      (1000, 132, 2048, False), (65, 257, 100, True)])
+def test_dense_fp32_matmul_on_the_matrix_cores(hip_backend, torch_cuda, m, n, k, wt):
+    """fp32 operands on the fp32 matrix instruction (exact products, fp32 accumulation in the instruction's order):
+    resident operands through the device entries, ragged tiles in every direction, K from one instruction step to many
+    slices, both layouts of B; against fp64 and against the tile kernel that takes the same call when the matrix-core
+    one is switched off. Products whose strides or alignment the matrix-core kernel does not read stay on the tile
+    kernel."""
+    torch = torch_cuda
+    rng = np.random.default_rng(m + n + k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((n, k) if wt else (k, n)).astype(np.float32)
+    want = a.astype(np.float64) @ (b.astype(np.float64).T if wt else b.astype(np.float64))
+
+    def run():
+        out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        if wt:
+            hip_backend.fp32_matmul_wt_dev(dev(torch, a), 0, dev(torch, b), 0, out, 0, m, n, k)
+        else:
+            hip_backend.fp32_matmul_dev(dev(torch, a), 0, k, dev(torch, b), 0, n, out, 0, n, m, n, k)
+        return out.cpu().numpy()
+
+    got = run()
+    assert hip_backend.last_kernel() == "sgemm_mfma_kernel"
+    close(got, want, rel=1e-5, abs_=2e-6 * np.sqrt(k) * 16)
+    try:
+        hip_backend.set_tuning("dense_mfma", 0)
+        tile = run()
+        assert hip_backend.last_kernel() == "sgemm_kernel"
+    finally:
+        hip_backend.set_tuning("dense_mfma", 1)
+    close(got, tile, rel=1e-5, abs_=2e-6 * np.sqrt(k) * 16)
+    if not wt:
+        # the same product out of a wider A at an offset of one float: not 16-byte aligned, the tile kernel's business
+        wide = np.zeros((m, k + 4), np.float32)
+        wide[:, 1:k + 1] = a
+        out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        hip_backend.fp32_matmul_dev(dev(torch, wide), 1, k + 4, dev(torch, b), 0, n, out, 0, n, m, n, k)
+        assert hip_backend.last_kernel() == "sgemm_kernel"
+        close(out.cpu().numpy(), want, rel=1e-5, abs_=2e-6 * np.sqrt(k) * 16)
+
+
 @pytest.mark.parametrize("kind,codec", [("bf16", "BFloat16"), ("fp16", "Float16")])
 def test_narrow_float_matmuls(hip_backend, torch_cuda, kind, codec):
     """Bf16MatmulKernel / Fp16MatmulKernel through the host entry: the oracle on the recorded inputs (with the formats'
