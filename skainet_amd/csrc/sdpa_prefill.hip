@@ -17,10 +17,15 @@
 //   1. kv_to_bf16_kernel: K -> bf16 [kv head][key][D], V -> bf16 transposed [kv head][D][key], keys padded with
 //      zeros to a multiple of 64. (The PV product contracts over keys, and an MFMA operand wants 8 consecutive
 //      contraction values per lane: V has to be read along keys, hence the transpose, done once per call.)
-//   2. sdpa_prefill_kernel: one workgroup = 4 waves = up to 4 query heads that share a KV head x 32 query
-//      positions (fewer heads per KV head: more query blocks per workgroup). Keys in blocks of 64: the K and V^T
-//      tiles of a block go global -> registers -> LDS (double-buffered, one barrier per block) and are shared by
-//      the 4 waves. Per wave and block:
+//   2. sdpa_prefill_kernel: one workgroup = two teams of 4 waves; a team = up to 4 query heads that share a KV head x
+//      32 query positions (fewer heads per KV head: more query blocks per team). The teams of workgroup i take query
+//      group G - 1 - i and query group i of the same KV head (groups 2 i + 1 and 2 i under a sliding window or without
+//      the causal rule, where neighbours share their key blocks): under the causal rule a late group (many keys) and an
+//      early one (few), so every workgroup carries the same work and one workgroup per CU keeps its SIMDs busy from
+//      start to end (with one group per workgroup, which two groups shared a CU was the dispatcher's choice: two late
+//      groups on one CU set the kernel's time). Keys in blocks of 64: the K and V^T tiles of a block go
+//      global -> registers -> LDS (double-buffered, one barrier per block) and are shared by the 8 waves; a block no
+//      wave of either team needs is never loaded. Per wave and block:
 //        S^T[key][query] = K_tile . Q^T           16 MFMAs (Q lives in registers, pre-multiplied by scale * log2 e)
 //        online softmax per query: a query is one accumulator COLUMN, so its 32 scores per 32-key tile sit in
 //          one lane pair (l, l ^ 32): the row statistics need a single cross-lane step
@@ -88,51 +93,53 @@ struct PrefillParams {
 };
 
 // One 64-key block of the bf16 K and V^T copies: global -> registers, and registers -> the LDS tiles.
+constexpr int PF_THREADS = 512;    // two teams of four waves
 template <int D>
-__device__ __forceinline__ void pf_load_block(pf_u32x4 (&kreg)[PF_KB * (D / 8) / 256], pf_u32x4 (&vreg)[D * (PF_KB / 8) / 256],
+__device__ __forceinline__ void pf_load_block(pf_u32x4 (&kreg)[PF_KB * (D / 8) / PF_THREADS], pf_u32x4 (&vreg)[D * (PF_KB / 8) / PF_THREADS],
                                               const __bf16* kbase, const __bf16* vbase, int spad, int k0, int tid) {
     constexpr int KCH = D / 8;
 #pragma unroll
-    for (int j = 0; j < PF_KB * KCH / 256; ++j) {
-        const int c = tid + 256 * j, key = c / KCH, ch = c % KCH;
+    for (int j = 0; j < PF_KB * KCH / PF_THREADS; ++j) {
+        const int c = tid + PF_THREADS * j, key = c / KCH, ch = c % KCH;
         kreg[j] = *reinterpret_cast<const pf_u32x4*>(kbase + (int64_t)(k0 + key) * D + 8 * ch);
     }
 #pragma unroll
-    for (int j = 0; j < D * (PF_KB / 8) / 256; ++j) {
-        const int c = tid + 256 * j, d = c / (PF_KB / 8), ch = c % (PF_KB / 8);
+    for (int j = 0; j < D * (PF_KB / 8) / PF_THREADS; ++j) {
+        const int c = tid + PF_THREADS * j, d = c / (PF_KB / 8), ch = c % (PF_KB / 8);
         vreg[j] = *reinterpret_cast<const pf_u32x4*>(vbase + (int64_t)d * spad + k0 + 8 * ch);
     }
 }
 template <int D>
-__device__ __forceinline__ void pf_store_block(const pf_u32x4 (&kreg)[PF_KB * (D / 8) / 256], const pf_u32x4 (&vreg)[D * (PF_KB / 8) / 256],
+__device__ __forceinline__ void pf_store_block(const pf_u32x4 (&kreg)[PF_KB * (D / 8) / PF_THREADS], const pf_u32x4 (&vreg)[D * (PF_KB / 8) / PF_THREADS],
                                                __bf16* kt, __bf16* vt, int tid) {
     constexpr int KCH = D / 8, KP = D + 8, VP = PF_KB + 8;
 #pragma unroll
-    for (int j = 0; j < PF_KB * KCH / 256; ++j) {
-        const int c = tid + 256 * j, key = c / KCH, ch = c % KCH;
+    for (int j = 0; j < PF_KB * KCH / PF_THREADS; ++j) {
+        const int c = tid + PF_THREADS * j, key = c / KCH, ch = c % KCH;
         *reinterpret_cast<pf_u32x4*>(kt + key * KP + 8 * ch) = kreg[j];
     }
 #pragma unroll
-    for (int j = 0; j < D * (PF_KB / 8) / 256; ++j) {
-        const int c = tid + 256 * j, d = c / (PF_KB / 8), ch = c % (PF_KB / 8);
+    for (int j = 0; j < D * (PF_KB / 8) / PF_THREADS; ++j) {
+        const int c = tid + PF_THREADS * j, d = c / (PF_KB / 8), ch = c % (PF_KB / 8);
         *reinterpret_cast<pf_u32x4*>(vt + d * VP + 8 * ch) = vreg[j];
     }
 }
 
 template <int D>
-__global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
+__global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillParams p) {
     constexpr int KP = D + 8;          // K tile row pitch (bf16): 16-byte aligned rows, 16 lanes of a b128 read on distinct banks
     constexpr int VP = PF_KB + 8;      // V^T tile row pitch (bf16)
     constexpr int NT = D / 16;         // MFMA steps along head_dim for S
     constexpr int ND = D / 32;         // 32-row tiles of O^T
     constexpr int KCH = D / 8;         // 16-byte chunks per K row
-    constexpr int K_LOADS = PF_KB * KCH / 256;       // 16-byte loads per thread for the K tile
-    constexpr int V_LOADS = D * (PF_KB / 8) / 256;   // and for the V^T tile
+    constexpr int K_LOADS = PF_KB * KCH / PF_THREADS;       // 16-byte loads per thread for the K tile
+    constexpr int V_LOADS = D * (PF_KB / 8) / PF_THREADS;   // and for the V^T tile
     extern __shared__ __attribute__((aligned(16))) uint8_t pf_smem[];       // 2 K tiles, then 2 V^T tiles
     __bf16* const ktile0 = reinterpret_cast<__bf16*>(pf_smem);
     __bf16* const vtile0 = ktile0 + 2 * PF_KB * KP;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6), team = wave_all >> 2, wave = wave_all & 3;
     const int col = lane & 31, h = lane >> 5;
     const int per_kv = p.heads / p.kv_heads;
     const int hpw = p.heads_per_wg;
@@ -141,11 +148,20 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
     const int kvh = blockIdx.y / head_groups;
     const int head = kvh * per_kv + (blockIdx.y % head_groups) * hpw + wave % hpw;
     const int b = blockIdx.z;
-    // causal: the workgroups with the most keys start first
-    const int qb_wg = p.causal ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
-    const int q0 = (qb_wg * qblocks_per_wg + wave / hpw) * PF_QW;          // first query position of this wave
-    const int q_wg_first = qb_wg * qblocks_per_wg * PF_QW;
-    const int q_wg_last = min(p.seq_q, (qb_wg + 1) * qblocks_per_wg * PF_QW) - 1;
+    // query groups (a team's share of the query positions). Causal over the whole prefix: team 0 takes group G - 1 - i,
+    // team 1 group i (equal work in every workgroup). Under a sliding window, or without the causal rule, every group
+    // has about the same work and neighbours share most of their key blocks: groups 2 i + 1 and 2 i. With an odd number
+    // of groups one group is team 0's alone.
+    const int q_per_group = qblocks_per_wg * PF_QW;
+    const int ngroups = (p.seq_q + q_per_group - 1) / q_per_group;
+    const bool adjacent = p.window > 0 || !p.causal;
+    const int g_early = adjacent ? 2 * (int)blockIdx.x : (int)blockIdx.x;
+    const int g_late = adjacent ? min(g_early + 1, ngroups - 1) : ngroups - 1 - (int)blockIdx.x;
+    const int my_group = team ? g_early : g_late;
+    const bool team_active = !(team == 1 && g_early == g_late);
+    const int q0 = my_group * q_per_group + (wave / hpw) * PF_QW;          // first query position of this wave
+    auto group_first = [&](int g) { return g * q_per_group; };
+    auto group_last = [&](int g) { return min(p.seq_q, (g + 1) * q_per_group) - 1; };
     const int shift = p.seq_kv - p.seq_q;                                   // absolute position of query 0
     const int len = p.lengths ? p.lengths[b] : p.seq_kv;
     // attended keys [first, end) of a query position: both bounds grow with the position
@@ -166,15 +182,19 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
     const int my_last_key = my_uniform ? p.seq_kv - 1 : end_of(my_qc) - 1;
     const bool wave_uniform = __ballot(my_uniform) != 0;
     const bool wg_uniform = __syncthreads_or(my_uniform) != 0;
-    // keys any wave of this workgroup needs: [kbeg, kend), whole blocks
-    const int kbeg = (wg_uniform || masked) ? 0 : first_of(q_wg_first);
-    const int kend = (wg_uniform || masked) ? p.seq_kv : end_of(q_wg_last);
-    const int blk_begin = kbeg / PF_KB;
-    const int nblocks = kend > kbeg ? (kend + PF_KB - 1) / PF_KB : blk_begin;
+    // keys any wave of this workgroup needs: the two teams' ranges (both bounds grow with the query position), whole
+    // blocks; between the early team's last block and the late team's first (a sliding window) lie blocks nobody needs
+    const bool all_keys = wg_uniform || masked;
+    const int e_beg = first_of(group_first(g_early)) / PF_KB, e_end = (end_of(group_last(g_early)) + PF_KB - 1) / PF_KB;
+    const int l_beg = first_of(group_first(g_late)) / PF_KB, l_end = (end_of(group_last(g_late)) + PF_KB - 1) / PF_KB;
+    const int blk_begin = all_keys ? 0 : min(e_beg, l_beg);
+    const int nblocks = all_keys ? (p.seq_kv + PF_KB - 1) / PF_KB : max(max(e_end, l_end), blk_begin);
+    auto needed = [&](int blk) { return all_keys || (blk >= e_beg && blk < e_end) || (blk >= l_beg && blk < l_end); };
+    auto next_needed = [&](int blk) { int nb = blk + 1; while (nb < nblocks && !needed(nb)) ++nb; return nb; };
     // this wave's 32 positions: the keys any of them attends, and the keys all of them attend
     const int q_wave_last = min(q0 + PF_QW - 1, p.seq_q - 1), q_wave_first = min(q0, p.seq_q - 1);
     const int wave_first_key = (wave_uniform || masked) ? 0 : first_of(q_wave_first);
-    const int wave_last_key = (wave_uniform || masked) ? p.seq_kv - 1 : end_of(q_wave_last) - 1;
+    const int wave_last_key = !team_active ? -1 : (wave_uniform || masked) ? p.seq_kv - 1 : end_of(q_wave_last) - 1;
     const int wave_common_first = first_of(q_wave_last), wave_common_last = end_of(q_wave_first) - 1;
 
     // Q fragment: lane (query col, half h) holds q[16 t + 8 h .. + 7] for every t, times scale * log2(e)
@@ -210,16 +230,18 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
         for (int e = 0; e < 16; ++e) oacc[i][e] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;     // per query (column); l_run is this lane's half of the keys
 
-    if (nblocks > blk_begin) {
-        pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, blk_begin * PF_KB, tid);
-        pf_store_block<D>(kreg, vreg, ktile0 + (blk_begin & 1) * (PF_KB * KP), vtile0 + (blk_begin & 1) * (D * VP), tid);
+    int blk = blk_begin;
+    while (blk < nblocks && !needed(blk)) ++blk;
+    if (blk < nblocks) {
+        pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, blk * PF_KB, tid);
+        pf_store_block<D>(kreg, vreg, ktile0, vtile0, tid);
     }
     __syncthreads();
 
-    for (int blk = blk_begin; blk < nblocks; ++blk) {
-        const int buf = blk & 1;
+    for (int buf = 0; blk < nblocks; buf ^= 1) {
         const int k0 = blk * PF_KB;
-        if (blk + 1 < nblocks) pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, k0 + PF_KB, tid);
+        const int nblk = next_needed(blk);
+        if (nblk < nblocks) pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, nblk * PF_KB, tid);
         if (k0 <= wave_last_key && k0 + PF_KB > wave_first_key) {     // wave-uniform: this wave has keys in the block
             // S^T tiles: s[j] covers keys k0 + 32 j .. + 31 (rows) x this wave's 32 queries (columns)
             pf_f32x16 s[2];
@@ -308,13 +330,14 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_kernel(PrefillParams p) {
                 }
             }
         }
-        if (blk + 1 < nblocks) pf_store_block<D>(kreg, vreg, ktile0 + (buf ^ 1) * (PF_KB * KP), vtile0 + (buf ^ 1) * (D * VP), tid);
+        if (nblk < nblocks) pf_store_block<D>(kreg, vreg, ktile0 + (buf ^ 1) * (PF_KB * KP), vtile0 + (buf ^ 1) * (D * VP), tid);
         __syncthreads();
+        blk = nblk;
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (my_q < p.seq_q) {
+    if (my_q < p.seq_q && team_active) {
         float* op = p.out + (((int64_t)b * p.heads + head) * p.seq_q + my_q) * D;
 #pragma unroll
         for (int i = 0; i < ND; ++i)
@@ -346,14 +369,15 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
     SKH_CHECK(hipGetLastError());
     const int per_kv = heads / kv_heads;
     const int hpw = per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1);
-    const int q_per_wg = (4 / hpw) * PF_QW;
+    const int q_per_group = (4 / hpw) * PF_QW;
+    const int ngroups = (seq_q + q_per_group - 1) / q_per_group;
     PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, window, right_context, lengths, hpw,
                     mask, mask_b, mask_h, mask_q, mask_k};
-    const dim3 grid((seq_q + q_per_wg - 1) / q_per_wg, kv_heads * (per_kv / hpw), batch);
+    const dim3 grid((ngroups + 1) / 2, kv_heads * (per_kv / hpw), batch);
     constexpr size_t smem = sizeof(__bf16) * (2 * PF_KB * (D + 8) + 2 * D * (PF_KB + 8));
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D>), smem);
     note_kernel("sdpa_prefill_kernel");
-    sdpa_prefill_kernel<D><<<grid, dim3(256), smem, s>>>(p);
+    sdpa_prefill_kernel<D><<<grid, dim3(PF_THREADS), smem, s>>>(p);
     SKH_CHECK(hipGetLastError());
     return 1;
 }
