@@ -56,17 +56,26 @@ __global__ __launch_bounds__(256) void kv_to_bf16_kernel(const float* __restrict
     const int64_t head = (int64_t)blockIdx.z * kv_heads + blockIdx.y;
     const float* ksrc = k + head * kv_capacity * D;
     const float* vsrc = v + head * kv_capacity * D;
-    // K: straight conversion, 4 floats per thread-step
-    for (int t = threadIdx.x; t < PF_KB * D / 4; t += 256) {
-        const int key = t / (D / 4), d4 = t % (D / 4);
-        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (k0 + key < seq_kv) x = *reinterpret_cast<const float4*>(ksrc + (int64_t)(k0 + key) * D + 4 * d4);
+    // K: straight conversion, 4 floats per thread-step; every load of the workgroup's 64 KB is requested before the
+    // first value is used (keys past the sequence: a clamped address, zeroed afterwards)
+    constexpr int STEPS = PF_KB * D / 4 / 256;
+    float4 xs[STEPS], ys[STEPS];
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int t = threadIdx.x + 256 * i, key = t / (D / 4), d4 = t % (D / 4);
+        const int64_t off = (int64_t)min(k0 + key, seq_kv - 1) * D + 4 * d4;
+        xs[i] = *reinterpret_cast<const float4*>(ksrc + off);
+        ys[i] = *reinterpret_cast<const float4*>(vsrc + off);
+    }
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int t = threadIdx.x + 256 * i, key = t / (D / 4), d4 = t % (D / 4);
+        const float keep = k0 + key < seq_kv ? 1.0f : 0.0f;
+        const float4 x = xs[i], y = ys[i];
         pf_bf16x4 o;
-        o[0] = (__bf16)x.x; o[1] = (__bf16)x.y; o[2] = (__bf16)x.z; o[3] = (__bf16)x.w;
+        o[0] = (__bf16)(x.x * keep); o[1] = (__bf16)(x.y * keep); o[2] = (__bf16)(x.z * keep); o[3] = (__bf16)(x.w * keep);
         *reinterpret_cast<pf_bf16x4*>(kb + (head * spad + k0 + key) * D + 4 * d4) = o;
-        float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (k0 + key < seq_kv) y = *reinterpret_cast<const float4*>(vsrc + (int64_t)(k0 + key) * D + 4 * d4);
-        tile[key][4 * d4] = y.x; tile[key][4 * d4 + 1] = y.y; tile[key][4 * d4 + 2] = y.z; tile[key][4 * d4 + 3] = y.w;
+        tile[key][4 * d4] = y.x * keep; tile[key][4 * d4 + 1] = y.y * keep; tile[key][4 * d4 + 2] = y.z * keep; tile[key][4 * d4 + 3] = y.w * keep;
     }
     __syncthreads();
     // V^T: thread-step = (d, 8 consecutive keys)
