@@ -304,10 +304,15 @@ __global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillPara
 #pragma unroll
                 for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[j][e]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run, mx);
+            // The reference point of the exponentials follows the running maximum lazily: it moves only when a block's
+            // maximum exceeds it by more than 8 (in units of ln 2; weights then stay below 2^8, far inside bf16 and fp32
+            // range, and the final division by the sum takes the common factor out). So the 64 output accumulators are
+            // rescaled in the few blocks where some query of the wave moves its reference -- for most waves the first
+            // block only -- instead of in every block.
+            const bool move = mx > m_run + 8.0f;                                      // also the first block (m_run = -inf) with any finite score
+            const float m_new = move ? mx : m_run;
             // a query of a padded row past seq_q, or a block wholly past a query's keys, can leave m_new at -inf
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);                // m_run = -inf -> 0
             float psum = 0.f;
             pf_bf16x8 pf[4];                                         // pf[2 j + g]: keys 16 g .. of tile j, this lane's 8 slots
 #pragma unroll
@@ -320,12 +325,16 @@ __global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillPara
                 pf[2 * j + 1] = pf_bf16x8{(__bf16)pr[8], (__bf16)pr[9], (__bf16)pr[10], (__bf16)pr[11],
                                           (__bf16)pr[12], (__bf16)pr[13], (__bf16)pr[14], (__bf16)pr[15]};
             }
-            l_run = l_run * alpha + psum;
+            if (__ballot(move) != 0) {                                               // wave-uniform
+                const float alpha = move ? __builtin_amdgcn_exp2f(m_run - m_use) : 1.0f;   // m_run = -inf -> 0
+                l_run *= alpha;
+#pragma unroll
+                for (int i = 0; i < ND; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
+            }
+            l_run += psum;
             m_run = m_new;
-#pragma unroll
-            for (int i = 0; i < ND; ++i)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) oacc[i][e] *= alpha;
             // O^T += V^T . P : A = V^T rows d, this lane's k-slots are keys 16 g + 4 h + {0..3} and 16 g + 8 + 4 h + {0..3}
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
