@@ -377,7 +377,8 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * of four waves per workgroup of that kernel, each with its own share of K: 1 or 2, default 2; rows with an odd number
  * of 256-element super-blocks always run one team), "gemm_ksw_stages" (activation tiles the one-team form keeps in LDS: 3 to 7,
  * default 5),
- * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_decode_split_keys" (least keys per split of
+ * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_prefill_teams" (query groups per workgroup of
+ * the matrix-core prompt kernel: 1, 2 = a late and an early group paired, 0 = paired where that still fills the chip), "sdpa_decode_split_keys" (least keys per split of
  * decode-shape attention, default 64), "sdpa_decode_gs" (query heads per workgroup of decode-shape attention: 1, 2 or 4, 0 = chosen from
  * the shape), "attn_merge_enable" (0: skainet_hip_attn_out_proj_dev always merges the key
  * splits in a launch of its own), "attn_merge_max_keys" (most keys per split for which that entry leaves the merge to

@@ -168,6 +168,7 @@ void set_gemm_ksw(int v);
 void set_gemm_ksw_teams(int v);
 void set_gemm_ksw_stages(int v);
 void set_sdpa_prefill_mfma(int v);
+void set_sdpa_prefill_teams(int v);
 void set_sdpa_decode_split_keys(int v);
 void set_q4k_ksplit_enable(int v);
 void set_q4k_mfma_enable(int v);
@@ -197,6 +198,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "gemm_ksw_teams")) { set_gemm_ksw_teams(value); return 0; }
     if (!strcmp(key, "gemm_ksw_stages")) { set_gemm_ksw_stages(value); return 0; }
     if (!strcmp(key, "sdpa_prefill_mfma")) { set_sdpa_prefill_mfma(value); return 0; }
+    if (!strcmp(key, "sdpa_prefill_teams")) { set_sdpa_prefill_teams(value); return 0; }
     if (!strcmp(key, "q4k_ksplit_enable")) { set_q4k_ksplit_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_enable")) { set_q4k_mfma_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_window")) { set_q4k_mfma_window(value); return 0; }

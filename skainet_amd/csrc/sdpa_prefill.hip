@@ -102,8 +102,8 @@ struct PrefillParams {
 };
 
 // One 64-key block of the bf16 K and V^T copies: global -> registers, and registers -> the LDS tiles.
-constexpr int PF_THREADS = 512;    // two teams of four waves
-template <int D>
+// PF_THREADS threads of a workgroup (one or two teams of four waves) stage a block together
+template <int D, int PF_THREADS>
 __device__ __forceinline__ void pf_load_block(pf_u32x4 (&kreg)[PF_KB * (D / 8) / PF_THREADS], pf_u32x4 (&vreg)[D * (PF_KB / 8) / PF_THREADS],
                                               const __bf16* kbase, const __bf16* vbase, int spad, int k0, int tid) {
     constexpr int KCH = D / 8;
@@ -118,7 +118,7 @@ __device__ __forceinline__ void pf_load_block(pf_u32x4 (&kreg)[PF_KB * (D / 8) /
         vreg[j] = *reinterpret_cast<const pf_u32x4*>(vbase + (int64_t)d * spad + k0 + 8 * ch);
     }
 }
-template <int D>
+template <int D, int PF_THREADS>
 __device__ __forceinline__ void pf_store_block(const pf_u32x4 (&kreg)[PF_KB * (D / 8) / PF_THREADS], const pf_u32x4 (&vreg)[D * (PF_KB / 8) / PF_THREADS],
                                                __bf16* kt, __bf16* vt, int tid) {
     constexpr int KCH = D / 8, KP = D + 8, VP = PF_KB + 8;
@@ -134,8 +134,11 @@ __device__ __forceinline__ void pf_store_block(const pf_u32x4 (&kreg)[PF_KB * (D
     }
 }
 
-template <int D>
-__global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillParams p) {
+// TEAMS 2: the paired form described above. TEAMS 1: one query group per workgroup of four waves (two workgroups per
+// CU), for calls whose paired grid would leave CUs without a workgroup.
+template <int D, int TEAMS>
+__global__ __launch_bounds__(256 * TEAMS, TEAMS == 1 ? 2 : 1) void sdpa_prefill_kernel(PrefillParams p) {
+    constexpr int PF_THREADS = 256 * TEAMS;
     constexpr int KP = D + 8;          // K tile row pitch (bf16): 16-byte aligned rows, 16 lanes of a b128 read on distinct banks
     constexpr int VP = PF_KB + 8;      // V^T tile row pitch (bf16)
     constexpr int NT = D / 16;         // MFMA steps along head_dim for S
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillPara
     __bf16* const vtile0 = ktile0 + 2 * PF_KB * KP;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6), team = wave_all >> 2, wave = wave_all & 3;
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6), team = TEAMS == 2 ? wave_all >> 2 : 0, wave = wave_all & 3;
     const int col = lane & 31, h = lane >> 5;
     const int per_kv = p.heads / p.kv_heads;
     const int hpw = p.heads_per_wg;
@@ -164,10 +167,15 @@ __global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillPara
     const int q_per_group = qblocks_per_wg * PF_QW;
     const int ngroups = (p.seq_q + q_per_group - 1) / q_per_group;
     const bool adjacent = p.window > 0 || !p.causal;
-    const int g_early = adjacent ? 2 * (int)blockIdx.x : (int)blockIdx.x;
-    const int g_late = adjacent ? min(g_early + 1, ngroups - 1) : ngroups - 1 - (int)blockIdx.x;
+    int g_early, g_late;
+    if (TEAMS == 2) {
+        g_early = adjacent ? 2 * (int)blockIdx.x : (int)blockIdx.x;
+        g_late = adjacent ? min(g_early + 1, ngroups - 1) : ngroups - 1 - (int)blockIdx.x;
+    } else {
+        g_late = g_early = p.causal ? ngroups - 1 - (int)blockIdx.x : (int)blockIdx.x;   // the groups with the most keys start first
+    }
     const int my_group = team ? g_early : g_late;
-    const bool team_active = !(team == 1 && g_early == g_late);
+    const bool team_active = TEAMS == 1 || !(team == 1 && g_early == g_late);
     const int q0 = my_group * q_per_group + (wave / hpw) * PF_QW;          // first query position of this wave
     auto group_first = [&](int g) { return g * q_per_group; };
     auto group_last = [&](int g) { return min(p.seq_q, (g + 1) * q_per_group) - 1; };
@@ -242,15 +250,15 @@ __global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillPara
     int blk = blk_begin;
     while (blk < nblocks && !needed(blk)) ++blk;
     if (blk < nblocks) {
-        pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, blk * PF_KB, tid);
-        pf_store_block<D>(kreg, vreg, ktile0, vtile0, tid);
+        pf_load_block<D, PF_THREADS>(kreg, vreg, kbase, vbase, p.spad, blk * PF_KB, tid);
+        pf_store_block<D, PF_THREADS>(kreg, vreg, ktile0, vtile0, tid);
     }
     __syncthreads();
 
     for (int buf = 0; blk < nblocks; buf ^= 1) {
         const int k0 = blk * PF_KB;
         const int nblk = next_needed(blk);
-        if (nblk < nblocks) pf_load_block<D>(kreg, vreg, kbase, vbase, p.spad, nblk * PF_KB, tid);
+        if (nblk < nblocks) pf_load_block<D, PF_THREADS>(kreg, vreg, kbase, vbase, p.spad, nblk * PF_KB, tid);
         if (k0 <= wave_last_key && k0 + PF_KB > wave_first_key) {     // wave-uniform: this wave has keys in the block
             // S^T tiles: s[j] covers keys k0 + 32 j .. + 31 (rows) x this wave's 32 queries (columns)
             pf_f32x16 s[2];
@@ -348,7 +356,7 @@ __global__ __launch_bounds__(PF_THREADS, 1) void sdpa_prefill_kernel(PrefillPara
                 }
             }
         }
-        if (nblk < nblocks) pf_store_block<D>(kreg, vreg, ktile0 + (buf ^ 1) * (PF_KB * KP), vtile0 + (buf ^ 1) * (D * VP), tid);
+        if (nblk < nblocks) pf_store_block<D, PF_THREADS>(kreg, vreg, ktile0 + (buf ^ 1) * (PF_KB * KP), vtile0 + (buf ^ 1) * (D * VP), tid);
         __syncthreads();
         blk = nblk;
     }
@@ -372,6 +380,8 @@ void* kernel_workspace(size_t bytes);   // shim.hip: per-thread scratch, grown o
 
 static std::atomic<int> g_prefill_mfma{1};
 void set_sdpa_prefill_mfma(int v) { g_prefill_mfma = v; }
+static std::atomic<int> g_prefill_teams{0};   // 0: chosen from the grid, 1: one query group per workgroup, 2: paired groups
+void set_sdpa_prefill_teams(int v) { if (v >= 0 && v <= 2) g_prefill_teams = v; }
 
 template <int D>
 static int launch_prefill_d(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
@@ -391,11 +401,19 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
     const int ngroups = (seq_q + q_per_group - 1) / q_per_group;
     PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, window, right_context, lengths, hpw,
                     mask, mask_b, mask_h, mask_q, mask_k};
-    const dim3 grid((ngroups + 1) / 2, kv_heads * (per_kv / hpw), batch);
+    // paired query groups where that still gives every CU a workgroup, else one group per (smaller) workgroup
+    const int64_t paired_wgs = (int64_t)((ngroups + 1) / 2) * kv_heads * (per_kv / hpw) * batch;
+    const bool paired = g_prefill_teams.load() == 0 ? paired_wgs >= num_cus() : g_prefill_teams.load() == 2;
+    const dim3 grid(paired ? (ngroups + 1) / 2 : ngroups, kv_heads * (per_kv / hpw), batch);
     constexpr size_t smem = sizeof(__bf16) * (2 * PF_KB * (D + 8) + 2 * D * (PF_KB + 8));
-    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D>), smem);
     note_kernel("sdpa_prefill_kernel");
-    sdpa_prefill_kernel<D><<<grid, dim3(PF_THREADS), smem, s>>>(p);
+    if (paired) {
+        SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D, 2>), smem);
+        sdpa_prefill_kernel<D, 2><<<grid, dim3(512), smem, s>>>(p);
+    } else {
+        SKH_SET_MAX_DYNAMIC_LDS_ONCE((&sdpa_prefill_kernel<D, 1>), smem);
+        sdpa_prefill_kernel<D, 1><<<grid, dim3(256), smem, s>>>(p);
+    }
     SKH_CHECK(hipGetLastError());
     return 1;
 }

@@ -206,12 +206,17 @@ def test_attention_prefill_mfma_window_and_key_lengths(hip_backend, torch_cuda, 
     v = rng.standard_normal((batch, kv_heads, skv, d)).astype(np.float32)
     scale = float(1 / np.sqrt(d))
     ln = None if lengths is None else np.asarray(lengths, np.int32)
-    got = gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, rc, ln)
-    assert hip_backend.last_kernel() == "sdpa_prefill_kernel"
     want = L.sdpa(q, k, v, scale, causal, window, rc, ln)
-    assert np.isfinite(got).all()
-    assert normalized_err(got, want, eps=1.0) <= 2e-2
-    assert np.sqrt(np.mean((got - want) ** 2)) <= 5e-3 * np.abs(want).max()
+    try:
+        for teams in (1, 2):        # one query group per workgroup; a late and an early (or two neighbouring) groups paired
+            hip_backend.set_tuning("sdpa_prefill_teams", teams)
+            got = gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, rc, ln)
+            assert hip_backend.last_kernel() == "sdpa_prefill_kernel"
+            assert np.isfinite(got).all()
+            assert normalized_err(got, want, eps=1.0) <= 2e-2
+            assert np.sqrt(np.mean((got - want) ** 2)) <= 5e-3 * np.abs(want).max()
+    finally:
+        hip_backend.set_tuning("sdpa_prefill_teams", 0)
     ones = np.ones_like(v)
     assert np.abs(gpu_sdpa(hip_backend, torch_cuda, q, k, ones, scale, causal, window, rc, ln) - 1.0).max() <= 1e-2
     hip_backend.set_tuning("sdpa_prefill_mfma", 0)
@@ -248,12 +253,17 @@ def test_attention_prefill_mfma_with_an_additive_mask(hip_backend, torch_cuda, b
         mask[..., 0] = np.minimum(mask[..., 0], 3.0)                   # and key 0 stays available
         mask[..., 0] = np.maximum(mask[..., 0], -3.0)
     ln = None if lengths is None else np.asarray(lengths, np.int32)
-    got = gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, 0, ln, mask)
-    assert hip_backend.last_kernel() == "sdpa_prefill_kernel"
     want = L.sdpa(q, k, v, scale, causal, window, 0, ln, mask)
-    assert np.isfinite(got).all()
-    assert normalized_err(got, want, eps=1.0) <= 2e-2
-    assert np.sqrt(np.mean((got - want) ** 2)) <= 5e-3 * np.abs(want).max()
+    try:
+        for teams in (1, 2):
+            hip_backend.set_tuning("sdpa_prefill_teams", teams)
+            got = gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, 0, ln, mask)
+            assert hip_backend.last_kernel() == "sdpa_prefill_kernel"
+            assert np.isfinite(got).all()
+            assert normalized_err(got, want, eps=1.0) <= 2e-2
+            assert np.sqrt(np.mean((got - want) ** 2)) <= 5e-3 * np.abs(want).max()
+    finally:
+        hip_backend.set_tuning("sdpa_prefill_teams", 0)
     hip_backend.set_tuning("sdpa_prefill_mfma", 0)
     try:
         close(gpu_sdpa(hip_backend, torch_cuda, q, k, v, scale, causal, window, 0, ln, mask), want)
