@@ -613,6 +613,63 @@ def measure_decoder_spi(workload, steps, warmup):
     return rec, ok
 
 
+UPLOAD_WORKLOADS = {"weight_upload_q4k_528mb": ("Q4_K", 229376, 4096)}   # name: (encoding, rows, cols)
+PCIE_PEAK_GBS = 64.0   # PCIe 5.0 x16, one direction, before protocol overhead
+
+
+def bench_upload(a):
+    """Host -> device rate of skainet_hip_weight_upload on one large packed weight (the bytes are never interpreted, so
+    they are random): from pageable memory through the library's page-locked chunks at the default setting and with the
+    staging off (one blocking copy), and from page-locked memory. A step is one upload; the best of `steps` is reported
+    (the host's page cache and clocks make the first calls slower), and the device copy is compared byte for byte."""
+    from skainet_amd import _lib, kernels
+    enc, rows, cols = UPLOAD_WORKLOADS[a.workload]
+    bs, nb = {"Q4_K": (256, 144)}[enc]
+    nbytes = rows * (cols // bs) * nb
+    steps = 6 if a.steps == 2000 else a.steps
+    src = np.random.default_rng(3).integers(0, 256, nbytes, dtype=np.uint8)
+    back = np.empty(nbytes, np.uint8)
+
+    def rate(arr, check):
+        best, ok = float("inf"), True
+        for i in range(steps):
+            t0 = time.perf_counter()
+            w = kernels.DeviceWeight.upload(enc, arr, rows, cols)
+            best = min(best, time.perf_counter() - t0)
+            if check and i == 0:
+                assert _lib.hip().skainet_hip_memcpy_d2h(back.ctypes.data, w.data_ptr, nbytes) == 0
+                ok = bool(np.array_equal(back, src))
+            w.close()
+        return nbytes / best / 1e9, best, ok
+
+    staged, best, ok = rate(src, True)
+    kernels.set_tuning("upload_chunk_mib", 0)
+    blocking, _, _ = rate(src, False)
+    kernels.set_tuning("upload_chunk_mib", 8)
+    pinned = kernels.PinnedBytes(nbytes)
+    pinned.array[:] = src
+    locked, _, ok2 = rate(pinned.array, True)
+    pinned.close()
+    t0 = time.perf_counter()
+    back[:] = src
+    host_copy = nbytes / (time.perf_counter() - t0) / 1e9
+    rec = {
+        "metric": "weight upload GB/s (pageable source)", "value": round(staged, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps,
+        "warmup": 0, "ms_per_step": round(best * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": a.workload, "encoding": enc, "rows": rows, "cols": cols, "bytes": nbytes,
+                   "timing": f"best of {steps} uploads, host clock around the call (it returns when the bytes are on the device)"},
+        "roofline": {"bound": "pcie", "achieved": round(staged, 2), "peak": PCIE_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(staged / PCIE_PEAK_GBS, 4), "traffic": None},
+        "extra": {"one_blocking_copy_GBps": round(blocking, 2), "page_locked_source_GBps": round(locked, 2),
+                  "host_memcpy_one_core_GBps": round(host_copy, 2), "device": _lib.hip().skainet_hip_device_name().decode()},
+    }
+    if not (ok and ok2):
+        rec["extra"]["PARITY_FAILED"] = True
+    print(json.dumps(rec))
+    sys.exit(0 if ok and ok2 else 1)
+
+
 def bench_decoder(a):
     if a.workload in SPI_DECODER_WORKLOADS:
         rec, ok = measure_decoder_spi(a.workload, 32 if a.steps == 2000 else a.steps, 4 if a.warmup == 200 else a.warmup)
@@ -630,7 +687,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000, help="timed steps (default 2000; 200 for the GEMM workloads)")
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(SPI_DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS) + sorted(DENSE_WORKLOADS))
+    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(SPI_DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS) + sorted(DENSE_WORKLOADS) + sorted(UPLOAD_WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
     ap.add_argument("--hbm-only", action="store_true", help="skip the cache-warm pass and the read probe, so every launch of the "
@@ -654,6 +711,8 @@ def main():
 
     if a.workload in DECODER_WORKLOADS or a.workload in SPI_DECODER_WORKLOADS:
         bench_decoder(a)
+    if a.workload in UPLOAD_WORKLOADS:
+        return bench_upload(a)
     if a.workload in DENSE_WORKLOADS:
         return bench_dense(a)
     if a.workload in ATTENTION_WORKLOADS:

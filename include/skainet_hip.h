@@ -85,6 +85,11 @@ SKAINET_HIP_API int32_t skainet_hip_free(void* device_ptr);
 SKAINET_HIP_API int32_t skainet_hip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
 SKAINET_HIP_API int32_t skainet_hip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
 SKAINET_HIP_API int32_t skainet_hip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes);
+/* Page-locked host memory for a loader to read packed weights into (wrap it as an off-heap MemorySegment, the kind of
+ * weight operand REF/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/NativeQ4KMemSegMatmulKernel.kt:39-44
+ * takes): skainet_hip_weight_upload from it is one DMA transfer with no staging copy on the host. NULL / -1 on failure. */
+SKAINET_HIP_API void* skainet_hip_host_alloc(size_t bytes);
+SKAINET_HIP_API int32_t skainet_hip_host_free(void* host_ptr);
 
 /* Elapsed-time measurement on the calling thread's stream (HIP events): begin, launch, end -> milliseconds. */
 SKAINET_HIP_API int32_t skainet_hip_timer_begin(void);
@@ -99,7 +104,10 @@ typedef struct skainet_hip_weight skainet_hip_weight;
 
 /* Copy `nbytes` packed bytes of a [rows, cols] weight to the device. `order` says how the host bytes are
  * laid out; the device copy is always canonical row-major (an input-block-major source is permuted on
- * the device, the inverse of API/PackedWeights.kt:63-93 toKernelOrder). NULL on failure. */
+ * the device, the inverse of API/PackedWeights.kt:63-93 toKernelOrder). Returns once the bytes are on the device: page-locked
+ * sources (skainet_hip_host_alloc) go as one transfer; pageable ones through page-locked chunks that a few host threads
+ * fill while earlier chunks are on the bus (the chunks, 64 MiB by default, are kept until the process ends; staged
+ * uploads from several threads take turns). NULL on failure. */
 SKAINET_HIP_API skainet_hip_weight* skainet_hip_weight_upload(
     const uint8_t* bytes, int64_t nbytes, int32_t encoding, int32_t order, int32_t rows, int32_t cols);
 /* Describe packed row-major bytes that already live on the device (not owned, not freed). */
@@ -361,7 +369,10 @@ SKAINET_HIP_API int32_t skainet_hip_graph_valid(const skainet_hip_graph* graph);
 SKAINET_HIP_API int32_t skainet_hip_graph_sync(skainet_hip_graph* graph);
 SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
 
-/* Launch-shape knobs for experiments (defaults are the measured best). Keys: "gemv_waves_per_cu",
+/* Launch-shape knobs for experiments (defaults are the measured best). Keys: "upload_chunk_mib" (size of the
+ * page-locked chunks skainet_hip_weight_upload stages pageable sources through, two per lane: 1 to 256 MiB, default 8;
+ * 0 = one blocking copy straight from the caller's memory), "upload_lanes" (host threads that fill those chunks, each
+ * with a stream of its own: 1 to 8, default 4), "gemv_waves_per_cu",
  * "q4k_rows_waves_per_cu" (resident waves per compute unit used to size the row shares, 0 = chosen from the shape),
  * "dense_mfma" (0: dense fp32 products stay on the vector-ALU tile kernel instead of the fp32 matrix instruction),
  * "gemv_stream_enable" (0: one-row Q8_0 / Q4_0 / Q5_0 / Q5_1 products stay on the row kernel instead of the one that

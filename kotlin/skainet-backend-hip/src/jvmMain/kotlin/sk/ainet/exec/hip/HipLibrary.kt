@@ -43,6 +43,9 @@ internal object HipLibrary {
     val h2d: MethodHandle? = bind("skainet_hip_memcpy_h2d", FunctionDescriptor.of(I, P, P, L))
     val d2h: MethodHandle? = bind("skainet_hip_memcpy_d2h", FunctionDescriptor.of(I, P, P, L))
     val d2d: MethodHandle? = bind("skainet_hip_memcpy_d2d", FunctionDescriptor.of(I, P, P, L))
+    /** Page-locked host memory for a loader to read packed weights into: `weightUpload` from it is one DMA transfer. */
+    val hostAlloc: MethodHandle? = bind("skainet_hip_host_alloc", FunctionDescriptor.of(P, L))
+    val hostFree: MethodHandle? = bind("skainet_hip_host_free", FunctionDescriptor.of(I, P))
 
     // ---- resident weights
     val weightUpload: MethodHandle? = bind("skainet_hip_weight_upload", FunctionDescriptor.of(P, P, L, I, I, I, I))

@@ -34,6 +34,8 @@ SIGNATURES = {
     "skainet_hip_memcpy_h2d": (_i32, [_vp, _vp, _sz]),
     "skainet_hip_memcpy_d2h": (_i32, [_vp, _vp, _sz]),
     "skainet_hip_memcpy_d2d": (_i32, [_vp, _vp, _sz]),
+    "skainet_hip_host_alloc": (_vp, [_sz]),
+    "skainet_hip_host_free": (_i32, [_vp]),
     "skainet_hip_timer_begin": (_i32, []),
     "skainet_hip_timer_end_ms": (_f32, []),
     "skainet_hip_weight_upload": (_vp, [_vp, _i64, _i32, _i32, _i32, _i32]),

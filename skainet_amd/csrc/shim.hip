@@ -14,7 +14,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
 #include <mutex>
+#include <thread>
 
 namespace skh {
 
@@ -70,6 +72,8 @@ static thread_local Scratch t_workspace;          // kernel scratch (attention s
 static thread_local Scratch t_stage[6];           // device staging of the host-pointer entries
 static thread_local Scratch t_fuse[2];            // normalised input / raw product of the unfused route of matmul_fused
 static thread_local Scratch t_pinned[2];          // page-locked host staging of skainet_hip_matmul_host (activations in, product out)
+static std::atomic<int> g_upload_chunk_mib{8};    // skainet_hip_weight_upload's page-locked chunks; 0: one blocking copy straight from the caller's memory
+static std::atomic<int> g_upload_lanes{4};        // host threads that fill them
 
 static std::mutex g_mutex;
 static int g_state = 0;        // 0 = not probed, 1 = usable, -1 = unusable
@@ -176,6 +180,88 @@ void* sync_scratch(size_t bytes) {
     }
     return t_sync;
 }
+// Host -> device copy of `bytes` bytes that returns when the data is on the device. Page-locked sources (the caller
+// read the file into memory from skainet_hip_host_alloc) go as ONE asynchronous copy at bus rate. Pageable sources go
+// through page-locked chunks: a lane owns two of them and a stream, and copies chunk j + 1 into one buffer while the
+// DMA engine moves chunk j out of the other. One host core fills a chunk at about half the bus rate, so large uploads
+// run several lanes on threads of their own, lane t taking chunks t, t + lanes, ...
+struct UploadLane {
+    void* pin[2] = {nullptr, nullptr};
+    size_t cap = 0;
+    hipEvent_t ev[2] = {nullptr, nullptr};
+    hipStream_t stream = nullptr;
+};
+constexpr int UPLOAD_MAX_LANES = 8;
+static UploadLane g_lanes[UPLOAD_MAX_LANES];     // made on first use, kept until the process ends
+static std::mutex g_upload_mutex;                // one staged upload at a time: they would share the bus anyway
+
+static hipError_t lane_prepare(UploadLane& l, size_t chunk) {
+    hipError_t e;
+    if (!l.stream && (e = hipStreamCreateWithFlags(&l.stream, hipStreamNonBlocking)) != hipSuccess) return e;
+    for (int b = 0; b < 2; ++b)
+        if (!l.ev[b] && (e = hipEventCreateWithFlags(&l.ev[b], hipEventDisableTiming)) != hipSuccess) return e;
+    if (l.cap < chunk) {
+        for (int b = 0; b < 2; ++b) {
+            if (l.pin[b]) { (void)hipHostFree(l.pin[b]); l.pin[b] = nullptr; }
+            l.cap = 0;
+            if ((e = hipHostMalloc(&l.pin[b], chunk, hipHostMallocDefault)) != hipSuccess) return e;
+        }
+        l.cap = chunk;
+    }
+    return hipSuccess;
+}
+static hipError_t lane_run(UploadLane& l, int lane, int lanes, uint8_t* dst, const uint8_t* src, size_t bytes, size_t chunk) {
+    hipError_t e;
+    int j = 0;
+    for (size_t off = (size_t)lane * chunk; off < bytes; off += (size_t)lanes * chunk, ++j) {
+        const int b = j & 1;
+        const size_t len = bytes - off < chunk ? bytes - off : chunk;
+        // the copy that last left this buffer (two of this lane's chunks ago) must be off the bus before it is overwritten
+        if (j >= 2 && (e = hipEventSynchronize(l.ev[b])) != hipSuccess) return e;
+        memcpy(l.pin[b], src + off, len);
+        if ((e = hipMemcpyAsync(dst + off, l.pin[b], len, hipMemcpyHostToDevice, l.stream)) != hipSuccess) return e;
+        if ((e = hipEventRecord(l.ev[b], l.stream)) != hipSuccess) return e;
+    }
+    return hipStreamSynchronize(l.stream);
+}
+static int staged_h2d(void* dst, const uint8_t* src, size_t bytes) {
+    if (bytes == 0) return 0;
+    const size_t chunk = (size_t)g_upload_chunk_mib.load() << 20;
+    bool pinned_src = false;
+    {
+        hipPointerAttribute_t attr;
+        const hipError_t e = hipPointerGetAttributes(&attr, src);
+        if (e == hipSuccess) pinned_src = attr.type == hipMemoryTypeHost;
+        else (void)hipGetLastError();                  // plain malloc memory: not known to the runtime
+    }
+    // `dst` is fresh memory that no queued work touches, so the lanes' own streams need not wait for the caller's; the
+    // call returns only when every lane's stream has drained, which orders the data before anything launched later
+    if (pinned_src) {
+        if (check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, t_stream), "hipMemcpy(weight)") != 0) return -1;
+        return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
+    }
+    if (chunk == 0 || bytes <= chunk) return check_hip(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice), "hipMemcpy(weight)");
+    const size_t chunks = (bytes + chunk - 1) / chunk;
+    int lanes = g_upload_lanes.load();
+    if ((size_t)lanes > chunks / 2) lanes = (int)(chunks / 2);      // a lane without two chunks of its own overlaps nothing
+    if (lanes < 1) lanes = 1;
+    std::lock_guard<std::mutex> lock(g_upload_mutex);
+    for (int t = 0; t < lanes; ++t)
+        if (check_hip(lane_prepare(g_lanes[t], chunk), "upload lane set-up") != 0) return -1;
+    hipError_t result[UPLOAD_MAX_LANES];
+    std::thread workers[UPLOAD_MAX_LANES];
+    const int device = g_device;
+    for (int t = 1; t < lanes; ++t)
+        workers[t] = std::thread([&, t] {
+            hipError_t e = hipSetDevice(device);
+            result[t] = e != hipSuccess ? e : lane_run(g_lanes[t], t, lanes, static_cast<uint8_t*>(dst), src, bytes, chunk);
+        });
+    result[0] = lane_run(g_lanes[0], 0, lanes, static_cast<uint8_t*>(dst), src, bytes, chunk);
+    for (int t = 1; t < lanes; ++t) workers[t].join();
+    for (int t = 0; t < lanes; ++t)
+        if (check_hip(result[t], "hipMemcpy(weight, staged)") != 0) return -1;
+    return 0;
+}
 float* sdpa_workspace(size_t bytes) { return static_cast<float*>(scratch_get(t_workspace, bytes)); }
 void* kernel_workspace(size_t bytes) { return scratch_get(t_workspace, bytes); }
 
@@ -232,10 +318,11 @@ int32_t skainet_hip_thread_release(void) {
     drop(t_workspace);
     for (Scratch& sc : t_stage) drop(sc);
     for (Scratch& sc : t_fuse) drop(sc);
-    for (Scratch& sc : t_pinned) {
+    auto drop_pinned = [&](Scratch& sc) {
         if (sc.ptr && check_hip(hipHostFree(sc.ptr), "hipHostFree(staging)") != 0) rc = -1;
         sc.ptr = nullptr; sc.cap = 0;
-    }
+    };
+    for (Scratch& sc : t_pinned) drop_pinned(sc);
     if (t_sync && check_hip(hipFree(t_sync), "hipFree(sync scratch)") != 0) rc = -1;
     t_sync = nullptr;
     if (t_ev0 && check_hip(hipEventDestroy(t_ev0), "hipEventDestroy") != 0) rc = -1;
@@ -253,6 +340,19 @@ int32_t skainet_hip_free(void* p) {
     if (!p) return 0;
     if (ensure_device() != 0) return -1;
     return check_hip(hipFree(p), "hipFree");
+}
+// Page-locked host memory for a loader to read packed weights into: an upload from it is one DMA transfer with no
+// staging copy on the host. Allocated, never registered (existing host memory cannot be pinned here).
+void* skainet_hip_host_alloc(size_t bytes) {
+    if (ensure_device() != 0) return nullptr;
+    void* p = nullptr;
+    if (check_hip(hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault), "hipHostMalloc") != 0) return nullptr;
+    return p;
+}
+int32_t skainet_hip_host_free(void* p) {
+    if (!p) return 0;
+    if (ensure_device() != 0) return -1;
+    return check_hip(hipHostFree(p), "hipHostFree");
 }
 int32_t skainet_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
     if (ensure_device() != 0) return -1;
@@ -289,6 +389,16 @@ float skainet_hip_timer_end_ms(void) {
 }
 int32_t skainet_hip_set_tuning(const char* key, int32_t value) {
     if (!key) return set_error("set_tuning: null key");
+    if (!strcmp(key, "upload_chunk_mib")) {
+        if (value < 0 || value > 256) return set_error("set_tuning: upload_chunk_mib must be 0 .. 256; got %d", value);
+        g_upload_chunk_mib = value;
+        return 0;
+    }
+    if (!strcmp(key, "upload_lanes")) {
+        if (value < 1 || value > UPLOAD_MAX_LANES) return set_error("set_tuning: upload_lanes must be 1 .. %d; got %d", UPLOAD_MAX_LANES, value);
+        g_upload_lanes = value;
+        return 0;
+    }
     if (set_tuning(key, value) != 0) return set_error("set_tuning: unknown key '%s'", key);
     return 0;
 }
@@ -314,11 +424,11 @@ skainet_hip_weight* skainet_hip_weight_upload(const uint8_t* bytes, int64_t nbyt
     if (check_hip(hipMalloc(&dev, (size_t)need), "hipMalloc(weight)") != 0) return nullptr;
     bool ok;
     if (order == SKAINET_HIP_ORDER_ROW_MAJOR) {
-        ok = check_hip(hipMemcpy(dev, bytes, (size_t)need, hipMemcpyHostToDevice), "hipMemcpy(weight)") == 0;
+        ok = staged_h2d(dev, bytes, (size_t)need) == 0;
     } else {
         void* tmp = nullptr;
         ok = check_hip(hipMalloc(&tmp, (size_t)need), "hipMalloc(weight staging)") == 0;
-        ok = ok && check_hip(hipMemcpy(tmp, bytes, (size_t)need, hipMemcpyHostToDevice), "hipMemcpy(weight)") == 0;
+        ok = ok && staged_h2d(tmp, bytes, (size_t)need) == 0;
         ok = ok && launch_relayout_to_row_major(static_cast<uint8_t*>(tmp), static_cast<uint8_t*>(dev), rows,
                                                 cols / block_elems(encoding), block_bytes(encoding)) == 0;
         ok = ok && check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize") == 0;

@@ -111,6 +111,32 @@ def to_kernel_order(encoding: str, row_major: np.ndarray, rows: int, blocks_per_
 EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
 
 
+class PinnedBytes:
+    """Page-locked host bytes from the library (skainet_hip_host_alloc) as a numpy uint8 array: read a weight file into
+    `.array` and DeviceWeight.upload moves it in one DMA transfer. The memory lives until close() / garbage collection;
+    `.array` must not be used afterwards."""
+
+    def __init__(self, nbytes: int):
+        _require_available()
+        self.nbytes = int(nbytes)
+        self.ptr = _lib.hip().skainet_hip_host_alloc(self.nbytes)
+        if not self.ptr:
+            raise HipError("host_alloc: " + _lib.last_error())
+        self.array = np.ctypeslib.as_array((C.c_uint8 * max(self.nbytes, 1)).from_address(self.ptr))[: self.nbytes]
+
+    def close(self) -> None:
+        if self.ptr:
+            self.array = None
+            _lib.hip().skainet_hip_host_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class DeviceWeight:
     """A packed [rows, cols] weight resident on the device (canonical row-major blocks)."""
 

@@ -342,3 +342,43 @@ def test_more_formats_spi_kernels_on_host_arrays(hip_backend, torch_cuda, enc):
     assert np.array_equal(out2, out[pad_y:pad_y + n])
     with pytest.raises(ValueError):
         kernel.matmul(x, 0, wbm, 0, k - 1, n, out, 0)
+
+
+def _device_bytes(kernels, w):
+    """The device copy of an uploaded weight, byte for byte."""
+    from skainet_amd import _lib
+    out = np.empty(w.nbytes, np.uint8)
+    assert _lib.hip().skainet_hip_memcpy_d2h(out.ctypes.data, w.data_ptr, out.size) == 0
+    return out
+
+
+@pytest.mark.parametrize("chunk_mib,lanes", [(0, 4), (1, 1), (1, 3), (1, 8), (8, 4)])
+def test_weight_upload_through_the_page_locked_chunks_is_byte_exact(hip_backend, torch_cuda, chunk_mib, lanes):
+    """A pageable source is staged through page-locked chunks, two per lane (one filled while the other is on the bus),
+    the lanes on host threads of their own: a weight of many chunks with a ragged last one, with fewer chunks than the
+    lanes could take, a weight smaller than a chunk, the staging switched off, a page-locked source (one transfer),
+    and the input-block-major order (permuted on the device) all leave the same bytes on the device."""
+    rng = np.random.default_rng(77 + chunk_mib + lanes)
+    try:
+        hip_backend.set_tuning("upload_chunk_mib", chunk_mib)
+        hip_backend.set_tuning("upload_lanes", lanes)
+        for enc, rows, cols in (("Q4_K", 4100, 4096), ("Q8_0", 37, 96), ("Q6_K", 3000, 2304)):
+            bs, nb = G.PACKED[enc][0], G.PACKED[enc][1]
+            per_row = cols // bs
+            packed = rng.integers(0, 256, rows * per_row * nb, dtype=np.uint8)      # upload never interprets the bytes
+            w = hip_backend.DeviceWeight.upload(enc, packed, rows, cols)
+            assert np.array_equal(_device_bytes(hip_backend, w), packed), (enc, "pageable")
+            w.close()
+            pinned = hip_backend.PinnedBytes(packed.size)
+            pinned.array[:] = packed
+            w = hip_backend.DeviceWeight.upload(enc, pinned.array, rows, cols)
+            assert np.array_equal(_device_bytes(hip_backend, w), packed), (enc, "page-locked")
+            w.close()
+            pinned.close()
+            block_major = np.ascontiguousarray(packed.reshape(rows, per_row, nb).transpose(1, 0, 2)).reshape(-1)
+            w = hip_backend.DeviceWeight.upload(enc, block_major, rows, cols, order=1)
+            assert np.array_equal(_device_bytes(hip_backend, w), packed), (enc, "block-major")
+            w.close()
+    finally:
+        hip_backend.set_tuning("upload_chunk_mib", 8)
+        hip_backend.set_tuning("upload_lanes", 4)
