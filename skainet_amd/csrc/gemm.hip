@@ -143,27 +143,36 @@ __device__ __forceinline__ float gemm_byte_to_float(uint32_t v) {
 // Per encoding: load_raw (global loads of a thread's 32 weights), decode_prepare (scales of the 32), and the decode of
 // part I (0..7, four weights) in two stages the main loop places separately: decode_codes<I> gathers the part's four
 // codes into the bytes of one dword, decode_pair<I, H> turns bytes 2 H and 2 H + 1 of it into two fp32 weights.
-struct RawQ4K { uint4 hdr, q0, q1; };
-struct RawQ6K { uint32_t ql[8], qh[8]; uint32_t sc, d; };
+// What is constant over the four steps of a 256-element super-block is loaded once per super-block into an Sb (load_sb)
+// and not with every step's codes: a step's loads are one instruction per 16 bytes and row, each touching as many cache
+// lines as the wave has rows, and their number, not their bytes, is what the weight side of the tile costs (Q6_K with
+// its two 2-byte loads of scales and d per task and step: 184.7 us per 512 x 32000 x 4096 product, 155 us without them).
+struct SbNone {};
+struct RawQ4K { uint4 q0, q1; };
+struct SbQ4K { uint4 hdr; };
+struct RawQ6K { uint32_t ql[8], qh[4]; };
+struct SbQ6K { u32x4_vec sc; uint32_t d; };          // the 16 int8 scales, the fp16 d
 struct RawQ80 { u32x4_vec lo, hi; uint32_t edge, odd; };   // aligned 32-byte body, the 2 bytes outside it, start parity
 
 // `e` = element offset inside the row, a multiple of 32.
 __device__ __forceinline__ void load_raw(RawQ4K& r, const uint8_t* row, int e) {
     const uint8_t* blk = row + (e >> 8) * Q4K_BYTES;
     const int g = (e & 255) >> 6;                     // 32-byte nibble group holding sub-blocks 2g, 2g+1
-    r.hdr = *reinterpret_cast<const uint4*>(blk);
     r.q0 = *reinterpret_cast<const uint4*>(blk + 16 + g * 32);
     r.q1 = *reinterpret_cast<const uint4*>(blk + 32 + g * 32);
+}
+__device__ __forceinline__ void load_sb(SbQ4K& sb, const uint8_t* row, int e) {
+    sb.hdr = *reinterpret_cast<const uint4*>(row + (e >> 8) * Q4K_BYTES);
 }
 // The decode of a thread's 32 weights is split into a header part and eight 4-weight parts (one per dword of
 // codes) so the main loop can place the parts between its MFMAs.
 struct DecQ4K { float scale, offset; int shift; };
-__device__ __forceinline__ void decode_prepare(const RawQ4K& r, int e, DecQ4K& c) {
+__device__ __forceinline__ void decode_prepare_k4(const uint4& hdr, int e, DecQ4K& c) {
     const int sb = (e & 255) >> 5;
-    const float d = half_bits_to_float_fast(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(r.hdr.x >> 16);
+    const float d = half_bits_to_float_fast(hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(hdr.x >> 16);
     // ggml get_scale_min_k4 on the 12 scale bytes s[0..11] (hdr.y = s[0..3], hdr.z = s[4..7], hdr.w = s[8..11])
     const int sh = (sb & 3) * 8;
-    const uint32_t sa = (r.hdr.y >> sh) & 0xFFu, sbm = (r.hdr.z >> sh) & 0xFFu, st = (r.hdr.w >> sh) & 0xFFu;
+    const uint32_t sa = (hdr.y >> sh) & 0xFFu, sbm = (hdr.z >> sh) & 0xFFu, st = (hdr.w >> sh) & 0xFFu;
     // both packings are evaluated and one is picked with a mask: a select written as a conditional becomes a branch
     // here, and a branch inside the K loop makes every wait behind it cover all the loads in flight
     const uint32_t hi = (uint32_t)-(int)(sb >> 2);            // sb >= 4: all ones
@@ -173,8 +182,9 @@ __device__ __forceinline__ void decode_prepare(const RawQ4K& r, int e, DecQ4K& c
     c.offset = dmin * (float)mn;
     c.shift = (sb & 1) * 4;
 }
+__device__ __forceinline__ void decode_prepare(const RawQ4K&, const SbQ4K& sb, int e, DecQ4K& c) { decode_prepare_k4(sb.hdr, e, c); }
 template <int I>
-__device__ __forceinline__ uint32_t decode_codes(const RawQ4K& r, const DecQ4K& c) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ4K& r, const SbQ4K&, const DecQ4K& c) {
     const uint32_t q = I == 0 ? r.q0.x : I == 1 ? r.q0.y : I == 2 ? r.q0.z : I == 3 ? r.q0.w
                      : I == 4 ? r.q1.x : I == 5 ? r.q1.y : I == 6 ? r.q1.z : r.q1.w;
     return (q >> c.shift) & 0x0F0F0F0Fu;
@@ -185,38 +195,47 @@ __device__ __forceinline__ void decode_pair(uint32_t v, const DecQ4K& c, float& 
     w1 = fmaf(gemm_byte_to_float<2 * H + 1>(v), c.scale, -c.offset);
 }
 
+// Q6_K: the pair of threads that shares a row's 64 elements of a step splits them by position inside the 32-element
+// quarters, not by quarter: thread `wsub` decodes positions 16 wsub .. 16 wsub + 15 of both quarters (elements
+// E + 16 wsub + .. and E + 32 + 16 wsub + ..). Its codes are then three runs of 16 bytes (low bits of either quarter, the
+// shared plane of high bits) that no other thread loads, where a thread that owns a whole quarter needs all 32 bytes of
+// the high-bit plane, the same 32 as its neighbour. park_elem gives the position of a thread's weights in the tile row.
 __device__ __forceinline__ void load_raw(RawQ6K& r, const uint8_t* row, int e) {
     const uint8_t* blk = row + (e >> 8) * Q6K_BYTES;
-    const int half = (e & 255) >> 7, kq = (e & 127) >> 5;   // quarter kq of the half: output offset 32 * kq
-    const uint8_t* ql = blk + half * 64 + (kq & 1) * 32;
-    const uint8_t* qh = blk + 128 + half * 32;
-    // two 16-byte loads per 32-byte run (2-byte aligned): 6 loads per task instead of 18, so that two steps of weights in
-    // flight stay far below the 63 loads a wave's memory counter can track
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const u32x4_vec l4 = load_u32x4_a2(ql + 16 * h), h4 = load_u32x4_a2(qh + 16 * h);
-        r.ql[4 * h] = l4.x; r.ql[4 * h + 1] = l4.y; r.ql[4 * h + 2] = l4.z; r.ql[4 * h + 3] = l4.w;
-        r.qh[4 * h] = h4.x; r.qh[4 * h + 1] = h4.y; r.qh[4 * h + 2] = h4.z; r.qh[4 * h + 3] = h4.w;
-    }
-    // the two int8 scales of this quarter: sc[half * 8 + 2 * kq] (elements 0..15) and [.. + 1] (elements 16..31)
-    r.sc = load_u16(blk + 192 + half * 8 + 2 * kq);
-    r.d = load_u16(blk + 208);
+    const int half = (e & 255) >> 7, wsub = (e >> 5) & 1;
+    const uint8_t* ql = blk + half * 64 + 16 * wsub;
+    const u32x4_vec la = load_u32x4_a2(ql), lb = load_u32x4_a2(ql + 32), h4 = load_u32x4_a2(blk + 128 + half * 32 + 16 * wsub);
+    r.ql[0] = la.x; r.ql[1] = la.y; r.ql[2] = la.z; r.ql[3] = la.w;
+    r.ql[4] = lb.x; r.ql[5] = lb.y; r.ql[6] = lb.z; r.ql[7] = lb.w;
+    r.qh[0] = h4.x; r.qh[1] = h4.y; r.qh[2] = h4.z; r.qh[3] = h4.w;
+}
+__device__ __forceinline__ void load_sb(SbQ6K& sb, const uint8_t* row, int e) {
+    const uint8_t* blk = row + (e >> 8) * Q6K_BYTES;
+    sb.sc = load_u32x4_a2(blk + 192);
+    sb.d = load_u16(blk + 208);
 }
 struct DecQ6K { float s0, s1, n0, n1; int nib, hs; };   // n = -32 s
-__device__ __forceinline__ void decode_prepare(const RawQ6K& r, int e, DecQ6K& c) {
-    const int kq = (e & 127) >> 5;
-    const float d = half_bits_to_float_fast(r.d);
-    c.s0 = d * (float)(int8_t)(r.sc & 0xFF);
-    c.s1 = d * (float)(int8_t)(r.sc >> 8);
+__device__ __forceinline__ void decode_prepare(const RawQ6K&, const SbQ6K& sb, int e, DecQ6K& c) {
+    // the step's quarters are kq and kq + 1 (kq 0 or 2) of its half; this thread's 16 positions of either lie in one
+    // 16-element scale group each: sc[8 half + 2 kq + wsub] and sc[8 half + 2 kq + 2 + wsub], bytes wsub and wsub + 2 of
+    // dword `step` (0..3) of the 16 scales
+    const int kq = (e & 127) >> 6 << 1, step = (e & 255) >> 6, wsub = (e >> 5) & 1;
+    const float d = half_bits_to_float_fast(sb.d);
+    // picked with masks (no branch, no indexed register)
+    const uint32_t m0 = (uint32_t)-(int)(step == 0), m1 = (uint32_t)-(int)(step == 1), m2 = (uint32_t)-(int)(step == 2), m3 = (uint32_t)-(int)(step == 3);
+    const uint32_t four = ((sb.sc.x & m0) | (sb.sc.y & m1) | (sb.sc.z & m2) | (sb.sc.w & m3)) >> (8 * wsub);
+    c.s0 = d * (float)(int8_t)(four & 0xFF);
+    c.s1 = d * (float)(int8_t)((four >> 16) & 0xFF);
     c.n0 = -32.f * c.s0;
     c.n1 = -32.f * c.s1;
     c.nib = (kq >> 1) * 4;
     c.hs = 2 * kq;
 }
 template <int I>
-__device__ __forceinline__ uint32_t decode_codes(const RawQ6K& r, const DecQ6K& c) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ6K& r, const SbQ6K&, const DecQ6K& c) {
+    // parts 0..3: quarter kq (bit pair kq of the high-bit bytes), parts 4..7: quarter kq + 1 (the next bit pair)
     const uint32_t lo = (r.ql[I] >> c.nib) & 0x0F0F0F0Fu;
-    const uint32_t hi = ((r.qh[I] >> c.hs) & 0x03030303u) << 4;
+    const uint32_t hi = ((r.qh[I & 3] >> (c.hs + (I < 4 ? 0 : 2))) & 0x03030303u) << 4;
     return lo | hi;                                          // four 6-bit codes, one per byte
 }
 template <int I, int H>
@@ -238,12 +257,12 @@ __device__ __forceinline__ void load_raw(RawQ80& r, const uint8_t* row, int e) {
     r.edge = load_u16(blk + (r.odd ? 0 : 32));
 }
 struct DecQ80 { float d; uint32_t drop; };
-__device__ __forceinline__ void decode_prepare(const RawQ80& r, int, DecQ80& c) {
+__device__ __forceinline__ void decode_prepare(const RawQ80& r, const SbNone&, int, DecQ80& c) {
     c.d = half_bits_to_float_fast(r.odd ? r.edge : (r.lo.x & 0xFFFFu));
     c.drop = r.odd ? 0u : 2u;                        // bytes in front of the codes in the loaded dwords
 }
 template <int I>
-__device__ __forceinline__ uint32_t decode_codes(const RawQ80& r, const DecQ80& c) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ80& r, const SbNone&, const DecQ80& c) {
     const uint32_t v[9] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w, r.edge};
     return __builtin_amdgcn_alignbyte(v[I + 1], v[I], c.drop);
 }
@@ -269,13 +288,13 @@ __device__ __forceinline__ void load_raw(RawQ45<FMT>& r, const uint8_t* row, int
 }
 struct DecQ45 { float d, add; };
 template <int FMT>
-__device__ __forceinline__ void decode_prepare(const RawQ45<FMT>& r, int, DecQ45& c) {
+__device__ __forceinline__ void decode_prepare(const RawQ45<FMT>& r, const SbNone&, int, DecQ45& c) {
     c.d = half_bits_to_float_fast(r.d);
     // w = d * code + add:  Q4_0 d * (code - 8),  Q5_0 d * (code5 - 16),  Q5_1 d * code5 + m
     c.add = FMT == 0 ? -8.f * c.d : (FMT == 1 ? -16.f * c.d : half_bits_to_float_fast(r.m));
 }
 template <int I, int FMT>
-__device__ __forceinline__ uint32_t decode_codes(const RawQ45<FMT>& r, const DecQ45&) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ45<FMT>& r, const SbNone&, const DecQ45&) {
     // parts 0..3: low nibbles of code dword I (elements 4I ..), parts 4..7: high nibbles of dword I - 4 (elements 16 + ..)
     uint32_t v = (r.q[I & 3] >> (I < 4 ? 0 : 4)) & 0x0F0F0F0Fu;
     if (FMT != 0) v |= ((((r.qh >> (4 * I)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;   // fifth bits 4I .. 4I + 3
@@ -288,30 +307,33 @@ __device__ __forceinline__ void decode_pair(uint32_t v, const DecQ45& c, float& 
 }
 
 // Q5_K: the Q4_K sub-block plus bit sb of the 32-byte fifth-bit plane at byte 16 (nibbles at byte 48).
-struct RawQ5K { uint4 hdr, q0, q1, h0, h1; };
+struct RawQ5K { uint4 q0, q1; };
+struct SbQ5K { uint4 hdr, h0, h1; };                // header and the fifth-bit plane: the same for all eight sub-blocks
 __device__ __forceinline__ void load_raw(RawQ5K& r, const uint8_t* row, int e) {
     const uint8_t* blk = row + (e >> 8) * Q5K_BYTES;
     const int g = (e & 255) >> 6;
-    r.hdr = *reinterpret_cast<const uint4*>(blk);
-    r.h0 = *reinterpret_cast<const uint4*>(blk + 16);
-    r.h1 = *reinterpret_cast<const uint4*>(blk + 32);
     r.q0 = *reinterpret_cast<const uint4*>(blk + 48 + g * 32);
     r.q1 = *reinterpret_cast<const uint4*>(blk + 64 + g * 32);
 }
+__device__ __forceinline__ void load_sb(SbQ5K& sb, const uint8_t* row, int e) {
+    const uint8_t* blk = row + (e >> 8) * Q5K_BYTES;
+    sb.hdr = *reinterpret_cast<const uint4*>(blk);
+    sb.h0 = *reinterpret_cast<const uint4*>(blk + 16);
+    sb.h1 = *reinterpret_cast<const uint4*>(blk + 32);
+}
 struct DecQ5K { float scale, offset; int shift, bit; };
-__device__ __forceinline__ void decode_prepare(const RawQ5K& r, int e, DecQ5K& c) {
-    const RawQ4K r4{r.hdr, r.q0, r.q1};
+__device__ __forceinline__ void decode_prepare(const RawQ5K&, const SbQ5K& sb, int e, DecQ5K& c) {
     DecQ4K c4;
-    decode_prepare(r4, e, c4);                       // same d / dmin / 6-bit scale and min packing
+    decode_prepare_k4(sb.hdr, e, c4);                // same d / dmin / 6-bit scale and min packing
     c.scale = c4.scale; c.offset = c4.offset; c.shift = c4.shift;
     c.bit = (e & 255) >> 5;
 }
 template <int I>
-__device__ __forceinline__ uint32_t decode_codes(const RawQ5K& r, const DecQ5K& c) {
+__device__ __forceinline__ uint32_t decode_codes(const RawQ5K& r, const SbQ5K& sb, const DecQ5K& c) {
     const uint32_t q = I == 0 ? r.q0.x : I == 1 ? r.q0.y : I == 2 ? r.q0.z : I == 3 ? r.q0.w
                      : I == 4 ? r.q1.x : I == 5 ? r.q1.y : I == 6 ? r.q1.z : r.q1.w;
-    const uint32_t h = I == 0 ? r.h0.x : I == 1 ? r.h0.y : I == 2 ? r.h0.z : I == 3 ? r.h0.w
-                     : I == 4 ? r.h1.x : I == 5 ? r.h1.y : I == 6 ? r.h1.z : r.h1.w;
+    const uint32_t h = I == 0 ? sb.h0.x : I == 1 ? sb.h0.y : I == 2 ? sb.h0.z : I == 3 ? sb.h0.w
+                     : I == 4 ? sb.h1.x : I == 5 ? sb.h1.y : I == 6 ? sb.h1.z : sb.h1.w;
     return ((q >> c.shift) & 0x0F0F0F0Fu) | (((h >> c.bit) & 0x01010101u) << 4);
 }
 template <int I, int H>
@@ -320,6 +342,19 @@ __device__ __forceinline__ void decode_pair(uint32_t v, const DecQ5K& c, float& 
     w1 = fmaf(gemm_byte_to_float<2 * H + 1>(v), c.scale, -c.offset);
 }
 
+__device__ __forceinline__ void load_sb(SbNone&, const uint8_t*, int) {}
+template <class Raw> struct SbOf { typedef SbNone type; };
+template <> struct SbOf<RawQ4K> { typedef SbQ4K type; };
+template <> struct SbOf<RawQ6K> { typedef SbQ6K type; };
+template <> struct SbOf<RawQ5K> { typedef SbQ5K type; };
+// Steps of 64 elements that one load_raw serves. Q6_K: the two steps of a 128-element half read the same 96 bytes (low
+// nibbles and bit pairs 0..3 of the fifth / sixth bit plane in the first, high nibbles and bit pairs 4..7 in the second),
+// so they are loaded once per half and decoded twice.
+template <class Raw> struct RawSteps { static constexpr int value = 1; };
+template <> struct RawSteps<RawQ6K> { static constexpr int value = 2; };
+// Element offset, inside a row's 64 elements of a step, of weights 8 i .. 8 i + 7 (i = 0..3) of thread `wsub` of the pair.
+template <class Raw> __device__ __forceinline__ int park_elem(int wsub, int i) { return 32 * wsub + 8 * i; }
+template <> __device__ __forceinline__ int park_elem<RawQ6K>(int wsub, int i) { return 32 * (i >> 1) + 16 * wsub + 8 * (i & 1); }
 template <class Raw> struct DecOf;
 template <> struct DecOf<RawQ4K> { typedef DecQ4K type; };
 template <> struct DecOf<RawQ6K> { typedef DecQ6K type; };
@@ -332,33 +367,33 @@ typedef __bf16 gemm_bf16x2 __attribute__((ext_vector_type(2)));
 // packed bf16 pair. The first item of a part gathers its codes into `codes`, the second reuses them: about seven
 // vector instructions for the first, five for the second -- what fits between two MFMAs without holding the matrix
 // core up.
-template <int I, int H, class Raw, class Dec>
-__device__ __forceinline__ uint32_t decode_item(const Raw& r, const Dec& c, uint32_t& codes) {
-    if (H == 0) codes = decode_codes<I>(r, c);
+template <int I, int H, class Raw, class Sb, class Dec>
+__device__ __forceinline__ uint32_t decode_item(const Raw& r, const Sb& sb, const Dec& c, uint32_t& codes) {
+    if (H == 0) codes = decode_codes<I>(r, sb, c);
     float w0, w1;
     decode_pair<I, H>(codes, c, w0, w1);
     return __builtin_bit_cast(uint32_t, gemm_bf16x2{(__bf16)w0, (__bf16)w1});
 }
 // item h with h a (constant-folded) loop variable
-template <class Raw, class Dec>
-__device__ __forceinline__ uint32_t decode_item_at(int h, const Raw& r, const Dec& c, uint32_t& codes) {
+template <class Raw, class Sb, class Dec>
+__device__ __forceinline__ uint32_t decode_item_at(int h, const Raw& r, const Sb& sb, const Dec& c, uint32_t& codes) {
     switch (h) {
-        case 0: return decode_item<0, 0>(r, c, codes);
-        case 1: return decode_item<0, 1>(r, c, codes);
-        case 2: return decode_item<1, 0>(r, c, codes);
-        case 3: return decode_item<1, 1>(r, c, codes);
-        case 4: return decode_item<2, 0>(r, c, codes);
-        case 5: return decode_item<2, 1>(r, c, codes);
-        case 6: return decode_item<3, 0>(r, c, codes);
-        case 7: return decode_item<3, 1>(r, c, codes);
-        case 8: return decode_item<4, 0>(r, c, codes);
-        case 9: return decode_item<4, 1>(r, c, codes);
-        case 10: return decode_item<5, 0>(r, c, codes);
-        case 11: return decode_item<5, 1>(r, c, codes);
-        case 12: return decode_item<6, 0>(r, c, codes);
-        case 13: return decode_item<6, 1>(r, c, codes);
-        case 14: return decode_item<7, 0>(r, c, codes);
-        default: return decode_item<7, 1>(r, c, codes);
+        case 0: return decode_item<0, 0>(r, sb, c, codes);
+        case 1: return decode_item<0, 1>(r, sb, c, codes);
+        case 2: return decode_item<1, 0>(r, sb, c, codes);
+        case 3: return decode_item<1, 1>(r, sb, c, codes);
+        case 4: return decode_item<2, 0>(r, sb, c, codes);
+        case 5: return decode_item<2, 1>(r, sb, c, codes);
+        case 6: return decode_item<3, 0>(r, sb, c, codes);
+        case 7: return decode_item<3, 1>(r, sb, c, codes);
+        case 8: return decode_item<4, 0>(r, sb, c, codes);
+        case 9: return decode_item<4, 1>(r, sb, c, codes);
+        case 10: return decode_item<5, 0>(r, sb, c, codes);
+        case 11: return decode_item<5, 1>(r, sb, c, codes);
+        case 12: return decode_item<6, 0>(r, sb, c, codes);
+        case 13: return decode_item<6, 1>(r, sb, c, codes);
+        case 14: return decode_item<7, 0>(r, sb, c, codes);
+        default: return decode_item<7, 1>(r, sb, c, codes);
     }
 }
 
@@ -400,8 +435,12 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     // to be used. Loads are unconditional (clamped rows, never stored) so a step's loads are in flight together.
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     typedef typename DecOf<Raw>::type Dec;
+    typedef typename SbOf<Raw>::type Sb;
     u32x4 aring[A_SLOTS][G_A_LOADS];
     Raw wring[2][G_W_TASKS];
+    // per-super-block constants of each task's row: those of the super-block being decoded, and those of the one after it,
+    // requested in the second of a super-block's four steps and taken over behind the fourth
+    Sb sb_cur[G_W_TASKS], sb_next[G_W_TASKS];
     auto step_k = [&](int step) { return k_begin + min(step, nsteps - 1) * GK; };   // loads past the end re-read the last step
     auto load_a_chunk = [&](int slot, int step, int j) __attribute__((always_inline)) {
         const int p = tid + G_THREADS * j, row = p >> 3, kp = p & 7;
@@ -424,8 +463,8 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     };
     uint32_t wp[G_W_TASKS][16];                                                         // packed bf16 pairs: weights 2 h, 2 h + 1
     auto park_w = [&](int stage, int t, int i) __attribute__((always_inline)) {         // weights 8 i .. 8 i + 7 of task t's 32
-        __bf16* dst = w_tile(stage) + (wrow + (G_THREADS / 2) * t) * GSTRIDE + 32 * wsub;
-        *reinterpret_cast<u32x4*>(dst + 8 * i) = u32x4{wp[t][4 * i], wp[t][4 * i + 1], wp[t][4 * i + 2], wp[t][4 * i + 3]};
+        __bf16* dst = w_tile(stage) + (wrow + (G_THREADS / 2) * t) * GSTRIDE + park_elem<Raw>(wsub, i);
+        *reinterpret_cast<u32x4*>(dst) = u32x4{wp[t][4 * i], wp[t][4 * i + 1], wp[t][4 * i + 2], wp[t][4 * i + 3]};
     };
 
     f32x16 acc[WTM][G_WTN];
@@ -454,7 +493,17 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
     //   behind the last N_STORES MFMAs       one LDS store each into the other stage: every weight chunk after its
     //                                        items, the activation chunks as late as possible, each followed by the
     //                                        global load that refills its ring register
-    auto step_body = [&](int stage, int slot_next, int step_next, int load_slot, int load_step) __attribute__((always_inline)) {
+    // `uc`: the step's position U in its super-block (0..3), a compile-time constant.
+    auto step_body = [&](auto uc, int stage, int slot_next, int step_next, int load_slot, int load_step) __attribute__((always_inline)) {
+        constexpr int U = decltype(uc)::value;
+        Sb (&sb_dec)[G_W_TASKS] = U == 3 ? sb_next : sb_cur;       // the step decoded during this one is step_next
+        // weight ring: a slot per step (requested two steps ahead), or per two steps (requested in the odd steps for the
+        // pair that starts three steps on; the slot's last decode was a step ago)
+        constexpr int RS = RawSteps<Raw>::value;
+        constexpr int w_slot_next = RS == 1 ? (U + 1) & 1 : ((U + 1) >> 1) & 1;
+        constexpr int w_load_slot = RS == 1 ? U & 1 : ((U + 3) >> 1) & 1;
+        constexpr bool w_load = RS == 1 || (U & 1);
+        const int w_load_step = RS == 1 ? load_step : load_step + 1;
         const int a_slot_next = A_SLOTS == 2 ? slot_next : 0;
         const int a_load_slot = A_SLOTS == 2 ? load_slot : 0, a_load_step = A_SLOTS == 2 ? load_step : step_next + 1;
         constexpr int N_MFMA = WTM * G_WTN * (GK / 16), N_HALVES = 16 * G_W_TASKS, N_STORES = G_A_LOADS + 4 * G_W_TASKS;
@@ -484,11 +533,12 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (q < G_W_TASKS) {
-                load_w_task(load_slot, load_step, q);
+                if (w_load) load_w_task(w_load_slot, w_load_step, q);
+                if (U == 1) load_sb(sb_next[q], wrow_ptr[q], step_k(step_next + 2));   // first step of the next super-block
                 __builtin_amdgcn_sched_barrier(0);
             } else if (q < FIRST_ITEM) {
                 const int t = q - G_W_TASKS;
-                decode_prepare(wring[slot_next][t], step_k(step_next) + 32 * wsub, dc[t]);
+                decode_prepare(wring[w_slot_next][t], sb_dec[t], step_k(step_next) + 32 * wsub, dc[t]);
                 __builtin_amdgcn_sched_barrier(0);
             } else if (q < FIRST_ITEM + N_GAPS) {
                 // decode item h sits behind MFMA FIRST_ITEM + h * N_GAPS / N_HALVES: evenly spread (the 256-row tiles have
@@ -497,7 +547,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
                 const int h0 = (g * N_HALVES + N_GAPS - 1) / N_GAPS, h1 = ((g + 1) * N_HALVES + N_GAPS - 1) / N_GAPS;
 #pragma clang loop unroll(full)
                 for (int hh = h0; hh < h1 && hh < N_HALVES; ++hh) {
-                    wp[hh / 16][hh % 16] = decode_item_at(hh % 16, wring[slot_next][hh / 16], dc[hh / 16], codes[hh / 16]);
+                    wp[hh / 16][hh % 16] = decode_item_at(hh % 16, wring[w_slot_next][hh / 16], sb_dec[hh / 16], dc[hh / 16], codes[hh / 16]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
@@ -514,38 +564,47 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if (U == 3) {
+#pragma unroll
+            for (int t = 0; t < G_W_TASKS; ++t) sb_cur[t] = sb_next[t];
+        }
     };
 
     // nsteps is a multiple of 4 (K chunks are whole 256-element groups) and > 0. The loop body is one straight-line
     // block (no branches), which is what lets the compiler's wait-count bookkeeping leave the newest step's loads in
     // flight while the older ones are parked.
     load_a(0, 0);
+#pragma unroll
+    for (int t = 0; t < G_W_TASKS; ++t) load_sb(sb_cur[t], wrow_ptr[t], step_k(0));
     load_w(0, 0);
 #pragma unroll
     for (int j = 0; j < G_A_LOADS; ++j) park_a(0, 0, j);
 #pragma unroll
     for (int t = 0; t < G_W_TASKS; ++t) {
         Dec d0;
-        decode_prepare(wring[0][t], step_k(0) + 32 * wsub, d0);
+        decode_prepare(wring[0][t], sb_cur[t], step_k(0) + 32 * wsub, d0);
         uint32_t codes0 = 0;
 #pragma unroll
-        for (int h = 0; h < 16; ++h) wp[t][h] = decode_item_at(h, wring[0][t], d0, codes0);
+        for (int h = 0; h < 16; ++h) wp[t][h] = decode_item_at(h, wring[0][t], sb_cur[t], d0, codes0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) park_w(0, t, i);
     }
     load_a(A_SLOTS == 2 ? 1 : 0, 1);
-    load_w(1, 1);
+    load_w(1, RawSteps<Raw>::value);                             // the ring's second slot: step 1, or steps 2 and 3
     __syncthreads();
-    for (int s0 = 0; s0 < nsteps; s0 += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int step = s0 + u;
-            // MFMAs of this step on stage u; step + 1 (ring slot u ^ 1) is decoded and parked in stage u ^ 1 meanwhile;
-            // ring slot u held this step's bytes (parked one step ago) and is refilled with the step after next (the
-            // wide tile's single activation slot: chunk by chunk behind its parking, with the step after next)
-            step_body(u, u ^ 1, step + 1, u, step + 2);
-            __syncthreads();
-        }
+    // One trip = the four steps of a super-block. Step s0 + u: MFMAs on stage u % 2; step + 1 (ring slot (u + 1) % 2) is
+    // decoded and parked in the other stage meanwhile; ring slot u % 2 held this step's bytes (parked one step ago) and
+    // is refilled with the step after next (the wide tile's single activation slot: chunk by chunk behind its parking,
+    // with the step after next)
+    for (int s0 = 0; s0 < nsteps; s0 += 4) {
+        step_body(std::integral_constant<int, 0>{}, 0, 1, s0 + 1, 0, s0 + 2);
+        __syncthreads();
+        step_body(std::integral_constant<int, 1>{}, 1, 0, s0 + 2, 1, s0 + 3);
+        __syncthreads();
+        step_body(std::integral_constant<int, 2>{}, 0, 1, s0 + 3, 0, s0 + 4);
+        __syncthreads();
+        step_body(std::integral_constant<int, 3>{}, 1, 0, s0 + 4, 1, s0 + 5);
+        __syncthreads();
     }
 
     float* cz = c + (int64_t)blockIdx.z * split_stride;      // split K: this split's partial product
