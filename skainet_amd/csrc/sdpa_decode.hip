@@ -85,10 +85,10 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
     float qr[GS][DPL];
 #pragma unroll
     for (int g = 0; g < GS; ++g) {
-        const float* qp = p.q + ((int64_t)b * p.heads + h0 + g) * D + sub * DPL;
+        const float* qp = p.q + ((int64_t)b * p.heads + h0 + g) * D + sub * 4;
 #pragma unroll
         for (int d = 0; d < DPL; d += 4) {
-            const float4 t = *reinterpret_cast<const float4*>(qp + d);
+            const float4 t = *reinterpret_cast<const float4*>(qp + 16 * d);   // float4 number d / 4 of the lane: elements 64 (d / 4) + 4 sub ..
             qr[g][d] = t.x * qscale; qr[g][d + 1] = t.y * qscale; qr[g][d + 2] = t.z * qscale; qr[g][d + 3] = t.w * qscale;
         }
     }
@@ -100,8 +100,11 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
         for (int d = 0; d < DPL; ++d) acc[g][d] = 0.f;
     }
 
-    const float* kb = p.k + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * DPL;
-    const float* vb = p.v + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * DPL;
+    // A lane's DPL elements of a row are float4s 64 elements apart (float4 number j: elements 64 j + 4 sub ..), so that the
+    // 16 lanes of a row read 256 consecutive bytes per load instruction and a row's cache lines are each touched once
+    // (with DPL consecutive elements per lane every instruction touched every line of the row).
+    const float* kb = p.k + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * 4;
+    const float* vb = p.v + ((int64_t)b * p.kv_heads + kvh) * p.kv_capacity * D + sub * 4;
     // The K / V rows of a pass (U groups of 4 keys per wave) are requested one pass ahead of their use, into the other of
     // two register sets: a split of 64 keys is two passes per wave, and both are in flight from the start.
     constexpr int STEP = 16 * U;
@@ -111,8 +114,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
             const int64_t off = (int64_t)min(k0 + 16 * u + kg, hi - 1) * D;   // a lane past the range re-reads the last row
 #pragma unroll
             for (int d = 0; d < DPL; d += 4) {
-                const float4 a = *reinterpret_cast<const float4*>(kb + off + d);
-                const float4 c = *reinterpret_cast<const float4*>(vb + off + d);
+                const float4 a = *reinterpret_cast<const float4*>(kb + off + 16 * d);
+                const float4 c = *reinterpret_cast<const float4*>(vb + off + 16 * d);
                 kr[u][d] = a.x; kr[u][d + 1] = a.y; kr[u][d + 2] = a.z; kr[u][d + 3] = a.w;
                 vr[u][d] = c.x; vr[u][d + 1] = c.y; vr[u][d + 2] = c.z; vr[u][d + 3] = c.w;
             }
@@ -182,8 +185,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
     // Merge the 16 running states of the workgroup (4 lane groups x 4 waves) through LDS: every lane parks its slice,
     // one 16-lane row per head works out the 16 weights 2^(m_s - max) and the weighted sum of the l_s, then each thread
     // sums its output elements over the states. (Merging lane groups by shuffles first cost 80 crossbar round trips and
-    // 16 exponentials per lane.) An element's position inside a state is permuted so that the 16 lanes of a row store
-    // 256 contiguous bytes: float4 number j of lane `sub` sits at j * 64 + sub * 4.
+    // 16 exponentials per lane.) A lane's float4 number j holds elements 64 j + 4 sub .. of the row, so the 16 lanes of
+    // a row store 256 contiguous bytes and a state lies in LDS in the row's own element order.
     const int state = wave * 4 + kg;
 #pragma unroll
     for (int g = 0; g < GS; ++g) {
@@ -224,8 +227,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_kernel(SdpaDecodeParams p) {
         const int64_t row = (int64_t)b * p.heads + h0 + g;
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {
-            const int i = i0 + e;
-            const int d = ((i & 63) >> 2) * DPL + (i >> 6) * 4 + (i & 3);
+            const int d = i0 + e;                                   // a state's layout in LDS is the row's own element order
             if (!p.part) {
                 p.out[row * D + d] = ls > 0.f ? o[e] / ls : 0.f;
             } else {
