@@ -167,22 +167,24 @@ __device__ __forceinline__ void load_sb(SbQ4K& sb, const uint8_t* row, int e) {
 // The decode of a thread's 32 weights is split into a header part and eight 4-weight parts (one per dword of
 // codes) so the main loop can place the parts between its MFMAs.
 struct DecQ4K { float scale, offset; int shift; };
+// UN: the step's position in its super-block (0..3), known where the K loop is unrolled: sub-block 2 UN + wsub. Which of
+// the two packings of the 6-bit scales applies (sub-blocks 0..3 / 4..7) is then decided at compile time; `e` gives wsub.
+template <int UN>
 __device__ __forceinline__ void decode_prepare_k4(const uint4& hdr, int e, DecQ4K& c) {
-    const int sb = (e & 255) >> 5;
+    const int wsub = (e >> 5) & 1;
     const float d = half_bits_to_float_fast(hdr.x & 0xFFFFu), dmin = half_bits_to_float_fast(hdr.x >> 16);
-    // ggml get_scale_min_k4 on the 12 scale bytes s[0..11] (hdr.y = s[0..3], hdr.z = s[4..7], hdr.w = s[8..11])
-    const int sh = (sb & 3) * 8;
+    // ggml get_scale_min_k4 on the 12 scale bytes s[0..11] (hdr.y = s[0..3], hdr.z = s[4..7], hdr.w = s[8..11]):
+    // byte (2 UN + wsub) % 4 of each
+    const int sh = (2 * (UN & 1) + wsub) * 8;
     const uint32_t sa = (hdr.y >> sh) & 0xFFu, sbm = (hdr.z >> sh) & 0xFFu, st = (hdr.w >> sh) & 0xFFu;
-    // both packings are evaluated and one is picked with a mask: a select written as a conditional becomes a branch
-    // here, and a branch inside the K loop makes every wait behind it cover all the loads in flight
-    const uint32_t hi = (uint32_t)-(int)(sb >> 2);            // sb >= 4: all ones
-    const uint32_t sc = ((sa & 63u) & ~hi) | (((st & 0xFu) | ((sa >> 6) << 4)) & hi);
-    const uint32_t mn = ((sbm & 63u) & ~hi) | (((st >> 4) | ((sbm >> 6) << 4)) & hi);
+    const uint32_t sc = UN < 2 ? (sa & 63u) : ((st & 0xFu) | ((sa >> 6) << 4));
+    const uint32_t mn = UN < 2 ? (sbm & 63u) : ((st >> 4) | ((sbm >> 6) << 4));
     c.scale = d * (float)sc;
     c.offset = dmin * (float)mn;
-    c.shift = (sb & 1) * 4;
+    c.shift = wsub * 4;
 }
-__device__ __forceinline__ void decode_prepare(const RawQ4K&, const SbQ4K& sb, int e, DecQ4K& c) { decode_prepare_k4(sb.hdr, e, c); }
+template <int UN>
+__device__ __forceinline__ void decode_prepare(const RawQ4K&, const SbQ4K& sb, int e, DecQ4K& c) { decode_prepare_k4<UN>(sb.hdr, e, c); }
 template <int I>
 __device__ __forceinline__ uint32_t decode_codes(const RawQ4K& r, const SbQ4K&, const DecQ4K& c) {
     const uint32_t q = I == 0 ? r.q0.x : I == 1 ? r.q0.y : I == 2 ? r.q0.z : I == 3 ? r.q0.w
@@ -215,15 +217,15 @@ __device__ __forceinline__ void load_sb(SbQ6K& sb, const uint8_t* row, int e) {
     sb.d = load_u16(blk + 208);
 }
 struct DecQ6K { float s0, s1, n0, n1; int nib, hs; };   // n = -32 s
+template <int UN>
 __device__ __forceinline__ void decode_prepare(const RawQ6K&, const SbQ6K& sb, int e, DecQ6K& c) {
-    // the step's quarters are kq and kq + 1 (kq 0 or 2) of its half; this thread's 16 positions of either lie in one
-    // 16-element scale group each: sc[8 half + 2 kq + wsub] and sc[8 half + 2 kq + 2 + wsub], bytes wsub and wsub + 2 of
-    // dword `step` (0..3) of the 16 scales
-    const int kq = (e & 127) >> 6 << 1, step = (e & 255) >> 6, wsub = (e >> 5) & 1;
+    // step UN (0..3) of the super-block: quarters kq and kq + 1 (kq 0 or 2) of half UN / 2; this thread's 16 positions of
+    // either lie in one 16-element scale group each: sc[4 UN + wsub] and sc[4 UN + 2 + wsub], bytes wsub and wsub + 2 of
+    // dword UN of the 16 scales
+    constexpr int kq = 2 * (UN & 1);
+    const int wsub = (e >> 5) & 1;
     const float d = half_bits_to_float_fast(sb.d);
-    // picked with masks (no branch, no indexed register)
-    const uint32_t m0 = (uint32_t)-(int)(step == 0), m1 = (uint32_t)-(int)(step == 1), m2 = (uint32_t)-(int)(step == 2), m3 = (uint32_t)-(int)(step == 3);
-    const uint32_t four = ((sb.sc.x & m0) | (sb.sc.y & m1) | (sb.sc.z & m2) | (sb.sc.w & m3)) >> (8 * wsub);
+    const uint32_t four = (UN == 0 ? sb.sc.x : UN == 1 ? sb.sc.y : UN == 2 ? sb.sc.z : sb.sc.w) >> (8 * wsub);
     c.s0 = d * (float)(int8_t)(four & 0xFF);
     c.s1 = d * (float)(int8_t)((four >> 16) & 0xFF);
     c.n0 = -32.f * c.s0;
@@ -257,6 +259,7 @@ __device__ __forceinline__ void load_raw(RawQ80& r, const uint8_t* row, int e) {
     r.edge = load_u16(blk + (r.odd ? 0 : 32));
 }
 struct DecQ80 { float d; uint32_t drop; };
+template <int UN>
 __device__ __forceinline__ void decode_prepare(const RawQ80& r, const SbNone&, int, DecQ80& c) {
     c.d = half_bits_to_float_fast(r.odd ? r.edge : (r.lo.x & 0xFFFFu));
     c.drop = r.odd ? 0u : 2u;                        // bytes in front of the codes in the loaded dwords
@@ -287,7 +290,7 @@ __device__ __forceinline__ void load_raw(RawQ45<FMT>& r, const uint8_t* row, int
     r.q[0] = q4.x; r.q[1] = q4.y; r.q[2] = q4.z; r.q[3] = q4.w;
 }
 struct DecQ45 { float d, add; };
-template <int FMT>
+template <int UN, int FMT>
 __device__ __forceinline__ void decode_prepare(const RawQ45<FMT>& r, const SbNone&, int, DecQ45& c) {
     c.d = half_bits_to_float_fast(r.d);
     // w = d * code + add:  Q4_0 d * (code - 8),  Q5_0 d * (code5 - 16),  Q5_1 d * code5 + m
@@ -322,11 +325,12 @@ __device__ __forceinline__ void load_sb(SbQ5K& sb, const uint8_t* row, int e) {
     sb.h1 = *reinterpret_cast<const uint4*>(blk + 32);
 }
 struct DecQ5K { float scale, offset; int shift, bit; };
+template <int UN>
 __device__ __forceinline__ void decode_prepare(const RawQ5K&, const SbQ5K& sb, int e, DecQ5K& c) {
     DecQ4K c4;
-    decode_prepare_k4(sb.hdr, e, c4);                // same d / dmin / 6-bit scale and min packing
+    decode_prepare_k4<UN>(sb.hdr, e, c4);            // same d / dmin / 6-bit scale and min packing
     c.scale = c4.scale; c.offset = c4.offset; c.shift = c4.shift;
-    c.bit = (e & 255) >> 5;
+    c.bit = 2 * UN + ((e >> 5) & 1);
 }
 template <int I>
 __device__ __forceinline__ uint32_t decode_codes(const RawQ5K& r, const SbQ5K& sb, const DecQ5K& c) {
@@ -538,7 +542,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
                 __builtin_amdgcn_sched_barrier(0);
             } else if (q < FIRST_ITEM) {
                 const int t = q - G_W_TASKS;
-                decode_prepare(wring[w_slot_next][t], sb_dec[t], step_k(step_next) + 32 * wsub, dc[t]);
+                decode_prepare<(U + 1) & 3>(wring[w_slot_next][t], sb_dec[t], step_k(step_next) + 32 * wsub, dc[t]);
                 __builtin_amdgcn_sched_barrier(0);
             } else if (q < FIRST_ITEM + N_GAPS) {
                 // decode item h sits behind MFMA FIRST_ITEM + h * N_GAPS / N_HALVES: evenly spread (the 256-row tiles have
@@ -582,7 +586,7 @@ __global__ __launch_bounds__(G_THREADS) void dequant_gemm_kernel(const __bf16* _
 #pragma unroll
     for (int t = 0; t < G_W_TASKS; ++t) {
         Dec d0;
-        decode_prepare(wring[0][t], sb_cur[t], step_k(0) + 32 * wsub, d0);
+        decode_prepare<0>(wring[0][t], sb_cur[t], step_k(0) + 32 * wsub, d0);
         uint32_t codes0 = 0;
 #pragma unroll
         for (int h = 0; h < 16; ++h) wp[t][h] = decode_item_at(h, wring[0][t], sb_cur[t], d0, codes0);
