@@ -173,6 +173,7 @@ void set_sdpa_decode_split_keys(int v);
 void set_q4k_ksplit_enable(int v);
 void set_q4k_mfma_enable(int v);
 void set_q4k_mfma_window(int v);
+void set_q4k_quads_stream_enable(int v);
 void set_attn_merge_enable(int v);
 void set_sdpa_decode_gs(int v);
 void set_attn_merge_max_keys(int v);
@@ -201,6 +202,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "sdpa_prefill_teams")) { set_sdpa_prefill_teams(value); return 0; }
     if (!strcmp(key, "q4k_ksplit_enable")) { set_q4k_ksplit_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_enable")) { set_q4k_mfma_enable(value); return 0; }
+    if (!strcmp(key, "q4k_quads_stream_enable")) { set_q4k_quads_stream_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_window")) { set_q4k_mfma_window(value); return 0; }
     if (!strcmp(key, "sdpa_decode_split_keys")) { set_sdpa_decode_split_keys(value); return 0; }
     if (!strcmp(key, "attn_merge_enable")) { set_attn_merge_enable(value); return 0; }

@@ -218,6 +218,30 @@ def test_q4k_three_to_eight_rows_on_the_matrix_instruction(hip_backend, torch_cu
         assert normalized_err(got[m - 1], alone[0]) <= 3e-4
 
 
+@pytest.mark.parametrize("n,m", [(4, 3), (5, 4), (37, 5), (130, 8), (1027, 7), (11008, 4), (11008, 8), (28672, 3), (40000, 8)])
+def test_q4k_three_to_eight_rows_streamed_through_lds_at_k_4096(hip_backend, torch_cuda, n, m):
+    """K = 4096: the batched kernel whose weight arrives through an LDS ring (one K slice per wave), on row counts that
+    leave ragged quads, ragged groups of quads and more than one round of workgroups; against the oracle and against the
+    register-fed kernel of the same arithmetic (another order of the fp32 sums)."""
+    k = 4096
+    packed = gaussian_weight(hip_backend, "Q4_K", n, k, 91) if n <= 11008 else random_valid_blocks("Q4_K", n * k // 256, 92)
+    x = np.random.default_rng(93 + m + n).standard_normal((m, k)).astype(np.float32)
+    x[m - 1, 7] = 33.0
+    got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+    assert hip_backend.last_kernel() == "q4k_gemv_quads_stream_kernel"
+    assert got.shape == (m, n) and not np.isnan(got).any()
+    rows = np.unique(np.concatenate([np.arange(min(n, 40)), np.arange(max(0, n - 40), n)]))
+    want = L.gemv("Q4_K", x, packed.reshape(n, -1)[rows].reshape(-1), len(rows))
+    assert normalized_err(got[:, rows], want) <= GEMV_TOL
+    try:
+        hip_backend.set_tuning("q4k_quads_stream_enable", 0)
+        fed = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemv_quads_kernel"
+    finally:
+        hip_backend.set_tuning("q4k_quads_stream_enable", 1)
+    assert normalized_err(got, fed) <= 2e-5
+
+
 def test_gemv_is_linear_and_deterministic_at_full_size(hip_backend, torch_cuda):
     """Size-independent properties at the benchmark shape: y(a*x1 + x2) == a*y(x1) + y(x2) within rounding; two runs agree bit for bit."""
     n, k = 11008, 4096
