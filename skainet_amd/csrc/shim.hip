@@ -251,13 +251,21 @@ static int staged_h2d(void* dst, const uint8_t* src, size_t bytes) {
     hipError_t result[UPLOAD_MAX_LANES];
     std::thread workers[UPLOAD_MAX_LANES];
     const int device = g_device;
-    for (int t = 1; t < lanes; ++t)
-        workers[t] = std::thread([&, t] {
-            hipError_t e = hipSetDevice(device);
-            result[t] = e != hipSuccess ? e : lane_run(g_lanes[t], t, lanes, static_cast<uint8_t*>(dst), src, bytes, chunk);
-        });
+    bool started[UPLOAD_MAX_LANES] = {};
+    for (int t = 1; t < lanes; ++t) {
+        try {
+            workers[t] = std::thread([&, t] {
+                hipError_t e = hipSetDevice(device);
+                result[t] = e != hipSuccess ? e : lane_run(g_lanes[t], t, lanes, static_cast<uint8_t*>(dst), src, bytes, chunk);
+            });
+            started[t] = true;
+        } catch (...) {}                                // no thread to be had: the caller runs that lane below
+    }
     result[0] = lane_run(g_lanes[0], 0, lanes, static_cast<uint8_t*>(dst), src, bytes, chunk);
-    for (int t = 1; t < lanes; ++t) workers[t].join();
+    for (int t = 1; t < lanes; ++t) {
+        if (started[t]) workers[t].join();
+        else result[t] = lane_run(g_lanes[t], t, lanes, static_cast<uint8_t*>(dst), src, bytes, chunk);
+    }
     for (int t = 0; t < lanes; ++t)
         if (check_hip(result[t], "hipMemcpy(weight, staged)") != 0) return -1;
     return 0;
