@@ -79,12 +79,21 @@ constexpr int MFMA_MAX_QUADS = 32;     // row quads per workgroup (bounds the fi
 constexpr int MFMA_XA_BYTES = 16 * 4 * MFMA_XROW * 4 + 16 * 16 + 16 * ATTN_MERGE_MAX_SPLITS * 4;
 // operand planes of 16 groups + {scale, sums} per group + the merge coefficients of up to 16 heads of a slice
 constexpr int MFMA_XC_OFFSET = 16 * 4 * MFMA_XROW * 4 + 16 * 16;
+// Bytes of a wave's ring: W + 1 quad slots of nli KB. The last slot doubles as the staging area of the activation
+// planes (the first W quads go into slots 0 .. W - 1, and the planes are in registers before the main loop asks for quad
+// W); where a slot is smaller than that area the ring is that much longer.
+__host__ __device__ constexpr uint32_t mfma_ring_bytes(int nli, int window) {
+    return (uint32_t)(window + 1) * nli * 1024u > (uint32_t)window * nli * 1024u + MFMA_XA_BYTES
+               ? (uint32_t)(window + 1) * nli * 1024u
+               : (uint32_t)window * nli * 1024u + MFMA_XA_BYTES;
+}
 
-// One wave's pass: K slices wave, wave + 4, ... (NSW of them), row quads [0, qt) of the workgroup, W quads in flight.
+// One wave's pass: K slices wave, wave + NW, ... (NSW of them; NW waves per workgroup), row quads [0, qt) of the workgroup,
+// W quads in flight.
 // Leaves one partial sum per (quad, lane) in `partials` (index: quad * 64 + (lane % 4) * 16 + lane / 4) and, with the
 // RMSNorm prologue, the sum of squares of this wave's activations in *ssq_out.
 // PRO: 0 plain activations, 1 RMSNorm prologue (x * gain, sum of squares), 2 activations = merge of attention partials.
-template <int NSW, int W, int PRO>
+template <int NSW, int W, int PRO, int NW>
 __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, const float* __restrict__ x, const float* __restrict__ gain,
                                               const AttnMergePrologue& am, int n, int r0, int qt, uint32_t row_bytes, int wave,
                                               int lane, uint8_t* ring, uint8_t* xa_stage, float* partials, float* ssq_out) {
@@ -126,7 +135,7 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
         for (int t = 0; t < NSW; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const uint32_t off = (uint32_t)((wave + 4 * t) * 1024 + (i * 64 + lane) * 4) * 4u;
+                const uint32_t off = (uint32_t)((wave + NW * t) * 1024 + (i * 64 + lane) * 4) * 4u;
                 mfma_plain_load16(xq[t][i], off, x);
                 if (PRO == 1) mfma_plain_load16(gq[t][i], off, gain);
             }
@@ -136,7 +145,7 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
     for (int u = 0; u < NLI; ++u) {
         const uint32_t p = min(64u * u + lane, (uint32_t)(NPQ - 1)), t = (p * 1821u) >> 18;       // p / 144 for p < 2^12
         const uint32_t rem = p - 144u * t, row4 = (rem * 1821u) >> 16, pc = rem - 36u * row4;    // rem / 36
-        loff[u] = __umul24(row4, row_bytes) + (wave + 4u * t) * 576u + pc * 16u;
+        loff[u] = __umul24(row4, row_bytes) + (wave + (uint32_t)NW * t) * 576u + pc * 16u;
     }
     const uint32_t max_off = (uint32_t)n * row_bytes - 16u;
     const uint32_t ring_addr = (uint32_t)(size_t)(__attribute__((address_space(3))) uint8_t*)ring;
@@ -280,8 +289,10 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
 // The epilogue is a template argument, not a run-time switch: what an epilogue reads besides a row's sum (residual
 // element, cos / sin pair) is requested at the start of the kernel and held in registers to the end, and with the switch
 // at run time every variant paid for those registers (the plain product ran 6.53 us where this form runs 6.15).
-template <int W, int PRO, int EPI>
-__global__ __launch_bounds__(256, PRO == 2 ? 1 : 2) void q4k_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x, float* y,
+// NW: waves per workgroup, 4 or 8 (eight for long rows: K is then split eight ways, a wave prepares and multiplies half
+// as many slices and two waves share a SIMD).
+template <int W, int PRO, int EPI, int NW>
+__global__ __launch_bounds__(64 * NW, (PRO == 2 || NW == 8) ? 1 : 2) void q4k_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x, float* y,
                                                                             int k, int n, int qt, const float* __restrict__ gain, float eps,
                                                                             const float* residual, RopeQkvEpilogue rope,
                                                                             AttnMergePrologue am) {
@@ -289,20 +300,21 @@ __global__ __launch_bounds__(256, PRO == 2 ? 1 : 2) void q4k_gemv_mfma_kernel(co
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nsl = k >> 10;                                   // slices of 1024 elements
-    const int nsw = (nsl - wave + 3) >> 2;                     // this wave's share (uniform)
-    const int ns_max = (nsl + 3) >> 2;
+    const int nsw = (nsl - wave + NW - 1) / NW;                // this wave's share (uniform)
+    const int ns_max = (nsl + NW - 1) / NW;
     const int nli_max = (144 * ns_max + 63) / 64;
-    const uint32_t ring_bytes = (uint32_t)(W + 1) * nli_max * 1024u;
-    uint8_t* ring = smem + wave * (ring_bytes + MFMA_XA_BYTES);
-    uint8_t* xa_stage = ring + ring_bytes;
-    float* partials_all = reinterpret_cast<float*>(smem + 4 * (ring_bytes + MFMA_XA_BYTES));   // [4 waves][qt][64]
-    float* ssq_lds = partials_all + 4 * qt * 64;
+    const uint32_t ring_bytes = mfma_ring_bytes(nli_max, W);
+    uint8_t* ring = smem + wave * ring_bytes;
+    uint8_t* xa_stage = ring + (uint32_t)W * (uint32_t)nli_max * 1024u;      // the ring's last slot: free until the main loop
+    float* partials_all = reinterpret_cast<float*>(smem + NW * ring_bytes);   // [NW waves][qt][64]
+    float* ssq_lds = partials_all + NW * qt * 64;
     float* partials = partials_all + wave * qt * 64;
     const int r0 = blockIdx.x * (4 * qt);
     const uint32_t row_bytes = (uint32_t)(k >> 8) * (uint32_t)Q4K_BYTES;
 
     // what the final pass will add or rotate with: one output row per 16 threads and round
-    constexpr int ROUNDS = MFMA_MAX_QUADS * 4 * 16 / 256;
+    constexpr int RPR = 4 * NW;                                 // rows per round
+    constexpr int ROUNDS = MFMA_MAX_QUADS * 4 / RPR;
     float pre_res[EPI == EPI_RESIDUAL ? ROUNDS : 1];
     f32x2_m pre_cs[EPI == EPI_ROPE_QKV ? ROUNDS : 1];
     int pos = 0;
@@ -311,9 +323,9 @@ __global__ __launch_bounds__(256, PRO == 2 ? 1 : 2) void q4k_gemv_mfma_kernel(co
         if (EPI == EPI_RESIDUAL || rope.table) {                                       // uniform
 #pragma unroll
             for (int it = 0; it < ROUNDS; ++it) {
-                const int row = min(r0 + it * 16 + (threadIdx.x >> 4), n - 1);
+                const int row = min(r0 + it * RPR + (threadIdx.x >> 4), n - 1);
                 if constexpr (EPI == EPI_RESIDUAL) pre_res[it] = 0.f; else pre_cs[it] = f32x2_m{1.f, 0.f};
-                if (it * 16 < 4 * qt) {
+                if (it * RPR < 4 * qt) {
                     if constexpr (EPI == EPI_RESIDUAL) mfma_plain_load4(pre_res[it], (uint32_t)row * 4u, residual);
                     else mfma_plain_load8(pre_cs[it], (uint32_t)((row % rope.head_dim) >> 1) * 8u, rope.table);
                 }
@@ -324,25 +336,33 @@ __global__ __launch_bounds__(256, PRO == 2 ? 1 : 2) void q4k_gemv_mfma_kernel(co
 
     float ssq = 0.f;
     switch (nsw) {
-        case 1: q4k_mfma_wave<1, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 2: if constexpr (PRO != 2) q4k_mfma_wave<2, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 3: if constexpr (W <= 2 && PRO != 2) q4k_mfma_wave<3, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 4: if constexpr (W <= 2 && PRO != 2) q4k_mfma_wave<4, W, PRO>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        default:                                               // K below 4 slices: this wave has none
+        case 1: q4k_mfma_wave<1, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 2: if constexpr (PRO != 2) q4k_mfma_wave<2, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 3: if constexpr (W <= 2 && PRO != 2 && NW == 4) q4k_mfma_wave<3, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 4: if constexpr (W <= 2 && PRO != 2 && NW == 4) q4k_mfma_wave<4, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        default:                                               // K below NW slices: this wave has none
             for (int i = lane; i < qt * 64; i += 64) partials[i] = 0.f;
     }
     if (PRO == 1 && lane == 0) ssq_lds[wave] = ssq;
     __syncthreads();
 
     float xscale = 1.0f;
-    if (PRO == 1) xscale = 1.0f / sqrtf(((ssq_lds[0] + ssq_lds[1]) + (ssq_lds[2] + ssq_lds[3])) * (1.0f / (float)k) + eps);
+    if (PRO == 1) {
+        float ss = (ssq_lds[0] + ssq_lds[1]) + (ssq_lds[2] + ssq_lds[3]);
+        if (NW == 8) ss += (ssq_lds[4] + ssq_lds[5]) + (ssq_lds[6] + ssq_lds[7]);
+        xscale = 1.0f / sqrtf(ss * (1.0f / (float)k) + eps);
+    }
     const int u = threadIdx.x & 15, pw = u >> 2, pp = u & 3;
 #pragma unroll
     for (int it = 0; it < ROUNDS; ++it) {
-        if (it * 16 >= 4 * qt) break;                          // uniform
-        const int rl = it * 16 + (threadIdx.x >> 4);           // row of the workgroup
+        if (it * RPR >= 4 * qt) break;                         // uniform
+        const int rl = it * RPR + (threadIdx.x >> 4);          // row of the workgroup
         const int rlc = min(rl, 4 * qt - 1);
-        const float4 p4 = *reinterpret_cast<const float4*>(partials_all + (pw * qt + (rlc >> 2)) * 64 + (rlc & 3) * 16 + pp * 4);
+        float4 p4 = *reinterpret_cast<const float4*>(partials_all + (pw * qt + (rlc >> 2)) * 64 + (rlc & 3) * 16 + pp * 4);
+        if (NW == 8) {                                         // waves 4 .. 7: a second float4 per thread
+            const float4 p8 = *reinterpret_cast<const float4*>(partials_all + ((pw + 4) * qt + (rlc >> 2)) * 64 + (rlc & 3) * 16 + pp * 4);
+            p4.x += p8.x; p4.y += p8.y; p4.z += p8.z; p4.w += p8.w;
+        }
         float val = row16_sum((p4.x + p4.y) + (p4.z + p4.w)) * xscale;
         const int row = r0 + rl;
         const bool live = u == 0 && rl < 4 * qt && row < n;
@@ -376,24 +396,26 @@ __global__ __launch_bounds__(256, PRO == 2 ? 1 : 2) void q4k_gemv_mfma_kernel(co
 
 static std::atomic<int> g_q4k_mfma_enable{1};
 void set_q4k_mfma_enable(int v) { g_q4k_mfma_enable = v; }
+static std::atomic<int> g_q4k_mfma_waves8{1};
+void set_q4k_mfma_waves8(int v) { g_q4k_mfma_waves8 = v != 0; }
 static std::atomic<int> g_q4k_mfma_window{0};      // 0: chosen from K
 void set_q4k_mfma_window(int v) { if (v == 0 || v == 2 || v == 3) g_q4k_mfma_window = v; }
 
 // quads in flight per wave: three while a quad is at most 5 KB per wave, two for the long rows (9 KB per quad and wave)
 static int mfma_window(int k) { return (((k >> 10) + 3) >> 2) >= 3 ? 2 : 3; }
 
-static size_t mfma_smem_bytes(int k, int qt, int window) {
-    const int ns_max = ((k >> 10) + 3) >> 2;
+static size_t mfma_smem_bytes(int k, int qt, int window, int nw) {
+    const int ns_max = ((k >> 10) + nw - 1) / nw;
     const int nli_max = (144 * ns_max + 63) / 64;
-    return (size_t)4 * ((size_t)(window + 1) * nli_max * 1024 + MFMA_XA_BYTES) + (size_t)4 * qt * 64 * sizeof(float) + 16;
+    return (size_t)nw * mfma_ring_bytes(nli_max, window) + (size_t)nw * qt * 64 * sizeof(float) + 32;
 }
 
-template <int W, int PRO, int EPI>
+template <int W, int PRO, int EPI, int NW = 4>
 static int launch_mfma_variant(int grid, size_t smem, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int qt,
                                const float* gain, float eps, const float* residual, const RopeQkvEpilogue& rope,
                                const AttnMergePrologue& am) {
-    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, PRO, EPI>), 160 * 1024);
-    q4k_gemv_mfma_kernel<W, PRO, EPI><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, rope, am);
+    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, PRO, EPI, NW>), 160 * 1024);
+    q4k_gemv_mfma_kernel<W, PRO, EPI, NW><<<dim3(grid), dim3(64 * NW), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, rope, am);
     SKH_CHECK(hipGetLastError());
     return 1;
 }
@@ -467,9 +489,18 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
     int window = g_q4k_mfma_window.load() > 0 ? g_q4k_mfma_window.load() : mfma_window(k);
     if (mfma_window(k) == 2) window = 2;                       // long rows: the wave's load counter holds 63
     if (merge) window = 3;
-    const size_t smem = mfma_smem_bytes(k, qt, window);
-    if (smem > 160 * 1024) return 0;
     const int pro = merge ? 2 : gain ? 1 : 0;
+    // long rows without a prologue (the decoder's down projection): eight waves, K split eight ways
+    if (g_q4k_mfma_waves8 && pro == 0 && k >= 8192 && epilogue <= EPI_RESIDUAL) {
+        const size_t smem8 = mfma_smem_bytes(k, qt, 2, 8);
+        if (smem8 <= 160 * 1024) {
+            note_kernel("q4k_gemv_mfma_kernel");
+            if (epilogue == EPI_NONE) return launch_mfma_variant<2, 0, EPI_NONE, 8>(grid, smem8, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am);
+            return launch_mfma_variant<2, 0, EPI_RESIDUAL, 8>(grid, smem8, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am);
+        }
+    }
+    const size_t smem = mfma_smem_bytes(k, qt, window, 4);
+    if (smem > 160 * 1024) return 0;
     if (window == 2) return launch_mfma<2>(pro, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
     return launch_mfma<3>(pro, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
 }
