@@ -173,6 +173,7 @@ void set_sdpa_decode_split_keys(int v);
 void set_q4k_ksplit_enable(int v);
 void set_q4k_mfma_enable(int v);
 void set_q4k_mfma_window(int v);
+void set_q4k_mfma_teams(int v);
 void set_q4k_mfma_waves8(int v);
 void set_q4k_quads_stream_enable(int v);
 void set_attn_merge_enable(int v);
@@ -205,6 +206,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q4k_mfma_enable")) { set_q4k_mfma_enable(value); return 0; }
     if (!strcmp(key, "q4k_quads_stream_enable")) { set_q4k_quads_stream_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_waves8")) { set_q4k_mfma_waves8(value); return 0; }
+    if (!strcmp(key, "q4k_mfma_teams")) { set_q4k_mfma_teams(value); return 0; }
     if (!strcmp(key, "q4k_mfma_window")) { set_q4k_mfma_window(value); return 0; }
     if (!strcmp(key, "sdpa_decode_split_keys")) { set_sdpa_decode_split_keys(value); return 0; }
     if (!strcmp(key, "attn_merge_enable")) { set_attn_merge_enable(value); return 0; }

@@ -93,22 +93,28 @@ __host__ __device__ constexpr uint32_t mfma_ring_bytes(int nli, int window) {
 // Leaves one partial sum per (quad, lane) in `partials` (index: quad * 64 + (lane % 4) * 16 + lane / 4) and, with the
 // RMSNorm prologue, the sum of squares of this wave's activations in *ssq_out.
 // PRO: 0 plain activations, 1 RMSNorm prologue (x * gain, sum of squares), 2 activations = merge of attention partials.
-template <int NSW, int W, int PRO, int NW>
+// T: teams. With T = 2 (K = 4096, one slice per wave) waves `wave` and `wave + NW` share slice `wave`: each prepares half
+// of its activation planes (the staging area is then one per slice, shared, and a workgroup barrier stands between its
+// writes and its reads), and team t takes the row quads t, t + 2, ... -- two waves per SIMD, the preparation not doubled.
+template <int NSW, int W, int PRO, int NW, int T>
 __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, const float* __restrict__ x, const float* __restrict__ gain,
                                               const AttnMergePrologue& am, int n, int r0, int qt, uint32_t row_bytes, int wave,
-                                              int lane, uint8_t* ring, uint8_t* xa_stage, float* partials, float* ssq_out) {
+                                              int team, int lane, uint8_t* ring, uint8_t* xa_stage, float* partials, float* ssq_out) {
     constexpr int NPQ = 144 * NSW;                 // 16-byte pieces of a quad in this wave's slices
     constexpr int NLI = (NPQ + 63) / 64;           // wave loads per quad
-    constexpr int NX = PRO == 2 ? 2 + 4 * ATTN_MERGE_MAX_SPLITS : NSW * 4 * (1 + PRO);        // activation (and gain) loads
+    constexpr int XI = 4 / T;                      // float4s of a slice this wave prepares per lane
+    constexpr int NX = PRO == 2 ? 2 + 4 * ATTN_MERGE_MAX_SPLITS : NSW * XI * (1 + PRO);       // activation (and gain) loads
     static_assert(NX + W * NLI <= 63, "loads in flight must fit the wave's counter");
     static_assert(PRO != 2 || NSW == 1, "the attention-merge prologue serves one slice per wave");
+    static_assert(T == 1 || (NSW == 1 && PRO != 2), "two teams: one slice per wave, plain or RMSNorm prologue");
+    const int nq = (qt - team + T - 1) / T;        // this wave's quads: team, team + T, ... (uniform; at least one)
     const int blk = lane >> 2, j = lane & 3, g = blk & 3, h = g & 1;
     const uint32_t sel = g < 2 ? (0x0C0C0000u | ((2 * h + 1) << 8) | (2 * h))
                                : (((2 * h + 1) << 24) | ((2 * h) << 16) | ((4 + 2 * h + 1) << 8) | (4 + 2 * h));
     const uint32_t m1 = g < 2 ? 0x3F3Fu : 0x0F0Fu, sh_min = g < 2 ? 0u : 4u;
 
     // activations (and gains) of this wave's slices first, the first W quads right behind them
-    u32x4_m xq[NSW][4], gq[PRO == 1 ? NSW : 1][4];
+    u32x4_m xq[NSW][XI], gq[PRO == 1 ? NSW : 1][XI];
     constexpr int MS = PRO == 2 ? ATTN_MERGE_MAX_SPLITS : 1;
     u32x4_m pq[PRO == 2 ? 4 : 1][MS];              // attention partials of the lane's four float4s, one per split
     f32x2_m mlq[2];                                // (max, sum) of the (head, split) pair this lane weighs, two rounds of 8 heads
@@ -134,10 +140,11 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
 #pragma unroll
         for (int t = 0; t < NSW; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int ii = 0; ii < XI; ++ii) {
+                const int i = team * XI + ii;
                 const uint32_t off = (uint32_t)((wave + NW * t) * 1024 + (i * 64 + lane) * 4) * 4u;
-                mfma_plain_load16(xq[t][i], off, x);
-                if (PRO == 1) mfma_plain_load16(gq[t][i], off, gain);
+                mfma_plain_load16(xq[t][ii], off, x);
+                if (PRO == 1) mfma_plain_load16(gq[t][ii], off, gain);
             }
     }
     uint32_t loff[NLI];
@@ -150,14 +157,16 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
     const uint32_t max_off = (uint32_t)n * row_bytes - 16u;
     const uint32_t ring_addr = (uint32_t)(size_t)(__attribute__((address_space(3))) uint8_t*)ring;
     constexpr uint32_t SLOT = NLI * 1024u;          // bytes of a quad in the ring; W + 1 slots
-    auto issue_quad = [&](int q) {                  // q uniform; rows past the weight are clamped (computed, never stored)
-        const uint32_t base = (uint32_t)(r0 + 4 * q) * row_bytes;
+    // q: index among this wave's quads (the workgroup's quad team + T q), uniform; rows past the weight are clamped
+    // (computed, never stored)
+    auto issue_quad = [&](int q) {
+        const uint32_t base = (uint32_t)(r0 + 4 * (team + T * q)) * row_bytes;
         const uint32_t slot = ring_addr + (uint32_t)(q % (W + 1)) * SLOT;
 #pragma unroll
         for (int u = 0; u < NLI; ++u) mfma_stream_to_lds(slot + 1024u * u, min(base + loff[u], max_off), w);
     };
 #pragma unroll
-    for (int q = 0; q < W; ++q) issue_quad(min(q, qt - 1));
+    for (int q = 0; q < W; ++q) issue_quad(min(q, nq - 1));
     if constexpr (PRO == 2) {
         mfma_wait_loads<W * NLI>(mlq[0]); mfma_wait_loads<W * NLI>(mlq[1]);
 #pragma unroll
@@ -194,7 +203,7 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
 #pragma unroll
         for (int t = 0; t < NSW; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { mfma_wait_loads<W * NLI>(xq[t][i]); if (PRO == 1) mfma_wait_loads<W * NLI>(gq[t][i]); }
+            for (int i = 0; i < XI; ++i) { mfma_wait_loads<W * NLI>(xq[t][i]); if (PRO == 1) mfma_wait_loads<W * NLI>(gq[t][i]); }
     }
 
     // activations of a slice: float4 number f = i * 64 + lane belongs to group f / 16 (the 16 lanes of a DPP row share a
@@ -207,12 +216,13 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
 #pragma unroll
     for (int t = 0; t < NSW; ++t) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float4 v = make_float4(__uint_as_float(xq[t][i].x), __uint_as_float(xq[t][i].y), __uint_as_float(xq[t][i].z), __uint_as_float(xq[t][i].w));
+        for (int ii = 0; ii < XI; ++ii) {
+            const int i = team * XI + ii;              // float4 number i * 64 + lane of the slice
+            float4 v = make_float4(__uint_as_float(xq[t][ii].x), __uint_as_float(xq[t][ii].y), __uint_as_float(xq[t][ii].z), __uint_as_float(xq[t][ii].w));
             if (PRO == 1) {
                 ssq = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ssq))));
-                v.x *= __uint_as_float(gq[t][i].x); v.y *= __uint_as_float(gq[t][i].y);
-                v.z *= __uint_as_float(gq[t][i].z); v.w *= __uint_as_float(gq[t][i].w);
+                v.x *= __uint_as_float(gq[t][ii].x); v.y *= __uint_as_float(gq[t][ii].y);
+                v.z *= __uint_as_float(gq[t][ii].z); v.w *= __uint_as_float(gq[t][ii].w);
             }
             const int G = i * 4 + (lane >> 4), tt = lane & 15;
             const float amax = row16_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
@@ -231,6 +241,7 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
             float* xs = reinterpret_cast<float*>(xs_lds + G);
             if ((tt & 7) == 0) { xs[0] = amax * (1.0f / 2097151.0f); xs[1 + (tt >> 3)] = s4 * inv; }
         }
+        if constexpr (T == 2) __syncthreads();         // the other team's half of the planes (every wave of the workgroup gets here)
         const uint4* src = reinterpret_cast<const uint4*>(xa_lds + (blk * 4 + j) * MFMA_XROW);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -245,7 +256,7 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
     // lane's read offsets inside a quad slot: header of (row j, super-block blk / 4 of the slice), then its two code pieces
     const uint32_t rd_hdr = (uint32_t)(j * 36 + (blk >> 2) * 9) * 16u, rd_q = rd_hdr + 16u + (uint32_t)g * 32u;
     const int widx = j * 16 + blk;
-    auto compute_quad = [&](int q) {
+    auto compute_quad = [&](int q) {                 // q: index among this wave's quads
         const uint8_t* slot = ring + (uint32_t)(q % (W + 1)) * SLOT;
         float total = 0.f;
 #pragma unroll
@@ -268,11 +279,11 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
             const int th = __mul24(dh[3], -4194304) + (((dh[2] << 8) + dh[1]) << 8) + dh[0];
             total = fmaf(s_grp[t], fmaf(dlo, (float)tl, fmaf(dhi, (float)th, -fmaf(mlo, xsl[t], mhi * xsh[t]))), total);
         }
-        partials[q * 64 + widx] = total;
+        partials[(team + T * q) * 64 + widx] = total;
     };
 
     // quads [0, base): wait for the quad, ask for the one W ahead, compute; the last W quads without new requests
-    const int base = max(qt - W, 0);
+    const int base = max(nq - W, 0);
     for (int q = 0; q < base; ++q) {
         mfma_wait_loads<(W - 1) * NLI>();
         mfma_wait_lds();                             // the slot about to be refilled has been read
@@ -282,38 +293,42 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
     mfma_static_for<0, W>([&](auto mc) {
         constexpr int m = decltype(mc)::value;
         mfma_wait_loads<(W - 1 - m) * NLI>();
-        if (base + m < qt) compute_quad(base + m);
+        if (base + m < nq) compute_quad(base + m);
     });
 }
 
 // The epilogue is a template argument, not a run-time switch: what an epilogue reads besides a row's sum (residual
 // element, cos / sin pair) is requested at the start of the kernel and held in registers to the end, and with the switch
 // at run time every variant paid for those registers (the plain product ran 6.53 us where this form runs 6.15).
-// NW: waves per workgroup, 4 or 8 (eight for long rows: K is then split eight ways, a wave prepares and multiplies half
-// as many slices and two waves share a SIMD).
-template <int W, int PRO, int EPI, int NW>
-__global__ __launch_bounds__(64 * NW, (PRO == 2 || NW == 8) ? 1 : 2) void q4k_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x, float* y,
+// NW: waves that split K, 4 or 8 (eight for long rows: a wave prepares and multiplies half as many slices and two waves
+// share a SIMD). T: teams of NW waves that split the workgroup's row quads (two at K = 4096: again two waves per SIMD,
+// and each prepares half of its slice's activation planes).
+template <int W, int PRO, int EPI, int NW, int T>
+__global__ __launch_bounds__(64 * NW * T, (PRO == 2 || NW * T == 8) ? 1 : 2) void q4k_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x, float* y,
                                                                             int k, int n, int qt, const float* __restrict__ gain, float eps,
                                                                             const float* residual, RopeQkvEpilogue rope,
                                                                             AttnMergePrologue am) {
     constexpr int epilogue = EPI;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = T == 1 ? wave_all : wave_all % NW, team = T == 1 ? 0 : wave_all / NW;
     const int nsl = k >> 10;                                   // slices of 1024 elements
     const int nsw = (nsl - wave + NW - 1) / NW;                // this wave's share (uniform)
     const int ns_max = (nsl + NW - 1) / NW;
     const int nli_max = (144 * ns_max + 63) / 64;
-    const uint32_t ring_bytes = mfma_ring_bytes(nli_max, W);
-    uint8_t* ring = smem + wave * ring_bytes;
-    uint8_t* xa_stage = ring + (uint32_t)W * (uint32_t)nli_max * 1024u;      // the ring's last slot: free until the main loop
-    float* partials_all = reinterpret_cast<float*>(smem + NW * ring_bytes);   // [NW waves][qt][64]
+    // One team: the planes' staging area is the ring's last slot (free until the main loop). Two teams: one area per slice,
+    // shared by its two waves, behind the rings.
+    const uint32_t ring_bytes = T == 1 ? mfma_ring_bytes(nli_max, W) : (uint32_t)(W + 1) * nli_max * 1024u;
+    uint8_t* ring = smem + wave_all * ring_bytes;
+    uint8_t* xa_stage = T == 1 ? ring + (uint32_t)W * (uint32_t)nli_max * 1024u : smem + NW * T * ring_bytes + wave * MFMA_XA_BYTES;
+    float* partials_all = reinterpret_cast<float*>(smem + NW * T * ring_bytes + (T == 1 ? 0 : NW * MFMA_XA_BYTES));   // [NW slices of K][qt][64]
     float* ssq_lds = partials_all + NW * qt * 64;
     float* partials = partials_all + wave * qt * 64;
     const int r0 = blockIdx.x * (4 * qt);
     const uint32_t row_bytes = (uint32_t)(k >> 8) * (uint32_t)Q4K_BYTES;
 
     // what the final pass will add or rotate with: one output row per 16 threads and round
-    constexpr int RPR = 4 * NW;                                 // rows per round
+    constexpr int RPR = 4 * NW * T;                             // rows per round
     constexpr int ROUNDS = MFMA_MAX_QUADS * 4 / RPR;
     float pre_res[EPI == EPI_RESIDUAL ? ROUNDS : 1];
     f32x2_m pre_cs[EPI == EPI_ROPE_QKV ? ROUNDS : 1];
@@ -336,20 +351,20 @@ __global__ __launch_bounds__(64 * NW, (PRO == 2 || NW == 8) ? 1 : 2) void q4k_ge
 
     float ssq = 0.f;
     switch (nsw) {
-        case 1: q4k_mfma_wave<1, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 2: if constexpr (PRO != 2) q4k_mfma_wave<2, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 3: if constexpr (W <= 2 && PRO != 2 && NW == 4) q4k_mfma_wave<3, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
-        case 4: if constexpr (W <= 2 && PRO != 2 && NW == 4) q4k_mfma_wave<4, W, PRO, NW>(w, x, gain, am, n, r0, qt, row_bytes, wave, lane, ring, xa_stage, partials, &ssq); break;
+        case 1: q4k_mfma_wave<1, W, PRO, NW, T>(w, x, gain, am, n, r0, qt, row_bytes, wave, team, lane, ring, xa_stage, partials, &ssq); break;
+        case 2: if constexpr (PRO != 2 && T == 1) q4k_mfma_wave<2, W, PRO, NW, T>(w, x, gain, am, n, r0, qt, row_bytes, wave, team, lane, ring, xa_stage, partials, &ssq); break;
+        case 3: if constexpr (W <= 2 && PRO != 2 && NW == 4 && T == 1) q4k_mfma_wave<3, W, PRO, NW, T>(w, x, gain, am, n, r0, qt, row_bytes, wave, team, lane, ring, xa_stage, partials, &ssq); break;
+        case 4: if constexpr (W <= 2 && PRO != 2 && NW == 4 && T == 1) q4k_mfma_wave<4, W, PRO, NW, T>(w, x, gain, am, n, r0, qt, row_bytes, wave, team, lane, ring, xa_stage, partials, &ssq); break;
         default:                                               // K below NW slices: this wave has none
             for (int i = lane; i < qt * 64; i += 64) partials[i] = 0.f;
     }
-    if (PRO == 1 && lane == 0) ssq_lds[wave] = ssq;
+    if (PRO == 1 && lane == 0) ssq_lds[wave_all] = ssq;
     __syncthreads();
 
     float xscale = 1.0f;
     if (PRO == 1) {
         float ss = (ssq_lds[0] + ssq_lds[1]) + (ssq_lds[2] + ssq_lds[3]);
-        if (NW == 8) ss += (ssq_lds[4] + ssq_lds[5]) + (ssq_lds[6] + ssq_lds[7]);
+        if (NW * T == 8) ss += (ssq_lds[4] + ssq_lds[5]) + (ssq_lds[6] + ssq_lds[7]);
         xscale = 1.0f / sqrtf(ss * (1.0f / (float)k) + eps);
     }
     const int u = threadIdx.x & 15, pw = u >> 2, pp = u & 3;
@@ -396,6 +411,8 @@ __global__ __launch_bounds__(64 * NW, (PRO == 2 || NW == 8) ? 1 : 2) void q4k_ge
 
 static std::atomic<int> g_q4k_mfma_enable{1};
 void set_q4k_mfma_enable(int v) { g_q4k_mfma_enable = v; }
+static std::atomic<int> g_q4k_mfma_teams{0};       // 0: chosen from the quads a workgroup owns
+void set_q4k_mfma_teams(int v) { if (v >= 0 && v <= 2) g_q4k_mfma_teams = v; }
 static std::atomic<int> g_q4k_mfma_waves8{1};
 void set_q4k_mfma_waves8(int v) { g_q4k_mfma_waves8 = v != 0; }
 static std::atomic<int> g_q4k_mfma_window{0};      // 0: chosen from K
@@ -404,18 +421,20 @@ void set_q4k_mfma_window(int v) { if (v == 0 || v == 2 || v == 3) g_q4k_mfma_win
 // quads in flight per wave: three while a quad is at most 5 KB per wave, two for the long rows (9 KB per quad and wave)
 static int mfma_window(int k) { return (((k >> 10) + 3) >> 2) >= 3 ? 2 : 3; }
 
-static size_t mfma_smem_bytes(int k, int qt, int window, int nw) {
+static size_t mfma_smem_bytes(int k, int qt, int window, int nw, int teams = 1) {
     const int ns_max = ((k >> 10) + nw - 1) / nw;
     const int nli_max = (144 * ns_max + 63) / 64;
-    return (size_t)nw * mfma_ring_bytes(nli_max, window) + (size_t)nw * qt * 64 * sizeof(float) + 32;
+    const size_t rings = teams == 1 ? (size_t)nw * mfma_ring_bytes(nli_max, window)
+                                    : (size_t)nw * teams * (window + 1) * nli_max * 1024 + (size_t)nw * MFMA_XA_BYTES;
+    return rings + (size_t)nw * qt * 64 * sizeof(float) + 32;
 }
 
-template <int W, int PRO, int EPI, int NW = 4>
+template <int W, int PRO, int EPI, int NW = 4, int T = 1>
 static int launch_mfma_variant(int grid, size_t smem, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n, int qt,
                                const float* gain, float eps, const float* residual, const RopeQkvEpilogue& rope,
                                const AttnMergePrologue& am) {
-    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, PRO, EPI, NW>), 160 * 1024);
-    q4k_gemv_mfma_kernel<W, PRO, EPI, NW><<<dim3(grid), dim3(64 * NW), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, rope, am);
+    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemv_mfma_kernel<W, PRO, EPI, NW, T>), 160 * 1024);
+    q4k_gemv_mfma_kernel<W, PRO, EPI, NW, T><<<dim3(grid), dim3(64 * NW * T), smem, s>>>(w, x, y, k, n, qt, gain, eps, residual, rope, am);
     SKH_CHECK(hipGetLastError());
     return 1;
 }
@@ -497,6 +516,29 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
             note_kernel("q4k_gemv_mfma_kernel");
             if (epilogue == EPI_NONE) return launch_mfma_variant<2, 0, EPI_NONE, 8>(grid, smem8, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am);
             return launch_mfma_variant<2, 0, EPI_RESIDUAL, 8>(grid, smem8, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am);
+        }
+    }
+    // K = 4096 with a plain or RMSNorm prologue: two teams of four waves (two waves per SIMD, the planes prepared once)
+    // where a workgroup owns enough quads: measured with two teams / one, 11 quads (11008 rows) 6.14 / 6.23 us, 28 quads
+    // (28672 rows) 11.87 / 12.14, but 6 quads (6144 rows) 4.81 / 4.53 and 4 quads (4096 rows) 4.05 / 3.85 -- the barrier
+    // between the halves of the preparation costs more than a short run of quads gains
+    const int teams = g_q4k_mfma_teams.load() != 0 ? g_q4k_mfma_teams.load() : (qt >= 8 ? 2 : 1);
+    if (teams == 2 && pro != 2 && k == 4096 && qt >= 2 && window == 3) {
+        const size_t smem2 = mfma_smem_bytes(k, qt, 3, 4, 2);
+        if (smem2 <= 160 * 1024) {
+            note_kernel("q4k_gemv_mfma_kernel");
+#define SKH_MFMA_T2(PRO, EPI) return launch_mfma_variant<3, PRO, EPI, 4, 2>(grid, smem2, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am)
+            if (pro == 1) {
+                if (epilogue == EPI_NONE) SKH_MFMA_T2(1, EPI_NONE);
+                if (epilogue == EPI_RESIDUAL) SKH_MFMA_T2(1, EPI_RESIDUAL);
+                if (epilogue == EPI_SWIGLU) SKH_MFMA_T2(1, EPI_SWIGLU);
+                SKH_MFMA_T2(1, EPI_ROPE_QKV);
+            }
+            if (epilogue == EPI_NONE) SKH_MFMA_T2(0, EPI_NONE);
+            if (epilogue == EPI_RESIDUAL) SKH_MFMA_T2(0, EPI_RESIDUAL);
+            if (epilogue == EPI_SWIGLU) SKH_MFMA_T2(0, EPI_SWIGLU);
+            SKH_MFMA_T2(0, EPI_ROPE_QKV);
+#undef SKH_MFMA_T2
         }
     }
     const size_t smem = mfma_smem_bytes(k, qt, window, 4);

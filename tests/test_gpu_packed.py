@@ -142,6 +142,71 @@ def test_q4k_decode_kernel_variants_agree_with_the_oracle(hip_backend, torch_cud
         hip_backend.set_tuning("q4k_mfma_enable", 1)
 
 
+@pytest.mark.parametrize("n", [8, 37, 515, 4096, 11008, 28672, 40000])
+def test_q4k_one_row_kernel_with_two_teams_of_waves(hip_backend, torch_cuda, n):
+    """K = 4096: two teams of four waves per workgroup (the teams split the row quads and each prepares half of a slice's
+    activation planes) against one team. Every (slice, quad) partial sum is formed by the same instructions in the same
+    order either way, so the results are the same bits: plain, with a residual, with the RMSNorm prologue, with SwiGLU."""
+    k = 4096
+    packed = gaussian_weight(hip_backend, "Q4_K", n, k, 61) if n <= 11008 else random_valid_blocks("Q4_K", n * k // 256, 62)
+    rng = np.random.default_rng(63 + n)
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    gain = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    res = rng.standard_normal((1, n)).astype(np.float32)
+    w = hip_backend.DeviceWeight.upload("Q4_K", packed, n, k)
+    xd, gd, rd = dev(torch_cuda, x), dev(torch_cuda, gain), dev(torch_cuda, res)
+
+    def run(teams):
+        hip_backend.set_tuning("q4k_mfma_teams", teams)
+        outs = []
+        for kw in ({}, {"residual": rd, "epilogue": 1}, {"gain": gd, "eps": 1e-5}, {"gain": gd, "eps": 1e-5, "epilogue": 2}):
+            cols = n // 2 if kw.get("epilogue") == 2 else n
+            if kw.get("epilogue") == 2 and n % 2:
+                continue
+            y = torch_cuda.full((1, cols), float("nan"), dtype=torch_cuda.float32, device="cuda")
+            w.matmul_fused(xd, 1, y, **kw)
+            assert hip_backend.last_kernel() == "q4k_gemv_mfma_kernel"
+            outs.append(y.cpu().numpy())
+        return outs
+
+    try:
+        one, two = run(1), run(2)
+    finally:
+        hip_backend.set_tuning("q4k_mfma_teams", 0)
+    assert normalized_err(one[0], L.gemv("Q4_K", x, packed, n)) <= GEMV_TOL
+    for a, b in zip(one, two):
+        assert not np.isnan(b).any()
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("n,k", [(4096, 14336), (2050, 8192), (517, 16384), (64, 12288)])
+def test_q4k_one_row_kernel_with_eight_waves_on_long_rows(hip_backend, torch_cuda, n, k):
+    """Rows of 8192 elements and more without a prologue: K split over eight waves instead of four (another order of the
+    fp32 sums), plain and with a residual, against the oracle and against the four-wave form."""
+    packed = gaussian_weight(hip_backend, "Q4_K", n, k, 51)
+    rng = np.random.default_rng(52 + n)
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    res = rng.standard_normal((1, n)).astype(np.float32)
+    w = hip_backend.DeviceWeight.upload("Q4_K", packed, n, k)
+    xd, rd = dev(torch_cuda, x), dev(torch_cuda, res)
+    want = L.gemv("Q4_K", x, packed, n)
+    outs = {}
+    try:
+        for eight in (1, 0):
+            hip_backend.set_tuning("q4k_mfma_waves8", eight)
+            y = torch_cuda.full((1, n), float("nan"), dtype=torch_cuda.float32, device="cuda")
+            w.matmul_fused(xd, 1, y)
+            assert hip_backend.last_kernel() == "q4k_gemv_mfma_kernel"
+            yr = torch_cuda.full((1, n), float("nan"), dtype=torch_cuda.float32, device="cuda")
+            w.matmul_fused(xd, 1, yr, residual=rd, epilogue=1)
+            outs[eight] = (y.cpu().numpy(), yr.cpu().numpy())
+            assert normalized_err(outs[eight][0], want) <= GEMV_TOL
+            assert normalized_err(outs[eight][1], want + res) <= GEMV_TOL
+    finally:
+        hip_backend.set_tuning("q4k_mfma_waves8", 1)
+    assert normalized_err(outs[1][0], outs[0][0]) <= 2e-5
+
+
 @pytest.mark.parametrize("slot64", [1, 0])
 @pytest.mark.parametrize("n,k", [(8000, 4096), (515, 4096), (70, 768), (33, 256), (257, 14336), (3, 16640)])
 def test_q6k_batch1_slot_variants_agree_with_the_oracle(hip_backend, torch_cuda, slot64, n, k):
