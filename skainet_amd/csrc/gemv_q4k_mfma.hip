@@ -523,11 +523,12 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
     // (28672 rows) 11.87 / 12.14, but 6 quads (6144 rows) 4.81 / 4.53 and 4 quads (4096 rows) 4.05 / 3.85 -- the barrier
     // between the halves of the preparation costs more than a short run of quads gains
     const int teams = g_q4k_mfma_teams.load() != 0 ? g_q4k_mfma_teams.load() : (qt >= 8 ? 2 : 1);
-    if (teams == 2 && pro != 2 && k == 4096 && qt >= 2 && window == 3) {
-        const size_t smem2 = mfma_smem_bytes(k, qt, 3, 4, 2);
+    // (two quads in flight per wave then: with two waves per SIMD 6.14 us at three, 5.98 at two, 6.95 at one)
+    if (teams == 2 && pro != 2 && k == 4096 && qt >= 2) {
+        const size_t smem2 = mfma_smem_bytes(k, qt, 2, 4, 2);
         if (smem2 <= 160 * 1024) {
             note_kernel("q4k_gemv_mfma_kernel");
-#define SKH_MFMA_T2(PRO, EPI) return launch_mfma_variant<3, PRO, EPI, 4, 2>(grid, smem2, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am)
+#define SKH_MFMA_T2(PRO, EPI) return launch_mfma_variant<2, PRO, EPI, 4, 2>(grid, smem2, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am)
             if (pro == 1) {
                 if (epilogue == EPI_NONE) SKH_MFMA_T2(1, EPI_NONE);
                 if (epilogue == EPI_RESIDUAL) SKH_MFMA_T2(1, EPI_RESIDUAL);
