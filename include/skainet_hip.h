@@ -383,7 +383,7 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * kernel and run the fp32 row-streaming one), "q4k_quads_stream_enable" (0: Q4_K products of 3 to 8 rows at K = 4096 stay on the
  * kernel that loads a lane's codes into registers instead of the one that streams the weight through an LDS ring),
  * "q4k_mfma_teams" (teams of four waves per workgroup of the one-row integer matrix-core kernel at K = 4096: 1, 2 = the
- * teams split the row quads and each wave prepares half of its slice's activations, 0 = two where a workgroup owns eight
+ * teams split the row quads and each wave prepares half of its slice's activations, 0 = two where a workgroup owns five
  * quads or more), "q4k_mfma_waves8" (0: the one-row integer matrix-core kernel keeps four waves per workgroup on rows of 8192 elements
  * and more instead of eight),
  * "q4k_mfma_window" (row quads the one-row integer matrix-core kernel keeps in flight per wave: 2 or 3,

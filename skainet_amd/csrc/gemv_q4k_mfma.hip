@@ -519,10 +519,10 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
         }
     }
     // K = 4096 with a plain or RMSNorm prologue: two teams of four waves (two waves per SIMD, the planes prepared once)
-    // where a workgroup owns enough quads: measured with two teams / one, 11 quads (11008 rows) 6.14 / 6.23 us, 28 quads
-    // (28672 rows) 11.87 / 12.14, but 6 quads (6144 rows) 4.81 / 4.53 and 4 quads (4096 rows) 4.05 / 3.85 -- the barrier
-    // between the halves of the preparation costs more than a short run of quads gains
-    const int teams = g_q4k_mfma_teams.load() != 0 ? g_q4k_mfma_teams.load() : (qt >= 8 ? 2 : 1);
+    // where a workgroup owns enough quads: measured with two teams / one, 28 quads (28672 rows) 11.64 / 12.09 us, 11 quads
+    // (11008 rows) 5.98 / 6.23, 6 quads (6144 rows) 4.43 / 4.51, but 4 quads (4096 rows) 3.91 / 3.83 -- the barrier between
+    // the halves of the preparation costs more than so short a run of quads gains
+    const int teams = g_q4k_mfma_teams.load() != 0 ? g_q4k_mfma_teams.load() : (qt >= 5 ? 2 : 1);
     // (two quads in flight per wave then: with two waves per SIMD 6.14 us at three, 5.98 at two, 6.95 at one)
     if (teams == 2 && pro != 2 && k == 4096 && qt >= 2) {
         const size_t smem2 = mfma_smem_bytes(k, qt, 2, 4, 2);
