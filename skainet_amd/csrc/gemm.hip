@@ -666,6 +666,12 @@ int launch_q4k_gemm_ksw(const __bf16* a, const uint8_t* w, float* c, int m, int 
 bool gemm_ksw_enabled();
 bool gemm_ksw_fits(int m, int n, int k);
 bool gemm_ksw_forced();
+size_t gemm_frag_activation_bytes(int m, int k);                                                              // gemm_q4k_frag.hip
+int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, hipStream_t s);
+int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s);
+bool gemm_frag_enabled();
+bool gemm_frag_fits(int m, int n, int k);
+bool gemm_frag_forced();
 
 static std::atomic<int> g_gemm_ksplit{0};   // 0 = choose from the tile count
 void set_gemm_ksplit(int v) { g_gemm_ksplit = v; }
@@ -714,7 +720,16 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         if (launch_q4k_gemm_ksw(a, w, epilogue != GEMM_EPI_NONE ? tmp : y, m, n, k, s) != 0) return -1;
         return finish();
     };
+    auto run_frag = [&]() -> int {                               // Q4_K: the same tiles, activations in fragment order
+        uint8_t* a = static_cast<uint8_t*>(kernel_workspace(gemm_frag_activation_bytes(m, k)));
+        if (!a) return -1;
+        if (launch_gemm_frag_prepass(x, gain, eps, a, m, k, s) != 0) return -1;
+        if (launch_q4k_gemm_frag(a, w, epilogue != GEMM_EPI_NONE ? tmp : y, m, n, k, s) != 0) return -1;
+        return finish();
+    };
     const bool ksw_ok = enc == ENC_Q4_K && gemm_ksw_fits(m, n, k) && g_gemm_wide.load() < 0 && g_gemm_rows.load() == 0;
+    const bool frag_ok = ksw_ok && gemm_frag_fits(m, n, k);
+    if (frag_ok && gemm_frag_forced()) return run_frag();
     if (ksw_ok && gemm_ksw_forced()) return run_ksw();
     // 128 activation rows per tile where there are no more than that (the weight is then decoded once, and half the
     // matrix work of the taller tile is not spent on rows that do not exist); the wide tile where it alone fills most of
@@ -752,7 +767,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         // products; its step is slower per tile row (0.31 us per 64 elements of K measured, 6.5 us per round outside the loop).
         // It wins where the tile kernel would have to split K across workgroups: 512 x 4096 x 4096 is such a shape.
         const int rounds = (((m + 127) / 128) * ((n + 63) / 64) + num_cus() - 1) / num_cus();
-        if (rounds * (6.5 + 0.31 * (k / GK)) < tile_estimate) return run_ksw();
+        if (rounds * (6.5 + 0.31 * (k / GK)) < tile_estimate) return frag_ok && gemm_frag_enabled() ? run_frag() : run_ksw();
     }
     if (ksplit > kgroups) ksplit = kgroups;
     const int k_chunk = ((kgroups + ksplit - 1) / ksplit) * 256;

@@ -1,0 +1,435 @@
+// Q4_K dequant-GEMM whose activations arrive in matrix-instruction fragment order:
+//   C[m, n] = sum_k A[m, k] * dequant(W[n, k]),  A fp32 [M, K] rounded to bf16 once, W packed Q4_K in canonical row-major
+//   GGUF order, products bf16 x bf16 on v_mfma_f32_32x32x16_bf16, fp32 accumulation, C fp32 [M, N].
+// A weight is code * (d * sc) - dmin * m in fp32 (one fused multiply-add), rounded to bf16 (nearest even): the arithmetic
+// of dequant_gemm_kernel (gemm.hip). Semantics: m rows = m scalar GEMVs,
+// /root/reference/skainet-backends/skainet-backend-cpu/src/commonMain/kotlin/sk/ainet/exec/kernel/PackedViewMatmulKernel.kt:69-108.
+//
+// Who owns what:
+//   * workgroup tile 128 (M) x 64 (N), eight waves (two per SIMD); every wave owns the WHOLE tile (4 x 2 matrix tiles of
+//     32 x 32: 128 accumulators; an activation fragment feeds two matrix instructions, a decoded weight fragment four)
+//     and whole super-blocks of K: wave w takes super-blocks w, w + 8, ... The partial tiles meet once, through LDS.
+//   * An activation element is needed by exactly one wave of the workgroup, so it never passes through LDS: the pass in
+//     front (gemm_frag_prepass_kernel) writes bf16 activations in the order the matrix instruction reads them -- the 64
+//     lanes x 16 bytes of the fragment of (row tile of 32, 16-element step) are 1 KB of consecutive memory -- and a
+//     wave's four fragment loads of a step are plain 16-byte loads into the registers the instruction reads, two steps
+//     ahead of their use. No barrier and no LDS traffic on the activation side.
+//   * The contraction order inside a step is a free permutation as long as both operands agree. A step is chosen so
+//     that a lane's 8 weights are the low and the high nibbles of ONE code dword: step t (0..3) of the 64-element group
+//     g of a super-block covers, for lane half h, elements 64 g + 16 h + 4 t + {0..3} (low nibbles, sub-block 2 g) and
+//     the same + 32 (high nibbles, sub-block 2 g + 1). A lane reads 16 code bytes per group and column tile from LDS.
+//   * Raw super-blocks (64 rows x 144 bytes) are fetched by loads that write LDS directly (global_load_lds_dwordx4), each
+//     wave its own super-blocks into its own two slots: no workgroup barrier in the loop at all.
+//   * Workgroup ids map to tiles so that the workgroups of one die (id mod 8) share activation row blocks and weight
+//     columns: each die's L2 fetches a rectangle of tiles, not every activation row.
+#include "common.h"
+
+#include <type_traits>
+
+namespace skh {
+
+typedef __bf16 frg_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 frg_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float frg_f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t frg_u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int FRG_M = 128, FRG_N = 64, FRG_WAVES = 8;
+constexpr int FRG_SLOT = FRG_N * 144;                         // one raw super-block of the tile's 64 weight rows: 9 wave loads
+constexpr int FRG_RED_PITCH = FRG_N + 4;                      // floats per row of a partial tile in the final exchange
+constexpr size_t FRG_LOOP_BYTES = (size_t)FRG_WAVES * 2 * FRG_SLOT;
+constexpr size_t FRG_RED_BYTES = (size_t)4 * FRG_M * FRG_RED_PITCH * sizeof(float);
+constexpr size_t FRG_SMEM = FRG_LOOP_BYTES > FRG_RED_BYTES ? FRG_LOOP_BYTES : FRG_RED_BYTES;
+
+// Bytes of the fragment-ordered bf16 copy of an [m, k] activation matrix: row tiles of 32 padded up to whole workgroup
+// tiles of 128 rows (the padding rows are zeros).
+size_t gemm_frag_activation_bytes(int m, int k) { return (size_t)((m + FRG_M - 1) / FRG_M) * FRG_M * (size_t)k * 2; }
+
+// Workgroup ids are handed to the eight dies round-robin, so die x runs ids x, x + 8, ... The GEMM gives die x the
+// consecutive positions x * (tiles / 8) .. of an order that walks `gm` row tiles for every column tile before it moves to
+// the next group of row tiles: a rectangle of tiles per die, which shares both operands inside that die's L2. (With a
+// tile count that is not a multiple of 8 the ids are taken in order.)
+struct FrgTileOrder { int gm, tiles_m, tiles_n; };
+__device__ __forceinline__ int frg_position(const FrgTileOrder& o, int id) {
+    const int tiles = o.tiles_m * o.tiles_n;
+    return (tiles & 7) == 0 ? (id & 7) * (tiles >> 3) + (id >> 3) : id;
+}
+__device__ __forceinline__ void frg_tile_of(const FrgTileOrder& o, int pos, int& mt, int& nt) {
+    const int per_group = o.gm * o.tiles_n, grp = pos / per_group, rem = pos - grp * per_group;
+    nt = rem / o.gm;
+    mt = grp * o.gm + (rem - nt * o.gm);
+}
+
+// Fragment order: the 16 bytes of lane (r, h) (r = lane % 32: activation row inside the row tile, h = lane / 32) for row
+// tile `it` and step s = 4 * (k / 64) + t sit at ((it * (K / 16) + s) * 64 + lane) * 16 and hold, as bf16,
+//   x[32 it + r][64 (s / 4) + 16 h + 4 t + 0..3] and x[32 it + r][64 (s / 4) + 32 + 16 h + 4 t + 0..3].
+// Thread (r, c) of a workgroup (c = 4 h + t) reads the two float4s and writes the piece: a wave reads eight row
+// segments of 128 bytes twice and writes eight runs of 128 bytes.
+__global__ __launch_bounds__(256) void gemm_frag_prepass_kernel(const float* __restrict__ in, uint8_t* __restrict__ out, int m, int k) {
+    const int gi = blockIdx.x, it = blockIdx.y;
+    const int r = threadIdx.x >> 3, c = threadIdx.x & 7;
+    const int row = 32 * it + r;
+    const float* src = in + (int64_t)min(row, m - 1) * k + 64 * gi + 4 * c;
+    float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 32);
+    if (row >= m) lo = hi = make_float4(0.f, 0.f, 0.f, 0.f);
+    frg_u32x4 v;
+    v.x = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)lo.x, (__bf16)lo.y});
+    v.y = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)lo.z, (__bf16)lo.w});
+    v.z = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)hi.x, (__bf16)hi.y});
+    v.w = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)hi.z, (__bf16)hi.w});
+    const int64_t steps = k >> 4, s = 4 * gi + (c & 3), lane = r + 32 * (c >> 2);
+    *reinterpret_cast<frg_u32x4*>(out + ((it * steps + s) * 64 + lane) * 16) = v;
+}
+
+// The same pass with an RMSNorm folded in: bf16(x / sqrt(mean(x^2) + eps) * gain), one workgroup per activation row
+// (rows past m: zeros), the row held in registers between the sum of squares and the scaling (k a multiple of 64, at
+// most 256 * 4 * V floats). A thread's float4 is half of a 16-byte piece.
+template <int V>
+__global__ __launch_bounds__(256) void gemm_frag_prepass_rmsnorm_kernel(const float* __restrict__ in, const float* __restrict__ gain,
+                                                                        uint8_t* __restrict__ out, int m, int k, float eps) {
+    __shared__ float red[4];
+    const int row = blockIdx.x;
+    const float4* x = reinterpret_cast<const float4*>(in + (int64_t)min(row, m - 1) * k);
+    const float4* g4 = reinterpret_cast<const float4*>(gain);
+    const int k4 = k >> 2;
+    float4 xr[V], gr[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        xr[j] = i < k4 && row < m ? x[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        gr[j] = i < k4 ? g4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j) { s = fmaf(xr[j].x, xr[j].x, s); s = fmaf(xr[j].y, xr[j].y, s); s = fmaf(xr[j].z, xr[j].z, s); s = fmaf(xr[j].w, xr[j].w, s); }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    const float scale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) * (1.0f / (float)k) + eps);
+    const int64_t steps = k >> 4, it = row >> 5;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i >= k4) continue;
+        const int gi = i >> 4, ci = i & 15, c = ci & 7, half = ci >> 3;
+        const int64_t st = 4 * gi + (c & 3), lane = (row & 31) + 32 * (c >> 2);
+        uint2 v;
+        v.x = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)(xr[j].x * scale * gr[j].x), (__bf16)(xr[j].y * scale * gr[j].y)});
+        v.y = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)(xr[j].z * scale * gr[j].z), (__bf16)(xr[j].w * scale * gr[j].w)});
+        *reinterpret_cast<uint2*>(out + ((it * steps + st) * 64 + lane) * 16 + 8 * half) = v;
+    }
+}
+
+// 16 bytes per lane from base + off straight into LDS at lds_addr + 16 * lane (M0 carries the LDS address); counted by
+// vmcnt like any other load, in issue order
+__device__ __forceinline__ void frg_dma16(uint32_t lds_addr, uint32_t off, const uint8_t* base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory");
+}
+
+// The eight 6-bit scales and minima of a super-block header (ggml get_scale_min_k4) as bytes of four dwords: sub-blocks
+// 0..3 and 4..7, each for scales and minima.
+struct FrgScales { float d, d16, dmin; uint32_t sc_lo, sc_hi, mn_lo, mn_hi; };
+__device__ __forceinline__ FrgScales frg_unpack(const frg_u32x4& hdr) {
+    FrgScales r;
+    r.d16 = half_bits_to_float_fast(hdr.x & 0xFFFFu) * 1048576.0f;    // high nibbles stay in place: 16 code 2^-24
+    r.d = r.d16 * 16.0f;                                              // low nibbles: code 2^-24
+    r.dmin = half_bits_to_float_fast(hdr.x >> 16);
+    r.sc_lo = hdr.y & 0x3F3F3F3Fu;
+    r.mn_lo = hdr.z & 0x3F3F3F3Fu;
+    r.sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+    r.mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+    return r;
+}
+// Group G (0..3) of a super-block: sub-block 2 G scales the low nibbles, 2 G + 1 the high ones.
+// Codes are not converted: masked into 16-bit fields (0x000F000F: the low nibbles of bytes 0 and 2, 0x00F000F0 their high
+// nibbles; the same on the dword shifted right by 8 for bytes 1 and 3) a field read as fp16 is the subnormal
+// code * 2^-24 (or 16 * code * 2^-24), which v_fma_mix_f32 widens exactly on its way into the fp32 multiply-add; the
+// powers of two go into the scales, so the products are the very fp32 values of converted codes.
+//   gs[0] = 2^24 d * sc[2G], gs[1] = dmin * m[2G], gs[2] = 2^20 d * sc[2G + 1], gs[3] = dmin * m[2G + 1]
+template <int G>
+__device__ __forceinline__ void frg_group_scales(const FrgScales& k, float (&gs)[4]) {
+    const uint32_t sc = G < 2 ? k.sc_lo : k.sc_hi, mn = G < 2 ? k.mn_lo : k.mn_hi;
+    gs[0] = k.d * ((G & 1) ? ubyte2_to_float(sc) : ubyte0_to_float(sc));
+    gs[1] = k.dmin * ((G & 1) ? ubyte2_to_float(mn) : ubyte0_to_float(mn));
+    gs[2] = k.d16 * ((G & 1) ? ubyte3_to_float(sc) : ubyte1_to_float(sc));
+    gs[3] = k.dmin * ((G & 1) ? ubyte3_to_float(mn) : ubyte1_to_float(mn));
+}
+typedef _Float16 frg_h2 __attribute__((ext_vector_type(2)));
+// the four weights of one nibble plane of a code dword (PLANE 0: low nibbles, 1: high) -> two dwords of bf16 pairs in
+// byte order; c8 = c >> 8
+template <int PLANE>
+__device__ __forceinline__ void frg_decode4(uint32_t c, uint32_t c8, float scale, float offset, uint32_t& lo, uint32_t& hi) {
+    constexpr uint32_t mask = PLANE ? 0x00F000F0u : 0x000F000Fu;
+    const frg_h2 b02 = __builtin_bit_cast(frg_h2, c & mask), b13 = __builtin_bit_cast(frg_h2, c8 & mask);
+    const float w0 = fmaf((float)b02.x, scale, -offset), w1 = fmaf((float)b13.x, scale, -offset);
+    const float w2 = fmaf((float)b02.y, scale, -offset), w3 = fmaf((float)b13.y, scale, -offset);
+    lo = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)w0, (__bf16)w1});
+    hi = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)w2, (__bf16)w3});
+}
+
+__global__ __launch_bounds__(64 * FRG_WAVES) void q4k_gemm_frag_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ w,
+                                                                       float* __restrict__ c, int m, int n, int k, FrgTileOrder order) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t frg_smem[];   // the kernel has no other LDS: offsets into it are LDS addresses
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col = lane & 31, kh = lane >> 5;
+
+    int mt, nt;
+    frg_tile_of(order, frg_position(order, blockIdx.x), mt, nt);
+    const int m0 = mt * FRG_M, n0 = nt * FRG_N;
+    const int nsb = k >> 8;
+    const int my_count = nsb > wv ? (nsb - wv + FRG_WAVES - 1) / FRG_WAVES : 0;   // this wave's super-blocks: wv, wv + 8, ...
+    const uint32_t row_bytes = (uint32_t)nsb * 144u;
+    const int64_t steps = k >> 4;
+
+    // activation fragments: row tile 4 mt + i, step s: 1 KB at ((4 mt + i) * steps + s) * 1024, this lane's 16 bytes
+    // Read through a buffer descriptor over this workgroup's four row tiles: the lane's constant 16 l is the vector
+    // offset, everything that moves is a scalar offset, so the address arithmetic stays on the scalar unit.
+    const uint32_t a_tile = (uint32_t)steps * 1024u;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(a) + (int64_t)(4 * mt) * a_tile, 0, 4 * a_tile, 0x00020000);
+    const uint32_t lane16 = 16u * lane;
+    // step u of this wave (16 per super-block): global step 16 * (wv + 8 * (u / 16)) + u % 16; past the end: the last one
+    const int last_u = 16 * my_count - 1;
+    auto load_frag = [&](int u, int i) -> frg_bf16x8 {
+        u = min(u, last_u);
+        const uint32_t soff = (uint32_t)(16 * (wv + FRG_WAVES * (u >> 4)) + (u & 15)) * 1024u + (uint32_t)i * a_tile;
+        return __builtin_bit_cast(frg_bf16x8, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, lane16, soff, 0));
+    };
+    auto load_frags = [&](frg_bf16x8 (&af)[4], int u) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[i] = load_frag(u, i);
+    };
+
+    // raw super-blocks: 576 pieces of 16 bytes in row order = 9 wave loads into this wave's slot (rows 144 bytes apart)
+    const uint32_t my_lds = (uint32_t)wv * 2u * FRG_SLOT;
+    uint32_t w_voff[9];
+#pragma unroll
+    for (int j = 0; j < 9; ++j) {
+        const int p = 64 * j + lane, row = (p * 7282) >> 16, pc = p - 9 * row;         // row = p / 9 for p < 576
+        w_voff[j] = (uint32_t)min(n0 + row, n - 1) * row_bytes + 16u * pc;             // rows past N: a valid copy, never stored
+    }
+    auto dma_w = [&](int slot, int q) __attribute__((always_inline)) {                 // this wave's q-th super-block
+        const uint8_t* base = w + (size_t)(wv + FRG_WAVES * q) * 144;                  // uniform
+#pragma unroll
+        for (int j = 0; j < 9; ++j) frg_dma16(my_lds + slot * FRG_SLOT + 1024u * j, w_voff[j], base);
+    };
+    // this lane's picks in a slot: rows col and col + 32; header 16 bytes, then per group 16 code bytes at 16 + 32 g + 16 kh
+    const uint32_t pick = my_lds + (uint32_t)col * 144u;
+    auto read_hdr = [&](FrgScales (&ks)[2], int slot) __attribute__((always_inline)) {
+        const uint8_t* q = frg_smem + (pick + slot * FRG_SLOT);
+        ks[0] = frg_unpack(*reinterpret_cast<const frg_u32x4*>(q));
+        ks[1] = frg_unpack(*reinterpret_cast<const frg_u32x4*>(q + 32 * 144));
+    };
+    auto read_codes = [&](frg_u32x4 (&codes)[2], int slot, int g) __attribute__((always_inline)) {
+        const uint8_t* q = frg_smem + (pick + slot * FRG_SLOT + 16 + 32 * g + 16 * kh);
+        codes[0] = *reinterpret_cast<const frg_u32x4*>(q);
+        codes[1] = *reinterpret_cast<const frg_u32x4*>(q + 32 * 144);
+    };
+
+    frg_f32x16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    if (my_count > 0) {
+        frg_bf16x8 af[2][4];                       // fragments of the step being multiplied and of the next one
+        uint32_t bw[2][2][4];                      // [set][column tile][dword]: decoded B operands
+        frg_u32x4 codes[2];                        // the code dwords of the group being decoded, per column tile
+        FrgScales ks[2];
+        float gs[2][4];
+
+        // Prologue: this wave's first two super-blocks into its slots, fragments of steps 0 and 1 into registers, weights
+        // of step 0 decoded.
+        load_frags(af[0], 0);
+        load_frags(af[1], 1);
+        dma_w(0, 0);
+        if (my_count > 1) dma_w(1, 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        read_hdr(ks, 0);
+        read_codes(codes, 0, 0);
+        frg_group_scales<0>(ks[0], gs[0]);
+        frg_group_scales<0>(ks[1], gs[1]);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            frg_decode4<0>(codes[j].x, codes[j].x >> 8, gs[j][0], gs[j][1], bw[0][j][0], bw[0][j][1]);
+            frg_decode4<1>(codes[j].x, codes[j].x >> 8, gs[j][2], gs[j][3], bw[0][j][2], bw[0][j][3]);
+        }
+
+        // One step: the 8 matrix instructions of step 16 q + P (fragments and weights in registers, set P & 1), and between
+        // them, in pinned program order, what prepares later steps:
+        //   behind each pair of matrix instructions on row tile i: the load of that fragment for two steps on
+        //   behind instructions 0, 2, 4, 6: the next step's weights decoded, four at a time
+        //   at the end of the third step of a group: the next group's code bytes read from LDS (the current ones are used
+        //   up; in the last group: the next super-block's header as well)
+        //   at the start of the last step of a group: the next group's scales
+        auto step_body = [&](auto pc, int q) __attribute__((always_inline)) {
+            constexpr int P = decltype(pc)::value, SET = P & 1, G = P >> 2, T = P & 3, NT = (T + 1) & 3, NG = (G + 1) & 3;
+            const int slot = q & 1, next_slot = G == 3 ? slot ^ 1 : slot;
+            frg_bf16x8 b[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = __builtin_bit_cast(frg_bf16x8, frg_u32x4{bw[SET][j][0], bw[SET][j][1], bw[SET][j][2], bw[SET][j][3]});
+            if (P == 0 && q >= 1 && q + 1 < my_count) {
+                // the slot of super-block q - 1 is free (its last bytes were read five steps ago): fetch super-block q + 1
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                dma_w(slot ^ 1, q + 1);
+            }
+            if (T == 3) {
+                frg_group_scales<NG>(ks[0], gs[0]);
+                frg_group_scales<NG>(ks[1], gs[1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma clang loop unroll(full)
+            for (int x = 0; x < 8; ++x) {
+                const int i = x >> 1, j = x & 1;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[SET][i], b[j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (j == 1) af[SET][i] = load_frag(16 * q + P + 2, i);
+                else {
+                    const int jj = i >> 1, half = i & 1;
+                    const uint32_t cw = NT == 0 ? codes[jj].x : NT == 1 ? codes[jj].y : NT == 2 ? codes[jj].z : codes[jj].w;
+                    if (half == 0) frg_decode4<0>(cw, cw >> 8, gs[jj][0], gs[jj][1], bw[SET ^ 1][jj][0], bw[SET ^ 1][jj][1]);
+                    else frg_decode4<1>(cw, cw >> 8, gs[jj][2], gs[jj][3], bw[SET ^ 1][jj][2], bw[SET ^ 1][jj][3]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (T == 2) {
+                if (G == 3) {
+                    // the next super-block: its slot was requested at least 14 steps (56 loads) ago and loads return in
+                    // issue order, so with at most 8 still in flight it has landed; this super-block's header was last
+                    // used three steps ago
+                    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                    read_hdr(ks, next_slot);
+                }
+                read_codes(codes, next_slot, NG);                         // dword 3 of the current group was decoded above
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        for (int q = 0; q < my_count; ++q) {                              // one super-block (sixteen steps) per trip
+            step_body(std::integral_constant<int, 0>{}, q);
+            step_body(std::integral_constant<int, 1>{}, q);
+            step_body(std::integral_constant<int, 2>{}, q);
+            step_body(std::integral_constant<int, 3>{}, q);
+            step_body(std::integral_constant<int, 4>{}, q);
+            step_body(std::integral_constant<int, 5>{}, q);
+            step_body(std::integral_constant<int, 6>{}, q);
+            step_body(std::integral_constant<int, 7>{}, q);
+            step_body(std::integral_constant<int, 8>{}, q);
+            step_body(std::integral_constant<int, 9>{}, q);
+            step_body(std::integral_constant<int, 10>{}, q);
+            step_body(std::integral_constant<int, 11>{}, q);
+            step_body(std::integral_constant<int, 12>{}, q);
+            step_body(std::integral_constant<int, 13>{}, q);
+            step_body(std::integral_constant<int, 14>{}, q);
+            step_body(std::integral_constant<int, 15>{}, q);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // nothing of this wave still writes or reads its slots
+    __syncthreads();
+
+    // The waves hold partial sums of the same 128 x 64 tile. Waves 4..7 park theirs in LDS and waves 0..3 add them to
+    // their own (same lane, same element: the addresses a lane reads are the ones its twin wrote); then waves 0..3 park
+    // the four remaining partial tiles and all eight waves add up a share of the rows and store it.
+    // Accumulator element e of lane l: row 8 (e / 4) + 4 (l / 32) + e % 4, column l % 32 of its 32 x 32 tile.
+    float* red = reinterpret_cast<float*>(frg_smem);
+    float* mine = red + (size_t)(wv & 3) * FRG_M * FRG_RED_PITCH;
+    auto tile_at = [&](int i, int j, int e) -> float& { return mine[(32 * i + 8 * (e >> 2) + 4 * kh + (e & 3)) * FRG_RED_PITCH + 32 * j + col]; };
+    if (wv >= 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
+    }
+    __syncthreads();
+    if (wv < 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] += tile_at(i, j, e);
+    }
+    __syncthreads();
+    if (wv < 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
+    }
+    __syncthreads();
+    const int c4 = (lane & 15) * 4;
+    constexpr int ROWS_PER_WAVE = FRG_M / FRG_WAVES;
+#pragma unroll
+    for (int it = 0; it < ROWS_PER_WAVE / 4; ++it) {
+        const int row = ROWS_PER_WAVE * wv + 4 * it + (lane >> 4);
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float4 t = *reinterpret_cast<const float4*>(red + ((size_t)v * FRG_M + row) * FRG_RED_PITCH + c4);
+            sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+        }
+        const int gr = m0 + row, gc = n0 + c4;
+        if (gr < m) {
+            float* dst = c + (int64_t)gr * n + gc;
+            if (gc + 3 < n && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) *reinterpret_cast<float4*>(dst) = sum;
+            else {
+                if (gc < n) dst[0] = sum.x;
+                if (gc + 1 < n) dst[1] = sum.y;
+                if (gc + 2 < n) dst[2] = sum.z;
+                if (gc + 3 < n) dst[3] = sum.w;
+            }
+        }
+    }
+}
+
+static std::atomic<int> g_gemm_frag{1};     // 0 never, 1 where the launcher's estimate favours it, 2 wherever it fits
+void set_gemm_frag(int v) { if (v >= 0 && v <= 2) g_gemm_frag = v; }
+bool gemm_frag_enabled() { return g_gemm_frag.load() != 0; }
+bool gemm_frag_forced() { return g_gemm_frag.load() == 2; }
+bool gemm_frag_fits(int m, int n, int k) {
+    return k % 256 == 0 && (uint64_t)n * (uint64_t)(k >> 8) * 144u < ((uint64_t)1 << 31) && gemm_frag_activation_bytes(m, k) < ((uint64_t)1 << 31) && (uint64_t)k * 256 < ((uint64_t)1 << 31);
+}
+
+// row tiles per group of the tile order: a die's share of the tiles is gm row tiles x (share / gm) column tiles and
+// its L2 fetches 256 gm + 36 share / gm bytes per element of K -- take the divisor of tiles_m with the least
+static FrgTileOrder frg_tile_order(int m, int n) {
+    FrgTileOrder o{1, (m + FRG_M - 1) / FRG_M, (n + FRG_N - 1) / FRG_N};
+    const double share = (double)o.tiles_m * o.tiles_n / 8.0;
+    double best = 0.0;
+    for (int g = 1; g <= o.tiles_m && g <= 8; ++g) {
+        if (o.tiles_m % g != 0) continue;
+        const double cost = 256.0 * g + 36.0 * share / g;
+        if (g == 1 || cost < best) { best = cost; o.gm = g; }
+    }
+    return o;
+}
+
+// The pass in front: x fp32 [m, k] (16-byte aligned, k a multiple of 64) -> the fragment-ordered bf16 copy `a`
+// (gemm_frag_activation_bytes(m, k) bytes); gain != null folds an RMSNorm in (k <= 16384).
+int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, hipStream_t s) {
+    const int row_tiles = (m + FRG_M - 1) / FRG_M * (FRG_M / 32);
+    if (!gain) gemm_frag_prepass_kernel<<<dim3(k / 64, row_tiles), dim3(256), 0, s>>>(x, a, m, k);
+    else if (k <= 256 * 4 * 4) gemm_frag_prepass_rmsnorm_kernel<4><<<dim3(row_tiles * 32), dim3(256), 0, s>>>(x, gain, a, m, k, eps);
+    else gemm_frag_prepass_rmsnorm_kernel<16><<<dim3(row_tiles * 32), dim3(256), 0, s>>>(x, gain, a, m, k, eps);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
+// C = A . W^T for activations already in fragment order; k a multiple of 256, operands 16-byte aligned. 0 on success.
+int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s) {
+    if (!gemm_frag_fits(m, n, k)) return set_error("gemm: operands of %d x %d x %d are outside this kernel's range", m, n, k);
+    const FrgTileOrder order = frg_tile_order(m, n);
+    note_kernel("q4k_gemm_frag_kernel");
+    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_frag_kernel), FRG_SMEM);
+    q4k_gemm_frag_kernel<<<dim3(order.tiles_m * order.tiles_n), dim3(64 * FRG_WAVES), FRG_SMEM, s>>>(a, w, c, m, n, k, order);
+    SKH_CHECK(hipGetLastError());
+    return 0;
+}
+
+}  // namespace skh

@@ -162,6 +162,34 @@ def test_q4k_gemm_with_k_split_over_the_waves(hip_backend, torch_cuda, m, n, k):
         hip_backend.set_tuning("gemm_ksw", 1)
         hip_backend.set_tuning("gemm_ksw_teams", 2)
         hip_backend.set_tuning("gemm_ksw_stages", 5)
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (9, 64, 256), (130, 70, 512), (128, 129, 1024), (300, 1000, 2304), (40, 200, 14336),
+                                   (257, 63, 768), (64, 512, 11008), (384, 1024, 4096)])
+def test_q4k_gemm_with_activations_in_fragment_order(hip_backend, torch_cuda, m, n, k):
+    """The Q4_K kernel whose activations are laid out by the pass in front in the order the matrix instruction reads them
+    (every wave: the whole 128 x 64 tile and whole super-blocks of K), forced on shapes with ragged row and column tiles,
+    fewer super-blocks than waves, uneven super-block counts per wave (43 and 56 super-blocks over 8 waves), tile counts
+    that are and are not a multiple of the eight dies; against the oracle (2e-2), against the same product with both
+    operands rounded to bf16 first (2e-4), and against the tile kernel."""
+    packed = gaussian_weight(hip_backend, "Q4_K", n, k, 900 + n)
+    x = np.random.default_rng(m * 7 + k).standard_normal((m, k)).astype(np.float32)
+    want = L.gemv("Q4_K", x, packed, n)
+    try:
+        hip_backend.set_tuning("gemm_frag", 2)
+        got = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemm_frag_kernel"
+        assert not np.isnan(got).any()
+        check(got, want)
+        check_exact(torch_cuda, "Q4_K", got, x, packed, n)
+        hip_backend.set_tuning("gemm_frag", 0)
+        hip_backend.set_tuning("gemm_ksw", 0)
+        tiles = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "dequant_gemm_kernel"
+        assert normalized_err(got, tiles) <= 1e-4          # same operands, another fp32 summation order
+    finally:
+        hip_backend.set_tuning("gemm_frag", 1)
+        hip_backend.set_tuning("gemm_ksw", 1)
     if (m, n, k) == (512, 4096, 4096):
         gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
-        assert hip_backend.last_kernel() == "q4k_gemm_ksw_kernel"      # the launcher's own choice for this shape
+        assert hip_backend.last_kernel() == "q4k_gemm_frag_kernel"     # the launcher's own choice for this shape
