@@ -177,6 +177,8 @@ void set_q4k_mfma_window(int v);
 void set_q4k_mfma_teams(int v);
 void set_q4k_mfma_waves8(int v);
 void set_q4k_quads_stream_enable(int v);
+void set_q4k_wide_enable(int v);
+void set_q4k_wide_min_batch(int v);
 void set_attn_merge_enable(int v);
 void set_sdpa_decode_gs(int v);
 void set_attn_merge_max_keys(int v);
@@ -207,6 +209,8 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q4k_ksplit_enable")) { set_q4k_ksplit_enable(value); return 0; }
     if (!strcmp(key, "q4k_mfma_enable")) { set_q4k_mfma_enable(value); return 0; }
     if (!strcmp(key, "q4k_quads_stream_enable")) { set_q4k_quads_stream_enable(value); return 0; }
+    if (!strcmp(key, "q4k_wide_enable")) { set_q4k_wide_enable(value); return 0; }
+    if (!strcmp(key, "q4k_wide_min_batch")) { set_q4k_wide_min_batch(value); return 0; }
     if (!strcmp(key, "q4k_mfma_waves8")) { set_q4k_mfma_waves8(value); return 0; }
     if (!strcmp(key, "q4k_mfma_teams")) { set_q4k_mfma_teams(value); return 0; }
     if (!strcmp(key, "q4k_mfma_window")) { set_q4k_mfma_window(value); return 0; }

@@ -502,8 +502,12 @@ static int launch_quads(hipStream_t s, const uint8_t* w, const float* x, float* 
 }
 
 // Returns 1 when this kernel took the product, 0 when the shape is outside its range, -1 on a launch error.
+int launch_q4k_gemv_wide(const uint8_t* w, const float* x, float* y, int k, int n, int batch);   // gemv_q4k_wide.hip
+
 int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int n, int batch) {
     if (batch < 3 || batch > 8) return 0;
+    // K = 4096: the kernel on the 16 x 16 x 32 matrix instruction
+    if (const int rc = launch_q4k_gemv_wide(w, x, y, k, n, batch)) return rc;
     if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) || (k & 255)) return 0;
     hipStream_t s = current_stream();
     // K = 4096 and offsets that fit 32 bits: the kernel that streams the weight through an LDS ring

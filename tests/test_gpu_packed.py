@@ -292,19 +292,51 @@ def test_q4k_three_to_eight_rows_streamed_through_lds_at_k_4096(hip_backend, tor
     packed = gaussian_weight(hip_backend, "Q4_K", n, k, 91) if n <= 11008 else random_valid_blocks("Q4_K", n * k // 256, 92)
     x = np.random.default_rng(93 + m + n).standard_normal((m, k)).astype(np.float32)
     x[m - 1, 7] = 33.0
-    got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
-    assert hip_backend.last_kernel() == "q4k_gemv_quads_stream_kernel"
-    assert got.shape == (m, n) and not np.isnan(got).any()
-    rows = np.unique(np.concatenate([np.arange(min(n, 40)), np.arange(max(0, n - 40), n)]))
-    want = L.gemv("Q4_K", x, packed.reshape(n, -1)[rows].reshape(-1), len(rows))
-    assert normalized_err(got[:, rows], want) <= GEMV_TOL
     try:
+        hip_backend.set_tuning("q4k_wide_enable", 0)
+        got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemv_quads_stream_kernel"
+        assert got.shape == (m, n) and not np.isnan(got).any()
+        rows = np.unique(np.concatenate([np.arange(min(n, 40)), np.arange(max(0, n - 40), n)]))
+        want = L.gemv("Q4_K", x, packed.reshape(n, -1)[rows].reshape(-1), len(rows))
+        assert normalized_err(got[:, rows], want) <= GEMV_TOL
         hip_backend.set_tuning("q4k_quads_stream_enable", 0)
         fed = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
         assert hip_backend.last_kernel() == "q4k_gemv_quads_kernel"
     finally:
         hip_backend.set_tuning("q4k_quads_stream_enable", 1)
+        hip_backend.set_tuning("q4k_wide_enable", 1)
     assert normalized_err(got, fed) <= 2e-5
+
+
+@pytest.mark.parametrize("n,m", [(1, 3), (4, 3), (5, 4), (16, 8), (17, 5), (37, 5), (130, 8), (1027, 7), (4096, 6), (11008, 3), (11008, 4),
+                                 (11008, 8), (28672, 5), (40000, 8)])
+def test_q4k_three_to_eight_rows_on_the_16x16x32_matrix_instruction(hip_backend, torch_cuda, n, m):
+    """K = 4096: the batched kernel on v_mfma_f32_16x16x32_bf16 (16 weight rows x one sub-block x 8 batch rows' hi and lo
+    parts per instruction, eight K slices per workgroup), on row counts that leave ragged units of 16 rows, workgroups
+    with one to eight units (fewer than the three requested up front, and more: the ring is refilled) and more than one
+    round of workgroups; against the oracle on the first and last rows, and against the 4x4x4 kernel of the same
+    arithmetic over the whole product (another order of the fp32 sums)."""
+    k = 4096
+    packed = gaussian_weight(hip_backend, "Q4_K", n, k, 91) if n <= 11008 else random_valid_blocks("Q4_K", n * k // 256, 92)
+    x = np.random.default_rng(93 + m + n).standard_normal((m, k)).astype(np.float32)
+    x[m - 1, 7] = 33.0
+    x[1, 512:576] = 0.0
+    try:
+        hip_backend.set_tuning("q4k_wide_min_batch", 3)      # by itself the launcher takes this kernel from 5 rows on
+        got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemv_wide_kernel"
+        assert got.shape == (m, n) and not np.isnan(got).any()
+        rows = np.unique(np.concatenate([np.arange(min(n, 40)), np.arange(max(0, n - 40), n)]))
+        want = L.gemv("Q4_K", x, packed.reshape(n, -1)[rows].reshape(-1), len(rows))
+        assert normalized_err(got[:, rows], want) <= GEMV_TOL
+        hip_backend.set_tuning("q4k_wide_enable", 0)
+        quads = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() in ("q4k_gemv_quads_stream_kernel", "q4k_gemv_quads_kernel")
+    finally:
+        hip_backend.set_tuning("q4k_wide_enable", 1)
+        hip_backend.set_tuning("q4k_wide_min_batch", 5)
+    assert normalized_err(got, quads) <= 3e-4      # two orders of fp32 sums, seen through this metric's floor of 1 % of the largest output
 
 
 def test_gemv_is_linear_and_deterministic_at_full_size(hip_backend, torch_cuda):
