@@ -18,7 +18,7 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(PKG, "build")
-HIP_SOURCES = ["shim.hip", "dequant.hip", "gemv.hip", "gemv_stream.hip", "gemv_q4k.hip", "gemv_q4k_mfma.hip", "gemv_q4k_quads.hip", "gemv_q4k_wide.hip", "gemm.hip", "gemm_q4k_ksw.hip", "gemm_q4k_frag.hip", "rows.hip", "sdpa.hip", "sdpa_decode.hip", "sdpa_prefill.hip", "dense.hip", "elementwise.hip"]
+HIP_SOURCES = ["shim.hip", "dequant.hip", "gemv.hip", "gemv_stream.hip", "gemv_q8_0_mfma.hip", "gemv_q4k.hip", "gemv_q4k_mfma.hip", "gemv_q4k_quads.hip", "gemv_q4k_wide.hip", "gemm.hip", "gemm_q4k_ksw.hip", "gemm_q4k_frag.hip", "rows.hip", "sdpa.hip", "sdpa_decode.hip", "sdpa_prefill.hip", "dense.hip", "elementwise.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
     # packed FP32 VALU ops are kept out of generated code on this target

@@ -187,6 +187,8 @@ int launch_q4k_gemv_rows(const uint8_t* w, const float* x, float* y, int k, int 
 int launch_q4k_gemv_quads(const uint8_t* w, const float* x, float* y, int k, int n, int batch);  // gemv_q4k_quads.hip
 int launch_gemv_stream(int enc, const uint8_t* w, const float* x, float* y, int k, int n);        // gemv_stream.hip
 void set_gemv_stream_enable(int v);
+int launch_q8_0_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n);                  // gemv_q8_0_mfma.hip
+void set_q8_0_mfma_enable(int v);
 void set_dense_mfma(int v);
 
 // Experiment knobs (defaults are the measured best): returns 0 when the key is known.
@@ -195,6 +197,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q4k_rows_waves_per_cu")) { set_q4k_rows_waves_per_cu(value); return 0; }
     if (!strcmp(key, "q6k_slot64")) { g_q6k_slot64 = value != 0; return 0; }
     if (!strcmp(key, "gemv_stream_enable")) { set_gemv_stream_enable(value); return 0; }
+    if (!strcmp(key, "q8_0_mfma_enable")) { set_q8_0_mfma_enable(value); return 0; }
     if (!strcmp(key, "dense_mfma")) { set_dense_mfma(value); return 0; }
     if (!strcmp(key, "gemm_wide")) { set_gemm_wide(value); return 0; }
     if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }
@@ -240,6 +243,12 @@ int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, 
             rc = left >= 3 ? launch_q4k_gemv_quads(w, xb, yb, k, n, nq) : launch_q4k_gemv_rows(w, xb, yb, k, n, left);
             if (rc < 0) return rc;
             if (rc == 1) { b0 += left >= 3 ? nq : left; continue; }
+        }
+        if (left == 1 && enc == ENC_Q8_0) {
+            // one row of Q8_0, K a multiple of 1024 up to 4096: the codes straight onto the integer matrix cores
+            rc = launch_q8_0_gemv_mfma(w, xb, yb, k, n);
+            if (rc < 0) return rc;
+            if (rc == 1) { b0 += 1; continue; }
         }
         if (left == 1 && enc != ENC_Q4_K) {
             // one row: the weight streamed through LDS in consecutive kilobytes, where the row shape allows it

@@ -248,17 +248,74 @@ def test_one_row_products_streamed_through_lds(hip_backend, torch_cuda, enc, n, 
     x = np.random.default_rng(63 + k).standard_normal((1, k)).astype(np.float32)
     x[0, 5] = -41.0
     want = L.gemv(enc, x, packed, n)
-    got = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x)
-    assert hip_backend.last_kernel() == ("gemv_stream_kernel" if eligible else "gemv_kernel")
-    assert not np.isnan(got).any()
-    assert normalized_err(got, want) <= GEMV_TOL
     try:
+        hip_backend.set_tuning("q8_0_mfma_enable", 0)       # (Q8_0 rows of 1024 to 4096 elements would take the matrix-core kernel)
+        got = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x)
+        assert hip_backend.last_kernel() == ("gemv_stream_kernel" if eligible else "gemv_kernel")
+        assert not np.isnan(got).any()
+        assert normalized_err(got, want) <= GEMV_TOL
         hip_backend.set_tuning("gemv_stream_enable", 0)
         rows = gpu_matmul(hip_backend, torch_cuda, enc, packed, n, k, x)
         assert hip_backend.last_kernel() == "gemv_kernel"
     finally:
         hip_backend.set_tuning("gemv_stream_enable", 1)
+        hip_backend.set_tuning("q8_0_mfma_enable", 1)
     assert normalized_err(got, rows) <= 2e-5
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (1000, 4096), (1027, 2048), (5000, 1024), (3, 4096), (1, 1024), (17, 3072),
+                                 (40000, 1024)])
+def test_q8_0_one_row_on_the_integer_matrix_cores(hip_backend, torch_cuda, n, k):
+    """One activation row against Q8_0, K a multiple of 1024 up to 4096: the int8 codes go onto v_mfma_i32_4x4x4_16b_i8 as
+    they lie, the activations as 22-bit fixed point per 64-element group. Against the exact-fp32 oracle (1e-3) and the
+    fp32 streaming kernel; shapes with one to four K slices, fewer quads than the four requested up front, ragged
+    quads, ring refills (more than four quads per workgroup) and more than one round of workgroups. Codes at the
+    extremes against a constant activation vector: the digit sums are at their largest."""
+    packed = gaussian_weight(hip_backend, "Q8_0", n, k, 61) if n * k >= 1 << 22 else random_valid_blocks("Q8_0", n * k // 32, 62 + n)
+    x = np.random.default_rng(63 + k).standard_normal((1, k)).astype(np.float32)
+    x[0, 5] = -41.0
+    want = L.gemv("Q8_0", x, packed, n)
+    got = gpu_matmul(hip_backend, torch_cuda, "Q8_0", packed, n, k, x)
+    assert hip_backend.last_kernel() == "q8_0_gemv_mfma_kernel"
+    assert not np.isnan(got).any()
+    err = normalized_err(got, want)
+    print(f"Q8_0 {n}x{k} on the matrix cores: {err:.2e}")
+    assert err <= GEMV_TOL
+    try:
+        hip_backend.set_tuning("q8_0_mfma_enable", 0)
+        fp32 = gpu_matmul(hip_backend, torch_cuda, "Q8_0", packed, n, k, x)
+        assert hip_backend.last_kernel() == "gemv_stream_kernel"
+    finally:
+        hip_backend.set_tuning("q8_0_mfma_enable", 1)
+    assert normalized_err(got, fp32) <= 1e-4
+    if n <= 1027:
+        # saturated codes (+127 / -127 rows) against constant activations: every digit sum at its extreme
+        blocks = np.frombuffer(packed, np.uint8).reshape(n, k // 32, 34).copy()
+        blocks[0::2, :, 2:] = 127
+        blocks[1::2, :, 2:] = 129                                   # -127
+        sat = blocks.reshape(-1)
+        for xc in (np.full((1, k), 3.25, np.float32), np.full((1, k), -1e-3, np.float32)):
+            got = gpu_matmul(hip_backend, torch_cuda, "Q8_0", sat, n, k, xc)
+            assert normalized_err(got, L.gemv("Q8_0", xc, sat, n)) <= GEMV_TOL
+
+
+def test_q8_0_matrix_core_kernel_keeps_non_finite_activations_loud(hip_backend, torch_cuda):
+    """The exact-fp32 product propagates a NaN or an infinity among the activations into every output; the fixed-point
+    kernel must not turn it into a finite number: the group's scale becomes NaN. A group of subnormal activations
+    contributes (next to) nothing, as in fp32."""
+    n, k = 64, 2048
+    packed = random_valid_blocks("Q8_0", n * k // 32, 7)
+    rng = np.random.default_rng(8)
+    for bad in (np.nan, np.inf, -np.inf):
+        x = rng.standard_normal((1, k)).astype(np.float32)
+        x[0, 700] = bad
+        got = gpu_matmul(hip_backend, torch_cuda, "Q8_0", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q8_0_gemv_mfma_kernel"
+        assert not np.isfinite(got).any(), bad
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    x[0, 128:192] = np.float32(1e-41) * rng.standard_normal(64).astype(np.float32)      # one group of subnormals
+    got = gpu_matmul(hip_backend, torch_cuda, "Q8_0", packed, n, k, x)
+    assert np.isfinite(got).all() and normalized_err(got, L.gemv("Q8_0", x, packed, n)) <= GEMV_TOL
 
 
 @pytest.mark.parametrize("n,k,m", [(5, 256, 3), (25, 1280, 8), (77, 2304, 7), (1000, 11008, 4), (11008, 4096, 6), (4096, 14336, 8),
