@@ -189,6 +189,7 @@ int launch_gemv_stream(int enc, const uint8_t* w, const float* x, float* y, int 
 void set_gemv_stream_enable(int v);
 int launch_q8_0_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n);                  // gemv_q8_0_mfma.hip
 void set_q8_0_mfma_enable(int v);
+void set_q8_0_mfma_per_cu(int v);
 void set_dense_mfma(int v);
 
 // Experiment knobs (defaults are the measured best): returns 0 when the key is known.
@@ -198,6 +199,7 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "q6k_slot64")) { g_q6k_slot64 = value != 0; return 0; }
     if (!strcmp(key, "gemv_stream_enable")) { set_gemv_stream_enable(value); return 0; }
     if (!strcmp(key, "q8_0_mfma_enable")) { set_q8_0_mfma_enable(value); return 0; }
+    if (!strcmp(key, "q8_0_mfma_per_cu")) { set_q8_0_mfma_per_cu(value); return 0; }
     if (!strcmp(key, "dense_mfma")) { set_dense_mfma(value); return 0; }
     if (!strcmp(key, "gemm_wide")) { set_gemm_wide(value); return 0; }
     if (!strcmp(key, "q4k_rows_enable")) { g_q4k_rows_enable = value; return 0; }

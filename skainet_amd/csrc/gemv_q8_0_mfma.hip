@@ -48,7 +48,7 @@ __host__ __device__ constexpr uint32_t q8m_ring_bytes(int window) { return (uint
 
 // W: quads in flight per wave (the ring has W slots: a slot is refilled once its quad is used up)
 template <int W>
-__global__ __launch_bounds__(256, 1) void q8_0_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+__global__ __launch_bounds__(256, W == 1 ? 4 : W == 2 ? 2 : 1) void q8_0_gemv_mfma_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                                 float* __restrict__ y, int k, int n, int qt) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q8m_smem[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -183,25 +183,34 @@ __global__ __launch_bounds__(256, 1) void q8_0_gemv_mfma_kernel(const uint8_t* _
 
 static std::atomic<int> g_q8_0_mfma_enable{1};
 void set_q8_0_mfma_enable(int v) { g_q8_0_mfma_enable = v != 0; }
+static std::atomic<int> g_q8_0_mfma_per_cu{2};      // workgroups per CU the grid is cut for (4096 x 4096, us per product: 1: 5.33, 2: 4.96, 3: 4.91 with one quad in flight, 4: 5.51)
+void set_q8_0_mfma_per_cu(int v) { if (v >= 1 && v <= 4) g_q8_0_mfma_per_cu = v; }
 
-// Returns 1 when this kernel took the product, 0 when the shape is outside its range, -1 on a launch error. One
-// activation row; K a multiple of 1024 up to 4096; the weight below 4 GiB; operands 16-byte aligned.
-int launch_q8_0_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n) {
-    constexpr int W = 4;
-    if (!g_q8_0_mfma_enable.load() || k < 1024 || (k & 1023) || k > 4096 || n < 1) return 0;
-    if ((uint64_t)(n + 4) * (uint64_t)(k >> 5) * Q80_BYTES >= ((uint64_t)1 << 32)) return 0;
-    if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return 0;
-    const int quads = (n + 3) / 4;
-    int qt = (quads + num_cus() - 1) / num_cus();
-    if (qt > Q8M_MAX_QUADS) qt = Q8M_MAX_QUADS;
-    const int grid = (quads + qt - 1) / qt;
+template <int W>
+static int launch_q8m(int grid, int qt, hipStream_t s, const uint8_t* w, const float* x, float* y, int k, int n) {
     const size_t smem = (size_t)4 * q8m_ring_bytes(W) + (size_t)4 * qt * 64 * sizeof(float);
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q8_0_gemv_mfma_kernel<W>), 160 * 1024);
     if (smem > 160 * 1024) return 0;
     note_kernel("q8_0_gemv_mfma_kernel");
-    q8_0_gemv_mfma_kernel<W><<<dim3(grid), dim3(256), smem, current_stream()>>>(w, x, y, k, n, qt);
+    q8_0_gemv_mfma_kernel<W><<<dim3(grid), dim3(256), smem, s>>>(w, x, y, k, n, qt);
     SKH_CHECK(hipGetLastError());
     return 1;
+}
+
+// Returns 1 when this kernel took the product, 0 when the shape is outside its range, -1 on a launch error. One
+// activation row; K a multiple of 1024 up to 4096; the weight below 4 GiB; operands 16-byte aligned.
+int launch_q8_0_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n) {
+    if (!g_q8_0_mfma_enable.load() || k < 1024 || (k & 1023) || k > 4096 || n < 1) return 0;
+    if ((uint64_t)(n + 4) * (uint64_t)(k >> 5) * Q80_BYTES >= ((uint64_t)1 << 32)) return 0;
+    if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return 0;
+    const int quads = (n + 3) / 4;
+    const int per_cu = g_q8_0_mfma_per_cu.load();
+    int qt = (quads + per_cu * num_cus() - 1) / (per_cu * num_cus());
+    if (qt > Q8M_MAX_QUADS) qt = Q8M_MAX_QUADS;
+    const int grid = (quads + qt - 1) / qt;
+    if (per_cu >= 3 && qt <= 4) return launch_q8m<1>(grid, qt, current_stream(), w, x, y, k, n);
+    if (per_cu == 2 && qt <= 8) return launch_q8m<2>(grid, qt, current_stream(), w, x, y, k, n);
+    return launch_q8m<4>(grid, qt, current_stream(), w, x, y, k, n);
 }
 
 }  // namespace skh
