@@ -70,6 +70,12 @@ SKAINET_HIP_API int32_t skainet_hip_compute_units(void);
 SKAINET_HIP_API const char* skainet_hip_last_kernel(void);
 /* Stream (a hipStream_t, NULL = the null stream) used by this thread's later device entries. */
 SKAINET_HIP_API int32_t skainet_hip_set_stream(void* stream);
+/* Give the calling thread a non-blocking stream of its own (made on first use, destroyed by
+ * skainet_hip_thread_release) and use it for this thread's later device entries. The null stream, the default, orders
+ * every thread's work behind every other's: a host that calls in from several threads (the reference's schedule
+ * workers) calls this once per thread. The caller then orders its own work on other streams against this thread's with
+ * skainet_hip_sync. No reference counterpart. 0 on success. */
+SKAINET_HIP_API int32_t skainet_hip_thread_stream(void);
 /* Wait for this thread's stream. */
 SKAINET_HIP_API int32_t skainet_hip_sync(void);
 /* Frees the calling thread's scratch (workspace, staging buffers of the host-pointer entries, counters, timer events)
@@ -120,8 +126,19 @@ SKAINET_HIP_API int64_t skainet_hip_weight_nbytes(const skainet_hip_weight* w);
 /* out[m, rows] = x[m, cols] . W^T, fp32 in and out, device pointers. What a ViewKernel registered for
  * matmul(F32 dense x packed BLOCKED_ROW_MAJOR) runs (API/MatmulKernels.kt:11-40; CPU twin
  * REF/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/FfmRowMajorKernels.kt:52-106).
- * m <= 8 streams the weight once per 4 rows (GEMV kernels, fp32 arithmetic, within 1e-3 of the exact fp32 product);
- * larger m uses the MFMA dequant-GEMM, which rounds activations and decoded weights to bf16 and accumulates in fp32
+ * m <= 8 streams the weight once per 4 (Q4_K: 8) rows, within 1e-3 of the exact fp32 product; the arithmetic class
+ * depends on format and m:
+ *   - Q4_K, m = 1, K a multiple of 1024 up to 16384, and Q8_0, m = 1, K a multiple of 1024 up to 4096: codes stay
+ *     integers, the activations are rounded to 22-bit fixed point against the largest magnitude of their 64-element
+ *     group and contracted on the int8 matrix instruction; scales and minima are applied in fp32 (measured 4e-5 / 2e-5
+ *     in the GEMV parity metric). A NaN or an infinity among the activations makes every output NaN.
+ *   - Q4_K, m = 3 .. 8: codes exact, an activation enters as bf16 hi + bf16 lo (16 to 17 significant bits) on the bf16
+ *     matrix instructions, fp32 sums (2e-4 in the metric).
+ *   - everything else (Q4_K m = 2 or other K, Q6_K, Q5_K, Q4_0, Q5_0, Q5_1, Q8_0 at other K): fp32 multiply-adds on
+ *     decoded codes, the reference's exact-fp32 products in another summation order.
+ *   skainet_hip_set_tuning("q4k_mfma_enable", 0) / ("q8_0_mfma_enable", 0) force the fp32 kernels at m = 1,
+ *   ("q4k_wide_enable", 0) + ("q4k_quads_stream_enable", 0) + ("q4k_rows_enable", 0) the fp32 slot kernel at every m.
+ * Larger m uses the MFMA dequant-GEMM, which rounds activations and decoded weights to bf16 and accumulates in fp32
  * (within 2e-2 of the largest output): the switch at m = 9 is a switch of precision class as well as of kernel, and
  * skainet_hip_matmul_kind_dev pins either one. */
 SKAINET_HIP_API int32_t skainet_hip_matmul_dev(const skainet_hip_weight* w, const float* x, int32_t m, float* out);
@@ -312,11 +329,15 @@ SKAINET_HIP_API int32_t skainet_hip_f32_reduce_axis_dev(const float* in, int32_t
 SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
 /* skainet_hip_f32_argmax_rows_dev for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid it). No counterpart in the reference. Same result (first maximum of each row);
- * the partial pairs and arrival counters live in a fixed 33 KiB array inside the library's code object instead of scratch
- * the library allocates, so the call makes no allocation of any kind. At most 64 rows per call (more is refused with
- * -1 and a message; cols is unbounded). Every call on a GPU shares that GPU's array: calls that overlap on one GPU
- * (two streams, two threads) race, calls on one stream are safe. */
+ * the partial pairs and arrival counters live in a fixed array inside the library's code object (8 slots of 33 KiB, 264
+ * KiB per GPU) instead of scratch the library allocates, so the call makes no allocation of any kind. At most 64 rows
+ * per call (more is refused with -1 and a message; cols is unbounded). A host thread is handed one slot on its first
+ * call and keeps it until the process ends (the library's streams are per host thread, so threads do not share
+ * counters); the ninth thread is refused with -1 and a message. Calls of ONE thread share its slot: issued on one stream
+ * they are safe, overlapping on two streams they race. */
 SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_noalloc_dev(const float* in, int32_t rows, int32_t cols, int32_t* out);
+/* The calling thread's slot of that array (handed out on first use), -1 when all are taken. Makes no device call. */
+SKAINET_HIP_API int32_t skainet_hip_f32_argmax_rows_noalloc_slot(void);
 
 /* Decoder glue the reference keeps in its external transformer repository (no counterpart in /root/reference; the
  * semantics are the standard Llama ones and are checked against closed forms):
@@ -357,7 +378,8 @@ SKAINET_HIP_API int32_t skainet_hip_i32_store_at_dev(int32_t* dst, const int32_t
  * allocates (a first call that grows the library's scratch) may run between begin and end: such a call fails with a
  * message instead of freeing memory under the capture, so run the sequence once eagerly first. A graph is tied to the
  * scratch addresses of its recording: when a later call on the thread makes the library reallocate scratch, the graph
- * is refused from then on (graph_valid / graph_launch). Only kernel launches are recorded. */
+ * is refused from then on (graph_valid / graph_launch). It is also tied to the thread that recorded it (scratch is per
+ * thread): graph_valid is 0 and graph_launch fails on any other thread. Only kernel launches are recorded. */
 typedef struct skainet_hip_graph skainet_hip_graph;
 SKAINET_HIP_API int32_t skainet_hip_graph_begin(void);
 SKAINET_HIP_API skainet_hip_graph* skainet_hip_graph_end(void);

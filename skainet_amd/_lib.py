@@ -27,6 +27,7 @@ SIGNATURES = {
     "skainet_hip_compute_units": (_i32, []),
     "skainet_hip_last_kernel": (C.c_char_p, []),
     "skainet_hip_set_stream": (_i32, [_vp]),
+    "skainet_hip_thread_stream": (_i32, []),
     "skainet_hip_sync": (_i32, []),
     "skainet_hip_thread_release": (_i32, []),
     "skainet_hip_malloc": (_vp, [_sz]),
@@ -92,6 +93,7 @@ SIGNATURES = {
     "skainet_hip_f32_add_dev": (_i32, [_vp, _vp, _vp, _i64]),
     "skainet_hip_f32_argmax_rows_dev": (_i32, [_vp, _i32, _i32, _vp]),
     "skainet_hip_f32_argmax_rows_noalloc_dev": (_i32, [_vp, _i32, _i32, _vp]),
+    "skainet_hip_f32_argmax_rows_noalloc_slot": (_i32, []),
     "skainet_hip_f32_rope_scatter_dev": (_i32, [_vp, _i64, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _i32, _i64, _i32]),
     "skainet_hip_decode_advance_dev": (_i32, [_vp, _vp, _vp, _vp, _i32]),
     "skainet_hip_i32_store_at_dev": (_i32, [_vp, _vp, _i32, _vp]),

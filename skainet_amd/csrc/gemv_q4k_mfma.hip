@@ -274,9 +274,12 @@ __device__ __forceinline__ void q4k_mfma_wave(const uint8_t* __restrict__ w, con
                 dl = __builtin_amdgcn_mfma_i32_4x4x4i8(xa[t][u], wlo, dl, 0, 0, 0);
                 dh = __builtin_amdgcn_mfma_i32_4x4x4i8(xa[t][8 + u], whi, dh, 0, 0, 0);
             }
-            // digits back together: ((top * 256 + mid) * 256 + low) - 64 * 65536 * (code sum)
-            const int tl = __mul24(dl[3], -4194304) + (((dl[2] << 8) + dl[1]) << 8) + dl[0];
-            const int th = __mul24(dh[3], -4194304) + (((dh[2] << 8) + dh[1]) << 8) + dh[0];
+            // digits back together: ((top * 256 + mid) * 256 + low) - 64 * 65536 * (code sum). The top term alone can pass
+            // 2^31 (top digit + 64 up to 96, codes up to 15, 32 of them) before the code sum takes the + 64 out again:
+            // the sum is formed modulo 2^32 on unsigned values (the true result fits 32 bits) and read as signed at the end.
+            const uint32_t ul = (uint32_t)dl[3] * 0xFFC00000u + ((((uint32_t)dl[2] << 8) + (uint32_t)dl[1]) << 8) + (uint32_t)dl[0];
+            const uint32_t uh = (uint32_t)dh[3] * 0xFFC00000u + ((((uint32_t)dh[2] << 8) + (uint32_t)dh[1]) << 8) + (uint32_t)dh[0];
+            const int tl = (int)ul, th = (int)uh;
             total = fmaf(s_grp[t], fmaf(dlo, (float)tl, fmaf(dhi, (float)th, -fmaf(mlo, xsl[t], mhi * xsh[t]))), total);
         }
         partials[(team + T * q) * 64 + widx] = total;
@@ -411,6 +414,19 @@ __global__ __launch_bounds__(64 * NW * T, (PRO == 2 || NW * T == 8) ? 1 : 2) voi
 
 static std::atomic<int> g_q4k_mfma_enable{1};
 void set_q4k_mfma_enable(int v) { g_q4k_mfma_enable = v; }
+static size_t mfma_smem_bytes(int k, int qt, int window, int nw, int teams);
+// Would launch_q4k_gemv_mfma take a product whose activations are the unmerged results of a one-query attention
+// (n outputs, k = heads * head_dim)? Every reason it can refuse that form, without launching anything: a caller that
+// leaves attention splits unmerged for it has no way back once the attention kernel has run.
+bool q4k_gemv_mfma_accepts_merge(int k, int n, int head_dim) {
+    if (!g_q4k_mfma_enable || k < 1024 || (k & 1023) || k > 4096 || n < 4) return false;
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return false;
+    if ((uint64_t)n * (uint64_t)(k >> 8) * Q4K_BYTES >= ((uint64_t)1 << 32)) return false;
+    const int quads = (n + 3) / 4;
+    int qt = (quads + num_cus() - 1) / num_cus();
+    if (qt > MFMA_MAX_QUADS) qt = MFMA_MAX_QUADS;
+    return mfma_smem_bytes(k, qt < 1 ? 1 : qt, 3, 4, 1) <= 160 * 1024;
+}
 static std::atomic<int> g_q4k_mfma_teams{0};       // 0: chosen from the quads a workgroup owns
 void set_q4k_mfma_teams(int v) { if (v >= 0 && v <= 2) g_q4k_mfma_teams = v; }
 static std::atomic<int> g_q4k_mfma_waves8{1};
@@ -421,7 +437,7 @@ void set_q4k_mfma_window(int v) { if (v == 0 || v == 2 || v == 3) g_q4k_mfma_win
 // quads in flight per wave: three while a quad is at most 5 KB per wave, two for the long rows (9 KB per quad and wave)
 static int mfma_window(int k) { return (((k >> 10) + 3) >> 2) >= 3 ? 2 : 3; }
 
-static size_t mfma_smem_bytes(int k, int qt, int window, int nw, int teams = 1) {
+static size_t mfma_smem_bytes(int k, int qt, int window, int nw, int teams) {
     const int ns_max = ((k >> 10) + nw - 1) / nw;
     const int nli_max = (144 * ns_max + 63) / 64;
     const size_t rings = teams == 1 ? (size_t)nw * mfma_ring_bytes(nli_max, window)
@@ -511,7 +527,7 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
     const int pro = merge ? 2 : gain ? 1 : 0;
     // long rows without a prologue (the decoder's down projection): eight waves, K split eight ways
     if (g_q4k_mfma_waves8 && pro == 0 && k >= 8192 && epilogue <= EPI_RESIDUAL) {
-        const size_t smem8 = mfma_smem_bytes(k, qt, 2, 8);
+        const size_t smem8 = mfma_smem_bytes(k, qt, 2, 8, 1);
         if (smem8 <= 160 * 1024) {
             note_kernel("q4k_gemv_mfma_kernel");
             if (epilogue == EPI_NONE) return launch_mfma_variant<2, 0, EPI_NONE, 8>(grid, smem8, current_stream(), w, x, y, k, n, qt, gain, eps, residual, rope, am);
@@ -542,7 +558,7 @@ int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int 
 #undef SKH_MFMA_T2
         }
     }
-    const size_t smem = mfma_smem_bytes(k, qt, window, 4);
+    const size_t smem = mfma_smem_bytes(k, qt, window, 4, 1);
     if (smem > 160 * 1024) return 0;
     if (window == 2) return launch_mfma<2>(pro, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);
     return launch_mfma<3>(pro, grid, smem, current_stream(), w, x, y, k, n, qt, gain, eps, residual, epilogue, rope, am);

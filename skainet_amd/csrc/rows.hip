@@ -499,7 +499,24 @@ int launch_argmax_rows(const float* in, int rows, int cols, int32_t* out) {
 // object: every GPU the library runs on holds its own copy until the process ends. In host code the array's name is
 // only a handle; the device address comes from hipGetSymbolAddress, once per device, and that address is what the
 // kernels are given.
-static __device__ __align__(256) unsigned char scratch[sizeof(ArgmaxScratch)];
+// Everything else in the library is per host thread (stream, scratch), so the array is cut into NOALLOC_SLOTS slots and
+// a host thread is handed one on its first call (an atomic counter; kept until the process ends): threads that each use
+// their own stream do not share counters. A thread that comes after the slots have run out is refused with a message.
+constexpr int NOALLOC_SLOTS = 8;
+constexpr size_t NOALLOC_SLOT_BYTES = (sizeof(ArgmaxScratch) + 255) & ~(size_t)255;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SLOTS * NOALLOC_SLOT_BYTES];
+static std::atomic<int> g_noalloc_next_slot{0};
+static thread_local int t_noalloc_slot = -1;
+// this thread's slot (handed out on first use), -1 when every slot is taken; no device call
+int argmax_noalloc_slot() {
+    if (t_noalloc_slot < 0) {
+        int s = g_noalloc_next_slot.load();
+        while (s < NOALLOC_SLOTS && !g_noalloc_next_slot.compare_exchange_weak(s, s + 1)) {}
+        if (s >= NOALLOC_SLOTS) return -1;
+        t_noalloc_slot = s;
+    }
+    return t_noalloc_slot;
+}
 constexpr int NOALLOC_MAX_DEVICES = 64;
 static void* g_noalloc_scratch[NOALLOC_MAX_DEVICES];    // per device, filled on first use
 static std::mutex g_noalloc_mutex;
@@ -509,6 +526,8 @@ __global__ void argmax_clear_kernel(ArgmaxScratch* __restrict__ sc, int rows) {
 }
 
 static ArgmaxScratch* noalloc_scratch() {
+    const int slot = argmax_noalloc_slot();
+    if (slot < 0) { set_error("argmax_rows_noalloc: all %d scratch slots are held by other host threads; use skainet_hip_f32_argmax_rows_dev", NOALLOC_SLOTS); return nullptr; }
     int dev = -1;
     if (check_hip(hipGetDevice(&dev), "hipGetDevice") != 0) return nullptr;
     if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) { set_error("argmax_rows_noalloc: device ordinal %d is beyond the %d this entry keeps scratch for", dev, NOALLOC_MAX_DEVICES); return nullptr; }
@@ -519,7 +538,7 @@ static ArgmaxScratch* noalloc_scratch() {
         if (!ptr) { set_error("argmax_rows_noalloc: no device address for the scratch array"); return nullptr; }
         g_noalloc_scratch[dev] = ptr;
     }
-    return static_cast<ArgmaxScratch*>(g_noalloc_scratch[dev]);
+    return reinterpret_cast<ArgmaxScratch*>(static_cast<unsigned char*>(g_noalloc_scratch[dev]) + (size_t)slot * NOALLOC_SLOT_BYTES);
 }
 
 int launch_argmax_rows_noalloc(const float* in, int rows, int cols, int32_t* out) {
@@ -545,6 +564,8 @@ int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int
 }
 
 }  // namespace skh
+
+extern "C" int32_t skainet_hip_f32_argmax_rows_noalloc_slot(void) { return skh::argmax_noalloc_slot(); }
 
 extern "C" int32_t skainet_hip_f32_argmax_rows_noalloc_dev(const float* in, int32_t rows, int32_t cols, int32_t* out) {
     if (skh::ensure_device() != 0) return -1;

@@ -375,6 +375,7 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
 int launch_q4k_gemv_mfma(const uint8_t* w, const float* x, float* y, int k, int n, const float* gain, float eps,
                          const float* residual, int epilogue, const RopeQkvEpilogue* rope_in,
                          const AttnMergePrologue* merge);   // gemv_q4k_mfma.hip
+bool q4k_gemv_mfma_accepts_merge(int k, int n, int head_dim);   // gemv_q4k_mfma.hip
 
 static std::atomic<int> g_attn_merge_enable{1};
 void set_attn_merge_enable(int v) { g_attn_merge_enable = v; }
@@ -389,7 +390,7 @@ int launch_attn_out_proj_q4k(const uint8_t* wo, int n, int k, const float* q, co
     if (!g_attn_merge_enable || k != heads * head_dim || k > 4096 || (k & 1023)) return 0;
     if (heads % kv_heads != 0 || seq_kv < 1 || kv_capacity < seq_kv) return 0;
     // dry checks of the projection first: once the attention kernel has run without a merge there is no way back
-    if ((reinterpret_cast<uintptr_t>(wo) & 15) || n < 4 || (uint64_t)n * (uint64_t)(k >> 8) * 144u >= ((uint64_t)1 << 32)) return 0;
+    if ((reinterpret_cast<uintptr_t>(wo) & 15) || !q4k_gemv_mfma_accepts_merge(k, n, head_dim)) return 0;
     if (residual && (reinterpret_cast<uintptr_t>(residual) & 3)) return 0;
     AttnMergePrologue am{};
     const int r = launch_sdpa_decode(q, k_cache, v_cache, nullptr, 1, heads, kv_heads, seq_kv, kv_capacity, head_dim, scale, window, 0,

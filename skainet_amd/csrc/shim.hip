@@ -173,6 +173,10 @@ static thread_local void* t_sync = nullptr;
 void* sync_scratch(size_t bytes) {
     if (bytes > SYNC_SCRATCH_BYTES) { set_error("sync scratch request of %zu bytes exceeds %zu", bytes, SYNC_SCRATCH_BYTES); return nullptr; }
     if (!t_sync) {
+        if (t_capture_stream) {
+            set_error("the cross-workgroup counters would be allocated while a graph capture is open: run the sequence once outside the capture first");
+            return nullptr;
+        }
         void* p = nullptr;
         if (check_hip(hipMalloc(&p, SYNC_SCRATCH_BYTES), "hipMalloc(sync scratch)") != 0) return nullptr;
         if (check_hip(hipMemset(p, 0, SYNC_SCRATCH_BYTES), "hipMemset(sync scratch)") != 0) { (void)hipFree(p); return nullptr; }
@@ -304,6 +308,16 @@ const char* skainet_hip_device_name(void) { return g_name; }
 int32_t skainet_hip_compute_units(void) { return g_cus; }
 const char* skainet_hip_last_kernel(void) { return t_last_kernel; }
 int32_t skainet_hip_set_stream(void* stream) { t_stream = static_cast<hipStream_t>(stream); return 0; }
+// A non-blocking stream of the calling thread's own, made on first use and kept until skainet_hip_thread_release: with
+// it the thread's device entries no longer queue behind every other thread's on the null stream.
+static thread_local hipStream_t t_own_stream = nullptr;
+int32_t skainet_hip_thread_stream(void) {
+    if (ensure_device() != 0) return -1;
+    if (t_capture_stream) return set_error("thread_stream: a graph capture is open on this thread");
+    if (!t_own_stream && check_hip(hipStreamCreateWithFlags(&t_own_stream, hipStreamNonBlocking), "hipStreamCreate") != 0) return -1;
+    t_stream = t_own_stream;
+    return 0;
+}
 int32_t skainet_hip_sync(void) {
     if (ensure_device() != 0) return -1;
     return check_hip(hipStreamSynchronize(t_stream), "hipStreamSynchronize");
@@ -322,6 +336,11 @@ int32_t skainet_hip_thread_release(void) {
         if (sc.ptr && check_hip(hipFree(sc.ptr), "hipFree(scratch)") != 0) rc = -1;
         sc.ptr = nullptr; sc.cap = 0;
     };
+    if (t_own_stream) {
+        if (t_stream == t_own_stream) t_stream = nullptr;
+        if (check_hip(hipStreamDestroy(t_own_stream), "hipStreamDestroy") != 0) rc = -1;
+        t_own_stream = nullptr;
+    }
     ++t_scratch_generation;                       // graphs recorded on this thread are stale from here on
     drop(t_workspace);
     for (Scratch& sc : t_stage) drop(sc);
@@ -598,7 +617,14 @@ float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, in
             // between its two events.
             hipEvent_t ev[65] = {};
             for (int r = 0; ok && r <= replays; ++r) ok = check_hip(hipEventCreate(&ev[r]), "hipEventCreate") == 0;
+            // every scratch buffer the products need is sized before the capture opens (one eager product per distinct
+            // weight shape is enough: the first weight stands for all, they share a shape in every caller); inside the
+            // capture a call that would still grow scratch fails instead of freeing memory under it
+            ok = ok && skainet_hip_matmul_kind_dev(weights[0], x, m, out, kind) == 0;
+            ok = ok && check_hip(hipStreamSynchronize(cap), "hipStreamSynchronize") == 0;
             ok = ok && check_hip(hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture") == 0;
+            hipStream_t outer_capture = t_capture_stream;
+            if (ok) t_capture_stream = cap;
             int step = 0;
             for (int i = 0; ok && i < 400; ++i, ++step) ok = skainet_hip_matmul_kind_dev(weights[step % nweights], x, m, out, kind) == 0;
             bool inner = ok && hipEventRecord(ev[0], cap) == hipSuccess;
@@ -607,6 +633,7 @@ float skainet_hip_matmul_repeat_dev(const skainet_hip_weight* const* weights, in
                 if (inner && hipEventRecord(ev[r + 1], cap) != hipSuccess) inner = false;
             }
             if (!inner) (void)hipGetLastError();
+            t_capture_stream = outer_capture;
             hipError_t e = hipStreamEndCapture(cap, &graph);
             ok = ok && check_hip(e, "hipStreamEndCapture") == 0;
             ok = ok && check_hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate") == 0;
@@ -796,7 +823,10 @@ int32_t skainet_hip_i32_increment_dev(int32_t* value, int32_t delta) {
 }
 
 // ---- HIP graphs: record this thread's device entries once, replay them with one launch ----
-struct skainet_hip_graph { hipGraph_t graph; hipGraphExec_t exec; uint64_t scratch_generation; };
+// A graph belongs to the thread that recorded it: the scratch addresses in it are that thread's, and so is the
+// generation counter they are checked against (`owner` points at the recording thread's counter; another thread's
+// launch is refused).
+struct skainet_hip_graph { hipGraph_t graph; hipGraphExec_t exec; uint64_t scratch_generation; const uint64_t* owner; };
 static thread_local hipStream_t t_capture_prev = nullptr;
 
 int32_t skainet_hip_graph_begin(void) {
@@ -827,13 +857,15 @@ skainet_hip_graph* skainet_hip_graph_end(void) {
         return nullptr;
     }
     (void)hipStreamDestroy(cap);   // replays run on the calling thread's stream, in order with its eager work
-    return new skainet_hip_graph{graph, exec, t_scratch_generation};
+    return new skainet_hip_graph{graph, exec, t_scratch_generation, &t_scratch_generation};
 }
 int32_t skainet_hip_graph_valid(const skainet_hip_graph* g) {
-    return g && g->scratch_generation == t_scratch_generation ? 1 : 0;
+    return g && g->owner == &t_scratch_generation && g->scratch_generation == t_scratch_generation ? 1 : 0;
 }
 int32_t skainet_hip_graph_launch(skainet_hip_graph* g) {
     if (!g) return set_error("graph_launch: null graph");
+    if (g->owner != &t_scratch_generation)
+        return set_error("graph_launch: refused, a graph is launched by the thread that recorded it (its scratch buffers are that thread's)");
     if (g->scratch_generation != t_scratch_generation)
         return set_error("graph_launch: refused, the library's scratch was reallocated after this graph was recorded "
                          "(generation %llu, now %llu); record it again",

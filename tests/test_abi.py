@@ -141,3 +141,28 @@ def test_kotlin_module_binds_the_header_as_declared():
     for accessor in ("matmulFp32", "matmulFp32Wt", "matmulBf16", "matmulFp16", "matmulQ4K", "matmulQ6K", "matmulQ5K", "matmulQ8_0",
                      "matmulQ4_0", "matmulQ5_0", "matmulQ5_1", "softmaxFp32", "normFp32", "attentionFp32"):
         assert f"override fun {accessor}()" in provider
+
+
+def test_no_alloc_argmax_hands_each_host_thread_a_slot_of_its_own():
+    """The arg-max entry that allocates nothing keeps its counters in a fixed array cut into 8 slots; a host thread gets
+    one on first use and keeps it (the library's streams are per thread). The hand-out makes no device call, so it is
+    checked here, in a fresh process: ten threads, each asking twice -- eight distinct slots 0..7, the same slot on the
+    second call, -1 for the two that come too late."""
+    import subprocess
+    import sys
+    code = (
+        "import ctypes, threading, sys\n"
+        f"lib = ctypes.CDLL({_lib.HIP_LIB_PATH!r})\n"
+        "f = lib.skainet_hip_f32_argmax_rows_noalloc_slot; f.restype = ctypes.c_int32\n"
+        "out = [None] * 10\n"
+        "gate = threading.Barrier(10)\n"
+        "def work(i):\n"
+        "    gate.wait(); a = f(); b = f(); gate.wait(); out[i] = (a, b)\n"
+        "ts = [threading.Thread(target=work, args=(i,)) for i in range(10)]\n"
+        "[t.start() for t in ts]; [t.join() for t in ts]\n"
+        "print(sorted(out))\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    got = eval(r.stdout.strip())
+    assert all(a == b for a, b in got)                                       # a thread keeps its slot
+    assert sorted(a for a, _ in got) == [-1, -1] + list(range(8))            # eight slots, then refusals

@@ -487,6 +487,28 @@ def test_graph_and_eager_decode_agree(small_model):
     assert np.array_equal(outs[0][2], outs[1][2])
 
 
+def test_decode_runs_with_the_one_row_matrix_core_kernel_switched_off(small_model):
+    """A decode step's attention leaves its key splits unmerged for the output projection only where that projection's
+    kernel will take them; with the kernel switched off the step falls back to attention + merge + product and gives
+    the same tokens (fp32 row kernels: the checker's bound holds as before)."""
+    from skainet_amd import kernels as kx
+    from skainet_amd.decoder import LlamaDecoder
+    cfg, w = small_model
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 6)
+    ref = LlamaDecoder(w, max_prefill=8)
+    first = ref.prefill(prompt)
+    toks = ref.decode(6, use_graph=False)
+    kx.set_tuning("q4k_mfma_enable", 0)
+    try:
+        dec = LlamaDecoder(w, max_prefill=8)
+        assert dec.prefill(prompt) == first
+        got = dec.decode(6, use_graph=False)
+        assert max_norm_err(dec.last_logits(), ref.last_logits()) < 1e-3
+    finally:
+        kx.set_tuning("q4k_mfma_enable", 1)
+    assert np.array_equal(got, toks)
+
+
 def test_prefill_rejects_oversized_prompt(small_model):
     from skainet_amd.decoder import LlamaDecoder
     cfg, w = small_model

@@ -560,3 +560,41 @@ def test_weight_upload_through_the_page_locked_chunks_is_byte_exact(hip_backend,
     finally:
         hip_backend.set_tuning("upload_chunk_mib", 8)
         hip_backend.set_tuning("upload_lanes", 4)
+
+
+@pytest.mark.parametrize("n,k", [(64, 4096), (37, 1024), (300, 8192)])
+def test_q4k_one_row_fixed_point_kernel_at_the_extremes_of_its_digit_sums(hip_backend, torch_cuda, n, k):
+    """Constant activations against saturated codes (all 15, all 0) with the largest scales: the top digit plane's sum
+    passes 2^31 before the code sum takes its offset out again, so the recombination must be modular; and the negative
+    mirror. Against the exact-fp32 oracle."""
+    blocks = random_valid_blocks("Q4_K", n * k // 256, 11).reshape(n, k // 256, 144).copy()
+    blocks[0::2, :, 16:] = 0xFF
+    blocks[1::2, :, 16:] = 0x00
+    blocks[:, :, 4:16] = 0xFF                                     # every 6-bit scale and minimum at 63
+    packed = blocks.reshape(-1)
+    for c in (7.5, -7.5, 1e-3):
+        x = np.full((1, k), c, np.float32)
+        got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemv_mfma_kernel"
+        assert normalized_err(got, L.gemv("Q4_K", x, packed, n)) <= GEMV_TOL
+
+
+def test_q4k_one_row_fixed_point_kernel_keeps_non_finite_activations_loud(hip_backend, torch_cuda):
+    """The exact-fp32 product (ScalarQ4_KMatmulKernel.kt:40-78) propagates a NaN or an infinity among the activations into
+    every output. The fixed-point kernel takes a group's largest magnitude with fmax (which drops a NaN) and scales by
+    its reciprocal (0 for an infinity) -- but the sub-block's fp32 activation sum, which the minima multiply, carries
+    the NaN or turns inf * 0 into one: no output stays finite. A group of subnormal activations contributes next to
+    nothing, as in fp32. With the RMSNorm prologue the sum of squares does the same."""
+    n, k = 64, 2048
+    packed = random_valid_blocks("Q4_K", n * k // 256, 7)
+    rng = np.random.default_rng(8)
+    for bad in (np.nan, np.inf, -np.inf):
+        x = rng.standard_normal((1, k)).astype(np.float32)
+        x[0, 700] = bad
+        got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+        assert hip_backend.last_kernel() == "q4k_gemv_mfma_kernel"
+        assert not np.isfinite(got).any(), bad
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    x[0, 128:192] = np.float32(1e-41) * rng.standard_normal(64).astype(np.float32)      # one group of subnormals
+    got = gpu_matmul(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+    assert np.isfinite(got).all() and normalized_err(got, L.gemv("Q4_K", x, packed, n)) <= GEMV_TOL

@@ -41,3 +41,34 @@ def test_argmax_noalloc_refuses_more_rows_than_its_scratch_holds(hip_backend, to
     assert lib.skainet_hip_f32_argmax_rows_noalloc_dev(y.data_ptr(), 64, 10, got.data_ptr()) == 0
     hip_backend.sync()
     assert got.cpu().tolist() == [int(r.argmax()) for r in y.cpu().numpy()]
+
+
+def test_argmax_noalloc_from_two_host_threads_at_once(hip_backend, torch_cuda):
+    """Two host threads, each on its own stream (the library's streams are per thread), call the entry over and over on
+    different inputs: each thread has a slot of the fixed array to itself, so no call sees the other's counters."""
+    import threading
+    torch = torch_cuda
+    lib = _lib.hip()
+    rng = np.random.default_rng(9)
+    data = [rng.standard_normal((3, 50000)).astype(np.float32) for _ in range(2)]
+    devs = [dev(torch, d) for d in data]
+    outs = [torch.full((40, 3), -1, dtype=torch.int32, device="cuda") for _ in range(2)]
+    errs = []
+
+    def work(t):
+        assert lib.skainet_hip_thread_stream() == 0, _lib.last_error()       # so that the two threads' kernels can overlap
+        for i in range(40):
+            if lib.skainet_hip_f32_argmax_rows_noalloc_dev(devs[t].data_ptr(), 3, 50000, outs[t][i].data_ptr()) != 0:
+                errs.append(_lib.last_error())
+        lib.skainet_hip_sync()
+        lib.skainet_hip_thread_release()
+
+    torch.cuda.synchronize()                                                 # the inputs are on the device before the threads start
+    ts = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert not errs, errs
+    torch.cuda.synchronize()
+    for t in range(2):
+        want = [int(r.argmax()) for r in data[t]]
+        assert (outs[t].cpu().numpy() == np.array(want, np.int32)).all()
