@@ -667,7 +667,7 @@ bool gemm_ksw_enabled();
 bool gemm_ksw_fits(int m, int n, int k);
 bool gemm_ksw_forced();
 size_t gemm_frag_activation_bytes(int m, int k);                                                              // gemm_q4k_frag.hip
-int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, hipStream_t s);
+int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, const uint8_t* w, int n, hipStream_t s);
 int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s);
 bool gemm_frag_enabled();
 bool gemm_frag_fits(int m, int n, int k);
@@ -723,7 +723,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     auto run_frag = [&]() -> int {                               // Q4_K: the same tiles, activations in fragment order
         uint8_t* a = static_cast<uint8_t*>(kernel_workspace(gemm_frag_activation_bytes(m, k)));
         if (!a) return -1;
-        if (launch_gemm_frag_prepass(x, gain, eps, a, m, k, s) != 0) return -1;
+        if (launch_gemm_frag_prepass(x, gain, eps, a, m, k, w, n, s) != 0) return -1;
         if (launch_q4k_gemm_frag(a, w, epilogue != GEMM_EPI_NONE ? tmp : y, m, n, k, s) != 0) return -1;
         return finish();
     };

@@ -168,6 +168,8 @@ void set_gemm_ksw(int v);
 void set_gemm_ksw_teams(int v);
 void set_gemm_ksw_stages(int v);
 void set_gemm_frag(int v);
+void set_gemm_frag_touch(int v);
+void set_gemm_frag_pieces(int v);
 void set_sdpa_prefill_mfma(int v);
 void set_sdpa_prefill_teams(int v);
 void set_sdpa_decode_split_keys(int v);
@@ -209,6 +211,8 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "gemm_ksw_teams")) { set_gemm_ksw_teams(value); return 0; }
     if (!strcmp(key, "gemm_ksw_stages")) { set_gemm_ksw_stages(value); return 0; }
     if (!strcmp(key, "gemm_frag")) { set_gemm_frag(value); return 0; }
+    if (!strcmp(key, "gemm_frag_touch")) { set_gemm_frag_touch(value); return 0; }
+    if (!strcmp(key, "gemm_frag_pieces")) { set_gemm_frag_pieces(value); return 0; }
     if (!strcmp(key, "sdpa_prefill_mfma")) { set_sdpa_prefill_mfma(value); return 0; }
     if (!strcmp(key, "sdpa_prefill_teams")) { set_sdpa_prefill_teams(value); return 0; }
     if (!strcmp(key, "q4k_ksplit_enable")) { set_q4k_ksplit_enable(value); return 0; }
