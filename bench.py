@@ -65,6 +65,10 @@ WORKLOADS = {
     "q4k_gemm_128x14336x4096": ("Q4_K", 14336, 4096, 128),
     "q6k_gemm_512x32000x4096": ("Q6_K", 32000, 4096, 512),
     "q4k_gemm_512x14336x4096": ("Q4_K", 14336, 4096, 512),
+    # the other products of a Llama-3-8B prefill of 512 tokens: fused gate/up, fused q/k/v, down
+    "q4k_gemm_512x28672x4096": ("Q4_K", 28672, 4096, 512),
+    "q4k_gemm_512x6144x4096": ("Q4_K", 6144, 4096, 512),
+    "q4k_gemm_512x4096x14336": ("Q4_K", 4096, 14336, 512),
     "q5k_gemm_512x4096x4096": ("Q5_K", 4096, 4096, 512),
     "q4_0_gemm_512x4096x4096": ("Q4_0", 4096, 4096, 512),
 }

@@ -767,7 +767,11 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
         // products; its step is slower per tile row (0.31 us per 64 elements of K measured, 6.5 us per round outside the loop).
         // It wins where the tile kernel would have to split K across workgroups: 512 x 4096 x 4096 is such a shape.
         const int rounds = (((m + 127) / 128) * ((n + 63) / 64) + num_cus() - 1) / num_cus();
-        if (rounds * (6.5 + 0.31 * (k / GK)) < tile_estimate) return frag_ok && gemm_frag_enabled() ? run_frag() : run_ksw();
+        // the same tiles with the activations in fragment order: measured 8 us per round outside the loop and 0.20 us per
+        // 64 elements of K (0.27 on rows longer than two super-blocks per wave, whose weight ring is refilled under way)
+        if (frag_ok && gemm_frag_enabled()) {
+            if (rounds * (8.0 + (k <= 4096 ? 0.20 : 0.27) * (k / GK)) < tile_estimate) return run_frag();
+        } else if (rounds * (6.5 + 0.31 * (k / GK)) < tile_estimate) return run_ksw();
     }
     if (ksplit > kgroups) ksplit = kgroups;
     const int k_chunk = ((kgroups + ksplit - 1) / ksplit) * 256;
