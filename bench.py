@@ -189,6 +189,9 @@ DECODER_WORKLOADS = {
 }
 # The same stack driven through host arrays only (the unchanged kernel SPI): see measure_decoder_spi.
 SPI_DECODER_WORKLOADS = {"llama3_8b_decode_spi": "llama3_8b_decode", "llama3_8b_8layers_decode_spi": "llama3_8b_8layers_decode"}
+# The same stack written against the generic resident-activation ops class (one device entry per op, nothing fused by
+# name): see measure_decoder_ops.
+OPS_DECODER_WORKLOADS = {"llama3_8b_decode_ops": "llama3_8b_decode", "llama3_8b_8layers_decode_ops": "llama3_8b_8layers_decode"}
 
 
 def cpu_baseline_decode(cfg, host, ctx):
@@ -365,10 +368,19 @@ def bench_dense(a):
 
 
 def bench_attention(a):
+    rec, ok = measure_attention(a.workload, a.steps, a.warmup, a.no_graph, a.skip_cpu)
+    print(json.dumps(rec).replace("NaN", "null"))
+    sys.exit(0 if ok else 1)
+
+
+def measure_attention(workload, steps_arg, warmup_arg, no_graph, skip_cpu):
     """Fused causal GQA attention, fp32 operands: prefill at 2048 (MFMA-class, flops counted dense as the reference's
-    scenarios do) and one-token decode against a 4096-long KV cache (HBM-bound: K and V are read once)."""
+    scenarios do) and one-token decode against a 4096-long KV cache (HBM-bound: K and V are read once). Returns
+    (record, ok)."""
     import torch
+    from types import SimpleNamespace
     from skainet_amd import _lib, kernels
+    a = SimpleNamespace(workload=workload, steps=steps_arg, warmup=warmup_arg, no_graph=no_graph, skip_cpu=skip_cpu)
     batch, sq, skv = ATTENTION_WORKLOADS[a.workload][:3]
     window = ATTENTION_WORKLOADS[a.workload][3] if len(ATTENTION_WORKLOADS[a.workload]) > 3 else 0
     heads, kvh, d = 32, 8, 128
@@ -461,8 +473,9 @@ def bench_attention(a):
         # the reference threads its attention rows over at most 4 pool participants once there are >= 512 rows
         cores = 4 if (kind == "reference" and not decode) else 1
         out_json["cpu_baseline"] = {"value": round(cpu_val, 4), "unit": unit, "cores": cores, "kind": kind, "sample": sample}
-    print(json.dumps(out_json).replace("NaN", "null"))
-    sys.exit(0 if err <= tol else 1)
+    del ks, vs, q, out
+    torch.cuda.empty_cache()
+    return out_json, err <= tol
 
 
 def measure_decoder(workload, steps, warmup, no_graph, skip_cpu):
@@ -617,6 +630,68 @@ def measure_decoder_spi(workload, steps, warmup):
     return rec, ok
 
 
+def measure_decoder_ops(workload, steps, warmup, no_graph):
+    """The decode step of `measure_decoder` through skainet_amd.ops.HipOps alone: what a model built with the NN DSL costs
+    when its TensorOps keeps activations resident -- 17 device entries per layer instead of the fused decoder's 5, every
+    intermediate a device tensor, the step recorded into a HIP graph. The fused decoder runs beside it on the same
+    weights: same prompt, logits compared, and its time per token at the same context for the comparison."""
+    from dataclasses import replace
+    from skainet_amd import _lib, kernels
+    from skainet_amd.decoder import LLAMA3_8B, LlamaDecoder, LlamaWeights
+    from skainet_amd.ops_decoder import OpsLlamaDecoder, OpsLlamaWeights
+    overrides, prompt_len, distinct = DECODER_WORKLOADS[OPS_DECODER_WORKLOADS[workload]]
+    cfg = replace(LLAMA3_8B, **overrides)
+    w = LlamaWeights(cfg, seed=20251125, distinct_layers=distinct)
+    ow = OpsLlamaWeights(w)
+    prompt = np.random.default_rng(7).integers(0, cfg.vocab, prompt_len)
+    fused = LlamaDecoder(w, max_prefill=prompt_len)
+    first_fused = fused.prefill(prompt)
+    dec = OpsLlamaDecoder(ow, max_prefill=prompt_len)
+    dec.prefill(prompt)                      # warm-up pass: sizes the library's scratch
+    kernels.sync()
+    with kernels.Timer() as t:
+        first = dec.prefill(prompt)
+    prefill_ms = t.ms
+    ref = fused.last_logits().astype(np.float64)
+    err = float(np.abs(dec.last_logits() - ref).max() / np.abs(ref).max())       # both prefills run the bf16 MFMA GEMM
+    ok = err < 2e-2 and bool(np.isfinite(dec.last_logits()).all())
+    dec.decode(max(1, warmup), use_graph=not no_graph)
+    fused.decode(max(1, warmup), use_graph=not no_graph)
+    pos0 = dec.position()
+    with kernels.Timer() as tm:
+        dec.run_steps(steps, use_graph=not no_graph)
+    ms_per_tok = tm.ms / steps
+    with kernels.Timer() as tm:
+        fused.run_steps(steps, use_graph=not no_graph)
+    fused_ms = tm.ms / steps
+    lg = dec.last_logits()
+    ok = ok and bool(np.isfinite(lg).all()) and dec.position() == pos0 + steps
+    alg = w.decode_bytes_per_token(pos0 + steps // 2)
+    gbs = alg / (ms_per_tok * 1e-3) / 1e9
+    rec = {
+        "metric": "decode tok/s", "value": round(1e3 / ms_per_tok, 2), "unit": "tok/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(ms_per_tok, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 (packed Q4_K / Q6_K weights)", "data": "synthetic",
+        "config": {"workload": workload, "layers": cfg.layers, "hidden": cfg.hidden, "heads": cfg.heads,
+                   "kv_heads": cfg.kv_heads, "head_dim": cfg.head_dim, "ffn": cfg.ffn, "vocab": cfg.vocab, "batch": 1,
+                   "prompt_tokens": prompt_len, "decoded_tokens": steps, "context_at_end": pos0 + steps,
+                   "route": "generic resident-activation ops class (HipOps): one device entry per tensor op, activations "
+                            "and KV cache resident, nothing fused by name",
+                   "launch": "host loop" if no_graph else "hip-graph replay of one decode step"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "extra": {"device_entries_per_token": dec.launches_per_token(), "prefill_ms": round(prefill_ms, 3),
+                  "fused_decoder_ms_per_token_same_context": round(fused_ms, 5),
+                  "prefill_logits_err_vs_fused_decoder": err, "first_token_equals_fused": bool(first == first_fused),
+                  "algorithmic_bytes_per_token": alg, "device": _lib.hip().skainet_hip_device_name().decode()},
+    }
+    if not ok:
+        rec["extra"]["PARITY_FAILED"] = True
+    dec.close()
+    fused.close()
+    return rec, ok
+
+
 UPLOAD_WORKLOADS = {"weight_upload_q4k_528mb": ("Q4_K", 229376, 4096)}   # name: (encoding, rows, cols)
 PCIE_PEAK_GBS = 64.0   # PCIe 5.0 x16, one direction, before protocol overhead
 
@@ -675,6 +750,10 @@ def bench_upload(a):
 
 
 def bench_decoder(a):
+    if a.workload in OPS_DECODER_WORKLOADS:
+        rec, ok = measure_decoder_ops(a.workload, 64 if a.steps == 2000 else a.steps, 4 if a.warmup == 200 else a.warmup, a.no_graph)
+        print(json.dumps(rec).replace("NaN", "null"))
+        sys.exit(0 if ok else 1)
     if a.workload in SPI_DECODER_WORKLOADS:
         rec, ok = measure_decoder_spi(a.workload, 32 if a.steps == 2000 else a.steps, 4 if a.warmup == 200 else a.warmup)
         print(json.dumps(rec).replace("NaN", "null"))
@@ -691,7 +770,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000, help="timed steps (default 2000; 200 for the GEMM workloads)")
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(SPI_DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS) + sorted(DENSE_WORKLOADS) + sorted(UPLOAD_WORKLOADS))
+    ap.add_argument("--workload", default="q4k_gemv_11008x4096_b1", choices=sorted(WORKLOADS) + sorted(DECODER_WORKLOADS) + sorted(SPI_DECODER_WORKLOADS) + sorted(OPS_DECODER_WORKLOADS) + sorted(ATTENTION_WORKLOADS) + sorted(DENSE_WORKLOADS) + sorted(UPLOAD_WORKLOADS))
     ap.add_argument("--no-graph", action="store_true", help="launch from the host loop instead of replaying a HIP graph")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline (profiling runs)")
     ap.add_argument("--hbm-only", action="store_true", help="skip the cache-warm pass and the read probe, so every launch of the "
@@ -713,14 +792,14 @@ def main():
         key, _, val = kv.partition("=")
         _lib.check(_lib.hip().skainet_hip_set_tuning(key.encode(), int(val)), "set_tuning")
 
-    if a.workload in DECODER_WORKLOADS or a.workload in SPI_DECODER_WORKLOADS:
+    if a.workload in DECODER_WORKLOADS or a.workload in SPI_DECODER_WORKLOADS or a.workload in OPS_DECODER_WORKLOADS:
         bench_decoder(a)
     if a.workload in UPLOAD_WORKLOADS:
         return bench_upload(a)
     if a.workload in DENSE_WORKLOADS:
         return bench_dense(a)
     if a.workload in ATTENTION_WORKLOADS:
-        bench_attention(a)
+        return bench_attention(a)
     default_run = a.workload == "q4k_gemv_11008x4096_b1" and not a.no_headline
     out, ok = measure_matmul(a.workload, a.steps, a.warmup, not a.no_graph, a.hbm_only, a.skip_cpu)
     if default_run:
@@ -733,17 +812,37 @@ def main():
             "steps": rec["steps"], "frac_of_bf16_mfma_peak": rec["roofline"]["frac"], "traffic": rec["roofline"]["traffic"],
             "dtype": rec["dtype"], "parity_ok": g_ok, "max_err_over_max": rec["extra"]["max_normalized_err_vs_fp64_decode_matmul"],
             "kernel": rec["extra"]["kernel"]}
-        d_steps, d_warm = (128, 8) if a.steps == 2000 else (min(a.steps, 256), min(a.warmup, 32))
-        rec, d_ok = measure_decoder("llama3_8b_decode", d_steps, d_warm, a.no_graph, True)
+        # the config's own 128 decoded tokens, whatever --steps says (a shorter run is a different workload)
+        rec, d_ok = measure_decoder("llama3_8b_decode", 128, 8, a.no_graph, True)
         headline["llama3_8b_decode"] = {
             "metric": rec["metric"], "value": rec["value"], "unit": rec["unit"], "ms_per_token": rec["ms_per_step"],
             "steps": rec["steps"], "frac_of_hbm_peak": rec["roofline"]["frac"], "prefill_ms": rec["extra"]["prefill_ms"],
             "prefill_tok_per_s": rec["extra"]["prefill_tok_per_s"], "context_at_end": rec["config"]["context_at_end"],
             "ms_per_token_at_context_limit": rec["extra"]["ms_per_token_at_context_limit"],
-            "context_limit": rec["extra"]["context_limit"], "dtype": rec["dtype"], "parity_ok": d_ok,
+            "context_limit": rec["extra"]["context_limit"], "dtype": rec["dtype"], "self_check_ok": d_ok,
             "weights": rec["config"]["weights"]}
-        out["extra"]["headline"] = headline
         ok = ok and g_ok and d_ok
+        # the remaining configurations of the baseline, each with the parity flag of its own fp64 check
+        short = a.steps != 2000
+        for wl in ("q8_0_gemv_4096x4096_b1", "q4k_gemv_11008x4096_b4", "q4k_gemv_11008x4096_b8", "q6k_gemm_512x32000x4096"):
+            gemm = WORKLOADS[wl][3] > 8
+            st, wu = ((100, 10) if gemm else (1000, 100)) if not short else (a.steps, a.warmup)
+            rec, w_ok = measure_matmul(wl, st, wu, not a.no_graph, True, True)
+            headline[wl] = {"metric": rec["metric"], "value": rec["value"], "unit": rec["unit"], "ms_per_step": rec["ms_per_step"],
+                            "steps": rec["steps"], "frac": rec["roofline"]["frac"], "bound": rec["roofline"]["bound"],
+                            "traffic": rec["roofline"]["traffic"], "dtype": rec["dtype"], "kernel": rec["extra"]["kernel"],
+                            "parity_ok": w_ok, "max_err": rec["extra"]["max_normalized_err_vs_fp64_decode_matmul"]}
+            ok = ok and w_ok
+        for wl in ("sdpa_prefill_2048", "sdpa_decode_4096_b1", "sdpa_decode_4096_b8"):
+            decode = ATTENTION_WORKLOADS[wl][1] == 1
+            st, wu = ((1000, 100) if decode else (20, 3)) if not short else (a.steps, a.warmup)
+            rec, w_ok = measure_attention(wl, st, wu, a.no_graph, True)
+            headline[wl] = {"metric": rec["metric"], "value": rec["value"], "unit": rec["unit"], "ms_per_step": rec["ms_per_step"],
+                            "steps": rec["steps"], "frac": rec["roofline"]["frac"], "bound": rec["roofline"]["bound"],
+                            "traffic": rec["roofline"]["traffic"], "dtype": rec["dtype"], "parity_ok": w_ok,
+                            "max_err": rec["extra"]["max_err_over_max_vs_torch_fp64"]}
+            ok = ok and w_ok
+        out["extra"]["headline"] = headline
     print(json.dumps(out).replace("NaN", "null"))
     sys.exit(0 if ok else 1)
 
