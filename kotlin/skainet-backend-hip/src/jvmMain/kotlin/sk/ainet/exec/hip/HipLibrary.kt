@@ -79,6 +79,23 @@ internal object HipLibrary {
         FunctionDescriptor.ofVoid(P, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P, I, I, I, I),
     )
 
+    // ---- device entries: every pointer in the GPU's memory, asynchronous on the calling thread's stream, 0 / -1
+    val sgemmDev: MethodHandle? = bind("skainet_hip_fp32_matmul_dev", FunctionDescriptor.of(I, P, I, I, P, I, I, P, I, I, I, I, I))
+    val sgemmWtDev: MethodHandle? = bind("skainet_hip_fp32_matmul_wt_dev", FunctionDescriptor.of(I, P, I, P, I, P, I, I, I, I))
+    val rmsNormDev: MethodHandle? = bind("skainet_hip_f32_rms_norm_dev", FunctionDescriptor.of(I, P, P, P, I, I, F))
+    val layerNormDev: MethodHandle? = bind("skainet_hip_f32_layer_norm_dev", FunctionDescriptor.of(I, P, P, P, P, I, I, F))
+    val softmaxDev: MethodHandle? = bind("skainet_hip_f32_softmax_rows_dev", FunctionDescriptor.of(I, P, P, I, I, I))
+    val sdpaDev: MethodHandle? = bind(
+        "skainet_hip_f32_sdpa_dev",
+        FunctionDescriptor.of(I, P, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P, I, I, I, I),
+    )
+    /** (op, a, a_mode, b, b_mode, out, n, inner): op 0 add, 1 sub, 2 mul, 3 div; mode 0 full, 1 scalar, 2 bias */
+    val binaryDev: MethodHandle? = bind("skainet_hip_f32_binary_dev", FunctionDescriptor.of(I, I, P, I, P, I, P, L, I))
+    /** (op, in, out, n): op 0 relu, 1 sigmoid, 2 silu, 3 gelu (tanh form), 4 gelu (erf form), 5 erf, 6 tanh */
+    val unaryDev: MethodHandle? = bind("skainet_hip_f32_unary_dev", FunctionDescriptor.of(I, I, P, P, L))
+    val reduceAllDev: MethodHandle? = bind("skainet_hip_f32_reduce_all_dev", FunctionDescriptor.of(I, P, L, I, P))
+    val reduceAxisDev: MethodHandle? = bind("skainet_hip_f32_reduce_axis_dev", FunctionDescriptor.of(I, P, I, I, I, I, P))
+
     /** Cheap, cached, false (not throwing) when the library or a gfx950 device is missing. */
     val usable: Boolean by lazy {
         runCatching {

@@ -27,8 +27,12 @@ import sk.ainet.lang.types.FP32
 /**
  * matmul(F32 dense contiguous x F32/<encoding> BLOCKED_ROW_MAJOR) on the device: all activation rows in one call
  * against a GGUF-ordered weight that is uploaded the first time its storage is seen and stays resident after that.
+ * The device twin of the CPU library's view kernel, registered under the same kernel key and serving the same operand
+ * classes (skainet-backends/skainet-backend-native-cpu/src/jvmMain/kotlin/sk/ainet/exec/kernel/FfmRowMajorKernels.kt:42-137,
+ * its pack :140-169).
  *
- * Per call: one copy of the rows into a native segment, `skainet_hip_matmul_host` (upload, product, download and one
+ * A resident activation ([HipDeviceStorage]) with a resident output runs `skainet_hip_matmul_dev` in place. A heap
+ * activation, per call: one copy of the rows into a native segment, `skainet_hip_matmul_host` (upload, product, download and one
  * wait on buffers the library keeps per thread), one copy back. Up to 8 rows run the weight-streaming GEMV kernels
  * (fp32 class, within 1e-3 of the exact product), more rows the matrix-core GEMM (bf16 operands, within 2e-2).
  */
@@ -40,6 +44,8 @@ public class HipRowMajorMatmulKernel internal constructor(
     override val key: KernelKey,
 ) : ViewKernel, MappedCapableKernel {
     override val name: String = "hip-rowmajor-${encoding.name}"
+
+    internal fun encodingOf(): TensorEncoding = encoding
 
     /** Weight handles by the identity of the storage that holds the packed bytes (a model's weights never move). */
     private val resident = IdentityHashMap<Storage, MemorySegment>()
@@ -57,6 +63,22 @@ public class HipRowMajorMatmulKernel internal constructor(
         require(out.shape[0] == rows && out.shape[1] == n) { "out must be [$rows, $n], was ${out.shape}" }
         check(w.layout.blockOrder == BlockOrder.ROW_MAJOR) { "$name reads canonical row-major weights; this one is ${w.layout.blockOrder}" }
         val fn = HipLibrary.matmulHost ?: return fallback(inputs, out, sink, "libskainet_hip unavailable")
+        val aDev = a.storage as? HipDeviceStorage
+        val oDev = out.storage as? HipDeviceStorage
+        if (aDev != null && oDev != null) {
+            // a resident activation into a resident output: the product runs where both already are, nothing is copied
+            if (!a.isContiguous || !out.isContiguous) return fallback(inputs, out, sink, "strided activation or output")
+            if (k % blockElems != 0) return fallback(inputs, out, sink, "inner dimension $k is not a multiple of $blockElems")
+            if (rows == 0 || n == 0) return
+            val dev = HipLibrary.matmulDev ?: return fallback(inputs, out, sink, "libskainet_hip unavailable")
+            val handle = handleFor(w) ?: return fallback(inputs, out, sink, "upload failed: ${HipLibrary.error()}")
+            val aPtr = MemorySegment.ofAddress(aDev.pointer().address() + a.layout.offsetElements * Float.SIZE_BYTES)
+            val oPtr = MemorySegment.ofAddress(oDev.pointer().address() + out.layout.offsetElements * Float.SIZE_BYTES)
+            val rc = dev.invoke(handle, aPtr, rows, oPtr) as Int
+            check(rc == 0) { "$name: ${HipLibrary.error()}" }
+            if (sink.isEnabled) sink.emit(TraceEvent.KernelRun(op = key.op, kernel = "$name (resident)", inputs = inputs.map { it.id }, output = out.id))
+            return
+        }
         val aHeap = a.storage as? Storage.Heap ?: return fallback(inputs, out, sink, "activation storage ${a.storage::class.simpleName}")
         val oHeap = out.storage as? Storage.Heap ?: return fallback(inputs, out, sink, "output storage ${out.storage::class.simpleName}")
         val activation = aHeap.floats ?: return fallback(inputs, out, sink, "activation is not a FloatArray")
@@ -64,10 +86,7 @@ public class HipRowMajorMatmulKernel internal constructor(
         if (!a.isContiguous || !out.isContiguous) return fallback(inputs, out, sink, "strided activation or output")
         if (k % blockElems != 0) return fallback(inputs, out, sink, "inner dimension $k is not a multiple of $blockElems")
         if (rows == 0 || n == 0) return
-        val handle = synchronized(resident) {
-            resident[w.storage] ?: (upload(w, n, k) ?: return fallback(inputs, out, sink, "upload failed: ${HipLibrary.error()}"))
-                .also { resident[w.storage] = it }
-        }
+        val handle = handleFor(w) ?: return fallback(inputs, out, sink, "upload failed: ${HipLibrary.error()}")
         Arena.ofConfined().use { arena ->
             val inSeg = arena.allocate(rows.toLong() * k * Float.SIZE_BYTES, 16)
             MemorySegment.copy(activation, aHeap.arrayOffset + a.layout.offsetElements.toInt(), inSeg, ValueLayout.JAVA_FLOAT, 0L, rows * k)
@@ -77,6 +96,11 @@ public class HipRowMajorMatmulKernel internal constructor(
             MemorySegment.copy(outSeg, ValueLayout.JAVA_FLOAT, 0L, output, oHeap.arrayOffset + out.layout.offsetElements.toInt(), rows * n)
         }
         if (sink.isEnabled) sink.emit(TraceEvent.KernelRun(op = key.op, kernel = name, inputs = inputs.map { it.id }, output = out.id))
+    }
+
+    /** The resident handle of the weight behind [w] ([n, k] packed rows), uploaded the first time its storage is seen; `null` when the upload fails. */
+    internal fun handleFor(w: TensorView): MemorySegment? = synchronized(resident) {
+        resident[w.storage] ?: upload(w, w.shape[0], w.shape[1])?.also { resident[w.storage] = it }
     }
 
     /**
@@ -154,6 +178,19 @@ public object HipRowMajorKernelPack : ViewKernelPack {
             KernelDispatch.register(kernel)
             installed += kernel
         }
+    }
+
+    /**
+     * The resident handle for a packed weight view (uploading it on first sight), for callers that run the device
+     * entries themselves ([HipOps]); `null` for an encoding, block order or inner dimension this pack does not serve.
+     */
+    @Synchronized
+    internal fun handleFor(w: TensorView): MemorySegment? {
+        install()
+        if (w.shape.rank != 2 || w.layout.blockOrder != BlockOrder.ROW_MAJOR) return null
+        val format = FORMATS.firstOrNull { it.encoding == w.format.encoding } ?: return null
+        if (w.shape[1] % format.elems != 0) return null
+        return installed.firstOrNull { it.encodingOf() == format.encoding }?.handleFor(w)
     }
 
     /** Device memory of every weight uploaded through this pack goes back to the device. */

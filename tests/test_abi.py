@@ -120,7 +120,7 @@ def test_kotlin_module_binds_the_header_as_declared():
     decls = _c_parameter_kinds()
     named = {m.group(1): m.group(2) for m in re.finditer(r"private val (\w+): FunctionDescriptor = (FunctionDescriptor\.\w+\([^)]*\))", src)}
     bound = re.findall(r'bind\(\s*"(skainet_hip_\w+)",\s*(FunctionDescriptor\.\w+\([^)]*\)|\w+)', src)
-    assert len(bound) >= 29
+    assert len(bound) >= 39
     for name, desc in bound:
         assert name in decls, f"{name} is not declared in the header"
         desc = named.get(desc, desc)
@@ -141,6 +141,27 @@ def test_kotlin_module_binds_the_header_as_declared():
     for accessor in ("matmulFp32", "matmulFp32Wt", "matmulBf16", "matmulFp16", "matmulQ4K", "matmulQ6K", "matmulQ5K", "matmulQ8_0",
                      "matmulQ4_0", "matmulQ5_0", "matmulQ5_1", "softmaxFp32", "normFp32", "attentionFp32"):
         assert f"override fun {accessor}()" in provider
+
+
+def test_resident_ops_class_serves_the_reference_method_set_in_both_languages():
+    """The resident-activation ops class overrides the methods the browser tier's resident ops class overrides
+    (WasmCpuOps.kt:180-428: the two matmuls, four binaries, six activations, two reductions, softmax / logSoftmax, the two
+    fused norms, attention) -- in the Kotlin text and in the Python mirror that the GPU tests drive -- and every device
+    entry the Kotlin class calls is bound in HipLibrary.kt (whose descriptors the test above holds against the header)."""
+    kdir = os.path.join(ROOT, "kotlin", "skainet-backend-hip", "src", "jvmMain", "kotlin", "sk", "ainet", "exec", "hip")
+    ops_kt = open(os.path.join(kdir, "HipOps.kt")).read()
+    lib_kt = open(os.path.join(kdir, "HipLibrary.kt")).read()
+    methods = ["matmul", "matmulWeightTransposed", "add", "subtract", "multiply", "divide", "relu", "sigmoid", "silu", "gelu",
+               "erf", "tanh", "sum", "mean", "softmax", "logSoftmax", "layerNorm", "rmsNorm", "scaledDotProductAttention"]
+    from skainet_amd import ops as py_ops
+    for name in methods:
+        assert re.search(r"override fun <T : DType, V> %s\(" % name, ops_kt), f"HipOps.kt does not override {name}"
+        snake = re.sub(r"(?<!^)(?=[A-Z])", "_", name).lower()
+        assert callable(getattr(py_ops.HipOps, snake, None)), f"ops.HipOps has no {snake}"
+    assert "fun <T : DType, V> toResident(" in ops_kt and callable(py_ops.HipOps.to_resident)
+    for handle in set(re.findall(r"HipLibrary\.(\w+)", ops_kt)):
+        assert re.search(r"\b(val|fun) %s\b" % handle, lib_kt), f"HipLibrary has no member {handle}"
+    assert "class HipTensorData" in open(os.path.join(kdir, "HipTensorData.kt")).read()
 
 
 def test_no_alloc_argmax_hands_each_host_thread_a_slot_of_its_own():
