@@ -303,6 +303,19 @@ SKAINET_HIP_API int32_t skainet_hip_attn_out_proj_dev(const skainet_hip_weight* 
                                                       int32_t seq_kv, int32_t kv_capacity, float scale, int32_t window,
                                                       const int32_t* lengths, const float* residual, float* out, float* attn_tmp);
 
+/* A gated MLP block in one call:
+ *   out[m, rows of w_down] = (residual ? residual : 0) + Wdown . swiglu(Wgate_up . rmsnorm(x)),
+ * x [m, cols of w_gate_up]; w_gate_up's rows are interleaved (gate_0, up_0, gate_1, up_1, ...), swiglu(g, u) =
+ * g / (1 + exp(-g)) * u; gain == NULL: no norm; `residual` may alias `out`. No reference counterpart as one call: the
+ * parts are the fused norm (f32_fused.c), two packed products and NAT:532-539's unary silu / binary mul / binary add.
+ * Prompt shapes (m > 8, packed weights): the (gate, up) product is parked once as fp32 pairs in the library's scratch and
+ * the pass that rounds the down projection's activations to bf16 takes the SwiGLU on the way (the activation is never
+ * stored as fp32), the residual is added where the down projection stores its tiles. Other shapes: the two
+ * skainet_hip_matmul_fused_dev calls in a row. Arithmetic class per row count as for skainet_hip_matmul_dev. */
+SKAINET_HIP_API int32_t skainet_hip_mlp_swiglu_dev(const skainet_hip_weight* w_gate_up, const skainet_hip_weight* w_down,
+                                                   const float* x, int32_t m, const float* gain, float eps,
+                                                   const float* residual, float* out);
+
 /* Decoder glue with the reference ops' semantics (device pointers):
  *   silu_mul: out[i] = gate[i] * (1 / (1 + exp(-gate[i]))) * up[i]   (NAT:532-539 unary op 2 then binary mul,
  *             REF/skainet-backend-native-cpu/native/src/f32_ops.c:222-244)

@@ -86,6 +86,7 @@ SIGNATURES = {
     "skainet_hip_f32_unary_dev": (_i32, [_i32, _vp, _vp, _i64]),
     "skainet_hip_f32_reduce_all_dev": (_i32, [_vp, _i64, _i32, _vp]),
     "skainet_hip_f32_reduce_axis_dev": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp]),
+    "skainet_hip_mlp_swiglu_dev": (_i32, [_vp, _vp, _vp, _i32, _vp, _f32, _vp, _vp]),
     "skainet_hip_attn_out_proj_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _vp, _vp]),
     "skainet_hip_f32_sdpa_cache_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _i32,
                                               _vp]),

@@ -63,6 +63,16 @@ __global__ __launch_bounds__(256) void gemm_prepass_kernel(const float* __restri
     }
 }
 
+// The same pass over rows of interleaved (gate, up) pairs: out[i] = bf16(silu(in[2 i]) * in[2 i + 1]), four per thread.
+__global__ __launch_bounds__(256) void gemm_prepass_swiglu_kernel(const float* __restrict__ in, __bf16* __restrict__ out, int64_t n4) {
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const float4 a = reinterpret_cast<const float4*>(in)[2 * i], b = reinterpret_cast<const float4*>(in)[2 * i + 1];
+    auto act = [](float g, float u) { return g * (1.0f / (1.0f + expf(-g))) * u; };
+    reinterpret_cast<bf16x4*>(out)[i] = bf16x4{(__bf16)act(a.x, a.y), (__bf16)act(a.z, a.w), (__bf16)act(b.x, b.y), (__bf16)act(b.z, b.w)};
+}
+
 // The same pass with an RMSNorm folded in: out = bf16(x / sqrt(mean(x^2) + eps) * gain), one workgroup per activation row,
 // the row held in registers between the sum of squares and the scaling (k a multiple of 4, at most 256 * 4 * V floats).
 template <int V>
@@ -667,8 +677,9 @@ bool gemm_ksw_enabled();
 bool gemm_ksw_fits(int m, int n, int k);
 bool gemm_ksw_forced();
 size_t gemm_frag_activation_bytes(int m, int k);                                                              // gemm_q4k_frag.hip
-int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, const uint8_t* w, int n, hipStream_t s);
-int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s);
+int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, const uint8_t* w, int n, hipStream_t s,
+                             bool pairs);
+int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s, const float* residual);
 bool gemm_frag_enabled();
 bool gemm_frag_fits(int m, int n, int k);
 bool gemm_frag_forced();
@@ -685,8 +696,10 @@ void set_gemm_rows(int v) { if (v == 0 || v == 2 || v == 4) g_gemm_rows = v; }
 // `tmp` ([m, n] floats, needed when an epilogue is asked for) takes the plain product when K is not split.
 // Returns 1, having launched nothing, when the shape is outside the tile kernel's range and a prologue or epilogue was
 // asked for (the caller composes the same arithmetic from separate launches).
+// x_pairs: x is [m, 2 k], rows of interleaved (gate, up) pairs, and the product's activation is their SwiGLU, taken in
+// the pass that rounds to bf16 (no gain then).
 int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y, const float* gain, float eps,
-                      const float* residual, int epilogue, float* tmp) {
+                      const float* residual, int epilogue, float* tmp, bool x_pairs) {
     if (m <= 0 || n <= 0) return 0;
     if (!is_packed(enc)) return set_error("gemm: unsupported encoding %d", enc);
     if (k <= 0 || k % block_elems(enc) != 0)
@@ -694,7 +707,8 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     // shapes the tile loader cannot take (a Q8_0 row that is not a whole number of 256-element groups: the K loop
     // runs pairs of 64-element steps over whole groups; unaligned operands) go through the row kernels: same result
     // to fp32 rounding, the weight streamed once per 4 rows
-    const bool fused = gain != nullptr || epilogue != GEMM_EPI_NONE;
+    const bool fused = gain != nullptr || epilogue != GEMM_EPI_NONE || x_pairs;
+    if (x_pairs && gain) return set_error("gemm: a SwiGLU prologue takes no RMSNorm gain");
     if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(x) & 15) ||
         (gain && ((reinterpret_cast<uintptr_t>(gain) & 15) || k > 256 * 4 * 16)) || (epilogue == GEMM_EPI_SWIGLU && (n & 1)) ||
         (epilogue != GEMM_EPI_NONE && !tmp))
@@ -702,7 +716,8 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     hipStream_t s = current_stream();
     auto round_activations = [&](__bf16* a) -> int {            // fp32 -> bf16, with the RMSNorm of a fused call folded in
         const int64_t n4 = (int64_t)m * k / 4;                  // k is a multiple of 64
-        if (!gain) gemm_prepass_kernel<<<dim3((unsigned)((n4 + 256 * PREPASS_UNROLL - 1) / (256 * PREPASS_UNROLL))), dim3(256), 0, s>>>(x, a, n4);
+        if (x_pairs) gemm_prepass_swiglu_kernel<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s>>>(x, a, n4);
+        else if (!gain) gemm_prepass_kernel<<<dim3((unsigned)((n4 + 256 * PREPASS_UNROLL - 1) / (256 * PREPASS_UNROLL))), dim3(256), 0, s>>>(x, a, n4);
         else if (k <= 256 * 4 * 4) gemm_prepass_rmsnorm_kernel<4><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
         else gemm_prepass_rmsnorm_kernel<16><<<dim3(m), dim3(256), 0, s>>>(x, gain, a, k, eps);
         SKH_CHECK(hipGetLastError());
@@ -723,9 +738,10 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
     auto run_frag = [&]() -> int {                               // Q4_K: the same tiles, activations in fragment order
         uint8_t* a = static_cast<uint8_t*>(kernel_workspace(gemm_frag_activation_bytes(m, k)));
         if (!a) return -1;
-        if (launch_gemm_frag_prepass(x, gain, eps, a, m, k, w, n, s) != 0) return -1;
-        if (launch_q4k_gemm_frag(a, w, epilogue != GEMM_EPI_NONE ? tmp : y, m, n, k, s) != 0) return -1;
-        return finish();
+        if (launch_gemm_frag_prepass(x, gain, eps, a, m, k, w, n, s, x_pairs) != 0) return -1;
+        // the residual is added where the tile is stored; only SwiGLU still parks the plain product
+        if (epilogue == GEMM_EPI_SWIGLU) return launch_q4k_gemm_frag(a, w, tmp, m, n, k, s, nullptr) != 0 ? -1 : finish();
+        return launch_q4k_gemm_frag(a, w, y, m, n, k, s, epilogue == GEMM_EPI_RESIDUAL ? residual : nullptr);
     };
     const bool ksw_ok = enc == ENC_Q4_K && gemm_ksw_fits(m, n, k) && g_gemm_wide.load() < 0 && g_gemm_rows.load() == 0;
     const bool frag_ok = ksw_ok && gemm_frag_fits(m, n, k);
@@ -804,7 +820,7 @@ int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, i
 }
 
 int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y) {
-    return launch_gemm_fused(enc, w, x, m, k, n, y, nullptr, 0.f, nullptr, GEMM_EPI_NONE, nullptr);
+    return launch_gemm_fused(enc, w, x, m, k, n, y, nullptr, 0.f, nullptr, GEMM_EPI_NONE, nullptr, false);
 }
 
 }  // namespace skh

@@ -96,7 +96,11 @@ __device__ __forceinline__ uint32_t frg_touch_weight(const FrgTouch& t, int id, 
 //   x[32 it + r][64 (s / 4) + 16 h + 4 t + 0..3] and x[32 it + r][64 (s / 4) + 32 + 16 h + 4 t + 0..3].
 // Thread (r, c) of a workgroup (c = 4 h + t) reads the two float4s and writes the piece: a wave reads eight row
 // segments of 128 bytes twice and writes eight runs of 128 bytes.
-template <int PIECES>
+// PAIRS: the input is [m, 2 k], rows of interleaved (gate, up) pairs, and the activation is their SwiGLU,
+// x[row][j] = silu(in[row][2 j]) * in[row][2 j + 1] (the arithmetic of swiglu_pairs_kernel): the product of a gate/up
+// projection goes into the down projection without its activation ever being stored as fp32.
+__device__ __forceinline__ float frg_silu_mul(float g, float u) { return g * (1.0f / (1.0f + expf(-g))) * u; }
+template <int PIECES, bool PAIRS = false>
 __global__ __launch_bounds__(256) void gemm_frag_prepass_kernel(const float* __restrict__ in, uint8_t* __restrict__ out, int m, int k,
                                                                 FrgTouch touch) {
     // a workgroup takes PIECES consecutive 64-element groups of one row tile; all its loads are issued before the first
@@ -104,10 +108,21 @@ __global__ __launch_bounds__(256) void gemm_frag_prepass_kernel(const float* __r
     const int g0 = blockIdx.x * PIECES, it = blockIdx.y;
     const int r = threadIdx.x >> 3, c = threadIdx.x & 7;
     const int row = 32 * it + r;
-    const float* src = in + (int64_t)min(row, m - 1) * k + 64 * g0 + 4 * c;
     float4 lo[PIECES], hi[PIECES];
+    if constexpr (PAIRS) {
+        const float* src = in + ((int64_t)min(row, m - 1) * k + 64 * g0 + 4 * c) * 2;
 #pragma unroll
-    for (int p = 0; p < PIECES; ++p) { lo[p] = *reinterpret_cast<const float4*>(src + 64 * p); hi[p] = *reinterpret_cast<const float4*>(src + 64 * p + 32); }
+        for (int p = 0; p < PIECES; ++p) {
+            const float4 a0 = *reinterpret_cast<const float4*>(src + 128 * p), a1 = *reinterpret_cast<const float4*>(src + 128 * p + 4);
+            const float4 b0 = *reinterpret_cast<const float4*>(src + 128 * p + 64), b1 = *reinterpret_cast<const float4*>(src + 128 * p + 68);
+            lo[p] = make_float4(frg_silu_mul(a0.x, a0.y), frg_silu_mul(a0.z, a0.w), frg_silu_mul(a1.x, a1.y), frg_silu_mul(a1.z, a1.w));
+            hi[p] = make_float4(frg_silu_mul(b0.x, b0.y), frg_silu_mul(b0.z, b0.w), frg_silu_mul(b1.x, b1.y), frg_silu_mul(b1.z, b1.w));
+        }
+    } else {
+        const float* src = in + (int64_t)min(row, m - 1) * k + 64 * g0 + 4 * c;
+#pragma unroll
+        for (int p = 0; p < PIECES; ++p) { lo[p] = *reinterpret_cast<const float4*>(src + 64 * p); hi[p] = *reinterpret_cast<const float4*>(src + 64 * p + 32); }
+    }
     __builtin_amdgcn_sched_barrier(0);                         // the pass's own loads are issued first
     const uint32_t seen = frg_touch_weight(touch, blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
     __builtin_amdgcn_sched_barrier(0);
@@ -214,7 +229,7 @@ __device__ __forceinline__ void frg_decode4(uint32_t c, uint32_t c8, float scale
 }
 
 __global__ __launch_bounds__(64 * FRG_WAVES) void q4k_gemm_frag_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ w,
-                                                                       float* __restrict__ c, int m, int n, int k, FrgTileOrder order) {
+                                                                       float* c, const float* residual, int m, int n, int k, FrgTileOrder order) {
     extern __shared__ __attribute__((aligned(16))) uint8_t frg_smem[];   // the kernel has no other LDS: offsets into it are LDS addresses
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -423,13 +438,17 @@ __global__ __launch_bounds__(64 * FRG_WAVES) void q4k_gemm_frag_kernel(const uin
         }
         const int gr = m0 + row, gc = n0 + c4;
         if (gr < m) {
+            // residual (may be c itself: every element is read and then written by this one thread): c = residual + product
             float* dst = c + (int64_t)gr * n + gc;
-            if (gc + 3 < n && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) *reinterpret_cast<float4*>(dst) = sum;
-            else {
-                if (gc < n) dst[0] = sum.x;
-                if (gc + 1 < n) dst[1] = sum.y;
-                if (gc + 2 < n) dst[2] = sum.z;
-                if (gc + 3 < n) dst[3] = sum.w;
+            const float* res = residual ? residual + (int64_t)gr * n + gc : nullptr;
+            if (gc + 3 < n && ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(res)) & 15) == 0) {
+                if (res) { const float4 t = *reinterpret_cast<const float4*>(res); sum.x = t.x + sum.x; sum.y = t.y + sum.y; sum.z = t.z + sum.z; sum.w = t.w + sum.w; }
+                *reinterpret_cast<float4*>(dst) = sum;
+            } else {
+                if (gc < n) dst[0] = (res ? res[0] : 0.f) + sum.x;
+                if (gc + 1 < n) dst[1] = (res ? res[1] : 0.f) + sum.y;
+                if (gc + 2 < n) dst[2] = (res ? res[2] : 0.f) + sum.z;
+                if (gc + 3 < n) dst[3] = (res ? res[3] : 0.f) + sum.w;
             }
         }
     }
@@ -464,11 +483,16 @@ void set_gemm_frag_touch(int v) { g_gemm_frag_touch = v != 0; }
 static std::atomic<int> g_gemm_frag_pieces{1};  // 64-element groups a workgroup of the plain pass takes (1, 2 or 4)
 void set_gemm_frag_pieces(int v) { if (v == 1 || v == 2 || v == 4) g_gemm_frag_pieces = v; }
 // `w` ([n, k] packed Q4_K, or null) is the weight of the product that follows: the plain pass touches its lines on the way.
-int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, const uint8_t* w, int n, hipStream_t s) {
+// `pairs`: x is [m, 2 k] rows of (gate, up) pairs and the activation their SwiGLU (no gain then).
+int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8_t* a, int m, int k, const uint8_t* w, int n, hipStream_t s,
+                             bool pairs) {
     const int row_tiles = (m + FRG_M - 1) / FRG_M * (FRG_M / 32);
     const FrgTouch touch{g_gemm_frag_touch.load() ? w : nullptr, (uint32_t)(k >> 8) * 144u, n, frg_tile_order(m, n)};
     const int pieces = g_gemm_frag_pieces.load();
-    if (!gain) {
+    if (pairs) {
+        if (gain) return set_error("gemm: a SwiGLU prologue takes no RMSNorm gain");
+        gemm_frag_prepass_kernel<1, true><<<dim3(k / 64, row_tiles), dim3(256), 0, s>>>(x, a, m, k, touch);
+    } else if (!gain) {
         if (pieces == 4 && k % 256 == 0) gemm_frag_prepass_kernel<4><<<dim3(k / 256, row_tiles), dim3(256), 0, s>>>(x, a, m, k, touch);
         else if (pieces >= 2 && k % 128 == 0) gemm_frag_prepass_kernel<2><<<dim3(k / 128, row_tiles), dim3(256), 0, s>>>(x, a, m, k, touch);
         else gemm_frag_prepass_kernel<1><<<dim3(k / 64, row_tiles), dim3(256), 0, s>>>(x, a, m, k, touch);
@@ -480,12 +504,13 @@ int launch_gemm_frag_prepass(const float* x, const float* gain, float eps, uint8
 }
 
 // C = A . W^T for activations already in fragment order; k a multiple of 256, operands 16-byte aligned. 0 on success.
-int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s) {
+// residual != null: c = residual + A . W^T (residual [m, n], may be c).
+int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, int n, int k, hipStream_t s, const float* residual) {
     if (!gemm_frag_fits(m, n, k)) return set_error("gemm: operands of %d x %d x %d are outside this kernel's range", m, n, k);
     const FrgTileOrder order = frg_tile_order(m, n);
     note_kernel("q4k_gemm_frag_kernel");
     SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_frag_kernel), FRG_SMEM);
-    q4k_gemm_frag_kernel<<<dim3(order.tiles_m * order.tiles_n), dim3(64 * FRG_WAVES), FRG_SMEM, s>>>(a, w, c, m, n, k, order);
+    q4k_gemm_frag_kernel<<<dim3(order.tiles_m * order.tiles_n), dim3(64 * FRG_WAVES), FRG_SMEM, s>>>(a, w, c, residual, m, n, k, order);
     SKH_CHECK(hipGetLastError());
     return 0;
 }

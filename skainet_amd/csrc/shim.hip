@@ -25,7 +25,7 @@ int launch_dequant(int enc, const uint8_t* w, int64_t nblocks, float* out, const
 int launch_gemv(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
 int launch_gemm(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y);
 int launch_gemm_fused(int enc, const uint8_t* w, const float* x, int m, int k, int n, float* y, const float* gain, float eps,
-                      const float* residual, int epilogue, float* tmp);
+                      const float* residual, int epilogue, float* tmp, bool x_pairs);
 int set_tuning(const char* key, int value);
 int launch_rms_norm(const float* in, const float* gamma, float* out, int rows, int cols, float eps);
 int launch_layer_norm(const float* in, const float* gamma, const float* beta, float* out, int rows, int cols, float eps);
@@ -70,7 +70,7 @@ static thread_local hipEvent_t t_ev0 = nullptr, t_ev1 = nullptr;
 struct Scratch { void* ptr = nullptr; size_t cap = 0; };
 static thread_local Scratch t_workspace;          // kernel scratch (attention split-K partials, GEMM staging)
 static thread_local Scratch t_stage[6];           // device staging of the host-pointer entries
-static thread_local Scratch t_fuse[2];            // normalised input / raw product of the unfused route of matmul_fused
+static thread_local Scratch t_fuse[3];            // normalised input / raw product of the unfused route of matmul_fused / (gate, up) product of the MLP entry
 static thread_local Scratch t_pinned[2];          // page-locked host staging of skainet_hip_matmul_host (activations in, product out)
 static std::atomic<int> g_upload_chunk_mib{8};    // skainet_hip_weight_upload's page-locked chunks; 0: one blocking copy straight from the caller's memory
 static std::atomic<int> g_upload_lanes{4};        // host threads that fill them
@@ -539,7 +539,7 @@ int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x
         // sums K splits (no split: a row kernel over the plain product, parked in tmp)
         float* tmp = epilogue != 0 ? static_cast<float*>(scratch_get(t_fuse[1], sizeof(float) * (size_t)m * w->rows)) : nullptr;
         if (epilogue != 0 && !tmp) return -1;
-        const int r = launch_gemm_fused(w->encoding, w->data, x, m, w->cols, w->rows, out, gain, eps, residual, epilogue, tmp);
+        const int r = launch_gemm_fused(w->encoding, w->data, x, m, w->cols, w->rows, out, gain, eps, residual, epilogue, tmp, false);
         if (r <= 0) return r;
     }
     const float* xin = x;
@@ -557,6 +557,44 @@ int32_t skainet_hip_matmul_fused_dev(const skainet_hip_weight* w, const float* x
     if (epilogue == 1) return launch_add(residual, y, out, (int64_t)m * w->rows);
     if (epilogue == 2) return launch_swiglu_pairs(y, out, (int64_t)m * (w->rows / 2));
     return 0;
+}
+// A gated MLP block: out = (residual ? residual : 0) + Wdown . swiglu(Wgate_up . rmsnorm(x)), Wgate_up's rows interleaved
+// (gate_0, up_0, gate_1, up_1, ...). Prompt shapes (m > 8) of packed weights: the (gate, up) product is parked once, as
+// fp32 pairs, and the pass that rounds the down projection's activations to bf16 takes the SwiGLU on the way -- the
+// activation itself is never stored as fp32 -- and the residual is added where the down projection stores its tiles.
+// Everything else is the two fused products in a row.
+int32_t skainet_hip_mlp_swiglu_dev(const skainet_hip_weight* w_gate_up, const skainet_hip_weight* w_down, const float* x, int32_t m,
+                                   const float* gain, float eps, const float* residual, float* out) {
+    if (ensure_device() != 0) return -1;
+    if (!w_gate_up || !w_down) return set_error("mlp_swiglu: null weight handle");
+    if (m <= 0) return 0;
+    if (!x || !out) return set_error("mlp_swiglu: null activation or output pointer");
+    if (w_gate_up->rows & 1) return set_error("mlp_swiglu: the gate/up weight needs an even row count; got %d", w_gate_up->rows);
+    if (w_down->cols != w_gate_up->rows / 2)
+        return set_error("mlp_swiglu: the down projection takes %d inputs, the gate/up product gives %d", w_down->cols, w_gate_up->rows / 2);
+    const int ffn = w_down->cols;
+    if (m > 8 && is_packed(w_gate_up->encoding) && is_packed(w_down->encoding)) {
+        float* pairs = static_cast<float*>(scratch_get(t_fuse[2], sizeof(float) * (size_t)m * w_gate_up->rows));
+        float* tmp = residual ? static_cast<float*>(scratch_get(t_fuse[1], sizeof(float) * (size_t)m * w_down->rows)) : nullptr;
+        if (!pairs || (residual && !tmp)) return -1;
+        int r = launch_gemm_fused(w_gate_up->encoding, w_gate_up->data, x, m, w_gate_up->cols, w_gate_up->rows, pairs, gain, eps, nullptr, 0,
+                                  nullptr, false);
+        if (r < 0) return -1;
+        if (r == 0) {
+            r = launch_gemm_fused(w_down->encoding, w_down->data, pairs, m, ffn, w_down->rows, out, nullptr, 0.f, residual, residual ? 1 : 0,
+                                  tmp, true);
+            if (r < 0) return -1;
+            if (r == 0) return 0;
+            // the down projection's shape is outside the tile kernels: finish from the parked pairs
+            float* act = static_cast<float*>(scratch_get(t_fuse[0], sizeof(float) * (size_t)m * ffn));
+            if (!act || launch_swiglu_pairs(pairs, act, (int64_t)m * ffn) != 0) return -1;
+            return skainet_hip_matmul_fused_dev(w_down, act, m, out, nullptr, 0.f, residual, residual ? 1 : 0);
+        }
+    }
+    float* act = static_cast<float*>(scratch_get(t_fuse[2], sizeof(float) * (size_t)m * ffn));
+    if (!act) return -1;
+    if (skainet_hip_matmul_fused_dev(w_gate_up, x, m, act, gain, eps, nullptr, 2) != 0) return -1;
+    return skainet_hip_matmul_fused_dev(w_down, act, m, out, nullptr, 0.f, residual, residual ? 1 : 0);
 }
 // One decode token's q/k/v projection with everything around it: out row = W . rmsnorm(x) (gain == NULL: no norm),
 // W's rows being [q | k | v] heads of head_dim; adjacent pairs of the q and k heads are rotated (RoPE, angle

@@ -369,8 +369,12 @@ class LlamaDecoder:
             if rows > 1:
                 kx.heads_to_rows_dev(self.attn, self.attn_rows, c.heads, rows, c.head_dim)
             L.wo.matmul_fused(self.attn_rows if rows > 1 else self.attn, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
-        L.w_gate_up.matmul_fused(self.h, rows, self.act, gain=L.ffn_norm, eps=c.rms_eps, epilogue=kx.EPI_SWIGLU)
-        L.w_down.matmul_fused(self.act, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
+        if rows > 8:
+            # prompt rows: the block in one call (the SwiGLU rides in the down projection's rounding pass)
+            L.w_gate_up.mlp_swiglu(L.w_down, self.h, rows, self.h, gain=L.ffn_norm, eps=c.rms_eps, residual=self.h)
+        else:
+            L.w_gate_up.matmul_fused(self.h, rows, self.act, gain=L.ffn_norm, eps=c.rms_eps, epilogue=kx.EPI_SWIGLU)
+            L.w_down.matmul_fused(self.act, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
 
     def _head(self, row: int) -> None:
         c = self.cfg

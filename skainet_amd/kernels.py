@@ -207,6 +207,12 @@ class DeviceWeight:
                                                        seq_kv, kv_capacity, scale, window, _ptr(lengths), _ptr(residual),
                                                        _ptr(out), _ptr(attn_tmp)), "attn_out_proj")
 
+    def mlp_swiglu(self, w_down: "DeviceWeight", x, m: int, out, gain=None, eps: float = 0.0, residual=None) -> None:
+        """self holds interleaved (gate, up) rows: out = (residual or 0) + Wdown . swiglu(self . rmsnorm(x))
+        (skainet_hip_mlp_swiglu_dev)."""
+        check(_lib.hip().skainet_hip_mlp_swiglu_dev(self._h, w_down._h, _ptr(x), m, _ptr(gain), eps, _ptr(residual), _ptr(out)),
+              "mlp_swiglu")
+
     def dequantize(self, out) -> None:
         check(_lib.hip().skainet_hip_dequantize_dev(self._h, _ptr(out)), "dequantize")
 

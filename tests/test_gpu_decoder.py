@@ -194,6 +194,58 @@ def test_matmul_fused_equals_composed(hip_backend, torch_cuda, enc, n, k, m):
         w.matmul_fused(d_x, m, out, epilogue=7)
 
 
+@pytest.mark.parametrize("enc,hidden,ffn,m", [("Q4_K", 512, 768, 40), ("Q4_K", 1024, 2816, 130), ("Q4_K", 256, 512, 3), ("Q6_K", 512, 512, 33),
+                                               ("Q8_0", 96, 160, 12), ("Q4_K", 4096, 14336, 64)])
+def test_mlp_swiglu_equals_float64_and_the_two_fused_products(hip_backend, torch_cuda, enc, hidden, ffn, m):
+    """The gated MLP block in one call against float64 arithmetic on the oracle-decoded weights (2e-2 of the largest output
+    for prompt rows on the bf16 matrix cores, 1e-3 for up to 8 rows) and against the two fused products it replaces, with
+    and without the norm and the residual (aliasing the output); Q4_K prompt rows run the fragment-order kernel for the
+    down projection when it is forced, with the SwiGLU in its rounding pass and the residual in its store."""
+    from oracle import lib as O
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(hidden + ffn + m)
+    pgu = kx.quantize(enc, (rng.standard_normal((2 * ffn, hidden)) * 0.05).astype(np.float32))
+    pdn = kx.quantize(enc, (rng.standard_normal((hidden, ffn)) * 0.05).astype(np.float32))
+    wgu_h = O.dequant(enc, pgu).reshape(2 * ffn, hidden).astype(np.float64)
+    wdn_h = O.dequant(enc, pdn).reshape(hidden, ffn).astype(np.float64)
+    wgu, wdn = kx.DeviceWeight.upload(enc, pgu, 2 * ffn, hidden), kx.DeviceWeight.upload(enc, pdn, hidden, ffn)
+    x = (rng.standard_normal((m, hidden)) * 2).astype(np.float32)
+    gain = (1 + 0.2 * rng.standard_normal(hidden)).astype(np.float32)
+    res = rng.standard_normal((m, hidden)).astype(np.float32)
+    eps = 1e-5
+    tol = 2e-2 if m > 8 else 1e-3
+    xd = x.astype(np.float64)
+    xn = xd / np.sqrt((xd * xd).mean(1, keepdims=True) + eps) * gain
+    d_x, d_gain = dev(torch, x), dev(torch, gain)
+    act = torch.empty((m, ffn), device="cuda")
+    for frag in ((1, 2) if enc == "Q4_K" and m > 8 else (1,)):
+        try:
+            kx.set_tuning("gemm_frag", frag)
+            for use_gain in (False, True):
+                p = (xn if use_gain else xd) @ wgu_h.T
+                a = p[:, 0::2] / (1 + np.exp(-p[:, 0::2])) * p[:, 1::2]
+                for use_res in (False, True):
+                    want = a @ wdn_h.T + (res if use_res else 0.0)
+                    out = dev(torch, res.copy()) if use_res else torch.full((m, hidden), 9.0, device="cuda")
+                    wgu.mlp_swiglu(wdn, d_x, m, out, gain=d_gain if use_gain else None, eps=eps, residual=out if use_res else None)
+                    kx.sync()
+                    if frag == 2:
+                        assert kx.last_kernel() == "q4k_gemm_frag_kernel"
+                    got = out.cpu().numpy()
+                    assert max_norm_err(got, want) < tol, (frag, use_gain, use_res)
+                    two = dev(torch, res.copy()) if use_res else torch.full((m, hidden), 9.0, device="cuda")
+                    wgu.matmul_fused(d_x, m, act, gain=d_gain if use_gain else None, eps=eps, epilogue=kx.EPI_SWIGLU)
+                    wdn.matmul_fused(act, m, two, residual=two if use_res else None, epilogue=kx.EPI_RESIDUAL if use_res else kx.EPI_NONE)
+                    kx.sync()
+                    # the same operands rounded at the same places: only the order of fp32 sums may differ
+                    assert max_norm_err(got, two.cpu().numpy().astype(np.float64)) < 1e-4, (frag, use_gain, use_res)
+        finally:
+            kx.set_tuning("gemm_frag", 1)
+    from skainet_amd._lib import HipError
+    with pytest.raises(HipError):
+        wdn.mlp_swiglu(wdn, d_x, m, act)                               # not a (gate, up) weight for this down projection
+
+
 @pytest.mark.parametrize("enc,heads,kvh,hd,k", [("Q4_K", 8, 2, 64, 512), ("Q4_K", 32, 8, 128, 4096), ("Q4_K", 3, 1, 64, 256),
                                                 ("Q6_K", 4, 2, 64, 512), ("Q4_K", 5, 1, 64, 1024), ("Q4_K", 8, 4, 128, 2048)])
 def test_matmul_qkv_rope_equals_product_then_rope(hip_backend, torch_cuda, enc, heads, kvh, hd, k):
