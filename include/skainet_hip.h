@@ -290,6 +290,12 @@ SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_dev(const float* q, const float* k,
 SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_cache_dev(const float* q, const float* k_cache, const float* v_cache, float* out,
     int32_t batch, int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t kv_capacity, int32_t head_dim,
     float scale, int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths);
+/* The same with the output laid out [batch, seq_q, heads, head_dim] -- token rows, which is what the output projection
+ * multiplies -- so a prompt pass needs no transposing launch between attention and projection. No reference counterpart
+ * (the reference's attention output is head-major, f32_fused.c:290-396; its callers transpose). */
+SKAINET_HIP_API int32_t skainet_hip_f32_sdpa_cache_rows_dev(const float* q, const float* k_cache, const float* v_cache, float* out,
+    int32_t batch, int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t kv_capacity, int32_t head_dim,
+    float scale, int32_t causal, int32_t window, int32_t right_context, const int32_t* lengths);
 /* One decode token's attention over the KV cache and the output projection behind it:
  *   out[rows of wo] = (residual ? residual : 0) + Wo . sdpa(q [heads, head_dim], cache [kv_heads, kv_capacity, head_dim]),
  * causal over seq_kv keys (or lengths[0] of them when `lengths` is given: a device-side key count, so a recorded graph

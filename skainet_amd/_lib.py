@@ -90,6 +90,8 @@ SIGNATURES = {
     "skainet_hip_attn_out_proj_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _vp, _vp]),
     "skainet_hip_f32_sdpa_cache_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _i32,
                                               _vp]),
+    "skainet_hip_f32_sdpa_cache_rows_dev": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _i32,
+                                                   _i32, _vp]),
     "skainet_hip_f32_silu_mul_dev": (_i32, [_vp, _vp, _vp, _i64]),
     "skainet_hip_f32_add_dev": (_i32, [_vp, _vp, _vp, _i64]),
     "skainet_hip_f32_argmax_rows_dev": (_i32, [_vp, _i32, _i32, _vp]),

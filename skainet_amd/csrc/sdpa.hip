@@ -181,7 +181,7 @@ int launch_sdpa_decode(const float* q, const float* k, const float* v, float* ou
 int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                         int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window,
                         int right_context, const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q,
-                        int mask_k);   // sdpa_prefill.hip
+                        int mask_k, int out_rows);   // sdpa_prefill.hip
 
 int launch_sdpa(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                 int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window, int right_context,
@@ -213,7 +213,7 @@ int launch_sdpa(const float* q, const float* k, const float* v, float* out, int 
     }
     if (seq_q > 1) {   // prompt shape: the matrix-core kernel, when it carries the shape (and the mask's layout)
         const int r = launch_sdpa_prefill(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale, causal,
-                                          window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k);
+                                          window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k, 0);
         if (r != 0) return r < 0 ? -1 : 0;
     }
     SdpaParams p{q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, head_dim, kv_capacity, scale, causal, window, right_context,

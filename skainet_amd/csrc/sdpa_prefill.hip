@@ -99,6 +99,7 @@ struct PrefillParams {
     int heads_per_wg;      // 1, 2 or 4 query heads of one KV head per workgroup
     const float* mask;         // additive mask or null; dims 1 or the full extent (heads: 1, kv_heads or heads)
     int mask_b, mask_h, mask_q, mask_k;
+    int out_rows;              // 0: out is [batch, heads, seq_q, D]; 1: [batch, seq_q, heads, D], token rows of a projection's input
 };
 
 // One 64-key block of the bf16 K and V^T copies: global -> registers, and registers -> the LDS tiles.
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(256 * TEAMS, TEAMS == 1 ? 2 : 1) void sdpa_prefill_
     const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     if (my_q < p.seq_q && team_active) {
-        float* op = p.out + (((int64_t)b * p.heads + head) * p.seq_q + my_q) * D;
+        float* op = p.out + (p.out_rows ? (((int64_t)b * p.seq_q + my_q) * p.heads + head) : (((int64_t)b * p.heads + head) * p.seq_q + my_q)) * D;
 #pragma unroll
         for (int i = 0; i < ND; ++i)
 #pragma unroll
@@ -386,7 +387,7 @@ void set_sdpa_prefill_teams(int v) { if (v >= 0 && v <= 2) g_prefill_teams = v; 
 template <int D>
 static int launch_prefill_d(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                             int seq_q, int seq_kv, int kv_capacity, float scale, int causal, int window, int right_context,
-                            const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k) {
+                            const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k, int out_rows) {
     const int spad = (seq_kv + PF_KB - 1) / PF_KB * PF_KB;
     const size_t elems = (size_t)batch * kv_heads * spad * D;
     __bf16* ws = static_cast<__bf16*>(kernel_workspace(2 * elems * sizeof(__bf16)));
@@ -400,7 +401,7 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
     const int q_per_group = (4 / hpw) * PF_QW;
     const int ngroups = (seq_q + q_per_group - 1) / q_per_group;
     PrefillParams p{q, kb, vt, out, heads, kv_heads, seq_q, seq_kv, spad, scale * 1.4426950408889634f, causal, window, right_context, lengths, hpw,
-                    mask, mask_b, mask_h, mask_q, mask_k};
+                    mask, mask_b, mask_h, mask_q, mask_k, out_rows};
     // paired query groups where that still gives every CU a workgroup, else one group per (smaller) workgroup
     const int64_t paired_wgs = (int64_t)((ngroups + 1) / 2) * kv_heads * (per_kv / hpw) * batch;
     const bool paired = g_prefill_teams.load() == 0 ? paired_wgs >= num_cus() : g_prefill_teams.load() == 2;
@@ -422,7 +423,7 @@ static int launch_prefill_d(const float* q, const float* k, const float* v, floa
 int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads,
                         int seq_q, int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window,
                         int right_context, const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q,
-                        int mask_k) {
+                        int mask_k, int out_rows) {
     if (!g_prefill_mfma) return 0;
     // a mask row is read four keys at a time: rows of a multiple of four keys from a 16-byte aligned base (or one value per row)
     if (mask && mask_k != 1 && ((mask_k & 3) || (reinterpret_cast<uintptr_t>(mask) & 15))) return 0;
@@ -431,8 +432,8 @@ int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* o
     if (batch > 65535 || (int64_t)kv_heads * heads > 65535) return 0;
     if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
          reinterpret_cast<uintptr_t>(out)) & 15) return 0;
-    if (head_dim == 64) return launch_prefill_d<64>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k);
-    return launch_prefill_d<128>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k);
+    if (head_dim == 64) return launch_prefill_d<64>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k, out_rows);
+    return launch_prefill_d<128>(q, k, v, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, scale, causal, window, right_context, lengths, mask, mask_b, mask_h, mask_q, mask_k, out_rows);
 }
 
 }  // namespace skh

@@ -46,6 +46,9 @@ int launch_narrow_matmul(const float* a, int64_t a_stride, const uint8_t* b, int
                          int m, int n, int k, int fp16);
 int launch_decode_advance(int32_t* pos, int32_t* kv_len, const int32_t* token, int32_t* log, int32_t capacity);
 int launch_heads_to_rows(const float* in, float* out, int heads, int tokens, int head_dim);
+int launch_sdpa_prefill(const float* q, const float* k, const float* v, float* out, int batch, int heads, int kv_heads, int seq_q,
+                        int seq_kv, int kv_capacity, int head_dim, float scale, int causal, int window, int right_context,
+                        const int32_t* lengths, const float* mask, int mask_b, int mask_h, int mask_q, int mask_k, int out_rows);
 int launch_i32_increment(int32_t* v, int32_t delta);
 int launch_stream_read(const void* p, int64_t bytes, int grid, uint32_t* sink);
 int launch_relayout_to_row_major(const uint8_t* src, uint8_t* dst, int rows, int bpr, int block_bytes);
@@ -768,6 +771,31 @@ int32_t skainet_hip_f32_sdpa_cache_dev(const float* q, const float* k_cache, con
     if (ensure_device() != 0) return -1;
     return launch_sdpa(q, k_cache, v_cache, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale, causal,
                        window, right_context, lengths, nullptr, 0, 0, 0, 0);
+}
+// skainet_hip_f32_sdpa_cache_dev with the output laid out [batch, seq_q, heads, head_dim]: token rows, the input of the
+// output projection as it is. Prompt shapes that the matrix-core kernel carries are stored that way by the kernel; every
+// other shape runs the head-major attention into scratch and one transposing pass per sequence.
+int32_t skainet_hip_f32_sdpa_cache_rows_dev(const float* q, const float* k_cache, const float* v_cache, float* out, int32_t batch,
+                                            int32_t heads, int32_t kv_heads, int32_t seq_q, int32_t seq_kv, int32_t kv_capacity,
+                                            int32_t head_dim, float scale, int32_t causal, int32_t window, int32_t right_context,
+                                            const int32_t* lengths) {
+    if (ensure_device() != 0) return -1;
+    if (batch <= 0 || heads <= 0 || kv_heads <= 0 || seq_q <= 0 || head_dim <= 0) return 0;
+    const bool plain = heads % kv_heads == 0 && window >= 0 && right_context >= 0 && (right_context == 0 || window != 0) &&
+                       kv_capacity >= seq_kv && seq_kv > 0;
+    if (plain && seq_q > 1) {
+        const int r = launch_sdpa_prefill(q, k_cache, v_cache, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale,
+                                          causal, window, right_context, lengths, nullptr, 0, 0, 0, 0, 1);
+        if (r != 0) return r < 0 ? -1 : 0;
+    }
+    const size_t per_seq = (size_t)heads * seq_q * head_dim;
+    float* tmp = static_cast<float*>(scratch_get(t_fuse[0], sizeof(float) * per_seq * batch));
+    if (!tmp) return -1;
+    if (launch_sdpa(q, k_cache, v_cache, tmp, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale, causal, window,
+                    right_context, lengths, nullptr, 0, 0, 0, 0) != 0) return -1;     // the argument rules and their messages are its own
+    for (int b = 0; b < batch; ++b)
+        if (launch_heads_to_rows(tmp + b * per_seq, out + b * per_seq, heads, seq_q, head_dim) != 0) return -1;
+    return 0;
 }
 // One decode token: out = (residual ? residual : 0) + Wo . sdpa(q, cache). Q4_K projections whose input is at most 4096
 // wide run as two launches (attention leaving its key splits unmerged, the projection merging them as it loads its

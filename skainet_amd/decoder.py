@@ -364,11 +364,10 @@ class LlamaDecoder:
             L.wo.attn_out_proj(self.q, kc, vc, c.heads, c.kv_heads, c.head_dim, seq_kv, c.ctx_max, scale, self.h, self.attn,
                                residual=self.h, lengths=kv_len_dev)
         else:
-            kx.sdpa_cache_dev(self.q, kc, vc, self.attn, 1, c.heads, c.kv_heads, rows, seq_kv, c.ctx_max, c.head_dim, scale,
-                              True, 0, 0, kv_len_dev)
-            if rows > 1:
-                kx.heads_to_rows_dev(self.attn, self.attn_rows, c.heads, rows, c.head_dim)
-            L.wo.matmul_fused(self.attn_rows if rows > 1 else self.attn, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
+            # attention straight into token rows: what the output projection multiplies
+            kx.sdpa_cache_rows_dev(self.q, kc, vc, self.attn_rows, 1, c.heads, c.kv_heads, rows, seq_kv, c.ctx_max, c.head_dim, scale,
+                                   True, 0, 0, kv_len_dev)
+            L.wo.matmul_fused(self.attn_rows, rows, self.h, residual=self.h, epilogue=kx.EPI_RESIDUAL)
         if rows > 8:
             # prompt rows: the block in one call (the SwiGLU rides in the down projection's rounding pass)
             L.w_gate_up.mlp_swiglu(L.w_down, self.h, rows, self.h, gain=L.ffn_norm, eps=c.rms_eps, residual=self.h)

@@ -299,6 +299,14 @@ def sdpa_cache_dev(q, k_cache, v_cache, out, batch, heads, kv_heads, seq_q, seq_
                                                     right_context, _ptr(key_lengths)), "sdpa_cache")
 
 
+def sdpa_cache_rows_dev(q, k_cache, v_cache, out, batch, heads, kv_heads, seq_q, seq_kv, kv_capacity, head_dim, scale,
+                        causal=False, window=0, right_context=0, key_lengths=None) -> None:
+    """sdpa_cache_dev with the output as token rows, [batch, seq_q, heads, head_dim] (skainet_hip_f32_sdpa_cache_rows_dev)."""
+    check(_lib.hip().skainet_hip_f32_sdpa_cache_rows_dev(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), batch, heads, kv_heads,
+                                                         seq_q, seq_kv, kv_capacity, head_dim, scale, int(causal), window,
+                                                         right_context, _ptr(key_lengths)), "sdpa_cache_rows")
+
+
 def silu_mul_dev(gate, up, out, n: int) -> None:
     check(_lib.hip().skainet_hip_f32_silu_mul_dev(_ptr(gate), _ptr(up), _ptr(out), n), "silu_mul")
 

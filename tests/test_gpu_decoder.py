@@ -306,6 +306,29 @@ def test_sdpa_cache_layout_matches_contiguous(hip_backend, torch_cuda):
         kx.sdpa_cache_dev(out_c, out_c, out_c, out_p, 1, 8, 2, 1, 40, 39, 64, 1.0)
 
 
+@pytest.mark.parametrize("b,h,hkv,sq,skv,cap,d", [(1, 32, 8, 512, 512, 2048, 128), (2, 8, 2, 40, 56, 64, 64), (2, 8, 2, 3, 37, 50, 64),
+                                                    (1, 4, 4, 1, 9, 16, 32)])
+def test_sdpa_cache_rows_is_the_head_major_result_transposed(hip_backend, torch_cuda, b, h, hkv, sq, skv, cap, d):
+    """Attention with the output as token rows ([batch, seq_q, heads, head_dim]: the matrix-core prompt kernel stores it that
+    way itself, other shapes go through a transposing pass) equals the head-major entry's result, element for element."""
+    torch, kx = torch_cuda, hip_backend
+    rng = np.random.default_rng(b + h + sq)
+    q = dev(torch, rng.standard_normal((b, h, sq, d)).astype(np.float32))
+    kc = dev(torch, rng.standard_normal((b, hkv, cap, d)).astype(np.float32))
+    vc = dev(torch, rng.standard_normal((b, hkv, cap, d)).astype(np.float32))
+    lens = dev(torch, np.array([skv, max(1, skv // 2)][:b], np.int32))
+    heads_major = torch.full((b, h, sq, d), 7.0, device="cuda")
+    rows = torch.full((b, sq, h, d), 9.0, device="cuda")
+    scale = float(1.0 / np.sqrt(d))
+    kx.sdpa_cache_dev(q, kc, vc, heads_major, b, h, hkv, sq, skv, cap, d, scale, True, 0, 0, lens)
+    kx.sdpa_cache_rows_dev(q, kc, vc, rows, b, h, hkv, sq, skv, cap, d, scale, True, 0, 0, lens)
+    kx.sync()
+    assert np.array_equal(rows.cpu().numpy(), heads_major.cpu().numpy().transpose(0, 2, 1, 3))
+    from skainet_amd._lib import HipError
+    with pytest.raises(HipError):
+        kx.sdpa_cache_rows_dev(q, kc, vc, rows, b, h, 3, sq, skv, cap, d, scale)        # heads not a multiple of kv_heads
+
+
 def test_graph_replays_match_eager(hip_backend, torch_cuda):
     """A recorded sequence (norm -> packed GEMV -> add -> counter) replayed several times, with eager work and
     synchronisation between the replays, gives the eager result every time."""
