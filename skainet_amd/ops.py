@@ -16,7 +16,7 @@ generic ops be recorded into a HIP graph. Without a scope an output owns a devic
 
 Beyond the reference's TensorOps set (the reference has no transformer; RoPE, the KV cache and the sampler live in an
 external repository) the class carries the four glue ops a decoder needs, marked as such below: `embedding_rows`,
-`rope_scatter`, `argmax_rows`, and integer `advance`.
+`rope_scatter`, `heads_to_rows` and `argmax_rows`.
 """
 from __future__ import annotations
 
@@ -59,6 +59,7 @@ class ForwardScope:
         self.capacity = int(capacity_bytes)
         self._top = 0
         self.high_water = 0
+        self.generation = 0          # resets so far: a tensor handed out before the last one is stale (Scope.kt:206-215)
 
     def allocate(self, nbytes: int) -> int:
         at = (self._top + 255) & ~255
@@ -69,9 +70,12 @@ class ForwardScope:
         return self._slab.ptr + at
 
     def reset(self) -> None:
+        """End of a step: every tensor handed out so far is invalid (its next use raises), the slab starts over."""
         self._top = 0
+        self.generation += 1
 
     def close(self) -> None:
+        self.generation += 1
         self._slab.close()
 
 
@@ -79,13 +83,24 @@ class HipTensor:
     """A dense tensor whose bytes are resident on the device (fp32 unless `dtype` says int32). `owner` keeps the
     allocation alive: an `_Allocation`, a `ForwardScope`, or another tensor (views)."""
 
-    __slots__ = ("shape", "ptr", "owner", "dtype")
+    __slots__ = ("shape", "_ptr", "owner", "dtype", "_scope", "_generation")
 
     def __init__(self, shape: Sequence[int], ptr: int, owner, dtype=np.float32):
         self.shape = tuple(int(s) for s in shape)
-        self.ptr = int(ptr)
+        self._ptr = int(ptr)
         self.owner = owner
         self.dtype = np.dtype(dtype)
+        # a tensor of a forward scope (or a view of one) lives until that scope's next reset
+        self._scope = owner if isinstance(owner, ForwardScope) else getattr(owner, "_scope", None)
+        self._generation = owner.generation if isinstance(owner, ForwardScope) else getattr(owner, "_generation", 0)
+
+    @property
+    def ptr(self) -> int:
+        """The device address; raises once the forward scope that handed the bytes out has been reset or closed (the
+        reference closes a scope's storages at reset, so a later use throws: Scope.kt:206-215)."""
+        if self._scope is not None and self._scope.generation != self._generation:
+            raise HipError(f"tensor {self.shape} belongs to a forward scope that has been reset since")
+        return self._ptr
 
     @property
     def volume(self) -> int:
@@ -140,6 +155,13 @@ class HipOps:
         self._lib = _lib.hip()
 
     # ---- operands and outputs -----------------------------------------------------------------------------------------
+    @staticmethod
+    def _live(*tensors) -> None:
+        """Operands are checked before an output is taken from the scope: a stale one raises without costing slab bytes."""
+        for t in tensors:
+            if isinstance(t, HipTensor):
+                t.ptr
+
     def _out(self, shape: Sequence[int], dtype=np.float32) -> HipTensor:
         n = int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize
         if self.scope is not None:
@@ -167,6 +189,7 @@ class HipOps:
             raise ValueError(f"Matrix multiplication shape mismatch: {a.shape} vs {b.shape}")
         m, k = a.shape
         n = b.shape[1]
+        self._live(a, b)
         out = self._out((m, n))
         if m and n:
             check(self._lib.skainet_hip_fp32_matmul_dev(a.ptr, 0, k, b.ptr, 0, n, out.ptr, 0, n, m, n, k), "matmul")
@@ -184,6 +207,7 @@ class HipOps:
         if not x.shape or x.shape[-1] != k:
             raise ValueError(f"matmulWeightTransposed shape mismatch: {x.shape} vs weight [{n}, {k}]")
         m = x.volume // k if k else 0
+        self._live(x, weight)
         out = self._out(x.shape[:-1] + (n,))
         if m and n:
             if isinstance(weight, HipTensor):
@@ -207,6 +231,7 @@ class HipOps:
     def _binary(self, op: str, a: HipTensor, b: HipTensor) -> HipTensor:
         shape = _broadcast_shape(a.shape, b.shape)
         am, bm = self._mode(a.shape, shape), self._mode(b.shape, shape)
+        self._live(a, b)
         out = self._out(shape)
         n = out.volume
         if n:
@@ -220,6 +245,7 @@ class HipOps:
 
     # ---- activations (WasmCpuOps.kt:281-312) -------------------------------------------------------------------------
     def _unary(self, op: str, t: HipTensor) -> HipTensor:
+        self._live(t)
         out = self._out(t.shape)
         if t.volume:
             kernels.unary_dev(op, t, out, t.volume)
@@ -234,6 +260,7 @@ class HipOps:
 
     # ---- reductions (WasmCpuOps.kt:316-348) --------------------------------------------------------------------------
     def _reduce(self, t: HipTensor, dim: Optional[int], mean: bool) -> HipTensor:
+        self._live(t)
         if dim is None:
             out = self._out(())
             kernels.reduce_all_dev(t, t.volume, out, mean)
@@ -259,6 +286,7 @@ class HipOps:
         if rank == 0 or dim % rank != rank - 1:
             raise ValueError("softmax runs over the last dimension")
         cols = t.shape[-1]
+        self._live(t)
         out = self._out(t.shape)
         if t.volume:
             kernels.softmax_rows_dev(t, out, t.volume // cols, cols, log)
@@ -268,19 +296,25 @@ class HipOps:
     def log_softmax(self, t, dim: int = -1): return self._softmax(t, dim, True)
 
     def rms_norm(self, x: HipTensor, gamma: Optional[HipTensor], eps: float) -> HipTensor:
+        if not x.shape:
+            raise ValueError("a norm needs a last dimension to run over")
         cols = x.shape[-1]
         if gamma is not None and gamma.volume != cols:
             raise ValueError(f"gamma of {gamma.shape} against rows of {cols}")
+        self._live(x, gamma)
         out = self._out(x.shape)
         if x.volume:
             kernels.rms_norm_dev(x, gamma, out, x.volume // cols, cols, eps)
         return out
 
     def layer_norm(self, x: HipTensor, gamma: Optional[HipTensor], beta: Optional[HipTensor], eps: float) -> HipTensor:
+        if not x.shape:
+            raise ValueError("a norm needs a last dimension to run over")
         cols = x.shape[-1]
         for name, p in (("gamma", gamma), ("beta", beta)):
             if p is not None and p.volume != cols:
                 raise ValueError(f"{name} of {p.shape} against rows of {cols}")
+        self._live(x, gamma, beta)
         out = self._out(x.shape)
         if x.volume:
             kernels.layer_norm_dev(x, gamma, beta, out, x.volume // cols, cols, eps)
@@ -302,6 +336,7 @@ class HipOps:
         skv = cap if seq_kv is None else int(seq_kv)
         if skv < 0 or skv > cap:
             raise ValueError(f"{skv} keys in caches of {cap} rows")
+        self._live(q, k, v, key_lengths)
         out = self._out(q.shape)
         if out.volume:
             kernels.sdpa_cache_dev(q, k, v, out, b, h, kvh, sq, skv, cap, d, float(scale if scale is not None else d ** -0.5),
@@ -313,6 +348,7 @@ class HipOps:
         """Rows `ids` ([count] int32, resident) of a packed embedding table, decoded to fp32 (the decode is the
         reference's, bit for bit: Q4_KTensorData.kt:133 and its siblings)."""
         count = ids.volume
+        self._live(ids)
         out = self._out((count, table.cols))
         check(self._lib.skainet_hip_dequantize_rows_dev(table._h, ids.ptr, count, out.ptr), "dequantize_rows")
         return out
@@ -330,6 +366,7 @@ class HipOps:
     def heads_to_rows(self, x: HipTensor) -> HipTensor:
         """[heads, tokens, head_dim] -> [tokens, heads * head_dim] (the reshape in front of the output projection)."""
         heads, tokens, hd = x.shape
+        self._live(x)
         out = self._out((tokens, heads * hd))
         kernels.heads_to_rows_dev(x, out, heads, tokens, hd)
         return out
@@ -337,6 +374,7 @@ class HipOps:
     def argmax_rows(self, t: HipTensor, out: Optional[HipTensor] = None) -> HipTensor:
         cols = t.shape[-1]
         rows = t.volume // cols
+        self._live(t, out)
         if out is None:
             out = self._out((rows,), np.int32)
         kernels.argmax_rows_dev(t, rows, cols, out)

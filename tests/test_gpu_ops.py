@@ -59,6 +59,37 @@ def test_elementwise_activations_and_reductions_stay_resident(ops):
     ops.scope.reset()
 
 
+def test_a_tensor_of_a_forward_scope_is_dead_after_the_reset(hip_backend):
+    """Per-step activations belong to their scope (Scope.kt:206-215: reset closes what was handed out, a later use
+    throws): a tensor, its views, and an op on it all raise after the reset; a tensor made after the reset lives at the
+    address the first one had; a tensor without a scope is not touched by any of it."""
+    from skainet_amd._lib import HipError
+    from skainet_amd.ops import ForwardScope, HipOps
+    scope = ForwardScope(1 << 20)
+    try:
+        o, free = HipOps(scope), HipOps()
+        keep = free.to_resident(np.arange(6, dtype=np.float32).reshape(2, 3))
+        t = o.to_resident(np.ones((4, 8), np.float32))
+        view = t.rows(1, 2).reshape(16)
+        first = t.ptr
+        assert o.add(t, t).numpy().sum() == 64.0
+        scope.reset()
+        for stale in (t, view):
+            with pytest.raises(HipError):
+                stale.numpy()
+        with pytest.raises(HipError):
+            o.relu(t)
+        again = o.to_resident(np.zeros((4, 8), np.float32))
+        assert again.ptr == first and again.numpy().sum() == 0.0
+        assert keep.numpy().tolist() == [[0.0, 1.0, 2.0], [3.0, 4.0, 5.0]]
+        with pytest.raises(HipError):
+            o.empty((1 << 20,))                                        # 4 MB out of a 1 MB slab
+    finally:
+        scope.close()
+    with pytest.raises(HipError):
+        again.numpy()                                                  # the scope is gone
+
+
 def test_softmax_norms_matmuls_and_attention(ops, hip_backend):
     rng = np.random.default_rng(2)
     x = rng.standard_normal((6, 50)).astype(np.float32) * 3
