@@ -33,12 +33,19 @@ typedef __bf16 frg_bf16x2 __attribute__((ext_vector_type(2)));
 typedef float frg_f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t frg_u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int FRG_M = 128, FRG_N = 64, FRG_WAVES = 8;
+constexpr int FRG_M = 128, FRG_N = 64;
 constexpr int FRG_SLOT = FRG_N * 144;                         // one raw super-block of the tile's 64 weight rows: 9 wave loads
 constexpr int FRG_RED_PITCH = FRG_N + 4;                      // floats per row of a partial tile in the final exchange
-constexpr size_t FRG_LOOP_BYTES = (size_t)FRG_WAVES * 2 * FRG_SLOT;
-constexpr size_t FRG_RED_BYTES = (size_t)4 * FRG_M * FRG_RED_PITCH * sizeof(float);
-constexpr size_t FRG_SMEM = FRG_LOOP_BYTES > FRG_RED_BYTES ? FRG_LOOP_BYTES : FRG_RED_BYTES;
+// Waves per workgroup: 8 (one workgroup per CU: the form for a weight whose tiles are one round over the chip) or 4 (two
+// workgroups per CU, for more tiles than CUs: while one of them is in its prologue, its exchange or its store -- phases
+// that use neither the matrix unit nor much of anything else -- the other is in its loop). LDS: the loop's rings (two
+// raw super-blocks per wave), reused by the final exchange: four whole partial tiles with 8 waves, four half tiles
+// (64 rows), twice, with 4.
+constexpr size_t frg_smem_bytes(int waves) {
+    const size_t loop = (size_t)waves * 2 * FRG_SLOT;
+    const size_t red = (size_t)4 * (waves == 8 ? FRG_M : FRG_M / 2) * FRG_RED_PITCH * sizeof(float);
+    return loop > red ? loop : red;
+}
 
 // Bytes of the fragment-ordered bf16 copy of an [m, k] activation matrix: row tiles of 32 padded up to whole workgroup
 // tiles of 128 rows (the padding rows are zeros).
@@ -228,7 +235,8 @@ __device__ __forceinline__ void frg_decode4(uint32_t c, uint32_t c8, float scale
     hi = __builtin_bit_cast(uint32_t, frg_bf16x2{(__bf16)w2, (__bf16)w3});
 }
 
-__global__ __launch_bounds__(64 * FRG_WAVES) void q4k_gemm_frag_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ w,
+template <int FRG_WAVES>
+__global__ __launch_bounds__(64 * FRG_WAVES, 2) void q4k_gemm_frag_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ w,
                                                                        float* c, const float* residual, int m, int n, int k, FrgTileOrder order) {
     extern __shared__ __attribute__((aligned(16))) uint8_t frg_smem[];   // the kernel has no other LDS: offsets into it are LDS addresses
     const int lane = threadIdx.x & 63;
@@ -391,51 +399,11 @@ __global__ __launch_bounds__(64 * FRG_WAVES) void q4k_gemm_frag_kernel(const uin
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // nothing of this wave still writes or reads its slots
     __syncthreads();
 
-    // The waves hold partial sums of the same 128 x 64 tile. Waves 4..7 park theirs in LDS and waves 0..3 add them to
-    // their own (same lane, same element: the addresses a lane reads are the ones its twin wrote); then waves 0..3 park
-    // the four remaining partial tiles and all eight waves add up a share of the rows and store it.
+    // The waves hold partial sums of the same 128 x 64 tile.
     // Accumulator element e of lane l: row 8 (e / 4) + 4 (l / 32) + e % 4, column l % 32 of its 32 x 32 tile.
     float* red = reinterpret_cast<float*>(frg_smem);
-    float* mine = red + (size_t)(wv & 3) * FRG_M * FRG_RED_PITCH;
-    auto tile_at = [&](int i, int j, int e) -> float& { return mine[(32 * i + 8 * (e >> 2) + 4 * kh + (e & 3)) * FRG_RED_PITCH + 32 * j + col]; };
-    if (wv >= 4) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
-    }
-    __syncthreads();
-    if (wv < 4) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] += tile_at(i, j, e);
-    }
-    __syncthreads();
-    if (wv < 4) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
-    }
-    __syncthreads();
     const int c4 = (lane & 15) * 4;
-    constexpr int ROWS_PER_WAVE = FRG_M / FRG_WAVES;
-#pragma unroll
-    for (int it = 0; it < ROWS_PER_WAVE / 4; ++it) {
-        const int row = ROWS_PER_WAVE * wv + 4 * it + (lane >> 4);
-        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const float4 t = *reinterpret_cast<const float4*>(red + ((size_t)v * FRG_M + row) * FRG_RED_PITCH + c4);
-            sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
-        }
+    auto store_row = [&](int row, float4 sum) __attribute__((always_inline)) {
         const int gr = m0 + row, gc = n0 + c4;
         if (gr < m) {
             // residual (may be c itself: every element is read and then written by this one thread): c = residual + product
@@ -451,6 +419,80 @@ __global__ __launch_bounds__(64 * FRG_WAVES) void q4k_gemm_frag_kernel(const uin
                 if (gc + 3 < n) dst[3] = (res ? res[3] : 0.f) + sum.w;
             }
         }
+    };
+    if constexpr (FRG_WAVES == 8) {
+        // Waves 4..7 park theirs in LDS and waves 0..3 add them to their own (same lane, same element: the addresses a
+        // lane reads are the ones its twin wrote); then waves 0..3 park the four remaining partial tiles and all eight
+        // waves add up a share of the rows and store it.
+        float* mine = red + (size_t)(wv & 3) * FRG_M * FRG_RED_PITCH;
+        auto tile_at = [&](int i, int j, int e) -> float& { return mine[(32 * i + 8 * (e >> 2) + 4 * kh + (e & 3)) * FRG_RED_PITCH + 32 * j + col]; };
+        if (wv >= 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
+        }
+        __syncthreads();
+        if (wv < 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[i][j][e] += tile_at(i, j, e);
+        }
+        __syncthreads();
+        if (wv < 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) tile_at(i, j, e) = acc[i][j][e];
+        }
+        __syncthreads();
+        constexpr int ROWS_PER_WAVE = FRG_M / 8;
+#pragma unroll
+        for (int it = 0; it < ROWS_PER_WAVE / 4; ++it) {
+            const int row = ROWS_PER_WAVE * wv + 4 * it + (lane >> 4);
+            float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float4 t = *reinterpret_cast<const float4*>(red + ((size_t)v * FRG_M + row) * FRG_RED_PITCH + c4);
+                sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+            }
+            store_row(row, sum);
+        }
+    } else {
+        // Four waves: the upper and the lower 64 rows in turn. Every wave parks its half tile, then adds up the four
+        // halves for its 16 of the 64 rows and stores them.
+        constexpr int HALF = FRG_M / 2;
+        float* mine = red + (size_t)wv * HALF * FRG_RED_PITCH;
+#pragma unroll
+        for (int ph = 0; ph < 2; ++ph) {
+            if (ph == 1) __syncthreads();                        // the first half's sums have been read
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        mine[(32 * ii + 8 * (e >> 2) + 4 * kh + (e & 3)) * FRG_RED_PITCH + 32 * j + col] = acc[2 * ph + ii][j][e];
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int row = 16 * wv + 4 * it + (lane >> 4);      // of the half
+                float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float4 t = *reinterpret_cast<const float4*>(red + ((size_t)v * HALF + row) * FRG_RED_PITCH + c4);
+                    sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+                }
+                store_row(HALF * ph + row, sum);
+            }
+        }
     }
 }
 
@@ -464,8 +506,11 @@ bool gemm_frag_fits(int m, int n, int k) {
 
 // row tiles per group of the tile order: a die's share of the tiles is gm row tiles x (share / gm) column tiles and
 // its L2 fetches 256 gm + 36 share / gm bytes per element of K -- take the divisor of tiles_m with the least
+static std::atomic<int> g_gemm_frag_gm{0};      // row tiles per group of the tile order: 0 = by the cost below, else forced (a divisor of the row-tile count)
+void set_gemm_frag_gm(int v) { if (v >= 0 && v <= 8) g_gemm_frag_gm = v; }
 static FrgTileOrder frg_tile_order(int m, int n) {
     FrgTileOrder o{1, (m + FRG_M - 1) / FRG_M, (n + FRG_N - 1) / FRG_N};
+    if (const int forced = g_gemm_frag_gm.load(); forced > 0 && o.tiles_m % forced == 0) { o.gm = forced; return o; }
     const double share = (double)o.tiles_m * o.tiles_n / 8.0;
     double best = 0.0;
     for (int g = 1; g <= o.tiles_m && g <= 8; ++g) {
@@ -480,6 +525,8 @@ static FrgTileOrder frg_tile_order(int m, int n) {
 // (gemm_frag_activation_bytes(m, k) bytes); gain != null folds an RMSNorm in (k <= 16384).
 static std::atomic<int> g_gemm_frag_touch{1};   // the pass in front touches the weight's lines (0: it does not)
 void set_gemm_frag_touch(int v) { g_gemm_frag_touch = v != 0; }
+static std::atomic<int> g_gemm_frag_waves{0};   // waves per workgroup of the product: 0 = 8 for one round of tiles, 4 (two workgroups per CU) for more; else 4 or 8
+void set_gemm_frag_waves(int v) { if (v == 0 || v == 4 || v == 8) g_gemm_frag_waves = v; }
 static std::atomic<int> g_gemm_frag_pieces{1};  // 64-element groups a workgroup of the plain pass takes (1, 2 or 4)
 void set_gemm_frag_pieces(int v) { if (v == 1 || v == 2 || v == 4) g_gemm_frag_pieces = v; }
 // `w` ([n, k] packed Q4_K, or null) is the weight of the product that follows: the plain pass touches its lines on the way.
@@ -512,8 +559,15 @@ int launch_q4k_gemm_frag(const uint8_t* a, const uint8_t* w, float* c, int m, in
     if (!gemm_frag_fits(m, n, k)) return set_error("gemm: operands of %d x %d x %d are outside this kernel's range", m, n, k);
     const FrgTileOrder order = frg_tile_order(m, n);
     note_kernel("q4k_gemm_frag_kernel");
-    SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_frag_kernel), FRG_SMEM);
-    q4k_gemm_frag_kernel<<<dim3(order.tiles_m * order.tiles_n), dim3(64 * FRG_WAVES), FRG_SMEM, s>>>(a, w, c, residual, m, n, k, order);
+    const int tiles = order.tiles_m * order.tiles_n;
+    const int waves = g_gemm_frag_waves.load() != 0 ? g_gemm_frag_waves.load() : (tiles > num_cus() ? 4 : 8);
+    if (waves == 4) {
+        SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_frag_kernel<4>), frg_smem_bytes(4));
+        q4k_gemm_frag_kernel<4><<<dim3(tiles), dim3(256), frg_smem_bytes(4), s>>>(a, w, c, residual, m, n, k, order);
+    } else {
+        SKH_SET_MAX_DYNAMIC_LDS_ONCE((&q4k_gemm_frag_kernel<8>), frg_smem_bytes(8));
+        q4k_gemm_frag_kernel<8><<<dim3(tiles), dim3(512), frg_smem_bytes(8), s>>>(a, w, c, residual, m, n, k, order);
+    }
     SKH_CHECK(hipGetLastError());
     return 0;
 }

@@ -170,6 +170,8 @@ void set_gemm_ksw_stages(int v);
 void set_gemm_frag(int v);
 void set_gemm_frag_touch(int v);
 void set_gemm_frag_pieces(int v);
+void set_gemm_frag_waves(int v);
+void set_gemm_frag_gm(int v);
 void set_sdpa_prefill_mfma(int v);
 void set_sdpa_prefill_teams(int v);
 void set_sdpa_decode_split_keys(int v);
@@ -213,6 +215,8 @@ int set_tuning(const char* key, int value) {
     if (!strcmp(key, "gemm_frag")) { set_gemm_frag(value); return 0; }
     if (!strcmp(key, "gemm_frag_touch")) { set_gemm_frag_touch(value); return 0; }
     if (!strcmp(key, "gemm_frag_pieces")) { set_gemm_frag_pieces(value); return 0; }
+    if (!strcmp(key, "gemm_frag_waves")) { set_gemm_frag_waves(value); return 0; }
+    if (!strcmp(key, "gemm_frag_gm")) { set_gemm_frag_gm(value); return 0; }
     if (!strcmp(key, "sdpa_prefill_mfma")) { set_sdpa_prefill_mfma(value); return 0; }
     if (!strcmp(key, "sdpa_prefill_teams")) { set_sdpa_prefill_teams(value); return 0; }
     if (!strcmp(key, "q4k_ksplit_enable")) { set_q4k_ksplit_enable(value); return 0; }

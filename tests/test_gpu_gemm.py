@@ -168,7 +168,8 @@ def test_q4k_gemm_with_k_split_over_the_waves(hip_backend, torch_cuda, m, n, k):
                                    (257, 63, 768), (64, 512, 11008), (384, 1024, 4096)])
 def test_q4k_gemm_with_activations_in_fragment_order(hip_backend, torch_cuda, m, n, k):
     """The Q4_K kernel whose activations are laid out by the pass in front in the order the matrix instruction reads them
-    (every wave: the whole 128 x 64 tile and whole super-blocks of K), forced on shapes with ragged row and column tiles,
+    (every wave: the whole 128 x 64 tile and whole super-blocks of K), in both of its forms (eight waves per workgroup,
+    and four with two workgroups per CU), forced on shapes with ragged row and column tiles,
     fewer super-blocks than waves, uneven super-block counts per wave (43 and 56 super-blocks over 8 waves), tile counts
     that are and are not a multiple of the eight dies; against the oracle (2e-2), against the same product with both
     operands rounded to bf16 first (2e-4), and against the tile kernel."""
@@ -177,11 +178,13 @@ def test_q4k_gemm_with_activations_in_fragment_order(hip_backend, torch_cuda, m,
     want = L.gemv("Q4_K", x, packed, n)
     try:
         hip_backend.set_tuning("gemm_frag", 2)
-        got = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
-        assert hip_backend.last_kernel() == "q4k_gemm_frag_kernel"
-        assert not np.isnan(got).any()
-        check(got, want)
-        check_exact(torch_cuda, "Q4_K", got, x, packed, n)
+        for waves in (8, 4):                       # one workgroup of eight waves per CU, or two of four
+            hip_backend.set_tuning("gemm_frag_waves", waves)
+            got = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
+            assert hip_backend.last_kernel() == "q4k_gemm_frag_kernel"
+            assert not np.isnan(got).any()
+            check(got, want)
+            check_exact(torch_cuda, "Q4_K", got, x, packed, n)
         hip_backend.set_tuning("gemm_frag", 0)
         hip_backend.set_tuning("gemm_ksw", 0)
         tiles = gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
@@ -189,6 +192,7 @@ def test_q4k_gemm_with_activations_in_fragment_order(hip_backend, torch_cuda, m,
         assert normalized_err(got, tiles) <= 1e-4          # same operands, another fp32 summation order
     finally:
         hip_backend.set_tuning("gemm_frag", 1)
+        hip_backend.set_tuning("gemm_frag_waves", 0)
         hip_backend.set_tuning("gemm_ksw", 1)
     if (m, n, k) == (512, 4096, 4096):
         gpu_gemm(hip_backend, torch_cuda, "Q4_K", packed, n, k, x)
