@@ -434,7 +434,15 @@ SKAINET_HIP_API void skainet_hip_graph_free(skainet_hip_graph* graph);
  * waves of a workgroup: 0 never, 1 where the launcher's estimate favours it, 2 wherever it fits), "gemm_ksw_teams" (teams
  * of four waves per workgroup of that kernel, each with its own share of K: 1 or 2, default 2; rows with an odd number
  * of 256-element super-blocks always run one team), "gemm_ksw_stages" (activation tiles the one-team form keeps in LDS: 3 to 7,
- * default 5),
+ * default 5), "gemm_frag" (the Q4_K kernel that reads its activations in matrix-fragment order: 0 never, 1 where the
+ * launcher's estimate favours it, 2 wherever it fits), "gemm_frag_waves" (waves per workgroup of that kernel: 8 = one
+ * workgroup per CU, 4 = two, 0 = eight for one round of tiles and four for more), "gemm_frag_gm" (row tiles per group of
+ * its tile order, 0 = by the launcher's traffic estimate), "gemm_frag_touch" (0: the pass in front of it does not touch the
+ * weight's lines), "gemm_frag_pieces" (64-element groups a workgroup of that pass takes: 1, 2 or 4),
+ * "q4k_wide_enable" (0: Q4_K products of 5 to 8 rows at K = 4096 stay on the 4 x 4 x 4 matrix-instruction kernel instead of
+ * the 16 x 16 x 32 one), "q4k_wide_min_batch" (fewest rows that kernel takes: 3 to 8, default 5), "q8_0_mfma_enable" (0:
+ * one-row Q8_0 products stay off the integer matrix cores), "q8_0_mfma_per_cu" (workgroups per CU of that kernel: 1, 2
+ * or 4, default 2),
  * "sdpa_prefill_mfma" (0: prompt-shape attention on the fp32 kernel), "sdpa_prefill_teams" (query groups per workgroup of
  * the matrix-core prompt kernel: 1, 2 = a late and an early group paired, 0 = paired where that still fills the chip), "sdpa_decode_split_keys" (least keys per split of
  * decode-shape attention, default 64), "sdpa_decode_gs" (query heads per workgroup of decode-shape attention: 1, 2 or 4, 0 = chosen from
