@@ -96,6 +96,27 @@ internal object HipLibrary {
     val reduceAllDev: MethodHandle? = bind("skainet_hip_f32_reduce_all_dev", FunctionDescriptor.of(I, P, L, I, P))
     val reduceAxisDev: MethodHandle? = bind("skainet_hip_f32_reduce_axis_dev", FunctionDescriptor.of(I, P, I, I, I, I, P))
 
+    // ---- fused device entries a decoder runtime on resident activations calls (no counterpart in the CPU library)
+    /** (w, x, m, out, gain, eps, residual, epilogue): epilogue 0 none, 1 += residual, 2 SwiGLU over interleaved (gate, up) rows */
+    val matmulFusedDev: MethodHandle? = bind("skainet_hip_matmul_fused_dev", FunctionDescriptor.of(I, P, P, I, P, P, F, P, I))
+    /** (w_gate_up, w_down, x, m, gain, eps, residual, out): out = residual + Wdown . swiglu(Wgate_up . rmsnorm(x)) */
+    val mlpSwigluDev: MethodHandle? = bind("skainet_hip_mlp_swiglu_dev", FunctionDescriptor.of(I, P, P, P, I, P, F, P, P))
+    /** attention over a [kvHeads, capacity, headDim] cache, output head-major / as token rows */
+    val sdpaCacheDev: MethodHandle? = bind(
+        "skainet_hip_f32_sdpa_cache_dev",
+        FunctionDescriptor.of(I, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P),
+    )
+    val sdpaCacheRowsDev: MethodHandle? = bind(
+        "skainet_hip_f32_sdpa_cache_rows_dev",
+        FunctionDescriptor.of(I, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P),
+    )
+    /** one decode token's attention + output projection (+ residual) */
+    val attnOutProjDev: MethodHandle? = bind(
+        "skainet_hip_attn_out_proj_dev",
+        FunctionDescriptor.of(I, P, P, P, P, I, I, I, I, I, F, I, P, P, P, P),
+    )
+    val argmaxRowsDev: MethodHandle? = bind("skainet_hip_f32_argmax_rows_dev", FunctionDescriptor.of(I, P, I, I, P))
+
     /** Cheap, cached, false (not throwing) when the library or a gfx950 device is missing. */
     val usable: Boolean by lazy {
         runCatching {
